@@ -1,0 +1,91 @@
+"""ctypes binding of libaccera_mi355x.so (the C ABI declared in include/accera_mi355x_gemm.h).
+
+There is no CPU fallback: if the shared library is missing, loading raises with the
+build command; if a call fails, the library's own error text is raised.
+"""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_DIR = os.path.join(_HERE, "lib")
+LIB_PATH = os.path.join(LIB_DIR, "libaccera_mi355x.so")
+INCLUDE_DIR = os.path.join(os.path.dirname(_HERE), "include")
+
+# element types / ops / status codes / variant ids (accera_mi355x_gemm.h)
+F32, F16, BF16, I8, I32 = 0, 1, 2, 3, 4
+PROLOGUE_NONE, PROLOGUE_SET0 = 0, 1
+EPILOGUE_NONE, EPILOGUE_RELU, EPILOGUE_RELU_NOCOND = 0, 1, 2
+OK, INVALID_ARGUMENT, UNSUPPORTED, HIP_ERROR = 0, 1, 2, 3
+VARIANT_AUTO, VARIANT_SKINNY_BASE, VARIANT_GENERIC, VARIANT_F32_MFMA = -1, 100, 200, 201
+
+EXPORTS = [
+    "acc950_init", "acc950_gemm_relu", "acc950_gemm_relu_ex", "acc950_gemm_relu_host",
+    "acc950_launch_geometry", "acc950_num_variants", "acc950_num_skinny_variants",
+    "acc950_variant_name", "acc950_last_error",
+]
+
+
+class Acc950Error(RuntimeError):
+    def __init__(self, code, message):
+        super().__init__(f"acc950 status {code}: {message}")
+        self.code = code
+
+
+_lib = None
+
+
+def lib():
+    """The loaded library (loads it on first use)."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            f"{LIB_PATH} is missing: build it with `python -c 'import __graft_entry__ as g; g.build()'` "
+            f"(or `make -C accera_amd/csrc`). There is no CPU fallback.")
+    L = ctypes.CDLL(LIB_PATH, mode=ctypes.RTLD_GLOBAL)
+    ci, i64, vp, cu = ctypes.c_int, ctypes.c_int64, ctypes.c_void_p, ctypes.c_uint
+    mat = [vp, i64, i64]
+    L.acc950_init.argtypes = [ci]
+    L.acc950_gemm_relu.argtypes = [ci, ci, ci, ci, ci] + mat * 3 + [ci, ci, vp]
+    L.acc950_gemm_relu_ex.argtypes = [ci, ci, ci, ci, ci] + mat * 3 + [ci, ci, ci, ci, vp]
+    L.acc950_gemm_relu_host.argtypes = [ci, ci, ci, ci, ci] + mat * 3 + [ci, ci]
+    L.acc950_launch_geometry.argtypes = [ci, ci, ci, ci, ci] + [i64] * 6 + [ci, ci, ctypes.POINTER(cu), ctypes.POINTER(cu),
+                                                                           ctypes.POINTER(cu), ctypes.POINTER(ci)]
+    L.acc950_variant_name.argtypes = [ci, ctypes.c_char_p, ctypes.c_size_t]
+    L.acc950_last_error.restype = ctypes.c_char_p
+    for name in EXPORTS:
+        if name != "acc950_last_error":
+            getattr(L, name).restype = ci
+    _lib = L
+    return L
+
+
+def check(rc):
+    if rc != OK:
+        raise Acc950Error(rc, lib().acc950_last_error().decode())
+
+
+def variant_name(variant):
+    buf = ctypes.create_string_buffer(128)
+    check(lib().acc950_variant_name(int(variant), buf, 128))
+    return buf.value.decode()
+
+
+def num_variants():
+    return lib().acc950_num_variants()
+
+
+def num_skinny_variants():
+    return lib().acc950_num_skinny_variants()
+
+
+def launch_geometry(in_type, out_type, M, N, K, a_strides, b_strides, c_strides, variant=VARIANT_AUTO, k_splits=0):
+    """(grid, block, dynamic_lds_bytes, chosen_variant) of the kernel a call would launch."""
+    grid = (ctypes.c_uint * 3)()
+    block = (ctypes.c_uint * 3)()
+    lds = ctypes.c_uint()
+    chosen = ctypes.c_int()
+    check(lib().acc950_launch_geometry(in_type, out_type, M, N, K, *a_strides, *b_strides, *c_strides, variant, k_splits,
+                                       grid, block, ctypes.byref(lds), ctypes.byref(chosen)))
+    return list(grid), list(block), lds.value, chosen.value

@@ -1,0 +1,417 @@
+// C ABI of the library (include/accera_mi355x_gemm.h): argument checking, kernel
+// selection, the host-pointer path and the launch-geometry query.
+#include "../../include/accera_mi355x_gemm.h"
+#include "common.h"
+#include "skinny.h"
+#include "variants.h"
+
+#include <cstdio>
+#include <cstring>
+#include <mutex>
+#include <string>
+
+using namespace acc950;
+
+namespace {
+
+thread_local std::string t_last_error;
+
+int fail(int code, const std::string& msg)
+{
+    t_last_error = msg;
+    return code;
+}
+int fail_hip(hipError_t e, const char* what)
+{
+    return fail(ACC950_HIP_ERROR, std::string(what) + ": " + hipGetErrorString(e));
+}
+
+int elem_size(int t)
+{
+    switch (t) {
+    case T_F32: case T_I32: return 4;
+    case T_F16: case T_BF16: return 2;
+    case T_I8: return 1;
+    default: return 0;
+    }
+}
+
+bool type_pair_ok(int in, int out)
+{
+    if (in == T_I8) return out == T_I32;
+    if (in == T_F32) return out == T_F32;
+    if (in == T_F16 || in == T_BF16) return out == T_F32 || out == T_F16 || out == T_BF16;
+    return false;
+}
+
+const MfmaVariant* mfma_table(int in_type, int* n)
+{
+    switch (in_type) {
+    case T_F16: return mfma_variants_f16(n);
+    case T_BF16: return mfma_variants_bf16(n);
+    case T_I8: return mfma_variants_i8(n);
+    default: *n = 0; return nullptr;
+    }
+}
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// Problem after validation; C is made row-major by computing the transposed product
+// C^T = B^T * A^T when the caller's C is column-major.
+struct Problem {
+    GemmArgs g;
+    bool have_pointers;
+};
+
+int make_problem(int in_type, int out_type, int M, int N, int K,
+                 const void* A, int64_t a_rs, int64_t a_cs, const void* B, int64_t b_rs, int64_t b_cs,
+                 void* C, int64_t c_rs, int64_t c_cs, int prologue, int epilogue, bool need_pointers, Problem* out)
+{
+    if (!type_pair_ok(in_type, out_type)) return fail(ACC950_INVALID_ARGUMENT, "unsupported input/output element type pair");
+    if (M < 0 || N < 0 || K < 0) return fail(ACC950_INVALID_ARGUMENT, "negative matrix dimension");
+    if (a_rs < 0 || a_cs < 0 || b_rs < 0 || b_cs < 0 || c_rs < 0 || c_cs < 0)
+        return fail(ACC950_INVALID_ARGUMENT, "negative strides are not supported");
+    if (prologue != PRO_NONE && prologue != PRO_SET0) return fail(ACC950_INVALID_ARGUMENT, "unknown prologue op");
+    if (epilogue != EPI_NONE && epilogue != EPI_RELU && epilogue != EPI_RELU_NOCOND)
+        return fail(ACC950_INVALID_ARGUMENT, "unknown epilogue op");
+    if (need_pointers && M > 0 && N > 0 && (!C || (K > 0 && (!A || !B))))
+        return fail(ACC950_INVALID_ARGUMENT, "null matrix pointer");
+    GemmArgs g{};
+    g.in_type = in_type; g.out_type = out_type;
+    g.prologue = prologue; g.epilogue = epilogue;
+    const bool transpose = c_cs != 1 && c_rs == 1 && N > 1;
+    if (!transpose) {
+        g.A = A; g.B = B; g.C = C; g.M = M; g.N = N; g.K = K;
+        g.a_rs = a_rs; g.a_cs = a_cs; g.b_rs = b_rs; g.b_cs = b_cs; g.c_rs = c_rs; g.c_cs = c_cs;
+    } else {
+        g.A = B; g.B = A; g.C = C; g.M = N; g.N = M; g.K = K;
+        g.a_rs = b_cs; g.a_cs = b_rs; g.b_rs = a_cs; g.b_cs = a_rs; g.c_rs = c_cs; g.c_cs = c_rs;
+    }
+    out->g = g;
+    out->have_pointers = need_pointers;
+    return ACC950_OK;
+}
+
+// ---- eligibility ------------------------------------------------------------------
+
+bool mfma_can_take(const MfmaVariant& v, const Problem& pb)
+{
+    const GemmArgs& g = pb.g;
+    if (g.M <= 0 || g.N <= 0 || g.K <= 0) return false;
+    const int es = elem_size(g.in_type), vec = 16 / es, bk = 128 / es;
+    if (g.a_cs != 1 || g.c_cs != 1) return false; // A row-major (K contiguous), C row-major
+    if (v.b_kc ? g.b_rs != 1 : g.b_cs != 1) return false;
+    const int64_t lda = g.a_rs, ldb = v.b_kc ? g.b_cs : g.b_rs;
+    if (lda % vec || ldb % vec) return false;
+    if (pb.have_pointers && (!aligned16(g.A) || !aligned16(g.B))) return false;
+    if (v.edge) {
+        if (g.K % vec) return false;
+        if (!v.b_kc && g.N % vec) return false;
+    } else {
+        if (g.M % v.bm || g.N % v.bn || g.K % bk) return false;
+    }
+    // per-lane global offsets of the direct fill are 32-bit
+    if ((int64_t)v.bm * lda * es >= (1ll << 31) || (int64_t)(v.b_kc ? v.bn : bk) * ldb * es >= (1ll << 31)) return false;
+    return true;
+}
+
+bool skinny_can_take(const Problem& pb)
+{
+    const GemmArgs& g = pb.g;
+    if (g.in_type != T_F16 && g.in_type != T_BF16) return false;
+    if (g.M < 1 || g.M > 8 || g.N < 8 || g.K < 2) return false;
+    if (g.a_cs != 1 || g.b_cs != 1 || g.c_cs != 1) return false;
+    if (g.N % 8 || g.K % 2 || g.b_rs % 8 || g.a_rs % 2) return false;
+    if (pb.have_pointers && (!aligned16(g.B) || (reinterpret_cast<uintptr_t>(g.A) & 3u))) return false;
+    return true;
+}
+
+// ---- scratch for the skinny kernels' K split -----------------------------------------
+std::mutex g_ws_mutex;
+float* g_scratch = nullptr;
+size_t g_scratch_floats = 0;
+unsigned* g_counters = nullptr;
+size_t g_counters_n = 0;
+
+hipError_t ensure_workspace(size_t floats, size_t counters)
+{
+    std::lock_guard<std::mutex> lock(g_ws_mutex);
+    if (floats > g_scratch_floats) {
+        if (g_scratch) { hipError_t e = hipFree(g_scratch); if (e != hipSuccess) return e; g_scratch = nullptr; g_scratch_floats = 0; }
+        size_t want = floats < (1u << 20) ? (1u << 20) : floats;
+        hipError_t e = hipMalloc((void**)&g_scratch, want * sizeof(float));
+        if (e != hipSuccess) return e;
+        g_scratch_floats = want;
+    }
+    if (counters > g_counters_n) {
+        if (g_counters) { hipError_t e = hipFree(g_counters); if (e != hipSuccess) return e; g_counters = nullptr; g_counters_n = 0; }
+        size_t want = counters < 4096 ? 4096 : counters;
+        hipError_t e = hipMalloc((void**)&g_counters, want * sizeof(unsigned));
+        if (e != hipSuccess) return e;
+        e = hipMemset(g_counters, 0, want * sizeof(unsigned));
+        if (e != hipSuccess) return e;
+        g_counters_n = want;
+    }
+    return hipSuccess;
+}
+
+int auto_skinny_variant(const GemmArgs&) { return 0; }
+
+int auto_skinny_splits(int variant, const GemmArgs& g)
+{
+    // enough workgroups to cover 256 CUs several times over, at least 128 k rows each
+    const int blocks = skinny_column_blocks(variant, g.N);
+    int splits = (2048 + blocks - 1) / blocks;
+    const int max_splits = g.K / 128 > 0 ? g.K / 128 : 1;
+    if (splits > max_splits) splits = max_splits;
+    if (splits < 1) splits = 1;
+    return splits;
+}
+
+// Preference order of MFMA tiles for the automatic choice: biggest tile that still
+// yields at least ~one workgroup per CU, else smaller tiles, else the edge kernel.
+int auto_mfma_variant(const Problem& pb)
+{
+    int n = 0;
+    const MfmaVariant* tab = mfma_table(pb.g.in_type, &n);
+    if (!tab) return -1;
+    struct Want { int bm, bn, wm, wn; bool direct, edge; };
+    const int64_t tiles256 = ((int64_t)pb.g.M / 256) * (pb.g.N / 256);
+    const Want big = {256, 256, 2, 2, true, false}, mid = {256, 128, 2, 2, true, false},
+               small = {128, 128, 2, 2, true, false}, edge = {128, 128, 2, 2, false, true};
+    Want order[4];
+    if (tiles256 >= 200) { order[0] = big; order[1] = mid; order[2] = small; }
+    else { order[0] = small; order[1] = mid; order[2] = big; }
+    order[3] = edge;
+    for (const Want& w : order)
+        for (int i = 0; i < n; ++i) {
+            const MfmaVariant& v = tab[i];
+            if (v.bm == w.bm && v.bn == w.bn && v.waves_m == w.wm && v.waves_n == w.wn && v.direct == w.direct &&
+                v.edge == w.edge && mfma_can_take(v, pb))
+                return i;
+        }
+    return -1;
+}
+
+struct Choice {
+    int variant;
+    int splits;
+};
+
+int choose(const Problem& pb, int variant, int k_splits, Choice* c)
+{
+    c->splits = 1;
+    if (variant == ACC950_VARIANT_AUTO) {
+        if (skinny_can_take(pb)) {
+            int sv = auto_skinny_variant(pb.g);
+            c->variant = ACC950_VARIANT_SKINNY_BASE + sv;
+            c->splits = k_splits > 0 ? k_splits : auto_skinny_splits(sv, pb.g);
+            return ACC950_OK;
+        }
+        if (f32_can_take(pb.g)) { c->variant = ACC950_VARIANT_F32_MFMA; return ACC950_OK; }
+        int mv = auto_mfma_variant(pb);
+        c->variant = mv >= 0 ? mv : ACC950_VARIANT_GENERIC;
+        return ACC950_OK;
+    }
+    if (variant == ACC950_VARIANT_GENERIC) { c->variant = variant; return ACC950_OK; }
+    if (variant == ACC950_VARIANT_F32_MFMA) {
+        if (!f32_can_take(pb.g)) return fail(ACC950_UNSUPPORTED, "the fp32 MFMA kernel needs fp32 inputs and K > 0");
+        c->variant = variant;
+        return ACC950_OK;
+    }
+    if (variant >= ACC950_VARIANT_SKINNY_BASE && variant < ACC950_VARIANT_SKINNY_BASE + skinny_num_variants()) {
+        if (!skinny_can_take(pb)) return fail(ACC950_UNSUPPORTED, "skinny kernel needs 16-bit inputs, M <= 8, row-major A/B/C, N % 8 == 0, K % 2 == 0");
+        c->variant = variant;
+        c->splits = k_splits > 0 ? k_splits : auto_skinny_splits(variant - ACC950_VARIANT_SKINNY_BASE, pb.g);
+        if (c->splits > pb.g.K / 2) c->splits = pb.g.K / 2;
+        return ACC950_OK;
+    }
+    int n = 0;
+    const MfmaVariant* tab = mfma_table(pb.g.in_type, &n);
+    if (variant < 0 || variant >= n) return fail(ACC950_INVALID_ARGUMENT, "unknown kernel variant");
+    if (!mfma_can_take(tab[variant], pb)) return fail(ACC950_UNSUPPORTED, "MFMA variant cannot take this shape / layout / alignment");
+    c->variant = variant;
+    return ACC950_OK;
+}
+
+int run(const Problem& pb, const Choice& c, hipStream_t stream, LaunchGeom* geom, bool dry_run)
+{
+    const GemmArgs& g = pb.g;
+    if (g.M == 0 || g.N == 0) {
+        if (geom) std::memset(geom, 0, sizeof(*geom));
+        return ACC950_OK;
+    }
+    hipError_t e;
+    if (c.variant == ACC950_VARIANT_GENERIC) {
+        e = launch_generic(g, stream, geom, dry_run);
+    } else if (c.variant == ACC950_VARIANT_F32_MFMA) {
+        e = launch_f32(g, stream, geom, dry_run);
+    } else if (c.variant >= ACC950_VARIANT_SKINNY_BASE) {
+        const int sv = c.variant - ACC950_VARIANT_SKINNY_BASE;
+        SkinnyArgs s{};
+        s.A = g.A; s.B = g.B; s.C = g.C; s.M = g.M; s.N = g.N; s.K = g.K;
+        s.a_rs = g.a_rs; s.b_rs = g.b_rs; s.c_rs = g.c_rs;
+        s.in_type = g.in_type; s.out_type = g.out_type; s.prologue = g.prologue; s.epilogue = g.epilogue;
+        s.splits = c.splits;
+        if (!dry_run && c.splits > 1) {
+            e = ensure_workspace(skinny_scratch_floats(sv, g.N, c.splits), (size_t)skinny_column_blocks(sv, g.N));
+            if (e != hipSuccess) return fail_hip(e, "workspace allocation");
+            s.scratch = g_scratch;
+            s.counters = g_counters;
+        }
+        e = launch_skinny(sv, s, stream, geom, dry_run);
+    } else {
+        int n = 0;
+        const MfmaVariant* tab = mfma_table(g.in_type, &n);
+        e = tab[c.variant].launch(g, stream, geom, dry_run);
+    }
+    if (e != hipSuccess) return fail_hip(e, "kernel launch");
+    return ACC950_OK;
+}
+
+// ---- device buffers of the host-pointer path (grow-only, one set per process) --------
+std::mutex g_host_mutex;
+struct DevBuf { void* p = nullptr; size_t bytes = 0; } g_dA, g_dB, g_dC;
+
+hipError_t reserve(DevBuf& b, size_t bytes)
+{
+    if (bytes <= b.bytes) return hipSuccess;
+    if (b.p) { hipError_t e = hipFree(b.p); if (e != hipSuccess) return e; b.p = nullptr; b.bytes = 0; }
+    hipError_t e = hipMalloc(&b.p, bytes);
+    if (e == hipSuccess) b.bytes = bytes;
+    return e;
+}
+
+size_t extent_elems(int rows, int cols, int64_t rs, int64_t cs)
+{
+    if (rows <= 0 || cols <= 0) return 0;
+    return (size_t)(1 + (int64_t)(rows - 1) * rs + (int64_t)(cols - 1) * cs);
+}
+
+} // namespace
+
+extern "C" {
+
+const char* acc950_last_error(void) { return t_last_error.c_str(); }
+
+int acc950_init(int device_id)
+{
+    hipError_t e = hipSetDevice(device_id);
+    if (e != hipSuccess) return fail_hip(e, "hipSetDevice");
+    hipDeviceProp_t prop;
+    e = hipGetDeviceProperties(&prop, device_id);
+    if (e != hipSuccess) return fail_hip(e, "hipGetDeviceProperties");
+    if (std::strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+        return fail(ACC950_UNSUPPORTED, std::string("this library is built for gfx950 only, device is ") + prop.gcnArchName);
+    return ACC950_OK;
+}
+
+int acc950_gemm_relu_ex(int in_type, int out_type, int M, int N, int K,
+                        const void* A, int64_t a_rs, int64_t a_cs, const void* B, int64_t b_rs, int64_t b_cs,
+                        void* C, int64_t c_rs, int64_t c_cs, int prologue, int epilogue, int variant, int k_splits,
+                        void* stream)
+{
+    Problem pb;
+    int rc = make_problem(in_type, out_type, M, N, K, A, a_rs, a_cs, B, b_rs, b_cs, C, c_rs, c_cs, prologue, epilogue, true, &pb);
+    if (rc) return rc;
+    Choice c;
+    rc = choose(pb, variant, k_splits, &c);
+    if (rc) return rc;
+    return run(pb, c, (hipStream_t)stream, nullptr, false);
+}
+
+int acc950_gemm_relu(int in_type, int out_type, int M, int N, int K,
+                     const void* A, int64_t a_rs, int64_t a_cs, const void* B, int64_t b_rs, int64_t b_cs,
+                     void* C, int64_t c_rs, int64_t c_cs, int prologue, int epilogue, void* stream)
+{
+    return acc950_gemm_relu_ex(in_type, out_type, M, N, K, A, a_rs, a_cs, B, b_rs, b_cs, C, c_rs, c_cs, prologue, epilogue,
+                               ACC950_VARIANT_AUTO, 0, stream);
+}
+
+int acc950_launch_geometry(int in_type, int out_type, int M, int N, int K,
+                           int64_t a_rs, int64_t a_cs, int64_t b_rs, int64_t b_cs, int64_t c_rs, int64_t c_cs,
+                           int variant, int k_splits, unsigned grid[3], unsigned block[3], unsigned* dyn_lds, int* chosen)
+{
+    Problem pb;
+    int rc = make_problem(in_type, out_type, M, N, K, nullptr, a_rs, a_cs, nullptr, b_rs, b_cs, nullptr, c_rs, c_cs,
+                          PRO_SET0, EPI_NONE, false, &pb);
+    if (rc) return rc;
+    Choice c;
+    rc = choose(pb, variant, k_splits, &c);
+    if (rc) return rc;
+    LaunchGeom geom{};
+    rc = run(pb, c, nullptr, &geom, true);
+    if (rc) return rc;
+    for (int i = 0; i < 3; ++i) { if (grid) grid[i] = geom.grid[i]; if (block) block[i] = geom.block[i]; }
+    if (dyn_lds) *dyn_lds = geom.dyn_lds;
+    if (chosen) *chosen = c.variant;
+    return ACC950_OK;
+}
+
+int acc950_gemm_relu_host(int in_type, int out_type, int M, int N, int K,
+                          const void* A, int64_t a_rs, int64_t a_cs, const void* B, int64_t b_rs, int64_t b_cs,
+                          void* C, int64_t c_rs, int64_t c_cs, int prologue, int epilogue)
+{
+    Problem check;
+    int rc = make_problem(in_type, out_type, M, N, K, A, a_rs, a_cs, B, b_rs, b_cs, C, c_rs, c_cs, prologue, epilogue, true, &check);
+    if (rc) return rc;
+    if (M == 0 || N == 0) return ACC950_OK;
+    const size_t a_bytes = extent_elems(M, K, a_rs, a_cs) * elem_size(in_type);
+    const size_t b_bytes = extent_elems(K, N, b_rs, b_cs) * elem_size(in_type);
+    const size_t c_bytes = extent_elems(M, N, c_rs, c_cs) * elem_size(out_type);
+    const bool c_dense = extent_elems(M, N, c_rs, c_cs) == (size_t)M * (size_t)N;
+
+    std::lock_guard<std::mutex> lock(g_host_mutex);
+    hipError_t e;
+    if ((e = reserve(g_dA, a_bytes ? a_bytes : 16)) != hipSuccess) return fail_hip(e, "hipMalloc(A)");
+    if ((e = reserve(g_dB, b_bytes ? b_bytes : 16)) != hipSuccess) return fail_hip(e, "hipMalloc(B)");
+    if ((e = reserve(g_dC, c_bytes)) != hipSuccess) return fail_hip(e, "hipMalloc(C)");
+    if (a_bytes && (e = hipMemcpy(g_dA.p, A, a_bytes, hipMemcpyHostToDevice)) != hipSuccess) return fail_hip(e, "copy A to device");
+    if (b_bytes && (e = hipMemcpy(g_dB.p, B, b_bytes, hipMemcpyHostToDevice)) != hipSuccess) return fail_hip(e, "copy B to device");
+    // C travels to the device when it is accumulated into, or when its extent has gaps
+    // that the copy back must not clobber
+    if (prologue == PRO_NONE || !c_dense)
+        if ((e = hipMemcpy(g_dC.p, C, c_bytes, hipMemcpyHostToDevice)) != hipSuccess) return fail_hip(e, "copy C to device");
+    rc = acc950_gemm_relu(in_type, out_type, M, N, K, g_dA.p, a_rs, a_cs, g_dB.p, b_rs, b_cs, g_dC.p, c_rs, c_cs,
+                          prologue, epilogue, nullptr);
+    if (rc) return rc;
+    if ((e = hipMemcpy(C, g_dC.p, c_bytes, hipMemcpyDeviceToHost)) != hipSuccess) return fail_hip(e, "copy C to host");
+    return ACC950_OK;
+}
+
+int acc950_num_variants(void)
+{
+    int n = 0;
+    mfma_variants_f16(&n);
+    return n;
+}
+
+int acc950_num_skinny_variants(void) { return skinny_num_variants(); }
+
+int acc950_variant_name(int variant, char* buf, size_t buf_len)
+{
+    if (!buf || buf_len == 0) return fail(ACC950_INVALID_ARGUMENT, "null buffer");
+    if (variant == ACC950_VARIANT_GENERIC) {
+        std::snprintf(buf, buf_len, "generic thread-bound 64x64 tile");
+        return ACC950_OK;
+    }
+    if (variant == ACC950_VARIANT_F32_MFMA) {
+        std::snprintf(buf, buf_len, "fp32 mfma 32x32 tile, K split over 4 waves");
+        return ACC950_OK;
+    }
+    if (variant >= ACC950_VARIANT_SKINNY_BASE && variant < ACC950_VARIANT_SKINNY_BASE + skinny_num_variants()) {
+        int lpr, waves;
+        skinny_variant_info(variant - ACC950_VARIANT_SKINNY_BASE, &lpr, &waves);
+        std::snprintf(buf, buf_len, "skinny cols/wg=%d waves=%d", lpr * 8, waves);
+        return ACC950_OK;
+    }
+    int n = 0;
+    const MfmaVariant* tab = mfma_variants_f16(&n);
+    if (variant < 0 || variant >= n) return fail(ACC950_INVALID_ARGUMENT, "unknown kernel variant");
+    const MfmaVariant& v = tab[variant];
+    std::snprintf(buf, buf_len, "mfma %dx%d waves %dx%d B=%s fill=%s%s", v.bm, v.bn, v.waves_m, v.waves_n,
+                  v.b_kc ? "col-major" : "row-major", v.direct ? "direct" : "registers", v.edge ? " edge" : "");
+    return ACC950_OK;
+}
+
+} // extern "C"

@@ -1,0 +1,101 @@
+// Shared declarations for the gfx950 GEMM+ReLU kernels and their host launchers.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace acc950 {
+
+// Element types (values match include/accera_mi355x_gemm.h).
+enum : int { T_F32 = 0, T_F16 = 1, T_BF16 = 2, T_I8 = 3, T_I32 = 4 };
+// Prologue / epilogue ops of the tensorized plan
+// (/root/reference/accera/python/accera/lang/Plan.py:208-379, fragment ops
+//  /root/reference/accera/acc-translate/src/Target/Cpp/CppPrinterUtils.h:630-655).
+enum : int { PRO_NONE = 0, PRO_SET0 = 1 };
+enum : int { EPI_NONE = 0, EPI_RELU = 1, EPI_RELU_NOCOND = 2 };
+
+// Arguments of one GEMM launch.  Strides are in elements.
+struct GemmArgs {
+    const void* A;
+    const void* B;
+    void* C;
+    int M, N, K;
+    int64_t a_rs, a_cs; // A[i,k] at i*a_rs + k*a_cs
+    int64_t b_rs, b_cs; // B[k,j] at k*b_rs + j*b_cs
+    int64_t c_rs, c_cs; // C[i,j] at i*c_rs + j*c_cs
+    int in_type, out_type;
+    int prologue, epilogue;
+    int tiles_m, tiles_n; // workgroup grid in tiles (MFMA kernels)
+};
+
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+typedef int i32x2 __attribute__((ext_vector_type(2)));
+typedef int i32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+
+#define ACC950_LDS __attribute__((address_space(3)))
+#define ACC950_GLOBAL __attribute__((address_space(1)))
+
+// ---- scalar conversions --------------------------------------------------------
+
+__device__ __forceinline__ float bf16_bits_to_float(uint16_t b) { return __uint_as_float((uint32_t)b << 16); }
+
+// float -> bfloat16 bits, round to nearest even, NaN kept quiet.  (The reference's
+// GPU store truncates, CppPrinterUtils.h:107-117; nearest-even is what its LLVM
+// host path and this library's oracle do.)
+__device__ __forceinline__ uint16_t float_to_bf16_bits(float f)
+{
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40u);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+
+__device__ __forceinline__ uint16_t float_to_f16_bits(float f)
+{
+    _Float16 h = (_Float16)f; // v_cvt_f16_f32: round to nearest even
+    return __builtin_bit_cast(uint16_t, h);
+}
+
+__device__ __forceinline__ float f16_bits_to_float(uint16_t b) { return (float)__builtin_bit_cast(_Float16, b); }
+
+// ---- fragment epilogue ops (CppPrinterUtils.h:630-643) ---------------------------
+// relu:                v > 0 ? v : 0     (NaN -> 0, -0 -> +0)
+// relu_no_conditional: v *= (v > 0)      (NaN stays NaN, negatives -> -0)
+template <typename T>
+__device__ __forceinline__ T apply_epilogue(T v, int epi)
+{
+    if (epi == EPI_RELU) return v > T(0) ? v : T(0);
+    if (epi == EPI_RELU_NOCOND) return v * T(v > T(0) ? 1 : 0);
+    return v;
+}
+
+// Store one float accumulator as the output element type.
+__device__ __forceinline__ void store_out(void* C, int out_type, int64_t idx, float v)
+{
+    if (out_type == T_F32) ((float*)C)[idx] = v;
+    else if (out_type == T_F16) ((uint16_t*)C)[idx] = float_to_f16_bits(v);
+    else ((uint16_t*)C)[idx] = float_to_bf16_bits(v);
+}
+__device__ __forceinline__ float load_out(const void* C, int out_type, int64_t idx)
+{
+    if (out_type == T_F32) return ((const float*)C)[idx];
+    if (out_type == T_F16) return f16_bits_to_float(((const uint16_t*)C)[idx]);
+    return bf16_bits_to_float(((const uint16_t*)C)[idx]);
+}
+
+// ---- host-side launch record -------------------------------------------------------
+struct LaunchGeom {
+    unsigned grid[3];
+    unsigned block[3];
+    unsigned dyn_lds;
+};
+
+typedef hipError_t (*LaunchFn)(const GemmArgs&, hipStream_t, LaunchGeom*, bool dry_run);
+
+} // namespace acc950

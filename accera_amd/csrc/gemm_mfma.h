@@ -1,0 +1,420 @@
+// LDS-tiled, double-buffered MFMA GEMM with the prologue/epilogue fused into the
+// accumulator write-back, for gfx950 (CDNA4) only.
+//
+// This is the hand-written replacement for what the reference's tensorized GPU plan
+// lowers to: per-warp MMA fragment loads / mma_sync passes / fragment store with
+// epilogue (/root/reference/accera/transforms/src/exec/ExecutionPlanToAffineLoweringPass.cpp:5986-6533),
+// the workgroup-cooperative block_copy of A/B tiles into shared memory
+// (/root/reference/accera/acc-translate/src/Target/Cpp/CppPrinterUtils.h:364-628),
+// its double buffering (ExecutionPlanToAffineLoweringPass.cpp:5240-5371) and the
+// accumulator (MMA_FRAGMENT) cache of C (:2705-2726).  None of that code is reused:
+//
+//  * MFMA: v_mfma_f32_32x32x16_{f16,bf16} and v_mfma_i32_32x32x32_i8 -- one
+//    instruction consumes 32 bytes of K per row, 16 bytes per lane.
+//  * An operand whose K index is contiguous in memory ("KC": row-major A,
+//    column-major B) is staged as [row][128 bytes of K] and read with one
+//    ds_read_b128 per fragment.  An operand whose M/N index is contiguous ("MC":
+//    row-major B) is staged as [k][row bytes] exactly as it lies in memory and read
+//    with the gfx950 LDS transpose reads ds_read_b64_tr_b16 / _tr_b8, which hand
+//    each lane the K-run of its own column.
+//  * 16-byte chunks are XOR-swizzled inside each LDS row so both the fragment reads
+//    and the tile fills are bank-conflict free without padding.
+//  * Tiles are filled either through registers (global_load_dwordx4 + ds_write_b128)
+//    or directly with global_load_lds_dwordx4, which needs no staging registers; in
+//    the direct form the swizzle is applied to the global address each lane fetches
+//    because the LDS destination of lane l is fixed at base + 16*l.
+//  * Two LDS buffers, one barrier per K tile: the fill of tile t+1 is issued before
+//    the MFMAs of tile t.
+//  * Workgroup ids are remapped so that each of the 8 XCDs (own L2 each) works on a
+//    compact rectangle of output tiles.
+#pragma once
+#include "common.h"
+#include <type_traits>
+
+namespace acc950 {
+
+enum : int { IN_F16 = 0, IN_BF16 = 1, IN_I8 = 2 };
+
+template <int IN> struct InTraits { static constexpr int ES = 2; using acc_t = f32x16; using scalar_t = float; };
+template <> struct InTraits<IN_I8> { static constexpr int ES = 1; using acc_t = i32x16; using scalar_t = int; };
+
+template <int IN>
+__device__ __forceinline__ void mfma32(const i32x4& a, const i32x4& b, typename InTraits<IN>::acc_t& c)
+{
+    if constexpr (IN == IN_F16)
+        c = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+    else if constexpr (IN == IN_BF16)
+        c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+    else
+        c = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c, 0, 0, 0);
+}
+
+// One K tile is 128 bytes of K for a KC operand, i.e. BK elements with BK*ES == 128.
+constexpr int KTILE_BYTES = 128;
+
+// Staging and fragment access for one operand tile of R rows (M or N extent).
+template <int IN, int R, bool KC, int NT>
+struct OperandTile {
+    static constexpr int ES = InTraits<IN>::ES;
+    static constexpr int BK = KTILE_BYTES / ES;          // K elements per tile
+    static constexpr int TILE_BYTES = R * KTILE_BYTES;   // same for KC and MC
+    static constexpr int CHUNKS = TILE_BYTES / 16;
+    static constexpr int PER_THREAD = CHUNKS / NT;
+    static_assert(CHUNKS % NT == 0, "tile must split evenly over the workgroup");
+    // MC: one LDS row is one k, holding R elements.
+    static constexpr int ROW_BYTES = KC ? KTILE_BYTES : R * ES;
+    static constexpr int CPR = ROW_BYTES / 16;           // 16-byte chunks per LDS row
+
+    // LDS chunk position -> chunk position of the same row after the swizzle (an involution).
+    __device__ static __forceinline__ int swizzle(int row, int c)
+    {
+        if constexpr (KC) return c ^ ((row >> 1) & 7);
+        else if constexpr (ES == 2) return c ^ (((row & 3) << 2) & (CPR - 1));
+        else return c ^ (((row & 7) << 1) & (CPR - 1));
+    }
+
+    // Byte offset in global memory of logical chunk (row, c) of the tile whose first
+    // row is r0 (M/N index) and first K element is k0.  ld = leading dimension in elements.
+    __device__ static __forceinline__ int64_t global_off(int row, int c, int r0, int k0, int64_t ld)
+    {
+        if constexpr (KC) return ((int64_t)(r0 + row) * ld + k0) * ES + c * 16;
+        else return ((int64_t)(k0 + row) * ld + r0) * ES + c * 16;
+    }
+
+    // EDGE: is logical chunk (row, c) inside the matrix?  (rmax = M or N, K multiple of 16/ES)
+    __device__ static __forceinline__ bool in_bounds(int row, int c, int r0, int k0, int rmax, int K)
+    {
+        if constexpr (KC) return (r0 + row) < rmax && (k0 + c * (16 / ES)) < K;
+        else return (k0 + row) < K && (r0 + c * (16 / ES)) < rmax;
+    }
+
+    // ---- register-staged fill ----
+    template <bool EDGE>
+    __device__ static __forceinline__ void load_global(i32x4 (&regs)[PER_THREAD], const char* base, int r0, int k0,
+                                                       int64_t ld, int rmax, int K, int tid)
+    {
+#pragma unroll
+        for (int i = 0; i < PER_THREAD; ++i) {
+            int id = tid + i * NT;
+            int row = id / CPR, c = id % CPR;
+            if constexpr (EDGE) {
+                if (in_bounds(row, c, r0, k0, rmax, K))
+                    regs[i] = *(const i32x4*)(base + global_off(row, c, r0, k0, ld));
+                else
+                    regs[i] = i32x4{0, 0, 0, 0};
+            } else {
+                regs[i] = *(const i32x4*)(base + global_off(row, c, r0, k0, ld));
+            }
+        }
+    }
+    __device__ static __forceinline__ void store_lds(const i32x4 (&regs)[PER_THREAD], char* lds, int tid)
+    {
+#pragma unroll
+        for (int i = 0; i < PER_THREAD; ++i) {
+            int id = tid + i * NT;
+            int row = id / CPR, c = id % CPR;
+            *(i32x4*)(lds + row * ROW_BYTES + swizzle(row, c) * 16) = regs[i];
+        }
+    }
+
+    // ---- direct global -> LDS fill (global_load_lds_dwordx4) ----
+    // Lane l of a wave writes LDS bytes [M0 + 16*l, +16), so LDS chunk position
+    // id = tid + i*NT is fixed and the lane fetches the logical chunk that the swizzle
+    // maps there.  The swizzle only depends on the low row bits, which are the same
+    // for every i, so one per-lane 32-bit offset serves all fills of the kernel and
+    // the rest of the address is wave-uniform (SGPR base, advanced per K tile).
+    static constexpr int ROWS_PER_PASS = NT / CPR; // rows covered by one fill instruction of the workgroup
+    static constexpr int SWIZZLE_PERIOD = KC ? 16 : (ES == 2 ? 4 : 8); // rows after which the swizzle repeats
+    static_assert(NT % CPR == 0 && ROWS_PER_PASS % SWIZZLE_PERIOD == 0, "swizzle must repeat every pass");
+
+    __device__ static __forceinline__ unsigned direct_lane_offset(int64_t ld, int tid)
+    {
+        int row = tid / CPR, cpos = tid % CPR;
+        return (unsigned)global_off(row, swizzle(row, cpos), 0, 0, ld);
+    }
+    // Uniform base of fill i for the tile at (r0, k0).
+    __device__ static __forceinline__ const char* direct_base(const char* base, int i, int r0, int k0, int64_t ld)
+    {
+        return base + global_off(i * ROWS_PER_PASS, 0, r0, k0, ld);
+    }
+    // The instruction is issued from inline assembly so that the compiler does not
+    // serialise later LDS reads of the *other* buffer behind it; the kernel waits with
+    // an explicit s_waitcnt vmcnt(0) before the barrier that publishes the tile.
+    __device__ static __forceinline__ void direct_issue(unsigned lds_addr, unsigned lane_off, const char* sbase)
+    {
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                     :
+                     : "s"(lds_addr), "v"(lane_off), "s"(sbase)
+                     : "memory");
+    }
+
+    // ---- fragment read: 32 rows starting at row0, k-step ks (32 bytes of K) ----
+    __device__ static __forceinline__ i32x4 read_frag(const char* lds, int row0, int ks, int lane)
+    {
+        if constexpr (KC) {
+            int row = row0 + (lane & 31);
+            int c = ks * 2 + (lane >> 5);
+            return *(const i32x4*)(lds + row * ROW_BYTES + swizzle(row, c) * 16);
+        } else if constexpr (ES == 2) {
+            // ds_read_b64_tr_b16: in each group of 16 lanes, lanes 4j..4j+3 point at k-row j
+            // (4 x 8 bytes = 16 columns); lane i receives column i of those 4 rows.
+            int h = lane >> 5, g = (lane >> 4) & 1, i = lane & 15;
+            int col_byte = (row0 + g * 16 + (i & 3) * 4) * 2;
+            int c = col_byte >> 4, within = col_byte & 15;
+            i32x4 out;
+#pragma unroll
+            for (int q = 0; q < 2; ++q) {
+                int k = ks * 16 + h * 8 + q * 4 + (i >> 2);
+                const char* p = lds + k * ROW_BYTES + swizzle(k, c) * 16 + within;
+                s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((ACC950_LDS s16x4*)p);
+                i32x2 w = __builtin_bit_cast(i32x2, v);
+                out[q * 2] = w[0];
+                out[q * 2 + 1] = w[1];
+            }
+            return out;
+        } else {
+            // ds_read_b64_tr_b8: lanes 2j, 2j+1 point at k-row j (2 x 8 bytes = 16 columns);
+            // lane i receives column i of those 8 rows.
+            int h = lane >> 5, g = (lane >> 4) & 1, i = lane & 15;
+            int col_byte = row0 + g * 16 + (i & 1) * 8;
+            int c = col_byte >> 4, within = col_byte & 15;
+            i32x4 out;
+#pragma unroll
+            for (int q = 0; q < 2; ++q) {
+                int k = ks * 32 + h * 16 + q * 8 + (i >> 1);
+                const char* p = lds + k * ROW_BYTES + swizzle(k, c) * 16 + within;
+                i32x2 w = __builtin_amdgcn_ds_read_tr8_b64_v2i32((ACC950_LDS i32x2*)p);
+                out[q * 2] = w[0];
+                out[q * 2 + 1] = w[1];
+            }
+            return out;
+        }
+    }
+};
+
+// Output tile -> (tile_m, tile_n).  Consecutive workgroup ids go to different XCDs
+// (id % 8), so ids are first regrouped per XCD and then walked in column-major order
+// inside bands of GROUP_M tile rows, which makes the tiles resident on one XCD at any
+// time a compact rectangle that shares A and B tiles through that XCD's L2.
+__device__ __forceinline__ void tile_coords(int pid, int tiles_m, int tiles_n, int& tm, int& tn)
+{
+    constexpr int XCDS = 8, GROUP_M = 4;
+    int total = tiles_m * tiles_n;
+    if (total % XCDS == 0) pid = (pid % XCDS) * (total / XCDS) + pid / XCDS;
+    int per_group = GROUP_M * tiles_n;
+    int group = pid / per_group;
+    int first_m = group * GROUP_M;
+    int gsz = tiles_m - first_m < GROUP_M ? tiles_m - first_m : GROUP_M;
+    int in_group = pid % per_group;
+    tm = first_m + in_group % gsz;
+    tn = in_group / gsz;
+}
+
+template <int IN, int BM, int BN, int WAVES_M, int WAVES_N, bool A_KC, bool B_KC, bool DIRECT, bool EDGE>
+__global__ void __launch_bounds__(WAVES_M* WAVES_N * 64) gemm_mfma_kernel(GemmArgs p)
+{
+    static_assert(!(DIRECT && EDGE), "edge tiles are zero-filled through registers");
+    constexpr int NT = WAVES_M * WAVES_N * 64;
+    constexpr int ES = InTraits<IN>::ES;
+    constexpr int BK = KTILE_BYTES / ES;
+    constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
+    constexpr int TM = WTM / 32, TN = WTN / 32;
+    static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wave tile is made of 32x32 MFMA blocks");
+    using TA = OperandTile<IN, BM, A_KC, NT>;
+    using TB = OperandTile<IN, BN, B_KC, NT>;
+    using acc_t = typename InTraits<IN>::acc_t;
+    using scalar_t = typename InTraits<IN>::scalar_t;
+    constexpr int STAGE_BYTES = TA::TILE_BYTES + TB::TILE_BYTES;
+
+    extern __shared__ __attribute__((aligned(1024))) char smem[];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int wr0 = (wave / WAVES_N) * WTM;
+    const int wc0 = (wave % WAVES_N) * WTN;
+
+    int tile_m, tile_n;
+    tile_coords(blockIdx.x, p.tiles_m, p.tiles_n, tile_m, tile_n);
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+
+    const char* Ab = (const char*)p.A;
+    const char* Bb = (const char*)p.B;
+    const int64_t lda = A_KC ? p.a_rs : p.a_cs; // KC: stride between rows; MC: stride between k
+    const int64_t ldb = B_KC ? p.b_cs : p.b_rs;
+
+    acc_t acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) acc[i][j] = acc_t{};
+
+    const int KT = (p.K + BK - 1) / BK;
+
+    // LDS byte address of the tile buffers as the hardware sees it (for M0).
+    const unsigned smem_addr = (unsigned)(size_t)(ACC950_LDS char*)smem;
+    const unsigned wave_lds = __builtin_amdgcn_readfirstlane((unsigned)(wave * 1024));
+    unsigned a_lane_off = 0, b_lane_off = 0;
+    if constexpr (DIRECT) {
+        a_lane_off = TA::direct_lane_offset(lda, tid);
+        b_lane_off = TB::direct_lane_offset(ldb, tid);
+    }
+    constexpr int FILLS_A = TA::PER_THREAD, FILLS_B = TB::PER_THREAD, FILLS = FILLS_A + FILLS_B;
+    // fill number f of the tile starting at K element k0 into stage buffer `stage`
+    auto issue_fill = [&](int f, int stage, int k0) {
+        if (f < FILLS_A)
+            TA::direct_issue(smem_addr + stage * STAGE_BYTES + wave_lds + f * NT * 16, a_lane_off,
+                             TA::direct_base(Ab, f, m0, k0, lda));
+        else
+            TB::direct_issue(smem_addr + stage * STAGE_BYTES + TA::TILE_BYTES + wave_lds + (f - FILLS_A) * NT * 16,
+                             b_lane_off, TB::direct_base(Bb, f - FILLS_A, n0, k0, ldb));
+    };
+
+    // MFMAs of one K tile.  Fragments are double-buffered across the four k-steps: the
+    // LDS reads of step ks+1 are issued between the MFMAs of step ks, one per MFMA
+    // slot, and (direct form) the fills of the next tile are spread over the slots too.
+    constexpr int SLOTS = TM * TN;
+    constexpr int FILLS_PER_SLOT = (FILLS + 4 * SLOTS - 1) / (4 * SLOTS);
+    constexpr int SLOT_STRIDE = FILLS_PER_SLOT > 1 ? 1 : (4 * SLOTS) / FILLS; // a fill every SLOT_STRIDE slots
+    auto mma_tile = [&](const char* sa, const char* sb, auto fill_tag, int fill_stage, int fill_k0) {
+        constexpr bool fill = decltype(fill_tag)::value;
+        i32x4 af[2][TM], bf[2][TN];
+#pragma unroll
+        for (int i = 0; i < TM; ++i) af[0][i] = TA::read_frag(sa, wr0 + i * 32, 0, lane);
+#pragma unroll
+        for (int j = 0; j < TN; ++j) bf[0][j] = TB::read_frag(sb, wc0 + j * 32, 0, lane);
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j) {
+                    const int slot = i * TN + j;
+                    mfma32<IN>(af[ks & 1][i], bf[ks & 1][j], acc[i][j]);
+                    if (ks < 3) {
+                        if (slot < TM) af[(ks + 1) & 1][slot] = TA::read_frag(sa, wr0 + slot * 32, ks + 1, lane);
+                        else if (slot - TM < TN) bf[(ks + 1) & 1][slot - TM] = TB::read_frag(sb, wc0 + (slot - TM) * 32, ks + 1, lane);
+                    }
+                    if constexpr (DIRECT) {
+                        const int gslot = ks * SLOTS + slot;
+                        if (fill && gslot % SLOT_STRIDE == 0) { // compile-time after unrolling
+#pragma unroll
+                            for (int u = 0; u < FILLS_PER_SLOT; ++u) {
+                                const int f = (gslot / SLOT_STRIDE) * FILLS_PER_SLOT + u;
+                                if (f < FILLS) issue_fill(f, fill_stage, fill_k0);
+                            }
+                        }
+                    }
+                }
+        }
+    };
+    static_assert(TM + TN <= SLOTS, "not enough MFMA slots to prefetch the next fragments");
+
+    if constexpr (DIRECT) {
+#pragma unroll
+        for (int f = 0; f < FILLS; ++f) issue_fill(f, 0, 0);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        for (int kt = 0; kt < KT - 1; ++kt) {
+            const int cur = kt & 1;
+            mma_tile(smem + cur * STAGE_BYTES, smem + cur * STAGE_BYTES + TA::TILE_BYTES, std::true_type{}, cur ^ 1, (kt + 1) * BK);
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __syncthreads();
+        }
+        {   // last tile: nothing left to fetch
+            const int cur = (KT - 1) & 1;
+            mma_tile(smem + cur * STAGE_BYTES, smem + cur * STAGE_BYTES + TA::TILE_BYTES, std::false_type{}, 0, 0);
+        }
+    } else {
+        i32x4 ra[TA::PER_THREAD], rb[TB::PER_THREAD];
+        TA::template load_global<EDGE>(ra, Ab, m0, 0, lda, p.M, p.K, tid);
+        TB::template load_global<EDGE>(rb, Bb, n0, 0, ldb, p.N, p.K, tid);
+        TA::store_lds(ra, smem, tid);
+        TB::store_lds(rb, smem + TA::TILE_BYTES, tid);
+        __syncthreads();
+        for (int kt = 0; kt < KT; ++kt) {
+            char* cur = smem + (kt & 1) * STAGE_BYTES;
+            char* nxt = smem + ((kt + 1) & 1) * STAGE_BYTES;
+            if (kt + 1 < KT) {
+                TA::template load_global<EDGE>(ra, Ab, m0, (kt + 1) * BK, lda, p.M, p.K, tid);
+                TB::template load_global<EDGE>(rb, Bb, n0, (kt + 1) * BK, ldb, p.N, p.K, tid);
+            }
+            mma_tile(cur, cur + TA::TILE_BYTES, std::false_type{}, 0, 0);
+            if (kt + 1 < KT) {
+                TA::store_lds(ra, nxt, tid);
+                TB::store_lds(rb, nxt + TA::TILE_BYTES, tid);
+            }
+            __syncthreads();
+        }
+    }
+
+    // Write-back: optional "+= C" (no SET prologue), epilogue op, narrowing store.
+    // MFMA 32x32 accumulator layout: register r of lane l holds
+    //   row = (r/4)*8 + (l/32)*4 + r%4,  column = l%32.
+    const int row_base = m0 + wr0 + (lane >> 5) * 4;
+    const int col_base = n0 + wc0 + (lane & 31);
+    auto for_each_acc = [&](auto&& fn) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int row = row_base + i * 32 + (r >> 2) * 8 + (r & 3);
+                    const int col = col_base + j * 32;
+                    if (EDGE && (row >= p.M || col >= p.N)) continue;
+                    acc[i][j][r] = fn(acc[i][j][r], (int64_t)row * p.c_rs + (int64_t)col * p.c_cs);
+                }
+    };
+    // epilogue as two selects on wave-uniform conditions (no per-element branches)
+    const bool is_relu = p.epilogue == EPI_RELU, is_nocond = p.epilogue == EPI_RELU_NOCOND;
+    auto epilogue = [&](scalar_t v) -> scalar_t {
+        scalar_t r = v > scalar_t(0) ? v : scalar_t(0);
+        scalar_t n = v * (v > scalar_t(0) ? scalar_t(1) : scalar_t(0));
+        return is_relu ? r : (is_nocond ? n : v);
+    };
+    if constexpr (IN == IN_I8) {
+        int* C = (int*)p.C;
+        if (p.prologue == PRO_NONE) for_each_acc([&](int v, int64_t idx) { return (int)((unsigned)v + (unsigned)C[idx]); });
+        for_each_acc([&](int v, int64_t idx) { C[idx] = epilogue(v); return v; });
+    } else {
+        if (p.prologue == PRO_NONE) {
+            if (p.out_type == T_F32) for_each_acc([&](float v, int64_t idx) { return v + ((const float*)p.C)[idx]; });
+            else if (p.out_type == T_F16) for_each_acc([&](float v, int64_t idx) { return v + f16_bits_to_float(((const uint16_t*)p.C)[idx]); });
+            else for_each_acc([&](float v, int64_t idx) { return v + bf16_bits_to_float(((const uint16_t*)p.C)[idx]); });
+        }
+        if (p.out_type == T_F32) for_each_acc([&](float v, int64_t idx) { ((float*)p.C)[idx] = epilogue(v); return v; });
+        else if (p.out_type == T_F16) for_each_acc([&](float v, int64_t idx) { ((uint16_t*)p.C)[idx] = float_to_f16_bits(epilogue(v)); return v; });
+        else for_each_acc([&](float v, int64_t idx) { ((uint16_t*)p.C)[idx] = float_to_bf16_bits(epilogue(v)); return v; });
+    }
+}
+
+// Host launcher for one kernel instantiation.
+template <int IN, int BM, int BN, int WAVES_M, int WAVES_N, bool A_KC, bool B_KC, bool DIRECT, bool EDGE>
+hipError_t launch_mfma(const GemmArgs& a, hipStream_t stream, LaunchGeom* geom, bool dry_run)
+{
+    constexpr int NT = WAVES_M * WAVES_N * 64;
+    constexpr int LDS = 2 * (BM + BN) * KTILE_BYTES;
+    auto kern = gemm_mfma_kernel<IN, BM, BN, WAVES_M, WAVES_N, A_KC, B_KC, DIRECT, EDGE>;
+    GemmArgs args = a;
+    args.tiles_m = (a.M + BM - 1) / BM;
+    args.tiles_n = (a.N + BN - 1) / BN;
+    if (geom) {
+        geom->grid[0] = (unsigned)(args.tiles_m * args.tiles_n);
+        geom->grid[1] = geom->grid[2] = 1;
+        geom->block[0] = NT;
+        geom->block[1] = geom->block[2] = 1;
+        geom->dyn_lds = LDS;
+    }
+    if (dry_run) return hipSuccess;
+    static bool attr_set = false; // per instantiation; benign if set twice
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
+        if (e != hipSuccess) return e;
+        attr_set = true;
+    }
+    hipLaunchKernelGGL(kern, dim3(args.tiles_m * args.tiles_n), dim3(NT), LDS, stream, args);
+    return hipGetLastError();
+}
+
+} // namespace acc950

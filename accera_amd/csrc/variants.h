@@ -1,0 +1,24 @@
+// Table entry describing one compiled MFMA GEMM kernel.
+#pragma once
+#include "common.h"
+
+namespace acc950 {
+
+struct MfmaVariant {
+    int bm, bn;          // block tile
+    int waves_m, waves_n;
+    bool a_kc, b_kc;     // operand has K contiguous in memory (else M/N contiguous)
+    bool direct;         // tile fill with global_load_lds (else through registers)
+    bool edge;           // handles M/N/K that are not tile multiples
+    LaunchFn launch;
+};
+
+const MfmaVariant* mfma_variants_f16(int* count);
+const MfmaVariant* mfma_variants_bf16(int* count);
+const MfmaVariant* mfma_variants_i8(int* count);
+
+bool f32_can_take(const GemmArgs& g);
+hipError_t launch_f32(const GemmArgs& a, hipStream_t stream, LaunchGeom* geom, bool dry_run);
+hipError_t launch_generic(const GemmArgs& a, hipStream_t stream, LaunchGeom* geom, bool dry_run);
+
+} // namespace acc950

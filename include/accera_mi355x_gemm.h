@@ -1,0 +1,133 @@
+/*
+ * accera_mi355x_gemm.h -- C ABI of the MI355X (gfx950) matmul + fused-epilogue kernels.
+ *
+ * The library replaces, for one GPU, what the reference's GPU plan path emits for an
+ * `acc.Nest` matmul with a fused elementwise epilogue (C += A*B, then ReLU): the
+ * generated `<fn>__gpu__` kernels and their host launcher stubs.  Each entry point
+ * below names the reference interface it stands in for.  Plain pointers and sizes
+ * only; no exceptions cross this boundary; every function returns an ACC950_* status.
+ *
+ * Matrices are described the way a .hat file describes an `affine_array`
+ * (/root/reference/accera/ir/src/TranslateToHeader.cpp:713-762): shape plus element
+ * strides (`affine_map`); row-major M x N has strides (N, 1), column-major (1, M).
+ */
+#ifndef ACCERA_MI355X_GEMM_H
+#define ACCERA_MI355X_GEMM_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#if defined(__cplusplus)
+extern "C" {
+#endif
+
+/* element types; the .hat element_type names are float, float16_t, bfloat16_t,
+ * int8_t, int32_t (TranslateToHeader.cpp:165-192, 329-400) */
+#define ACC950_F32 0
+#define ACC950_F16 1
+#define ACC950_BF16 2
+#define ACC950_I8 3
+#define ACC950_I32 4
+
+/* prologue / epilogue ops of plan.tensorize
+ * (/root/reference/accera/python/accera/lang/Plan.py:208-379;
+ *  device helpers /root/reference/accera/acc-translate/src/Target/Cpp/CppPrinterUtils.h:630-655) */
+#define ACC950_PROLOGUE_NONE 0 /* C = epilogue(C + A*B) */
+#define ACC950_PROLOGUE_SET0 1 /* C = epilogue(A*B)     (MMAFragmentOp.SET with 0) */
+#define ACC950_EPILOGUE_NONE 0
+#define ACC950_EPILOGUE_RELU 1           /* v > 0 ? v : 0 */
+#define ACC950_EPILOGUE_RELU_NOCOND 2    /* v *= (v > 0)  */
+
+/* status codes */
+#define ACC950_OK 0
+#define ACC950_INVALID_ARGUMENT 1 /* bad type pair, negative size, null pointer, unknown op */
+#define ACC950_UNSUPPORTED 2      /* the requested kernel variant cannot take this problem */
+#define ACC950_HIP_ERROR 3        /* a HIP call failed; see acc950_last_error() */
+
+/* kernel selection for acc950_gemm_relu_ex */
+#define ACC950_VARIANT_AUTO (-1)
+#define ACC950_VARIANT_SKINNY_BASE 100 /* 100 + i : streaming kernel i for M <= 8 */
+#define ACC950_VARIANT_GENERIC 200     /* thread-bound kernel, any shape / stride / type */
+#define ACC950_VARIANT_F32_MFMA 201    /* fp32 MFMA kernel (fp32 inputs) */
+
+/*
+ * Selects the device and checks that it is a gfx950 part.  Optional: the other entry
+ * points use the current HIP device.  Stands in for hatlib's device selection
+ * (`device_id=` of hat.run_benchmark, /root/reference/tools/benchmarkers/accera_gemm.py:612-626).
+ */
+int acc950_init(int device_id);
+
+/*
+ * C = epilogue((prologue == SET0 ? 0 : C) + A * B) on DEVICE pointers, asynchronously on
+ * `stream` (a hipStream_t, or NULL for the default stream).  A is M x K, B is K x N,
+ * C is M x N.  in_type F16/BF16 -> out_type F32/F16/BF16 (fp32 accumulate);
+ * I8 -> I32 (exact, wrap-around); F32 -> F32.
+ *
+ * Replaces the generated host launcher `fn(A,B,C){ fn__gpu__<<<grid,block,lds>>>(A,B,C); }`
+ * which likewise takes device pointers
+ * (/root/reference/accera/acc-translate/src/Target/Cpp/GpuDialectCppPrinter.cpp:532-561)
+ * and the kernel body the tensorize / cache / bind lowering produces
+ * (/root/reference/accera/transforms/src/exec/ExecutionPlanToAffineLoweringPass.cpp:5986-6533).
+ */
+int acc950_gemm_relu(int in_type, int out_type, int M, int N, int K,
+                     const void* A, int64_t a_row_stride, int64_t a_col_stride,
+                     const void* B, int64_t b_row_stride, int64_t b_col_stride,
+                     void* C, int64_t c_row_stride, int64_t c_col_stride,
+                     int prologue, int epilogue, void* stream);
+
+/*
+ * Same, with the kernel variant chosen by the caller: the counterpart of building one
+ * point of the reference's tuning space (tile sizes, cache strategy, double buffering:
+ * /root/reference/tools/benchmarkers/accera_gemm.py:187-348).  `variant` is
+ * ACC950_VARIANT_AUTO, an index < acc950_num_variants() into the MFMA table,
+ * ACC950_VARIANT_SKINNY_BASE + i, ACC950_VARIANT_F32_MFMA or ACC950_VARIANT_GENERIC.  `k_splits` (skinny
+ * kernels only; 0 = automatic) splits K over workgroups.
+ */
+int acc950_gemm_relu_ex(int in_type, int out_type, int M, int N, int K,
+                        const void* A, int64_t a_row_stride, int64_t a_col_stride,
+                        const void* B, int64_t b_row_stride, int64_t b_col_stride,
+                        void* C, int64_t c_row_stride, int64_t c_col_stride,
+                        int prologue, int epilogue, int variant, int k_splits, void* stream);
+
+/*
+ * Same computation on HOST pointers, synchronous: copies A, B (and C when it is
+ * accumulated into) to the device, runs the kernel, copies C back.  This is the
+ * calling convention of a HAT_DYNAMIC package function `void f(T* A, T* B, T* C)` as
+ * hatlib calls it with NumPy arrays
+ * (/root/reference/README.md:118-136; /root/reference/accera/python/accera/Package.py:776-784);
+ * the per-function symbols of a package forward to this entry point.
+ */
+int acc950_gemm_relu_host(int in_type, int out_type, int M, int N, int K,
+                          const void* A, int64_t a_row_stride, int64_t a_col_stride,
+                          const void* B, int64_t b_row_stride, int64_t b_col_stride,
+                          void* C, int64_t c_row_stride, int64_t c_col_stride,
+                          int prologue, int epilogue);
+
+/*
+ * Launch record of the kernel acc950_gemm_relu_ex would run for this problem, without
+ * running it: grid[3], block[3], dynamic LDS bytes, and the variant actually chosen.
+ * The structural counterpart of the `launch_parameters` / `dynamic_shared_mem_bytes`
+ * fields the reference regex-parses out of its generated source
+ * (/root/reference/accera/python/accera/Package.py:25-28, 714-743).
+ */
+int acc950_launch_geometry(int in_type, int out_type, int M, int N, int K,
+                           int64_t a_row_stride, int64_t a_col_stride,
+                           int64_t b_row_stride, int64_t b_col_stride,
+                           int64_t c_row_stride, int64_t c_col_stride,
+                           int variant, int k_splits,
+                           unsigned grid[3], unsigned block[3], unsigned* dynamic_lds_bytes, int* chosen_variant);
+
+/* Number of MFMA table variants, and a human-readable description of any variant id
+ * ("mfma 256x256 waves 2x2 B=row-major fill=direct", ...).  Returns ACC950_INVALID_ARGUMENT
+ * for an unknown id. */
+int acc950_num_variants(void);
+int acc950_num_skinny_variants(void);
+int acc950_variant_name(int variant, char* buf, size_t buf_len);
+
+/* Text of the last error on the calling thread ("" if none). */
+const char* acc950_last_error(void);
+
+#if defined(__cplusplus)
+}
+#endif
+#endif /* ACCERA_MI355X_GEMM_H */

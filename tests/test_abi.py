@@ -1,0 +1,74 @@
+"""The C-ABI library loads without a GPU and exports every symbol the header declares;
+argument checking and the launch-geometry query run on the host alone."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from accera_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared():
+    text = open(os.path.join(ROOT, "include", "accera_mi355x_gemm.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(acc950_\w+)\s*\(", text)))
+
+
+def test_every_declared_symbol_is_exported():
+    names = _declared()
+    assert len(names) >= 9 and set(_lib.EXPORTS) == set(names)
+    L = ctypes.CDLL(_lib.LIB_PATH)
+    for n in names:
+        assert getattr(L, n) is not None, n
+
+
+def test_variant_table_is_described():
+    assert _lib.num_variants() >= 8 and _lib.num_skinny_variants() >= 1
+    names = [_lib.variant_name(v) for v in range(_lib.num_variants())]
+    assert len(set(names)) == len(names)
+    assert any("direct" in n for n in names) and any("edge" in n for n in names)
+    assert "skinny" in _lib.variant_name(_lib.VARIANT_SKINNY_BASE)
+    with pytest.raises(_lib.Acc950Error):
+        _lib.variant_name(57)
+
+
+# launch geometry expectations for the BASELINE configurations: grid = tiles of the block
+# tile, block = waves * 64 (Plan.py:937-956 derives the same quantities from the bound indices;
+# mfma_tests.py:2562,2572 pins them as <<<dim3(...), dim3(...)>>> strings)
+def test_launch_geometry_of_the_configs():
+    g, b, lds, v = _lib.launch_geometry(_lib.F16, _lib.F32, 4096, 4096, 4096, (4096, 1), (4096, 1), (4096, 1))
+    name = _lib.variant_name(v)
+    bm, bn = map(int, re.search(r"mfma (\d+)x(\d+)", name).groups())
+    assert g == [(4096 // bm) * (4096 // bn), 1, 1] and b[0] % 64 == 0 and lds == 2 * (bm + bn) * 128
+    g, b, lds, v = _lib.launch_geometry(_lib.BF16, _lib.BF16, 4096, 3072, 768, (768, 1), (1, 768), (3072, 1))
+    assert "B=col-major" in _lib.variant_name(v)
+    g, b, lds, v = _lib.launch_geometry(_lib.I8, _lib.I32, 8192, 8192, 8192, (8192, 1), (8192, 1), (8192, 1))
+    assert "mfma" in _lib.variant_name(v)
+    g, b, lds, v = _lib.launch_geometry(_lib.F16, _lib.F16, 8, 11008, 4096, (4096, 1), (11008, 1), (11008, 1))
+    assert "skinny" in _lib.variant_name(v) and g[0] * g[1] >= 256
+    g, b, lds, v = _lib.launch_geometry(_lib.F32, _lib.F32, 512, 512, 512, (512, 1), (512, 1), (512, 1))
+    assert v == _lib.VARIANT_F32_MFMA and g[:2] == [16, 16]
+    # unaligned shapes fall to the thread-bound kernel, explicit variants refuse them
+    g, b, lds, v = _lib.launch_geometry(_lib.F16, _lib.F32, 100, 71, 40, (40, 1), (71, 1), (71, 1))
+    assert v == _lib.VARIANT_GENERIC and g[:2] == [2, 2]
+    with pytest.raises(_lib.Acc950Error) as e:
+        _lib.launch_geometry(_lib.F16, _lib.F32, 100, 71, 40, (40, 1), (71, 1), (71, 1), variant=0)
+    assert e.value.code == _lib.UNSUPPORTED
+
+
+def test_argument_checking_on_the_host():
+    with pytest.raises(_lib.Acc950Error) as e:
+        _lib.launch_geometry(_lib.I8, _lib.F32, 64, 64, 64, (64, 1), (64, 1), (64, 1))
+    assert e.value.code == _lib.INVALID_ARGUMENT and "type pair" in str(e.value)
+    with pytest.raises(_lib.Acc950Error):
+        _lib.launch_geometry(_lib.F16, _lib.F32, -1, 64, 64, (64, 1), (64, 1), (64, 1))
+    with pytest.raises(_lib.Acc950Error):
+        _lib.launch_geometry(_lib.F16, _lib.F32, 64, 64, 64, (-64, 1), (64, 1), (64, 1))
+    # null pointers are rejected before anything is launched
+    rc = _lib.lib().acc950_gemm_relu(_lib.F16, _lib.F32, 64, 64, 64, None, 64, 1, None, 64, 1, None, 64, 1, 1, 1, None)
+    assert rc == _lib.INVALID_ARGUMENT and b"null" in _lib.lib().acc950_last_error()
+    # empty problems are a no-op
+    assert _lib.lib().acc950_gemm_relu(_lib.F16, _lib.F32, 0, 64, 64, None, 64, 1, None, 64, 1, None, 64, 1, 1, 1, None) == 0

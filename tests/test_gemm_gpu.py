@@ -1,0 +1,306 @@
+"""GPU parity tests: every kernel family of libaccera_mi355x.so, called through the C
+ABI on device memory, against the CPU oracle on the same seeded inputs.
+
+Integer results must be bit-exact; float results are held to the tolerances the
+reference's own tests use (rtol 1e-3 for fp32 output of fp16/bf16 inputs, 1e-2 for
+fp16/bf16 output: mfma_tests.py:2047,2083,2553-2577), with signed data so that ReLU
+really clips (the reference's ReLU tests use non-negative inputs only).
+"""
+import numpy as np
+import pytest
+
+import oracle as ora
+from tests.util import assert_matches, make_input, out_zeros, to_device, to_host
+
+pytestmark = pytest.mark.gpu
+
+PAIRS = [("f16", "f32"), ("f16", "f16"), ("bf16", "f32"), ("bf16", "bf16"), ("i8", "i32")]
+
+
+def run_case(in_type, out_type, M, N, K, b_layout="row", c_layout="row", variant=-1, splits=0,
+             prologue=ora.PRO_SET0, epilogue=ora.EPI_RELU, seed=0, dist="uniform", expect_variant=None):
+    import accera_amd as acc
+    import torch
+    rng = np.random.default_rng(seed)
+    A = make_input(rng, (M, K), in_type, dist)
+    B = make_input(rng, (K, N), in_type, dist)
+    if b_layout == "col":
+        B = np.asfortranarray(B)
+    if prologue == ora.PRO_NONE:
+        C0 = make_input(rng, (M, N), "i8", dist).astype(np.int32) * 1000 if out_type == "i32" else \
+            make_input(rng, (M, N), out_type, dist)
+    else:
+        # poison C so that a kernel that wrongly reads it cannot pass
+        C0 = np.full((M, N), 77, np.int32) if out_type == "i32" else make_input(rng, (M, N), out_type, dist)
+    if c_layout == "col":
+        C0 = np.asfortranarray(C0)
+    dA, dB, dC = to_device(A, in_type), to_device(B, in_type), to_device(C0, out_type)
+    assert dB.stride() == ((1, K) if b_layout == "col" else (N, 1))
+    acc.gemm_relu(dA, dB, dC, prologue=prologue, epilogue=epilogue, variant=variant, k_splits=splits)
+    torch.cuda.synchronize()
+    got = to_host(dC, out_type)
+    want = ora.gemm_relu_exact(A, B, C0, in_type, out_type, prologue, epilogue)
+    assert_matches(got, want, out_type, K)
+    if epilogue == ora.EPI_RELU and M * N >= 64:
+        w = ora.widen(want, out_type)
+        assert (w == 0).any() and (w > 0).any(), "test data must exercise both ReLU branches"
+    return got
+
+
+def _variants(b_layout):
+    from accera_amd import _lib
+    names = [(v, _lib.variant_name(v)) for v in range(_lib.num_variants())]
+    key = "B=col-major" if b_layout == "col" else "B=row-major"
+    return [(v, n) for v, n in names if key in n]
+
+
+# ---- every MFMA variant, every input type, both B layouts --------------------------------
+@pytest.mark.parametrize("in_type,out_type", [("f16", "f32"), ("bf16", "bf16"), ("i8", "i32")])
+@pytest.mark.parametrize("b_layout", ["row", "col"])
+def test_mfma_all_variants(in_type, out_type, b_layout):
+    bk = 128 if in_type == "i8" else 64
+    for v, name in _variants(b_layout):
+        print("variant", v, name, in_type, b_layout, flush=True)
+        # two tiles in each direction, three K tiles (odd count exercises both LDS buffers)
+        run_case(in_type, out_type, 512, 512, 3 * bk, b_layout=b_layout, variant=v, seed=v)
+        if "edge" in name:
+            # ragged M, N (multiple of the 16-byte vector only) and a K tail
+            run_case(in_type, out_type, 200, 144, 336 if in_type == "i8" else 176, b_layout=b_layout, variant=v, seed=100 + v)
+
+
+@pytest.mark.parametrize("in_type,out_type", PAIRS)
+def test_mfma_auto_output_types(in_type, out_type):
+    run_case(in_type, out_type, 256, 384, 512, seed=3)
+    run_case(in_type, out_type, 256, 384, 512, seed=4, prologue=ora.PRO_NONE)
+    run_case(in_type, out_type, 256, 384, 512, seed=5, epilogue=ora.EPI_RELU_NOCOND, b_layout="col")
+    run_case(in_type, out_type, 256, 384, 512, seed=6, epilogue=ora.EPI_NONE, prologue=ora.PRO_NONE)
+
+
+def test_mfma_single_k_tile_and_many_tiles():
+    run_case("f16", "f32", 128, 128, 64, seed=7)          # K loop runs once (no prefetch)
+    run_case("f16", "f32", 1024, 1536, 128, seed=8)       # many tiles: exercises the XCD / group remap
+    run_case("i8", "i32", 768, 1280, 256, seed=9, variant=5)  # tile count not a multiple of 8 XCDs
+    run_case("bf16", "f32", 1280, 768, 1024, seed=10)     # reference size 1280x768x1024 (mfma_tests.py:2007-2272)
+
+
+def test_mfma_tile_map_covers_every_tile_once():
+    """Identity-like check of the workgroup -> tile map: C = A @ I must reproduce A in
+    every tile, for tile grids that are / are not multiples of the XCD count and group size."""
+    import accera_amd as acc
+    import torch
+    for (M, N) in [(256, 128), (640, 384), (1152, 1664), (2048, 2048)]:
+        K = N
+        rng = np.random.default_rng(M + N)
+        A = make_input(rng, (M, K), "f16")
+        I = np.eye(K, N, dtype=np.float16)
+        dC = to_device(out_zeros(M, N, "f32"), "f32")
+        acc.gemm_relu(to_device(A, "f16"), to_device(I, "f16"), dC, epilogue=acc.EPILOGUE_NONE)
+        torch.cuda.synchronize()
+        assert np.array_equal(to_host(dC, "f32"), A.astype(np.float32)), (M, N)
+
+
+# ---- edge kernel and generic kernel: sizes of the reference's boundary tests ---------------
+@pytest.mark.parametrize("shape", [(16, 16, 1264), (64, 64, 96), (960, 1024, 1024), (100, 72, 40), (16, 16, 16), (128, 16, 16)])
+@pytest.mark.parametrize("in_type,out_type", [("f16", "f32"), ("bf16", "f32"), ("i8", "i32")])
+def test_boundary_shapes(shape, in_type, out_type):
+    M, N, K = shape  # 16x16x1264: mfma_tests.py:2242-2272; 16/128 x K=16: :2579-2602
+    run_case(in_type, out_type, M, N, K, seed=sum(shape))
+
+
+@pytest.mark.parametrize("in_type,out_type", PAIRS + [("f32", "f32")])
+@pytest.mark.parametrize("shape", [(33, 47, 29), (1, 1, 1), (65, 130, 7), (64, 93, 64)])
+def test_generic_kernel_any_shape(in_type, out_type, shape):
+    M, N, K = shape
+    run_case(in_type, out_type, M, N, K, variant=200, seed=sum(shape))
+    run_case(in_type, out_type, M, N, K, variant=200, seed=sum(shape) + 1, b_layout="col", c_layout="col", prologue=ora.PRO_NONE)
+
+
+def test_column_major_c_uses_transposed_product():
+    run_case("f16", "f32", 256, 384, 256, c_layout="col", seed=21)
+    run_case("i8", "i32", 256, 384, 256, c_layout="col", b_layout="col", seed=22)
+    run_case("bf16", "bf16", 384, 256, 192, c_layout="col", seed=23, prologue=ora.PRO_NONE)
+
+
+def test_strided_views_with_padding():
+    """Leading dimensions larger than the logical width (sub-matrix views)."""
+    import accera_amd as acc
+    import torch
+    rng = np.random.default_rng(31)
+    M, N, K = 256, 256, 192
+    Abig = make_input(rng, (M, K + 64), "f16")
+    Bbig = make_input(rng, (K, N + 128), "f16")
+    Cbig = np.full((M, N + 8), -5.0, np.float32)
+    dA, dB, dC = to_device(Abig, "f16"), to_device(Bbig, "f16"), to_device(Cbig, "f32")
+    acc.gemm_relu(dA[:, :K], dB[:, :N], dC[:, :N])
+    torch.cuda.synchronize()
+    got = to_host(dC, "f32")
+    want = ora.gemm_relu_exact(Abig[:, :K], Bbig[:, :N], None, "f16", "f32")
+    assert_matches(got[:, :N], want, "f32", K)
+    assert np.all(got[:, N:] == -5.0)  # padding untouched
+
+
+# ---- fp32 kernel ------------------------------------------------------------------------------
+@pytest.mark.parametrize("shape", [(512, 512, 512), (64, 32, 8), (100, 70, 52), (33, 47, 29), (256, 256, 1000)])
+@pytest.mark.parametrize("b_layout", ["row", "col"])
+def test_f32_mfma_kernel(shape, b_layout):
+    M, N, K = shape
+    got = run_case("f32", "f32", M, N, K, b_layout=b_layout, seed=41)
+    # fp32 products: must be far better than a reduced-precision input path could give
+    rng = np.random.default_rng(41)
+    A, B = make_input(rng, (M, K), "f32"), make_input(rng, (K, N), "f32")
+    want = np.maximum(A.astype(np.float64) @ B.astype(np.float64), 0)
+    assert np.abs(got - want).max() < 1e-4 * max(1, np.sqrt(K) / 8)
+    run_case("f32", "f32", M, N, K, b_layout=b_layout, seed=42, prologue=ora.PRO_NONE, epilogue=ora.EPI_RELU_NOCOND)
+
+
+def test_readme_quickstart_shape_and_data():
+    """README.md:118-136: A,B ~ U[0,1) 512x512 fp32, C zeros, atol 1e-3."""
+    import accera_amd as acc
+    import torch
+    rng = np.random.default_rng(1001)
+    A = rng.random((512, 512), dtype=np.float32)
+    B = rng.random((512, 512), dtype=np.float32)
+    C = np.zeros((512, 512), np.float32)
+    dC = to_device(C, "f32")
+    acc.gemm_relu(to_device(A, "f32"), to_device(B, "f32"), dC, prologue=acc.PROLOGUE_NONE)
+    torch.cuda.synchronize()
+    np.testing.assert_allclose(to_host(dC, "f32"), np.maximum(C + A @ B, 0.0), atol=1e-3)
+
+
+# ---- skinny streaming kernel -----------------------------------------------------------------
+@pytest.mark.parametrize("in_type,out_type", [("f16", "f16"), ("f16", "f32"), ("bf16", "bf16")])
+def test_skinny_all_variants_and_splits(in_type, out_type):
+    from accera_amd import _lib
+    for sv in range(_lib.num_skinny_variants()):
+        for splits in (1, 3, 8):
+            print("skinny", sv, _lib.variant_name(100 + sv), "splits", splits, flush=True)
+            run_case(in_type, out_type, 8, 1024 + 64, 1024, variant=100 + sv, splits=splits, seed=sv * 10 + splits, dist="normal")
+    # ragged: M < 8, N not a multiple of the column block, K not a multiple of the k step
+    run_case(in_type, out_type, 5, 1000, 998, variant=100, splits=4, seed=77, dist="normal")
+    run_case(in_type, out_type, 1, 8, 2, variant=100, splits=1, seed=78, dist="normal", epilogue=ora.EPI_NONE)
+    run_case(in_type, out_type, 8, 2048, 512, seed=79, dist="normal", prologue=ora.PRO_NONE)
+
+
+def test_skinny_repeated_launches_reuse_counters():
+    """The K-split arrival counters must return to zero after every launch."""
+    for rep in range(3):
+        run_case("f16", "f16", 8, 4096, 2048, variant=100, splits=8, seed=90 + rep, dist="normal")
+    run_case("f16", "f16", 8, 512, 2048, variant=103, splits=5, seed=95, dist="normal")
+
+
+# ---- closed forms: bit-exact expectations ------------------------------------------------------
+@pytest.mark.parametrize("in_type,out_type", [("f16", "f32"), ("bf16", "f32"), ("i8", "i32"), ("f32", "f32")])
+def test_permutation_matrix_is_bit_exact(in_type, out_type):
+    import accera_amd as acc
+    import torch
+    rng = np.random.default_rng(51)
+    M, K = 256, 256
+    A = make_input(rng, (M, K), in_type)
+    perm = rng.permutation(K)
+    P = np.zeros((K, K), np.float32)
+    P[perm, np.arange(K)] = 1
+    Pm = {"f32": P, "f16": P.astype(np.float16), "bf16": ora.to_bf16(P), "i8": P.astype(np.int8)}[in_type]
+    dC = to_device(out_zeros(M, K, out_type), out_type)
+    acc.gemm_relu(to_device(A, in_type), to_device(Pm, in_type), dC)
+    torch.cuda.synchronize()
+    want = np.maximum(ora.widen(A, in_type)[:, perm], 0)
+    assert np.array_equal(ora.widen(to_host(dC, out_type), out_type), want)
+
+
+def test_reference_constant_fill_known_answers():
+    """A=2, B=3, C=0.42 -> 6K + 0.42 (docs/Tutorials/Hello_MatMul.md:165-237, K=256;
+    docs/Tutorials/Optimized_MatMul.md:204-280, K=128)."""
+    import accera_amd as acc
+    import torch
+    for K, expected in [(256, 1536.42), (128, 768.42)]:
+        for t in ("f32", "f16"):
+            A = np.full((128, K), 2.0, ora.NP_STORAGE[t])
+            B = np.full((K, 256), 3.0, ora.NP_STORAGE[t])
+            dC = to_device(np.full((128, 256), 0.42, np.float32), "f32")
+            acc.gemm_relu(to_device(A, t), to_device(B, t), dC, prologue=acc.PROLOGUE_NONE)
+            torch.cuda.synchronize()
+            np.testing.assert_allclose(to_host(dC, "f32"), expected, rtol=1e-6)
+
+
+def test_int8_extremes_are_exact():
+    import accera_amd as acc
+    import torch
+    M = N = 256
+    K = 1024
+    A = np.full((M, K), -128, np.int8)
+    B = np.full((K, N), -128, np.int8)
+    dC = to_device(out_zeros(M, N, "i32"), "i32")
+    acc.gemm_relu(to_device(A, "i8"), to_device(B, "i8"), dC)
+    torch.cuda.synchronize()
+    assert np.all(to_host(dC, "i32") == K * 16384)
+    B[:] = 127
+    dC = to_device(out_zeros(M, N, "i32"), "i32")
+    acc.gemm_relu(to_device(A, "i8"), to_device(B, "i8"), dC, epilogue=acc.EPILOGUE_NONE)
+    torch.cuda.synchronize()
+    assert np.all(to_host(dC, "i32") == -K * 128 * 127)
+
+
+@pytest.mark.parametrize("variant", [-1, 200])
+@pytest.mark.parametrize("epi", [ora.EPI_RELU, ora.EPI_RELU_NOCOND])
+def test_relu_special_values(variant, epi):
+    """epilogue(C0 + 0): relu maps NaN, -0, -inf to +0; relu_no_conditional keeps NaN and
+    turns -inf into NaN (-inf * 0).  CppPrinterUtils.h:630-643."""
+    import accera_amd as acc
+    import torch
+    M, N, K = 128, 128, 64
+    vals = np.array([-0.0, np.nan, np.inf, -np.inf, -3.5, 2.25, 0.0, 1e-38], np.float32)
+    C0 = np.tile(vals, (M, N // len(vals)))
+    A = np.zeros((M, K), np.float16)
+    B = np.zeros((K, N), np.float16)
+    dC = to_device(C0, "f32")
+    acc.gemm_relu(to_device(A, "f16"), to_device(B, "f16"), dC, prologue=acc.PROLOGUE_NONE, epilogue=epi, variant=variant)
+    torch.cuda.synchronize()
+    got = to_host(dC, "f32")
+    want = C0.copy()
+    ora.gemm_relu(A, B, want, "f16", "f32", prologue=ora.PRO_NONE, epilogue=epi)
+    assert np.array_equal(np.isnan(got), np.isnan(want))
+    ok = ~np.isnan(want)
+    assert np.array_equal(got[ok], want[ok])
+    assert np.array_equal(np.signbit(got[ok]), np.signbit(want[ok]))
+
+
+def test_linearity_and_k_split_invariance_full_size_int8():
+    """Size-independent property at a large size: for int8, A@[B1|B2] computed as one
+    N=2048 problem equals the two N=1024 problems, and equals int64 NumPy on sampled rows."""
+    import accera_amd as acc
+    import torch
+    rng = np.random.default_rng(61)
+    M, N, K = 2048, 2048, 4096
+    A, B = make_input(rng, (M, K), "i8"), make_input(rng, (K, N), "i8")
+    dA, dB = to_device(A, "i8"), to_device(B, "i8")
+    dC = to_device(out_zeros(M, N, "i32"), "i32")
+    acc.gemm_relu(dA, dB, dC, epilogue=acc.EPILOGUE_NONE)
+    dC1 = to_device(out_zeros(M, N // 2, "i32"), "i32")
+    acc.gemm_relu(dA, dB[:, : N // 2], dC1, epilogue=acc.EPILOGUE_NONE)
+    torch.cuda.synchronize()
+    C = to_host(dC, "i32")
+    assert np.array_equal(C[:, : N // 2], to_host(dC1, "i32"))
+    rows = rng.choice(M, 16, replace=False)
+    assert np.array_equal(C[rows], (A[rows].astype(np.int64) @ B.astype(np.int64)).astype(np.int32))
+    # checksum of checksums: sum_j C[i,j] = A[i,:] . (B 1)
+    assert np.array_equal(C.astype(np.int64).sum(axis=1), A.astype(np.int64) @ B.astype(np.int64).sum(axis=1))
+
+
+# ---- error behaviour of the C ABI ---------------------------------------------------------------
+def test_errors_are_reported_not_thrown():
+    import accera_amd as acc
+    import torch
+    A = torch.zeros((64, 64), dtype=torch.int8, device="cuda")
+    Cf = torch.zeros((64, 64), dtype=torch.float32, device="cuda")
+    with pytest.raises(acc.Acc950Error) as e:
+        acc.gemm_relu(A, A, Cf)  # int8 -> fp32 is not a supported pair
+    assert e.value.code == 1
+    Ah = torch.zeros((100, 72), dtype=torch.float16, device="cuda")
+    Ch = torch.zeros((100, 100), dtype=torch.float32, device="cuda")
+    with pytest.raises(acc.Acc950Error) as e:
+        acc.gemm_relu(Ah, Ah.t(), Ch, variant=0)  # 256x256 tile variant cannot take 100x100
+    assert e.value.code == 2
+    with pytest.raises(acc.Acc950Error):
+        acc.gemm_relu(Ah, Ah.t(), Ch, variant=57)
+    with pytest.raises(ValueError):
+        acc.gemm_relu(Ah.cpu(), Ah.t(), Ch)  # no CPU path
