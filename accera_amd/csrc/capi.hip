@@ -98,7 +98,7 @@ bool mfma_can_take(const MfmaVariant& v, const Problem& pb)
 {
     const GemmArgs& g = pb.g;
     if (g.M <= 0 || g.N <= 0 || g.K <= 0) return false;
-    const int es = elem_size(g.in_type), vec = 16 / es, bk = 128 / es;
+    const int es = elem_size(g.in_type), vec = 16 / es, bk = v.kb / es;
     if (g.a_cs != 1 || g.c_cs != 1) return false; // A row-major (K contiguous), C row-major
     if (v.b_kc ? g.b_rs != 1 : g.b_cs != 1) return false;
     const int64_t lda = g.a_rs, ldb = v.b_kc ? g.b_cs : g.b_rs;
@@ -175,10 +175,10 @@ int auto_mfma_variant(const Problem& pb)
     int n = 0;
     const MfmaVariant* tab = mfma_table(pb.g.in_type, &n);
     if (!tab) return -1;
-    struct Want { int bm, bn, wm, wn; bool direct, edge; };
+    struct Want { int bm, bn, wm, wn; bool direct, edge; int kb, stages; };
     const int64_t tiles256 = ((int64_t)pb.g.M / 256) * (pb.g.N / 256);
-    const Want big = {256, 256, 2, 2, true, false}, mid = {256, 128, 2, 2, true, false},
-               small = {128, 128, 2, 2, true, false}, edge = {128, 128, 2, 2, false, true};
+    const Want big = {256, 256, 2, 4, true, false, 128, 2}, mid = {256, 128, 2, 2, true, false, 128, 3},
+               small = {128, 128, 2, 2, true, false, 128, 2}, edge = {128, 128, 2, 2, false, true, 128, 2};
     Want order[4];
     if (tiles256 >= 200) { order[0] = big; order[1] = mid; order[2] = small; }
     else { order[0] = small; order[1] = mid; order[2] = big; }
@@ -187,7 +187,7 @@ int auto_mfma_variant(const Problem& pb)
         for (int i = 0; i < n; ++i) {
             const MfmaVariant& v = tab[i];
             if (v.bm == w.bm && v.bn == w.bn && v.waves_m == w.wm && v.waves_n == w.wn && v.direct == w.direct &&
-                v.edge == w.edge && mfma_can_take(v, pb))
+                v.edge == w.edge && v.kb == w.kb && v.stages == w.stages && mfma_can_take(v, pb))
                 return i;
         }
     return -1;
@@ -409,8 +409,8 @@ int acc950_variant_name(int variant, char* buf, size_t buf_len)
     const MfmaVariant* tab = mfma_variants_f16(&n);
     if (variant < 0 || variant >= n) return fail(ACC950_INVALID_ARGUMENT, "unknown kernel variant");
     const MfmaVariant& v = tab[variant];
-    std::snprintf(buf, buf_len, "mfma %dx%d waves %dx%d B=%s fill=%s%s", v.bm, v.bn, v.waves_m, v.waves_n,
-                  v.b_kc ? "col-major" : "row-major", v.direct ? "direct" : "registers", v.edge ? " edge" : "");
+    std::snprintf(buf, buf_len, "mfma %dx%d kb%d waves %dx%d B=%s fill=%s stages=%d%s", v.bm, v.bn, v.kb, v.waves_m, v.waves_n,
+                  v.b_kc ? "col-major" : "row-major", v.direct ? "direct" : "registers", v.stages, v.edge ? " edge" : "");
     return ACC950_OK;
 }
 

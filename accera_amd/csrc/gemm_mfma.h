@@ -1,4 +1,4 @@
-// LDS-tiled, double-buffered MFMA GEMM with the prologue/epilogue fused into the
+// LDS-tiled, multi-stage MFMA GEMM with the prologue/epilogue fused into the
 // accumulator write-back, for gfx950 (CDNA4) only.
 //
 // This is the hand-written replacement for what the reference's tensorized GPU plan
@@ -12,7 +12,7 @@
 //  * MFMA: v_mfma_f32_32x32x16_{f16,bf16} and v_mfma_i32_32x32x32_i8 -- one
 //    instruction consumes 32 bytes of K per row, 16 bytes per lane.
 //  * An operand whose K index is contiguous in memory ("KC": row-major A,
-//    column-major B) is staged as [row][128 bytes of K] and read with one
+//    column-major B) is staged as [row][KB bytes of K] and read with one
 //    ds_read_b128 per fragment.  An operand whose M/N index is contiguous ("MC":
 //    row-major B) is staged as [k][row bytes] exactly as it lies in memory and read
 //    with the gfx950 LDS transpose reads ds_read_b64_tr_b16 / _tr_b8, which hand
@@ -23,8 +23,9 @@
 //    or directly with global_load_lds_dwordx4, which needs no staging registers; in
 //    the direct form the swizzle is applied to the global address each lane fetches
 //    because the LDS destination of lane l is fixed at base + 16*l.
-//  * Two LDS buffers, one barrier per K tile: the fill of tile t+1 is issued before
-//    the MFMAs of tile t.
+//  * STAGES LDS buffers, one barrier per K tile: the fill of tile t+STAGES-1 is
+//    issued at the start of the MFMAs of tile t, and only the fills of tile t+1 are
+//    waited for (s_waitcnt vmcnt(n) with the younger fills still in flight).
 //  * Workgroup ids are remapped so that each of the 8 XCDs (own L2 each) works on a
 //    compact rectangle of output tiles.
 #pragma once
@@ -49,29 +50,42 @@ __device__ __forceinline__ void mfma32(const i32x4& a, const i32x4& b, typename 
         c = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c, 0, 0, 0);
 }
 
-// One K tile is 128 bytes of K for a KC operand, i.e. BK elements with BK*ES == 128.
-constexpr int KTILE_BYTES = 128;
+template <int N>
+__device__ __forceinline__ void wait_vmcnt()
+{
+    static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
 
-// Staging and fragment access for one operand tile of R rows (M or N extent).
-template <int IN, int R, bool KC, int NT>
+// Staging and fragment access for one operand tile of R rows (M or N extent) and KB
+// bytes of K (64 or 128), i.e. BK = KB / element-size K elements.
+template <int IN, int R, bool KC, int NT, int KB>
 struct OperandTile {
+    static_assert(KB == 64 || KB == 128, "K tile is 64 or 128 bytes");
     static constexpr int ES = InTraits<IN>::ES;
-    static constexpr int BK = KTILE_BYTES / ES;          // K elements per tile
-    static constexpr int TILE_BYTES = R * KTILE_BYTES;   // same for KC and MC
+    static constexpr int BK = KB / ES;                   // K elements per tile
+    static constexpr int KSTEPS = KB / 32;               // MFMA steps per tile
+    static constexpr int TILE_BYTES = R * KB;            // same for KC and MC
     static constexpr int CHUNKS = TILE_BYTES / 16;
     static constexpr int PER_THREAD = CHUNKS / NT;
     static_assert(CHUNKS % NT == 0, "tile must split evenly over the workgroup");
-    // MC: one LDS row is one k, holding R elements.
-    static constexpr int ROW_BYTES = KC ? KTILE_BYTES : R * ES;
+    // KC: one LDS row is one matrix row (KB bytes); MC: one LDS row is one k (R elements).
+    static constexpr int ROW_BYTES = KC ? KB : R * ES;
     static constexpr int CPR = ROW_BYTES / 16;           // 16-byte chunks per LDS row
 
-    // LDS chunk position -> chunk position of the same row after the swizzle (an involution).
+    // LDS chunk position <-> logical chunk of the same row (an involution).
+    //  KC, 128-byte rows: a 16-lane read phase touches rows r..r+15 at one chunk; rows
+    //      two apart are 256 bytes (all banks) apart, so the row pair index picks the chunk.
+    //  KC,  64-byte rows: four rows fill the 256-byte bank span, so row/4 picks the chunk.
+    //  MC: a transpose read touches 4 (16-bit) or 8 (8-bit) consecutive k rows, which are
+    //      a multiple of 256 bytes apart; k picks a 64- / 32-byte group inside the row.
     __device__ static __forceinline__ int swizzle(int row, int c)
     {
-        if constexpr (KC) return c ^ ((row >> 1) & 7);
+        if constexpr (KC) return KB == 128 ? c ^ ((row >> 1) & 7) : c ^ ((row >> 2) & 3);
         else if constexpr (ES == 2) return c ^ (((row & 3) << 2) & (CPR - 1));
         else return c ^ (((row & 7) << 1) & (CPR - 1));
     }
+    static constexpr int SWIZZLE_PERIOD = KC ? 16 : (ES == 2 ? 4 : 8); // rows after which it repeats
 
     // Byte offset in global memory of logical chunk (row, c) of the tile whose first
     // row is r0 (M/N index) and first K element is k0.  ld = leading dimension in elements.
@@ -124,7 +138,6 @@ struct OperandTile {
     // for every i, so one per-lane 32-bit offset serves all fills of the kernel and
     // the rest of the address is wave-uniform (SGPR base, advanced per K tile).
     static constexpr int ROWS_PER_PASS = NT / CPR; // rows covered by one fill instruction of the workgroup
-    static constexpr int SWIZZLE_PERIOD = KC ? 16 : (ES == 2 ? 4 : 8); // rows after which the swizzle repeats
     static_assert(NT % CPR == 0 && ROWS_PER_PASS % SWIZZLE_PERIOD == 0, "swizzle must repeat every pass");
 
     __device__ static __forceinline__ unsigned direct_lane_offset(int64_t ld, int tid)
@@ -138,8 +151,8 @@ struct OperandTile {
         return base + global_off(i * ROWS_PER_PASS, 0, r0, k0, ld);
     }
     // The instruction is issued from inline assembly so that the compiler does not
-    // serialise later LDS reads of the *other* buffer behind it; the kernel waits with
-    // an explicit s_waitcnt vmcnt(0) before the barrier that publishes the tile.
+    // serialise later LDS reads of the *other* buffers behind it; the kernel waits with
+    // an explicit s_waitcnt vmcnt(n) before the barrier that publishes the tile.
     __device__ static __forceinline__ void direct_issue(unsigned lds_addr, unsigned lane_off, const char* sbase)
     {
         asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
@@ -210,18 +223,33 @@ __device__ __forceinline__ void tile_coords(int pid, int tiles_m, int tiles_n, i
     tn = in_group / gsz;
 }
 
-template <int IN, int BM, int BN, int WAVES_M, int WAVES_N, bool A_KC, bool B_KC, bool DIRECT, bool EDGE>
-__global__ void __launch_bounds__(WAVES_M* WAVES_N * 64) gemm_mfma_kernel(GemmArgs p)
-{
+// Compile-time description of one kernel instantiation.
+template <int IN_, int BM_, int BN_, int WAVES_M_, int WAVES_N_, bool A_KC_, bool B_KC_, bool DIRECT_, bool EDGE_, int KB_, int STAGES_>
+struct MfmaConfig {
+    static constexpr int IN = IN_, BM = BM_, BN = BN_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_, KB = KB_, STAGES = STAGES_;
+    static constexpr bool A_KC = A_KC_, B_KC = B_KC_, DIRECT = DIRECT_, EDGE = EDGE_;
+    static constexpr int NT = WAVES_M * WAVES_N * 64;
+    static constexpr int LDS_BYTES = STAGES * (BM + BN) * KB;
     static_assert(!(DIRECT && EDGE), "edge tiles are zero-filled through registers");
-    constexpr int NT = WAVES_M * WAVES_N * 64;
+    static_assert(DIRECT || STAGES == 2, "the register-staged fill is double-buffered");
+    static_assert(STAGES >= 2 && STAGES <= 4, "2 to 4 LDS stages");
+    static_assert(LDS_BYTES <= 160 * 1024, "LDS budget of one CU");
+};
+
+template <typename Cfg>
+__global__ void __launch_bounds__(Cfg::NT) gemm_mfma_kernel(GemmArgs p)
+{
+    constexpr int IN = Cfg::IN, BM = Cfg::BM, BN = Cfg::BN, WAVES_M = Cfg::WAVES_M, WAVES_N = Cfg::WAVES_N;
+    constexpr int KB = Cfg::KB, STAGES = Cfg::STAGES, NT = Cfg::NT;
+    constexpr bool A_KC = Cfg::A_KC, B_KC = Cfg::B_KC, DIRECT = Cfg::DIRECT, EDGE = Cfg::EDGE;
     constexpr int ES = InTraits<IN>::ES;
-    constexpr int BK = KTILE_BYTES / ES;
+    constexpr int BK = KB / ES;
+    constexpr int KSTEPS = KB / 32;
     constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
     constexpr int TM = WTM / 32, TN = WTN / 32;
     static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wave tile is made of 32x32 MFMA blocks");
-    using TA = OperandTile<IN, BM, A_KC, NT>;
-    using TB = OperandTile<IN, BN, B_KC, NT>;
+    using TA = OperandTile<IN, BM, A_KC, NT, KB>;
+    using TB = OperandTile<IN, BN, B_KC, NT, KB>;
     using acc_t = typename InTraits<IN>::acc_t;
     using scalar_t = typename InTraits<IN>::scalar_t;
     constexpr int STAGE_BYTES = TA::TILE_BYTES + TB::TILE_BYTES;
@@ -270,60 +298,98 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64) gemm_mfma_kernel(GemmAr
                              b_lane_off, TB::direct_base(Bb, f - FILLS_A, n0, k0, ldb));
     };
 
-    // MFMAs of one K tile.  Fragments are double-buffered across the four k-steps: the
-    // LDS reads of step ks+1 are issued between the MFMAs of step ks, one per MFMA
-    // slot, and (direct form) the fills of the next tile are spread over the slots too.
+    // MFMAs of one K tile.  Fragments are double-buffered across the k-steps: the LDS
+    // reads of step ks+1 are issued between the MFMAs of step ks, one per MFMA slot,
+    // and (direct form) the fills of a later tile go out with the first MFMA slots so
+    // that they have the rest of this tile, and the following ones, to land.  With
+    // CROSS the reads issued during the last k-step fetch step 0 of the *next* tile
+    // (already published), so no LDS latency is exposed after the barrier.  A
+    // sched_barrier after every slot pins this order against the machine scheduler.
     constexpr int SLOTS = TM * TN;
-    constexpr int FILLS_PER_SLOT = (FILLS + 4 * SLOTS - 1) / (4 * SLOTS);
-    constexpr int SLOT_STRIDE = FILLS_PER_SLOT > 1 ? 1 : (4 * SLOTS) / FILLS; // a fill every SLOT_STRIDE slots
-    auto mma_tile = [&](const char* sa, const char* sb, auto fill_tag, int fill_stage, int fill_k0) {
-        constexpr bool fill = decltype(fill_tag)::value;
-        i32x4 af[2][TM], bf[2][TN];
+    constexpr int FILLS_PER_SLOT = (FILLS + SLOTS - 1) / SLOTS; // all fills within the first k-step
+    static_assert(TM + TN <= SLOTS, "not enough MFMA slots to prefetch the next fragments");
+    static_assert(KSTEPS % 2 == 0, "fragment buffers alternate per k-step and must line up across tiles");
+    i32x4 af[2][TM], bf[2][TN];
+    auto load_first_frags = [&](const char* sa, const char* sb) {
 #pragma unroll
         for (int i = 0; i < TM; ++i) af[0][i] = TA::read_frag(sa, wr0 + i * 32, 0, lane);
 #pragma unroll
         for (int j = 0; j < TN; ++j) bf[0][j] = TB::read_frag(sb, wc0 + j * 32, 0, lane);
+    };
+    auto mma_tile = [&](const char* sa, const char* sb, const char* next_sa, const char* next_sb, auto fill_tag,
+                        auto cross_tag, int fill_stage, int fill_k0) {
+        constexpr bool fill = decltype(fill_tag)::value;
+        constexpr bool cross = decltype(cross_tag)::value;
 #pragma unroll
-        for (int ks = 0; ks < 4; ++ks) {
+        for (int ks = 0; ks < KSTEPS; ++ks) {
+            const bool last = ks + 1 == KSTEPS;
+            const char* ra = last ? next_sa : sa;
+            const char* rb = last ? next_sb : sb;
+            const int rks = last ? 0 : ks + 1;
 #pragma unroll
             for (int i = 0; i < TM; ++i)
 #pragma unroll
                 for (int j = 0; j < TN; ++j) {
                     const int slot = i * TN + j;
                     mfma32<IN>(af[ks & 1][i], bf[ks & 1][j], acc[i][j]);
-                    if (ks < 3) {
-                        if (slot < TM) af[(ks + 1) & 1][slot] = TA::read_frag(sa, wr0 + slot * 32, ks + 1, lane);
-                        else if (slot - TM < TN) bf[(ks + 1) & 1][slot - TM] = TB::read_frag(sb, wc0 + (slot - TM) * 32, ks + 1, lane);
+                    if (!last || cross) {
+                        // B fragments first: the first MFMAs of the next step need bf[0] and af[0]
+                        if (slot < TN) bf[(ks + 1) & 1][slot] = TB::read_frag(rb, wc0 + slot * 32, rks, lane);
+                        else if (slot - TN < TM) af[(ks + 1) & 1][slot - TN] = TA::read_frag(ra, wr0 + (slot - TN) * 32, rks, lane);
                     }
-                    if constexpr (DIRECT) {
-                        const int gslot = ks * SLOTS + slot;
-                        if (fill && gslot % SLOT_STRIDE == 0) { // compile-time after unrolling
+                    if constexpr (DIRECT && fill) {
+                        if (ks == 0) {
 #pragma unroll
                             for (int u = 0; u < FILLS_PER_SLOT; ++u) {
-                                const int f = (gslot / SLOT_STRIDE) * FILLS_PER_SLOT + u;
+                                const int f = slot * FILLS_PER_SLOT + u;
                                 if (f < FILLS) issue_fill(f, fill_stage, fill_k0);
                             }
                         }
                     }
+                    __builtin_amdgcn_sched_barrier(0);
                 }
         }
     };
-    static_assert(TM + TN <= SLOTS, "not enough MFMA slots to prefetch the next fragments");
 
     if constexpr (DIRECT) {
+        // D tiles are in flight beyond the one being computed; AHEAD of them are already
+        // published (landed and behind a barrier) when a tile starts.
+        constexpr int D = STAGES - 1;
+        constexpr int AHEAD = STAGES >= 3 ? 2 : 1;
+        constexpr bool CROSS = AHEAD >= 2;
+        constexpr int YOUNGER = (D - AHEAD) * FILLS; // fills allowed to be outstanding at the end of a tile
+        using cross_t = std::integral_constant<bool, CROSS>;
 #pragma unroll
-        for (int f = 0; f < FILLS; ++f) issue_fill(f, 0, 0);
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        for (int s = 0; s < D; ++s)
+            if (s < KT) {
+#pragma unroll
+                for (int f = 0; f < FILLS; ++f) issue_fill(f, s, s * BK);
+            }
+        if (KT >= D) wait_vmcnt<YOUNGER>();
+        else wait_vmcnt<0>();
         __syncthreads();
-        for (int kt = 0; kt < KT - 1; ++kt) {
-            const int cur = kt & 1;
-            mma_tile(smem + cur * STAGE_BYTES, smem + cur * STAGE_BYTES + TA::TILE_BYTES, std::true_type{}, cur ^ 1, (kt + 1) * BK);
-            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        if constexpr (CROSS) load_first_frags(smem, smem + TA::TILE_BYTES);
+        int kt = 0;
+        // steady state: tile kt+D exists and is fetched now
+        for (; kt + D < KT; ++kt) {
+            const char* cur = smem + (kt % STAGES) * STAGE_BYTES;
+            const char* nxt = smem + ((kt + 1) % STAGES) * STAGE_BYTES;
+            if constexpr (!CROSS) load_first_frags(cur, cur + TA::TILE_BYTES);
+            mma_tile(cur, cur + TA::TILE_BYTES, nxt, nxt + TA::TILE_BYTES, std::true_type{}, cross_t{}, (kt + D) % STAGES,
+                     (kt + D) * BK);
+            wait_vmcnt<YOUNGER>(); // tile kt+AHEAD has landed
             __syncthreads();
         }
-        {   // last tile: nothing left to fetch
-            const int cur = (KT - 1) & 1;
-            mma_tile(smem + cur * STAGE_BYTES, smem + cur * STAGE_BYTES + TA::TILE_BYTES, std::false_type{}, 0, 0);
+        // drain: nothing left to fetch (the cross prefetch of the last tile reads a stale buffer, unused)
+        for (; kt < KT; ++kt) {
+            const char* cur = smem + (kt % STAGES) * STAGE_BYTES;
+            const char* nxt = smem + ((kt + 1) % STAGES) * STAGE_BYTES;
+            if constexpr (!CROSS) load_first_frags(cur, cur + TA::TILE_BYTES);
+            mma_tile(cur, cur + TA::TILE_BYTES, nxt, nxt + TA::TILE_BYTES, std::false_type{}, cross_t{}, 0, 0);
+            if (kt + 1 < KT) {
+                wait_vmcnt<0>();
+                __syncthreads();
+            }
         }
     } else {
         i32x4 ra[TA::PER_THREAD], rb[TB::PER_THREAD];
@@ -339,7 +405,8 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64) gemm_mfma_kernel(GemmAr
                 TA::template load_global<EDGE>(ra, Ab, m0, (kt + 1) * BK, lda, p.M, p.K, tid);
                 TB::template load_global<EDGE>(rb, Bb, n0, (kt + 1) * BK, ldb, p.N, p.K, tid);
             }
-            mma_tile(cur, cur + TA::TILE_BYTES, std::false_type{}, 0, 0);
+            load_first_frags(cur, cur + TA::TILE_BYTES);
+            mma_tile(cur, cur + TA::TILE_BYTES, cur, cur + TA::TILE_BYTES, std::false_type{}, std::false_type{}, 0, 0);
             if (kt + 1 < KT) {
                 TA::store_lds(ra, nxt, tid);
                 TB::store_lds(rb, nxt + TA::TILE_BYTES, tid);
@@ -390,30 +457,28 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64) gemm_mfma_kernel(GemmAr
 }
 
 // Host launcher for one kernel instantiation.
-template <int IN, int BM, int BN, int WAVES_M, int WAVES_N, bool A_KC, bool B_KC, bool DIRECT, bool EDGE>
+template <typename Cfg>
 hipError_t launch_mfma(const GemmArgs& a, hipStream_t stream, LaunchGeom* geom, bool dry_run)
 {
-    constexpr int NT = WAVES_M * WAVES_N * 64;
-    constexpr int LDS = 2 * (BM + BN) * KTILE_BYTES;
-    auto kern = gemm_mfma_kernel<IN, BM, BN, WAVES_M, WAVES_N, A_KC, B_KC, DIRECT, EDGE>;
+    auto kern = gemm_mfma_kernel<Cfg>;
     GemmArgs args = a;
-    args.tiles_m = (a.M + BM - 1) / BM;
-    args.tiles_n = (a.N + BN - 1) / BN;
+    args.tiles_m = (a.M + Cfg::BM - 1) / Cfg::BM;
+    args.tiles_n = (a.N + Cfg::BN - 1) / Cfg::BN;
     if (geom) {
         geom->grid[0] = (unsigned)(args.tiles_m * args.tiles_n);
         geom->grid[1] = geom->grid[2] = 1;
-        geom->block[0] = NT;
+        geom->block[0] = Cfg::NT;
         geom->block[1] = geom->block[2] = 1;
-        geom->dyn_lds = LDS;
+        geom->dyn_lds = Cfg::LDS_BYTES;
     }
     if (dry_run) return hipSuccess;
     static bool attr_set = false; // per instantiation; benign if set twice
     if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
+        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES);
         if (e != hipSuccess) return e;
         attr_set = true;
     }
-    hipLaunchKernelGGL(kern, dim3(args.tiles_m * args.tiles_n), dim3(NT), LDS, stream, args);
+    hipLaunchKernelGGL(kern, dim3(args.tiles_m * args.tiles_n), dim3(Cfg::NT), Cfg::LDS_BYTES, stream, args);
     return hipGetLastError();
 }
 

@@ -10,6 +10,8 @@ struct MfmaVariant {
     bool a_kc, b_kc;     // operand has K contiguous in memory (else M/N contiguous)
     bool direct;         // tile fill with global_load_lds (else through registers)
     bool edge;           // handles M/N/K that are not tile multiples
+    int kb;              // bytes of K per tile (64 or 128)
+    int stages;          // LDS buffers
     LaunchFn launch;
 };
 

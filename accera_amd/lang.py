@@ -1,0 +1,547 @@
+"""The slice of Accera's Python DSL that describes the matmul (+ fused ReLU) hot path.
+
+Scripts written against the reference -- the README quick start
+(/root/reference/README.md:52-92) and the GPU matmul / matmul+ReLU plans of
+/root/reference/accera/python/accera/test/mfma_tests.py:58-101,359-432 -- run against
+this module with `import accera_amd as acc`:
+
+    A = acc.Array(role=acc.Role.INPUT, element_type=acc.ScalarType.float16, shape=(M, K))
+    ...
+    nest = acc.Nest(shape=(M, N, K)); i, j, k = nest.get_indices()
+    @nest.iteration_logic
+    def _(): C[i, j] += A[i, k] * B[k, j]
+    plan = nest.create_schedule().create_plan(acc.Target(acc.Target.Model.AMD_MI355X))
+    plan.tensorize(..., prologue_op=acc.MMAFragmentOp.SET, prologue_arg=0, epilogue_op=acc.MMAFragmentOp.ReLU)
+    package.add(plan, args=(A, B, C), base_name="matmul_relu")
+    package.build("pkg", format=acc.Package.Format.HAT_DYNAMIC, output_dir=...)
+
+There is no compiler behind it.  `Package.add` pattern-matches the recorded logic to
+`C[i,j] += A[i,k] * B[k,j]` optionally fused with `C[i,j] = max(C[i,j], 0)` -- exactly the
+pattern the reference's tensorization matcher accepts
+(/root/reference/accera/transforms/src/exec/ExecutionPlanToAffineLoweringPass.cpp:5986-6167) --
+and binds the function to the prebuilt gfx950 kernels of libaccera_mi355x.so; schedule and
+plan transformations (tile, reorder, cache, bind, unroll, ...) are accepted and recorded,
+because the kernels embody their own tiling, caching and binding.  Anything that is not this
+pattern raises NotImplementedError.  `Package.build` emits `<name>.hat` + `<name>.so`.
+"""
+import enum
+import hashlib
+import os
+import subprocess
+
+from . import _lib
+from . import hat as _hat
+
+
+class Role(enum.Enum):
+    INPUT = "input"
+    INPUT_OUTPUT = "input_output"
+    OUTPUT = "output"
+    CONST = "const"
+    TEMP = "temp"
+
+
+class ScalarType(enum.Enum):
+    float32 = ("float", _lib.F32)
+    float16 = ("float16_t", _lib.F16)
+    bfloat16 = ("bfloat16_t", _lib.BF16)
+    int8 = ("int8_t", _lib.I8)
+    int32 = ("int32_t", _lib.I32)
+
+    @property
+    def c_name(self):
+        return self.value[0]
+
+    @property
+    def lib_id(self):
+        return self.value[1]
+
+
+class MMAFragmentOp(enum.Enum):  # /root/reference/docs/Reference/enumerations/MMAFragmentOp.md
+    NONE = 0
+    ReLU = 1
+    ReLU_NoConditional = 2
+    SET = 3
+    SCALE = 4
+
+
+class MMAShape(enum.Enum):
+    """Accepted for source compatibility (/root/reference/accera/ir/include/value/ValueMMAOp.h:27-49);
+    the gfx950 kernels always issue the 32x32 MFMA with 32 bytes of K per step."""
+    M64xN64xK1_B4 = 0
+    M64xN64xK1_B2 = 1
+    M32xN32xK2_B1 = 2
+    M16xN16xK4_B1 = 3
+    M64xN64xK4_B4 = 4
+    M64xN64xK4_B2 = 5
+    M32xN32xK8_B1 = 6
+    M16xN16xK16_B1 = 7
+    M64xN64xK2_B4 = 8
+    M64xN64xK2_B2 = 9
+    M32xN32xK4_B1 = 10
+    M16xN16xK8_B1 = 11
+    M32xN32xK16_B1 = 12   # gfx950 native: v_mfma_f32_32x32x16_{f16,bf16}
+    M32xN32xK32_B1 = 13   # gfx950 native: v_mfma_i32_32x32x32_i8
+
+
+class MMASchedulingPolicy(enum.Enum):
+    PASS_ORDER = 0
+    BLOCK_ORDER = 1
+
+
+class CacheStrategy(enum.Enum):
+    BLOCKED = 0
+    STRIPED = 1
+
+
+class _MemorySpace(enum.Enum):
+    NONE = 0
+    GLOBAL = 1
+    SHARED = 2
+    PRIVATE = 3
+    MMA_FRAGMENT = 4
+
+
+class Target:
+    """Device description.  Only the HOST default and the MI355X GPU exist here; the
+    tensor-core table row is the gfx950 analogue of MI100_TENSORCORE_INFO
+    (/root/reference/accera/python/accera/Targets.py:748-830)."""
+
+    class Model(enum.Enum):
+        HOST = "HOST"
+        AMD_MI355X = "AMD MI355X"
+
+    class Category(enum.Enum):
+        CPU = 0
+        GPU = 1
+
+    class Runtime(enum.Enum):
+        NONE = 0
+        ROCM = 1
+
+    class _GridUnit(enum.Enum):
+        BLOCK_X = 0
+        BLOCK_Y = 1
+        BLOCK_Z = 2
+        THREAD_X = 3
+        THREAD_Y = 4
+        THREAD_Z = 5
+        WARP_X = 6
+        WARP_Y = 7
+
+    class _GridUnits:
+        def __getattr__(self, name):
+            return Target._GridUnit[name]
+
+    # (input type, output type) -> MMA shapes the hardware runs natively
+    MI355X_TENSORCORE_INFO = {
+        (ScalarType.float16, ScalarType.float32): [MMAShape.M32xN32xK16_B1],
+        (ScalarType.bfloat16, ScalarType.float32): [MMAShape.M32xN32xK16_B1],
+        (ScalarType.int8, ScalarType.int32): [MMAShape.M32xN32xK32_B1],
+        (ScalarType.float32, ScalarType.float32): [MMAShape.M32xN32xK2_B1],
+    }
+
+    def __init__(self, model=None, category=None, runtime=None):
+        if isinstance(model, str):
+            model = Target.Model(model)
+        self.model = model or Target.Model.HOST
+        gpu = self.model == Target.Model.AMD_MI355X or category == Target.Category.GPU
+        self.category = Target.Category.GPU if gpu else Target.Category.CPU
+        self.runtime = Target.Runtime.ROCM if gpu else Target.Runtime.NONE
+        self.name = self.model.value
+        self.GridUnit = Target._GridUnits()
+        self.MemorySpace = _MemorySpace
+        self.warp_size = 64
+        self.compute_units = 256
+        self.max_shared_memory_per_block = 160 * 1024
+        self.tensor_core_info = Target.MI355X_TENSORCORE_INFO
+
+
+Target.HOST = Target()
+
+
+# ---- expression recording ---------------------------------------------------------------------
+
+class Index:
+    _count = 0
+
+    def __init__(self, name=None):
+        Index._count += 1
+        self.name = name or f"i{Index._count}"
+
+    def __repr__(self):
+        return self.name
+
+
+class _Expr:
+    def __mul__(self, other):
+        return _Bin("mul", self, _wrap(other))
+
+    __rmul__ = __mul__
+
+    def __add__(self, other):
+        return _Bin("add", self, _wrap(other))
+
+    __radd__ = __add__
+
+
+class _Const(_Expr):
+    def __init__(self, v):
+        self.v = v
+
+
+class _Bin(_Expr):
+    def __init__(self, op, a, b):
+        self.op, self.a, self.b = op, a, b
+
+
+class _Cast(_Expr):
+    def __init__(self, x, t):
+        self.x, self.t = x, t
+
+
+class _Ref(_Expr):
+    def __init__(self, array, idx):
+        self.array, self.idx = array, tuple(idx)
+
+    def __iadd__(self, other):
+        return _Bin("add", self, _wrap(other))
+
+
+def _wrap(x):
+    return x if isinstance(x, _Expr) else _Const(x)
+
+
+def _strip_cast(e):
+    while isinstance(e, _Cast):
+        e = e.x
+    return e
+
+
+def max(a, b):  # noqa: A001 - mirrors acc.max
+    return _Bin("max", _wrap(a), _wrap(b))
+
+
+def min(a, b):  # noqa: A001
+    return _Bin("min", _wrap(a), _wrap(b))
+
+
+def cast(x, t):
+    return _Cast(_wrap(x), t)
+
+
+_recording = []  # stack of statement lists
+
+
+class Array:
+    class Layout(enum.Enum):
+        FIRST_MAJOR = 0   # row-major   (/root/reference/accera/python/accera/lang/Layout.py:11-33)
+        LAST_MAJOR = 1    # column-major
+        DEFERRED = 2
+
+    def __init__(self, role, element_type=ScalarType.float32, layout=None, shape=None, name="", **_):
+        if shape is None or len(shape) != 2:
+            raise NotImplementedError("this build handles 2-D arrays (matrices) only")
+        self.role = role
+        self.element_type = element_type
+        self.layout = layout or Array.Layout.FIRST_MAJOR
+        self.shape = tuple(int(s) for s in shape)
+        self.name = name
+
+    @property
+    def strides(self):
+        r, c = self.shape
+        return (c, 1) if self.layout == Array.Layout.FIRST_MAJOR else (1, r)
+
+    def __getitem__(self, idx):
+        return _Ref(self, idx)
+
+    def __setitem__(self, idx, value):
+        if not _recording:
+            raise RuntimeError("array assignment outside of an iteration_logic function")
+        _recording[-1].append((_Ref(self, idx), _wrap(value)))
+
+
+class Nest:
+    def __init__(self, shape):
+        self.shape = tuple(int(s) for s in shape)
+        self.indices = tuple(Index() for _ in self.shape)
+        self.statements = []
+
+    def get_indices(self):
+        return self.indices if len(self.indices) > 1 else self.indices[0]
+
+    def iteration_logic(self, fn):
+        _recording.append([])
+        try:
+            fn()
+        finally:
+            self.statements += _recording.pop()
+        return fn
+
+    def create_schedule(self):
+        return Schedule([self])
+
+    def create_plan(self, target=None):
+        return self.create_schedule().create_plan(target)
+
+
+class Schedule:
+    """Loop transformations are recorded, not applied: the gfx950 kernels carry their own
+    tiling (reference semantics: /root/reference/accera/python/accera/lang/Schedule.py)."""
+
+    def __init__(self, nests, fused=False, partial=None):
+        self.nests = nests
+        self.fused = fused
+        self.partial = partial
+        self.commands = []
+        if fused:
+            # fused indices, then the fusing index f, then the unfused ones (Schedule.py:522-628)
+            first = nests[0]
+            self.indices = list(first.indices[:partial]) + [Index("f")] + [ix for n in nests for ix in n.indices[partial:]]
+        else:
+            self.indices = list(nests[0].indices)
+
+    def get_indices(self):
+        return tuple(self.indices)
+
+    def split(self, index, size):
+        inner = Index(f"{index.name}i")
+        self.indices.insert(self.indices.index(index) + 1, inner)
+        self.commands.append(("split", index, size))
+        return inner
+
+    def tile(self, shape):
+        return tuple(self.split(ix, sz) for ix, sz in shape.items())
+
+    def reorder(self, *order):
+        order = order[0] if len(order) == 1 and isinstance(order[0], (tuple, list)) else order
+        self.commands.append(("reorder", tuple(order)))
+        self.indices = list(order)
+
+    def skew(self, *a, **k):
+        self.commands.append(("skew", a, k))
+
+    def pad(self, *a, **k):
+        self.commands.append(("pad", a, k))
+
+    def create_plan(self, target=None):
+        return Plan(self, target or Target.HOST)
+
+
+def fuse(*schedules, partial=None):
+    scheds = schedules[0] if len(schedules) == 1 and isinstance(schedules[0], (tuple, list)) else schedules
+    nests = [n for s in scheds for n in s.nests]
+    if partial is None:
+        partial = len(nests[0].shape)
+    return Schedule(nests, fused=True, partial=partial)
+
+
+class Plan:
+    """Execution-plan calls of the reference (Plan.py:134-703, 793-956).  `tensorize` carries
+    semantics (prologue / epilogue op); the rest selects nothing here and is recorded."""
+
+    def __init__(self, schedule, target):
+        self.schedule = schedule
+        self.target = target
+        self.commands = []
+        self.prologue_op, self.prologue_arg = MMAFragmentOp.NONE, 0
+        self.epilogue_op, self.epilogue_arg = MMAFragmentOp.NONE, 0
+
+    def tensorize(self, indices, mma_shape=None, use_static_offsets=False, num_total_passes=1, num_fused_passes=None,
+                  scheduling_policy=MMASchedulingPolicy.PASS_ORDER, prologue_op=MMAFragmentOp.NONE, prologue_arg=0,
+                  epilogue_op=MMAFragmentOp.NONE, epilogue_arg=0, **_):
+        if prologue_op not in (MMAFragmentOp.NONE, MMAFragmentOp.SET) or (prologue_op == MMAFragmentOp.SET and prologue_arg != 0):
+            raise NotImplementedError("prologue must be NONE or SET 0")
+        if epilogue_op not in (MMAFragmentOp.NONE, MMAFragmentOp.ReLU, MMAFragmentOp.ReLU_NoConditional):
+            raise NotImplementedError("epilogue must be NONE, ReLU or ReLU_NoConditional")
+        self.prologue_op, self.prologue_arg = prologue_op, prologue_arg
+        self.epilogue_op, self.epilogue_arg = epilogue_op, epilogue_arg
+        self.commands.append(("tensorize", mma_shape, num_total_passes))
+
+    def _record(name):
+        def f(self, *a, **k):
+            self.commands.append((name, a, k))
+            return None
+        return f
+
+    cache = _record("cache")
+    bind = _record("bind")
+    unroll = _record("unroll")
+    vectorize = _record("vectorize")
+    parallelize = _record("parallelize")
+    kernelize = _record("kernelize")
+    del _record
+
+
+# ---- pattern match to the GEMM (+ReLU) hot path -------------------------------------------------
+
+class _GemmSpec:
+    def __init__(self, A, B, C, M, N, K, prologue, epilogue):
+        self.A, self.B, self.C, self.M, self.N, self.K = A, B, C, M, N, K
+        self.prologue, self.epilogue = prologue, epilogue
+
+
+def _match(source):
+    plan = source if isinstance(source, Plan) else None
+    sched = plan.schedule if plan else (source if isinstance(source, Schedule) else source.create_schedule())
+    nests = sched.nests
+    unsupported = NotImplementedError(
+        "this build compiles exactly one pattern: C[i,j] += A[i,k] * B[k,j], optionally fused with C[i,j] = max(C[i,j], 0)")
+    if len(nests) not in (1, 2) or len(nests[0].shape) != 3 or len(nests[0].statements) != 1:
+        raise unsupported
+    mm = nests[0]
+    i, j, k = mm.indices
+    dst, val = mm.statements[0]
+    val = _strip_cast(val)
+    if not (isinstance(val, _Bin) and val.op == "add"):
+        raise unsupported
+    acc_ref, prod = _strip_cast(val.a), _strip_cast(val.b)
+    if not (isinstance(acc_ref, _Ref) and acc_ref.array is dst.array and acc_ref.idx == (i, j) and dst.idx == (i, j)):
+        raise unsupported
+    if not (isinstance(prod, _Bin) and prod.op == "mul"):
+        raise unsupported
+    a, b = _strip_cast(prod.a), _strip_cast(prod.b)
+    if not (isinstance(a, _Ref) and isinstance(b, _Ref)):
+        raise unsupported
+    if a.idx == (k, j) and b.idx == (i, k):
+        a, b = b, a
+    if a.idx != (i, k) or b.idx != (k, j):
+        raise unsupported
+    M, N, K = mm.shape
+    A, B, C = a.array, b.array, dst.array
+    if A.shape != (M, K) or B.shape != (K, N) or C.shape != (M, N):
+        raise ValueError(f"array shapes {A.shape}, {B.shape}, {C.shape} do not match the nest {mm.shape}")
+    epilogue = _lib.EPILOGUE_NONE
+    if len(nests) == 2:
+        relu = nests[1]
+        if not (sched.fused and sched.partial == 2 and relu.shape == (M, N) and len(relu.statements) == 1):
+            raise unsupported
+        i2, j2 = relu.indices
+        rdst, rval = relu.statements[0]
+        rval = _strip_cast(rval)
+        ok = (rdst.array is C and rdst.idx == (i2, j2) and isinstance(rval, _Bin) and rval.op == "max")
+        if ok:
+            x, z = _strip_cast(rval.a), _strip_cast(rval.b)
+            if isinstance(x, _Const):
+                x, z = z, x
+            ok = isinstance(x, _Ref) and x.array is C and x.idx == (i2, j2) and isinstance(z, _Const) and z.v == 0
+        if not ok:
+            raise unsupported
+        epilogue = _lib.EPILOGUE_RELU
+    prologue = _lib.PROLOGUE_NONE
+    if plan:
+        if plan.prologue_op == MMAFragmentOp.SET:
+            prologue = _lib.PROLOGUE_SET0
+        if plan.epilogue_op == MMAFragmentOp.ReLU:
+            epilogue = _lib.EPILOGUE_RELU
+        elif plan.epilogue_op == MMAFragmentOp.ReLU_NoConditional:
+            epilogue = _lib.EPILOGUE_RELU_NOCOND
+    return _GemmSpec(A, B, C, M, N, K, prologue, epilogue)
+
+
+# ---- package -------------------------------------------------------------------------------------
+
+class Package:
+    class Format(enum.Flag):
+        HAT_DYNAMIC = enum.auto()
+        HAT_STATIC = enum.auto()
+        MLIR = enum.auto()
+        DEFAULT = HAT_DYNAMIC
+
+    class Mode(enum.Enum):
+        RELEASE = "Release"
+        DEBUG = "Debug"
+
+    class Platform(enum.Enum):
+        HOST = "host"
+        LINUX = "linux"
+
+    def __init__(self):
+        self._functions = []
+        self._description = {}
+
+    def add(self, source, args, base_name="", parameters=None, function_opts=None, auxiliary=None):
+        """Bind one function to the package; returns its full name `<base_name>_<16 hex>`
+        (/root/reference/accera/python/accera/Package.py:203-259, 310-335)."""
+        spec = _match(source)
+        args = tuple(args)
+        if set(map(id, args)) != {id(spec.A), id(spec.B), id(spec.C)} or len(args) != 3:
+            raise ValueError("args must be exactly the three arrays used by the nest")
+        if spec.A.element_type != spec.B.element_type:
+            raise ValueError("A and B must have the same element type")
+        sig = repr((base_name, [(a.role.value, a.element_type.c_name, a.shape, a.layout.name) for a in args],
+                    spec.prologue, spec.epilogue, sorted((parameters or {}).items())))
+        name = f"{base_name}_{hashlib.md5(sig.encode()).hexdigest()[:16]}"
+        self._functions.append(dict(name=name, base_name=base_name, spec=spec, args=args, auxiliary=auxiliary or {},
+                                    parameters=parameters or {}))
+        return name
+
+    def add_description(self, author=None, license=None, other=None, version=None):
+        self._description.update({k: v for k, v in dict(author=author, license=license, version=version).items() if v})
+        self._description.setdefault("other", {}).update(other or {})
+
+    def _stub_source(self):
+        lines = ["/* generated by accera_amd.Package.build: HAT entry points forwarding to libaccera_mi355x.so */",
+                 "#include <stdint.h>", "#include <stdio.h>", '#include "accera_mi355x_gemm.h"', ""]
+        for f in self._functions:
+            s = f["spec"]
+            order = {id(a): n for a, n in zip(f["args"], ("a0", "a1", "a2"))}
+            pa, pb, pc = order[id(s.A)], order[id(s.B)], order[id(s.C)]
+            call_args = (f"{s.A.element_type.lib_id}, {s.C.element_type.lib_id}, {s.M}, {s.N}, {s.K}, "
+                         f"{pa}, {s.A.strides[0]}, {s.A.strides[1]}, {pb}, {s.B.strides[0]}, {s.B.strides[1]}, "
+                         f"{pc}, {s.C.strides[0]}, {s.C.strides[1]}, {s.prologue}, {s.epilogue}")
+            lines += [
+                f"void {f['name']}(void* a0, void* a1, void* a2)", "{",
+                f"    if (acc950_gemm_relu_host({call_args}) != ACC950_OK)",
+                f"        fprintf(stderr, \"{f['name']}: %s\\n\", acc950_last_error());", "}",
+                "/* same function on device pointers, asynchronous on `stream` (hipStream_t or NULL) */",
+                f"int {f['name']}__device(void* a0, void* a1, void* a2, void* stream)", "{",
+                f"    return acc950_gemm_relu({call_args}, stream);", "}", ""]
+        return "\n".join(lines)
+
+    def build(self, name, format=None, mode=None, platform=None, tolerance=1e-5, output_dir=None, **_):
+        """Emit `<output_dir>/<name>.hat` and `<name>.so` (HAT_DYNAMIC).  Returns the list of
+        files written (Package.py:551-788 returns the same kind of list)."""
+        fmt = format or Package.Format.DEFAULT
+        if not (fmt & Package.Format.HAT_DYNAMIC):
+            raise NotImplementedError("only Package.Format.HAT_DYNAMIC is produced by this build")
+        output_dir = os.path.abspath(output_dir or os.getcwd())
+        os.makedirs(output_dir, exist_ok=True)
+        if not os.path.exists(_lib.LIB_PATH):
+            raise RuntimeError(f"{_lib.LIB_PATH} is missing; build the kernel library first")
+        c_path = os.path.join(output_dir, f"{name}.c")
+        so_path = os.path.join(output_dir, f"{name}.so")
+        hat_path = os.path.join(output_dir, f"{name}.hat")
+        with open(c_path, "w") as f:
+            f.write(self._stub_source())
+        rel = os.path.relpath(_lib.LIB_DIR, output_dir)
+        cmd = ["gcc", "-shared", "-fPIC", "-O2", "-o", so_path, c_path, f"-I{_lib.INCLUDE_DIR}", f"-L{_lib.LIB_DIR}",
+               "-laccera_mi355x", f"-Wl,-rpath,$ORIGIN/{rel}", f"-Wl,-rpath,{_lib.LIB_DIR}"]
+        subprocess.check_call(cmd)
+
+        functions = []
+        for f in self._functions:
+            s = f["spec"]
+            arguments = []
+            for a in f["args"]:
+                ct = a.element_type.c_name
+                arguments.append(_hat.Argument(name=a.name, declared_type=f"{ct}*", element_type=ct, usage=a.role.value,
+                                               shape=list(a.shape), affine_map=list(a.strides)))
+            grid, block, lds, variant = _lib.launch_geometry(s.A.element_type.lib_id, s.C.element_type.lib_id, s.M, s.N, s.K,
+                                                             s.A.strides, s.B.strides, s.C.strides)
+            aux = {"accera": {"base_name": f["base_name"], "parameters": {k: str(v) for k, v in f["parameters"].items()}},
+                   # structural counterpart of the device-function record of the reference's GPU packages
+                   # (Package.py:714-743): launch geometry of the kernel behind this entry point
+                   "accera_mi355x": {"device_entry": f"{f['name']}__device", "kernel": _lib.variant_name(variant),
+                                     "launch_parameters": grid + block, "dynamic_shared_mem_bytes": lds,
+                                     "prologue": s.prologue, "epilogue": s.epilogue}}
+            aux.update(f["auxiliary"])
+            functions.append(_hat.Function(name=f["name"], base_name=f["base_name"], arguments=arguments, auxiliary=aux))
+        _hat.write_hat(hat_path, name, functions, link_target=f"{name}.so",
+                       author=self._description.get("author", ""), version=self._description.get("version", ""),
+                       license_url=self._description.get("license", ""),
+                       required_gpu={"runtime": "ROCM", "model": "AMD MI355X", "instruction_set_version": "gfx950"},
+                       compiled_with={"compiler": "hipcc (kernels), gcc (entry points)", "flags": "--offload-arch=gfx950 -O3",
+                                      "libraries": ["libaccera_mi355x.so"]})
+        return [hat_path, so_path]

@@ -6,6 +6,8 @@ reference's own tests use (rtol 1e-3 for fp32 output of fp16/bf16 inputs, 1e-2 f
 fp16/bf16 output: mfma_tests.py:2047,2083,2553-2577), with signed data so that ReLU
 really clips (the reference's ReLU tests use non-negative inputs only).
 """
+import re
+
 import numpy as np
 import pytest
 
@@ -58,11 +60,12 @@ def _variants(b_layout):
 @pytest.mark.parametrize("in_type,out_type", [("f16", "f32"), ("bf16", "bf16"), ("i8", "i32")])
 @pytest.mark.parametrize("b_layout", ["row", "col"])
 def test_mfma_all_variants(in_type, out_type, b_layout):
-    bk = 128 if in_type == "i8" else 64
     for v, name in _variants(b_layout):
         print("variant", v, name, in_type, b_layout, flush=True)
-        # two tiles in each direction, three K tiles (odd count exercises both LDS buffers)
-        run_case(in_type, out_type, 512, 512, 3 * bk, b_layout=b_layout, variant=v, seed=v)
+        # two tiles in each direction; K tile counts below, at and above the pipeline depth
+        kb = int(re.search(r"kb(\d+)", name).group(1)) // (1 if in_type == "i8" else 2)
+        for k_tiles in (1, 2, 3, 7):
+            run_case(in_type, out_type, 512, 512, k_tiles * kb, b_layout=b_layout, variant=v, seed=v + k_tiles)
         if "edge" in name:
             # ragged M, N (multiple of the 16-byte vector only) and a K tail
             run_case(in_type, out_type, 200, 144, 336 if in_type == "i8" else 176, b_layout=b_layout, variant=v, seed=100 + v)

@@ -1,0 +1,228 @@
+"""HAT package boundary: the DSL slice records the README quick start, Package.build emits a
+.hat that is valid TOML *and* a valid C header, and the hatlib-style loader validates
+arguments.  The GPU-marked tests call the package functions on NumPy arrays."""
+import os
+import subprocess
+
+import numpy as np
+import pytest
+
+import accera_amd as acc
+import oracle as ora
+from accera_amd import hat
+
+
+def _quickstart_package(tmp, M=512, N=512, K=512):
+    """README.md:52-92, with `import accera_amd as acc`."""
+    A = acc.Array(role=acc.Role.INPUT, shape=(M, K))
+    B = acc.Array(role=acc.Role.INPUT, shape=(K, N))
+    C = acc.Array(role=acc.Role.INPUT_OUTPUT, shape=(M, N))
+    matmul = acc.Nest(shape=(M, N, K))
+    i1, j1, k1 = matmul.get_indices()
+
+    @matmul.iteration_logic
+    def _():
+        C[i1, j1] += A[i1, k1] * B[k1, j1]
+
+    relu = acc.Nest(shape=(M, N))
+    i2, j2 = relu.get_indices()
+
+    @relu.iteration_logic
+    def _():
+        C[i2, j2] = acc.max(C[i2, j2], 0.0)
+
+    package = acc.Package()
+    schedule = acc.fuse(matmul.create_schedule(), relu.create_schedule(), partial=2)
+    package.add(schedule, args=(A, B, C), base_name="matmul_relu_fusion_naive")
+    i, j, f, k = schedule.get_indices()
+    ii, jj = schedule.tile({i: 16, j: 16})
+    schedule.reorder(j, i, f, k, jj, ii)
+    plan = schedule.create_plan()
+    plan.unroll(ii)
+    package.add(plan, args=(A, B, C), base_name="matmul_relu_fusion_transformed")
+    files = package.build(name="hello_accera", format=acc.Package.Format.HAT_DYNAMIC, output_dir=str(tmp))
+    return files
+
+
+def _gpu_plan_package(tmp, in_t, out_t, M, N, K, b_layout=None, epilogue=None, base_name="matmul_relu"):
+    """mfma_tests.py:359-432 (`_matmul_relu`): tensorized plan with SET prologue and ReLU epilogue."""
+    target = acc.Target(acc.Target.Model.AMD_MI355X)
+    A = acc.Array(role=acc.Role.INPUT, element_type=in_t, shape=(M, K))
+    B = acc.Array(role=acc.Role.INPUT, element_type=in_t, shape=(K, N), layout=b_layout or acc.Array.Layout.FIRST_MAJOR)
+    C = acc.Array(role=acc.Role.INPUT_OUTPUT, element_type=out_t, shape=(M, N))
+    nest = acc.Nest(shape=(M, N, K))
+    i, j, k = nest.get_indices()
+
+    @nest.iteration_logic
+    def _():
+        C[i, j] += A[i, k] * B[k, j]
+
+    schedule = nest.create_schedule()
+    ii, jj, kk = schedule.tile({i: 16, j: 16, k: 16})
+    schedule.reorder(i, j, k, ii, jj, kk)
+    plan = schedule.create_plan(target)
+    plan.bind({i: target.GridUnit.BLOCK_Y, j: target.GridUnit.BLOCK_X, ii: target.GridUnit.WARP_Y, jj: target.GridUnit.WARP_X})
+    plan.tensorize(indices=(ii, jj, kk), mma_shape=acc.MMAShape.M32xN32xK16_B1, prologue_op=acc.MMAFragmentOp.SET,
+                   prologue_arg=0, epilogue_op=epilogue or acc.MMAFragmentOp.ReLU)
+    plan.cache(A, index=ii, double_buffer=True, location=target.MemorySpace.SHARED)
+    plan.cache(C, index=ii, location=target.MemorySpace.MMA_FRAGMENT)
+    package = acc.Package()
+    name = package.add(plan, args=(A, B, C), base_name=base_name)
+    files = package.build(name="gpu_pkg", output_dir=str(tmp))
+    return files, name
+
+
+def test_quickstart_builds_a_valid_hat(tmp_path):
+    hat_path, so_path = _quickstart_package(tmp_path)
+    assert os.path.exists(hat_path) and os.path.exists(so_path)
+    doc = hat.parse(hat_path)
+    fns = doc["functions"]
+    assert len(fns) == 2
+    for name, rec in fns.items():
+        assert rec["name"] == name and rec["calling_convention"] == "cdecl"
+        assert name.rsplit("_", 1)[0] in ("matmul_relu_fusion_naive", "matmul_relu_fusion_transformed")
+        assert len(name.rsplit("_", 1)[1]) == 16
+        usages = [a["usage"] for a in rec["arguments"]]
+        assert usages == ["input", "input", "input_output"]
+        for a in rec["arguments"]:
+            # docs/Tutorials/Optimized_MatMul.md:176-187: row-major 2-D float arrays
+            assert a["logical_type"] == "affine_array" and a["declared_type"] == "float*" and a["element_type"] == "float"
+            assert a["shape"] == [512, 512] and a["affine_map"] == [512, 1] and a["affine_offset"] == 0
+        assert rec["return"]["declared_type"] == "void"
+        aux = rec["auxiliary"]["accera_mi355x"]
+        assert len(aux["launch_parameters"]) == 6 and aux["epilogue"] == acc.EPILOGUE_RELU and aux["prologue"] == acc.PROLOGUE_NONE
+    assert doc["dependencies"]["link_target"] == "hello_accera.so"
+    assert doc["target"]["required"]["GPU"]["instruction_set_version"] == "gfx950"
+    assert "void (*matmul_relu_fusion_naive)(float*, float*, float*)" in doc["declaration"]["code"]
+
+
+def test_hat_is_a_valid_c_header_and_links(tmp_path):
+    """Second class of callers: C programs that include the .hat and call the alias
+    (docs/Tutorials/Hello_MatMul.md:165-237).  Compile and link only; running needs a GPU."""
+    hat_path, so_path = _quickstart_package(tmp_path)
+    main_c = tmp_path / "main.c"
+    main_c.write_text('#include "hello_accera.hat"\n'
+                      "static float A[512*512], B[512*512], C[512*512];\n"
+                      "int main(int argc, char** argv) { if (argc > 1) matmul_relu_fusion_transformed(A, B, C); return 0; }\n")
+    exe = tmp_path / "main"
+    subprocess.check_call(["gcc", "-o", str(exe), str(main_c), f"-I{tmp_path}", str(so_path),
+                           f"-Wl,-rpath,{tmp_path}"])
+    subprocess.check_call([str(exe)])  # argc == 1: loads every library, calls nothing
+    subprocess.check_call(["g++", "-fsyntax-only", "-x", "c++", str(main_c), f"-I{tmp_path}"])
+
+
+def test_column_major_and_types_are_recorded(tmp_path):
+    (hat_path, _), name = _gpu_plan_package(tmp_path, acc.ScalarType.bfloat16, acc.ScalarType.bfloat16, 4096, 3072, 768,
+                                            b_layout=acc.Array.Layout.LAST_MAJOR)
+    rec = hat.parse(hat_path)["functions"][name]
+    a, b, c = rec["arguments"]
+    assert a["element_type"] == "bfloat16_t" and a["declared_type"] == "bfloat16_t*"
+    assert b["shape"] == [768, 3072] and b["affine_map"] == [1, 768]     # column-major B
+    assert c["affine_map"] == [3072, 1]
+    aux = rec["auxiliary"]["accera_mi355x"]
+    assert "B=col-major" in aux["kernel"] and aux["prologue"] == acc.PROLOGUE_SET0 and aux["epilogue"] == acc.EPILOGUE_RELU
+    assert aux["dynamic_shared_mem_bytes"] > 0 and aux["device_entry"] == name + "__device"
+
+
+def test_only_the_matmul_pattern_is_accepted():
+    A = acc.Array(role=acc.Role.INPUT, shape=(8, 8))
+    B = acc.Array(role=acc.Role.INPUT, shape=(8, 8))
+    C = acc.Array(role=acc.Role.INPUT_OUTPUT, shape=(8, 8))
+    nest = acc.Nest(shape=(8, 8, 8))
+    i, j, k = nest.get_indices()
+
+    @nest.iteration_logic
+    def _():
+        C[i, j] += A[i, k] + B[k, j]  # not a product
+
+    with pytest.raises(NotImplementedError):
+        acc.Package().add(nest, args=(A, B, C), base_name="bad")
+    nest2 = acc.Nest(shape=(8, 8, 8))
+    i, j, k = nest2.get_indices()
+
+    @nest2.iteration_logic
+    def _():
+        C[i, j] += A[i, k] * B[j, k]  # B indexed (j, k): not B[k, j]
+
+    with pytest.raises(NotImplementedError):
+        acc.Package().add(nest2, args=(A, B, C), base_name="bad")
+
+
+def test_loader_validates_arguments_before_calling(tmp_path):
+    hat_path, _ = _quickstart_package(tmp_path, 64, 64, 64)
+    pkg, functions = hat.load(hat_path)
+    assert set(n.rsplit("_", 1)[0] for n in functions.names if n[-1].isdigit() or True) >= {"matmul_relu_fusion_naive"}
+    f = functions["matmul_relu_fusion_transformed"]     # alias -> first function with that base name
+    assert f is functions[f.name] and f.name.startswith("matmul_relu_fusion_transformed_")
+    A = np.zeros((64, 64), np.float32)
+    with pytest.raises(ValueError, match="expected 3 arguments"):
+        f(A, A)
+    with pytest.raises(ValueError, match="dtype"):
+        f(A.astype(np.float64), A, A)
+    with pytest.raises(ValueError, match="shape"):
+        f(np.zeros((64, 32), np.float32), A, A)
+    with pytest.raises(ValueError, match="strides"):
+        f(np.asfortranarray(np.ones((64, 64), np.float32)), A, A)
+    with pytest.raises(TypeError):
+        f([1, 2], A, A)
+
+
+# ---------------------------------------------------------------------------------------------
+@pytest.mark.gpu
+def test_readme_quickstart_end_to_end(tmp_path):
+    """README.md:118-136, verbatim apart from the import."""
+    hat_path, _ = _quickstart_package(tmp_path)
+    _, functions = hat.load(hat_path)
+    rng = np.random.default_rng(1001)
+    A_test = rng.random((512, 512)).astype(np.float32)
+    B_test = rng.random((512, 512)).astype(np.float32)
+    for base in ("matmul_relu_fusion_transformed", "matmul_relu_fusion_naive"):
+        C_test = np.zeros((512, 512)).astype(np.float32)
+        C_numpy = np.maximum(C_test + A_test @ B_test, 0.0)
+        functions[base](A_test, B_test, C_test)
+        np.testing.assert_allclose(C_test, C_numpy, atol=1e-3)
+    # the function accumulates into C (no SET prologue): signed data, non-zero C
+    A_s, B_s = (A_test - 0.5), (B_test - 0.5)
+    C0 = rng.standard_normal((512, 512)).astype(np.float32)
+    C_test = C0.copy()
+    functions["matmul_relu_fusion_naive"](A_s, B_s, C_test)
+    want = ora.gemm_relu_exact(A_s, B_s, C0, "f32", "f32", ora.PRO_NONE, ora.EPI_RELU)
+    np.testing.assert_allclose(C_test, want, atol=1e-3)
+    assert (C_test == 0).any() and (C_test > 0).any()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("in_t,out_t,shape,b_layout", [
+    (acc.ScalarType.float16, acc.ScalarType.float32, (256, 384, 512), None),
+    (acc.ScalarType.bfloat16, acc.ScalarType.bfloat16, (256, 256, 192), acc.Array.Layout.LAST_MAJOR),
+    (acc.ScalarType.int8, acc.ScalarType.int32, (256, 256, 256), None),
+    (acc.ScalarType.float16, acc.ScalarType.float16, (8, 1024, 512), None),
+    (acc.ScalarType.float32, acc.ScalarType.float32, (16, 16, 16), None),     # mfma_tests.py:2579-2602 sizes
+    (acc.ScalarType.float32, acc.ScalarType.float32, (128, 128, 16), None),
+])
+def test_tensorized_plan_package_on_numpy_arrays(tmp_path, in_t, out_t, shape, b_layout):
+    M, N, K = shape
+    (hat_path, _), name = _gpu_plan_package(tmp_path, in_t, out_t, M, N, K, b_layout)
+    _, functions = hat.load(hat_path)
+    tn = {acc.ScalarType.float16: "f16", acc.ScalarType.bfloat16: "bf16", acc.ScalarType.int8: "i8",
+          acc.ScalarType.float32: "f32", acc.ScalarType.int32: "i32"}
+    it, ot = tn[in_t], tn[out_t]
+    from tests.util import assert_matches, make_input
+    rng = np.random.default_rng(5)
+    A, B = make_input(rng, (M, K), it), make_input(rng, (K, N), it)
+    if b_layout is not None:
+        B = np.asfortranarray(B)
+    C = np.full((M, N), 3, ora.NP_STORAGE[ot])   # SET prologue: the old content must not matter
+    functions[name](A, B, C)
+    assert_matches(C, ora.gemm_relu_exact(A, B, None, it, ot), ot, K)
+
+
+@pytest.mark.gpu
+def test_run_benchmark_reports_hatlib_style_rows(tmp_path):
+    hat_path, _ = _quickstart_package(tmp_path, 256, 256, 256)
+    results = hat.run_benchmark(hat_path, batch_size=5, min_time_in_sec=0.2, input_sets_minimum_size_MB=2)
+    assert len(results) == 2
+    for r in results:
+        assert r.function_name.startswith("matmul_relu_fusion_")
+        assert 0 < r.min_of_means <= r.median_of_means and r.min_of_means <= r.mean
+        assert r.mean_of_small_means <= r.mean and r.robust_mean > 0
