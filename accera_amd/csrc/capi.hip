@@ -122,6 +122,8 @@ bool skinny_can_take(const Problem& pb)
     if (g.M < 1 || g.M > 8 || g.N < 8 || g.K < 2) return false;
     if (g.a_cs != 1 || g.b_cs != 1 || g.c_cs != 1) return false;
     if (g.N % 8 || g.K % 2 || g.b_rs % 8 || g.a_rs % 2) return false;
+    // per-lane offsets of the direct-to-LDS fills are 32-bit
+    if ((int64_t)g.K * g.b_rs * 2 >= (1ll << 32) || (int64_t)8 * g.a_rs * 2 >= (1ll << 32)) return false;
     if (pb.have_pointers && (!aligned16(g.B) || (reinterpret_cast<uintptr_t>(g.A) & 3u))) return false;
     return true;
 }
@@ -159,10 +161,12 @@ int auto_skinny_variant(const GemmArgs&) { return 0; }
 
 int auto_skinny_splits(int variant, const GemmArgs& g)
 {
-    // enough workgroups to cover 256 CUs several times over, at least 128 k rows each
+    // One workgroup per column block streams all of K unless that leaves most CUs idle;
+    // splitting K costs a trip through the scratch buffer, so it is only used to reach
+    // about one workgroup per CU, with at least 256 k rows per slice.
     const int blocks = skinny_column_blocks(variant, g.N);
-    int splits = (2048 + blocks - 1) / blocks;
-    const int max_splits = g.K / 128 > 0 ? g.K / 128 : 1;
+    int splits = blocks >= 128 ? 1 : (256 + blocks - 1) / blocks;
+    const int max_splits = g.K / 256 > 0 ? g.K / 256 : 1;
     if (splits > max_splits) splits = max_splits;
     if (splits < 1) splits = 1;
     return splits;
@@ -400,9 +404,9 @@ int acc950_variant_name(int variant, char* buf, size_t buf_len)
         return ACC950_OK;
     }
     if (variant >= ACC950_VARIANT_SKINNY_BASE && variant < ACC950_VARIANT_SKINNY_BASE + skinny_num_variants()) {
-        int lpr, waves;
-        skinny_variant_info(variant - ACC950_VARIANT_SKINNY_BASE, &lpr, &waves);
-        std::snprintf(buf, buf_len, "skinny cols/wg=%d waves=%d", lpr * 8, waves);
+        int lpr, waves, depth;
+        skinny_variant_info(variant - ACC950_VARIANT_SKINNY_BASE, &lpr, &waves, &depth);
+        std::snprintf(buf, buf_len, "skinny cols/wg=%d waves=%d depth=%d", lpr * 8, waves, depth);
         return ACC950_OK;
     }
     int n = 0;

@@ -9,14 +9,18 @@
 //
 // Work split
 //   * grid.x = column blocks of CB = 8*LPR columns, grid.y = K splits.
-//   * inside a wave, lane = kp*LPR + cg: cg picks 8 adjacent columns (one 16-byte load
-//     per B row), kp picks a pair of adjacent k rows, so a wave instruction pair
-//     covers 2*(64/LPR) rows x CB columns; rows are dealt round-robin to the waves.
+//   * inside a wave, lane = kp*LPR + cg: cg picks 8 adjacent columns (16 bytes of a B
+//     row), kp picks a pair of adjacent k rows, so one wave step covers 2*(64/LPR) rows
+//     x CB columns; steps are dealt round-robin to the waves of the workgroup.
+//   * every wave is an independent streaming engine: it owns a ring of DEPTH slots in
+//     LDS and fills them with global_load_lds (no staging registers): per step two
+//     16-byte-per-lane loads for the two B rows and one 4-byte-per-lane load for the
+//     matching A pairs, laid out [k pair][m].  DEPTH steps are in flight per wave at all
+//     times (s_waitcnt vmcnt(3*(DEPTH-1)) admits the oldest), which is what hides the
+//     HBM latency; there is no barrier in the streaming phase.
 //   * two k rows are interleaved with v_perm_b32 into (k, k+1) half pairs and
 //     multiplied with the matching A pair by v_dot2_f32_f16 / v_dot2_f32_bf16
 //     (2 MACs per lane per instruction, fp32 accumulate): 8x8 accumulators per lane.
-//   * A (at most 8 x K) is staged once per workgroup in LDS as [k pair][m] so that a
-//     lane fetches its 8 pairs with two ds_read_b128.
 //   * at the end the 64/LPR partial sums held by different lanes are combined with a
 //     halving butterfly (each step exchanges half of the live values with the lane
 //     32, 16, 8 ... away), then across waves through LDS, then -- when the K range is
@@ -42,16 +46,18 @@ __device__ __forceinline__ float dot2(unsigned a, unsigned b, float c)
     }
 }
 
-// LPR: lanes per B row segment (8 columns each); WAVES: waves per workgroup.
-template <bool BF16, int LPR, int WAVES>
+// LPR: lanes per B row segment (8 columns each); WAVES: waves per workgroup;
+// DEPTH: ring slots (steps in flight) per wave.
+template <bool BF16, int LPR, int WAVES, int DEPTH>
 __global__ void __launch_bounds__(WAVES * 64) gemm_skinny_kernel(SkinnyArgs p)
 {
-    constexpr int NT = WAVES * 64;
-    constexpr int NKP = 64 / LPR;        // k pairs per wave instruction
+    constexpr int NKP = 64 / LPR;        // k pairs per wave step
     constexpr int CB = LPR * 8;          // columns per workgroup
     constexpr int VPL = 64 / NKP;        // values per lane after the butterfly
+    constexpr int SLOT_BYTES = 2048 + 256; // two B rows (64 lanes x 16 B each) + A pairs (64 x 4 B)
+    constexpr int RING_BYTES = DEPTH * SLOT_BYTES;
+    static_assert(3 * (DEPTH - 1) < 64, "vmcnt is a 6-bit counter");
     extern __shared__ __attribute__((aligned(16))) char smem[];
-    unsigned* sA = (unsigned*)smem;      // [k pair][8] half pairs
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int kp = lane / LPR, cg = lane % LPR;
@@ -65,15 +71,35 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_skinny_kernel(SkinnyArgs p)
     const int pair_end = min(pair_begin + pairs_per_split, pairs_total);
     const int npairs = max(pair_end - pair_begin, 0);
 
-    // stage A[0..8) x [2*pair_begin, 2*pair_end) as [pair][m]; rows >= M are zero
-    const unsigned* A32 = (const unsigned*)p.A;
-    for (int e = tid; e < npairs * 8; e += NT) {
-        int m = e / npairs, pr = e % npairs;
-        unsigned v = 0;
-        if (m < p.M) v = A32[((int64_t)m * p.a_rs) / 2 + pair_begin + pr];
-        sA[pr * 8 + m] = v;
-    }
-    __syncthreads();
+    constexpr int STEP = WAVES * NKP; // k pairs per workgroup pass
+    const int iters = (npairs + STEP - 1) / STEP;
+
+    // wave-private ring in LDS
+    char* ring = smem + wave * RING_BYTES;
+    const unsigned ring_addr = __builtin_amdgcn_readfirstlane((unsigned)(size_t)(ACC950_LDS char*)ring);
+
+    // per-lane global byte offsets relative to the (uniform) base of a step; lanes outside
+    // the matrix fetch a valid address (column 0 / pair 0) and are masked at the MACs
+    const int64_t row_bytes = p.b_rs * 2;
+    const char* Bb = (const char*)p.B + (int64_t)(2 * pair_begin) * row_bytes;
+    const char* Ab = (const char*)p.A + (int64_t)pair_begin * 4;
+    const int am = lane & 7, akp = lane >> 3;            // A fill: lane -> (pair akp of the step, row am)
+    auto issue = [&](int it, int slot) {
+        const int pr = it * STEP + wave * NKP + kp;      // this lane's pair for B
+        const int prc = pr < npairs ? pr : 0;
+        const unsigned boff = (unsigned)((int64_t)(2 * prc) * row_bytes + (int64_t)(col_ok ? col0 : 0) * 2);
+        const int apr = it * STEP + wave * NKP + (akp < NKP ? akp : 0);
+        const int aprc = apr < npairs ? apr : 0;
+        const unsigned aoff = (unsigned)((int64_t)(am < p.M ? am : 0) * p.a_rs * 2 + (int64_t)aprc * 4);
+        const unsigned dst = ring_addr + slot * SLOT_BYTES;
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2\n\t"
+                     "s_mov_b32 m0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %4, %2\n\t"
+                     "s_mov_b32 m0, %5\n\ts_nop 0\n\tglobal_load_lds_dword %6, %7"
+                     :
+                     : "s"(dst), "v"(boff), "s"(Bb), "s"(dst + 1024), "v"(boff + (unsigned)row_bytes), "s"(dst + 2048),
+                       "v"(aoff), "s"(Ab)
+                     : "memory");
+    };
 
     float acc[8][8];
 #pragma unroll
@@ -81,50 +107,41 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_skinny_kernel(SkinnyArgs p)
 #pragma unroll
         for (int n = 0; n < 8; ++n) acc[m][n] = 0.f;
 
-    const char* Bb = (const char*)p.B;
-    const int64_t row_bytes = p.b_rs * 2;
-    constexpr int STEP = WAVES * NKP; // k pairs per workgroup pass
-    const int iters = (npairs + STEP - 1) / STEP;
-    constexpr int U = 4;
-    for (int it0 = 0; it0 < iters; it0 += U) {
-        u32x4 b0[U], b1[U];
-        int pr[U];
+    // prologue: DEPTH steps in flight (steps past the end re-fetch a valid address, unused)
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-            pr[u] = (it0 + u) * STEP + wave * NKP + kp;
-            const bool ok = col_ok && pr[u] < npairs;
-            b0[u] = u32x4{0, 0, 0, 0};
-            b1[u] = u32x4{0, 0, 0, 0};
-            if (ok) {
-                const char* g = Bb + (int64_t)(2 * (pair_begin + pr[u])) * row_bytes + (int64_t)col0 * 2;
-                b0[u] = __builtin_nontemporal_load((const u32x4*)g);
-                b1[u] = __builtin_nontemporal_load((const u32x4*)(g + row_bytes));
-            }
-        }
+    for (int d = 0; d < DEPTH; ++d) issue(d, d);
+
+    for (int it0 = 0; it0 < iters; it0 += DEPTH) {
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const bool in_range = pr[u] < npairs;
-            const int prc = in_range ? pr[u] : 0;
-            u32x4 a_lo = *(const u32x4*)(sA + prc * 8);
-            u32x4 a_hi = *(const u32x4*)(sA + prc * 8 + 4);
-            if (!in_range) { // keep 0 * inf out of the sums
-                a_lo = u32x4{0, 0, 0, 0};
-                a_hi = u32x4{0, 0, 0, 0};
-            }
-            unsigned bp[8];
+        for (int d = 0; d < DEPTH; ++d) {
+            const int it = it0 + d;
+            // the 3 loads of step `it` are the oldest outstanding ones
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(3 * (DEPTH - 1)) : "memory");
+            const char* slot = ring + d * SLOT_BYTES;
+            const u32x4 b0 = *(const u32x4*)(slot + lane * 16);
+            const u32x4 b1 = *(const u32x4*)(slot + 1024 + lane * 16);
+            const u32x4 a_lo = *(const u32x4*)(slot + 2048 + kp * 32);
+            const u32x4 a_hi = *(const u32x4*)(slot + 2048 + kp * 32 + 16);
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); // slot is in registers: it may be refilled
+            issue(it + DEPTH, d);
+            const int pr = it * STEP + wave * NKP + kp;
+            if (pr < npairs && it < iters && col_ok) {
+                unsigned bp[8];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                bp[2 * j] = __builtin_amdgcn_perm(b1[u][j], b0[u][j], 0x05040100u);     // (B[k][n], B[k+1][n]), n even
-                bp[2 * j + 1] = __builtin_amdgcn_perm(b1[u][j], b0[u][j], 0x07060302u); // n odd
-            }
+                for (int j = 0; j < 4; ++j) {
+                    bp[2 * j] = __builtin_amdgcn_perm(b1[j], b0[j], 0x05040100u);     // (B[k][n], B[k+1][n]), n even
+                    bp[2 * j + 1] = __builtin_amdgcn_perm(b1[j], b0[j], 0x07060302u); // n odd
+                }
 #pragma unroll
-            for (int m = 0; m < 8; ++m) {
-                const unsigned am = m < 4 ? a_lo[m & 3] : a_hi[m & 3];
+                for (int m = 0; m < 8; ++m) {
+                    const unsigned amv = m < 4 ? a_lo[m & 3] : a_hi[m & 3];
 #pragma unroll
-                for (int n = 0; n < 8; ++n) acc[m][n] = dot2<BF16>(am, bp[n], acc[m][n]);
+                    for (int n = 0; n < 8; ++n) acc[m][n] = dot2<BF16>(amv, bp[n], acc[m][n]);
+                }
             }
         }
     }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // drain the look-ahead fills before the LDS is reused
 
     // ---- reduce over the NKP lane groups: halving butterfly ----
     // before: lane holds v[e], e = m*8+n, partial over its own k pairs
@@ -148,7 +165,7 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_skinny_kernel(SkinnyArgs p)
         live = half;
     }
 
-    // ---- reduce over waves through LDS (reuses the A staging area) ----
+    // ---- reduce over waves through LDS (reuses the rings) ----
     __syncthreads();
     float* red = (float*)smem; // [wave][VPL][64]
     if (wave > 0) {
@@ -177,33 +194,41 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_skinny_kernel(SkinnyArgs p)
     }
 
     // ---- K split over workgroups: partial sums to scratch, last arrival finishes ----
+    // The partial sums are written as agent-scope relaxed atomics (written through to the
+    // level of the memory system that all XCDs share), so no cache-wide write-back is
+    // needed: the stores only have to be acknowledged (vmcnt = 0) before this workgroup
+    // takes its ticket.
     float* part = p.scratch + ((int64_t)blockIdx.y * gridDim.x + blockIdx.x) * (64 * LPR);
 #pragma unroll
-    for (int j = 0; j < VPL; ++j) part[j * 64 + lane] = v[j];
-    __threadfence();
+    for (int j = 0; j < VPL; ++j) __hip_atomic_store(part + j * 64 + lane, v[j], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     unsigned ticket = 0;
-    if (lane == 0) ticket = atomicAdd(p.counters + blockIdx.x, 1u);
+    if (lane == 0) ticket = __hip_atomic_fetch_add(p.counters + blockIdx.x, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     ticket = __shfl(ticket, 0, 64);
     if (ticket != (unsigned)p.splits - 1) return;
-    __threadfence();
+    // last arrival: drop any stale copies of the scratch lines from this XCD's caches, then
+    // read all slices with ordinary pipelined loads and add them in split order
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+    float sum[VPL];
 #pragma unroll
-    for (int j = 0; j < VPL; ++j) {
-        float s = 0.f;
-        for (int sp = 0; sp < p.splits; ++sp)
-            s += __builtin_nontemporal_load(p.scratch + ((int64_t)sp * gridDim.x + blockIdx.x) * (64 * LPR) + j * 64 + lane);
-        finish((j + VPL * kp) >> 3, (j + VPL * kp) & 7, s);
+    for (int j = 0; j < VPL; ++j) sum[j] = 0.f;
+    for (int sp = 0; sp < p.splits; ++sp) {
+        const float* src = p.scratch + ((int64_t)sp * gridDim.x + blockIdx.x) * (64 * LPR) + lane;
+#pragma unroll
+        for (int j = 0; j < VPL; ++j) sum[j] += src[j * 64];
     }
+#pragma unroll
+    for (int j = 0; j < VPL; ++j) finish((j + VPL * kp) >> 3, (j + VPL * kp) & 7, sum[j]);
     if (lane == 0) p.counters[blockIdx.x] = 0; // ready for the next launch
 }
 
-template <bool BF16, int LPR, int WAVES>
+template <bool BF16, int LPR, int WAVES, int DEPTH>
 hipError_t launch_one(const SkinnyArgs& a, hipStream_t stream, LaunchGeom* geom, bool dry_run)
 {
     constexpr int CB = LPR * 8;
-    auto kern = gemm_skinny_kernel<BF16, LPR, WAVES>;
-    const int pairs_per_split = (a.K / 2 + a.splits - 1) / a.splits;
-    unsigned lds = (unsigned)pairs_per_split * 32u;
-    const unsigned red = (WAVES - 1) * (64 / (64 / LPR)) * 64 * 4;
+    auto kern = gemm_skinny_kernel<BF16, LPR, WAVES, DEPTH>;
+    unsigned lds = WAVES * DEPTH * (2048 + 256);
+    const unsigned red = (WAVES - 1) * LPR * 64 * 4;
     if (lds < red) lds = red;
     dim3 grid((a.N + CB - 1) / CB, a.splits, 1), block(WAVES * 64, 1, 1);
     if (geom) {
@@ -213,33 +238,34 @@ hipError_t launch_one(const SkinnyArgs& a, hipStream_t stream, LaunchGeom* geom,
     }
     if (dry_run) return hipSuccess;
     if (lds > 160 * 1024) return hipErrorInvalidValue;
-    static unsigned attr_lds = 0;
-    if (lds > 64 * 1024 && lds > attr_lds) {
-        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    static bool attr_set = false;
+    if (lds > 64 * 1024 && !attr_set) {
+        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return e;
-        attr_lds = 160 * 1024;
+        attr_set = true;
     }
     hipLaunchKernelGGL(kern, grid, block, lds, stream, a);
     return hipGetLastError();
 }
 
 struct SkinnyVariant {
-    int lpr, waves;
+    int lpr, waves, depth;
     hipError_t (*f16)(const SkinnyArgs&, hipStream_t, LaunchGeom*, bool);
     hipError_t (*bf16)(const SkinnyArgs&, hipStream_t, LaunchGeom*, bool);
 };
-#define SV(LPR, W) { LPR, W, &launch_one<false, LPR, W>, &launch_one<true, LPR, W> }
-const SkinnyVariant kSkinny[] = { SV(8, 4), SV(8, 8), SV(8, 16), SV(16, 4), SV(16, 8), SV(4, 8), SV(4, 4) };
+#define SV(LPR, W, D) { LPR, W, D, &launch_one<false, LPR, W, D>, &launch_one<true, LPR, W, D> }
+const SkinnyVariant kSkinny[] = { SV(8, 4, 8), SV(8, 8, 4), SV(8, 8, 8), SV(8, 4, 4), SV(8, 16, 4), SV(8, 16, 2), SV(16, 4, 8), SV(16, 8, 4), SV(32, 4, 8) };
 #undef SV
 constexpr int kNumSkinny = (int)(sizeof(kSkinny) / sizeof(kSkinny[0]));
 
 } // namespace
 
 int skinny_num_variants() { return kNumSkinny; }
-void skinny_variant_info(int v, int* lpr, int* waves)
+void skinny_variant_info(int v, int* lpr, int* waves, int* depth)
 {
     *lpr = kSkinny[v].lpr;
     *waves = kSkinny[v].waves;
+    *depth = kSkinny[v].depth;
 }
 int skinny_column_blocks(int v, int N) { return (N + kSkinny[v].lpr * 8 - 1) / (kSkinny[v].lpr * 8); }
 size_t skinny_scratch_floats(int v, int N, int splits)

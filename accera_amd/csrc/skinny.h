@@ -19,7 +19,7 @@ struct SkinnyArgs {
 };
 
 int skinny_num_variants();
-void skinny_variant_info(int v, int* lanes_per_row, int* waves);
+void skinny_variant_info(int v, int* lanes_per_row, int* waves, int* depth);
 int skinny_column_blocks(int v, int N);
 size_t skinny_scratch_floats(int v, int N, int splits);
 hipError_t launch_skinny(int v, const SkinnyArgs& a, hipStream_t stream, LaunchGeom* geom, bool dry_run);

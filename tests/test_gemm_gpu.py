@@ -189,6 +189,7 @@ def test_skinny_repeated_launches_reuse_counters():
     for rep in range(3):
         run_case("f16", "f16", 8, 4096, 2048, variant=100, splits=8, seed=90 + rep, dist="normal")
     run_case("f16", "f16", 8, 512, 2048, variant=103, splits=5, seed=95, dist="normal")
+    run_case("f16", "f16", 8, 11008, 4096, splits=7, seed=96, dist="normal")  # the decode shape itself
 
 
 # ---- closed forms: bit-exact expectations ------------------------------------------------------
