@@ -12,14 +12,14 @@ from . import _lib  # noqa: F401
 from ._lib import (Acc950Error, EPILOGUE_NONE, EPILOGUE_RELU, EPILOGUE_RELU_NOCOND, PROLOGUE_NONE,  # noqa: F401
                    PROLOGUE_SET0, VARIANT_AUTO, VARIANT_F32_MFMA, VARIANT_GENERIC, VARIANT_SKINNY_BASE)
 
-__all__ = ["gemm_relu", "hat"]
+__all__ = ["gemm_relu", "GemmCall", "hat"]
 
 
 def __getattr__(name):
     # torch and the DSL are imported on first use so that `import accera_amd` stays light
-    if name == "gemm_relu":
-        from .gemm import gemm_relu
-        return gemm_relu
+    if name in ("gemm_relu", "GemmCall"):
+        from . import gemm
+        return getattr(gemm, name)
     if name == "hat":
         import importlib
         return importlib.import_module(".hat", __name__)

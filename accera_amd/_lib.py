@@ -21,7 +21,7 @@ VARIANT_AUTO, VARIANT_SKINNY_BASE, VARIANT_GENERIC, VARIANT_F32_MFMA = -1, 100, 
 EXPORTS = [
     "acc950_init", "acc950_gemm_relu", "acc950_gemm_relu_ex", "acc950_gemm_relu_host",
     "acc950_launch_geometry", "acc950_num_variants", "acc950_num_skinny_variants",
-    "acc950_variant_name", "acc950_last_error",
+    "acc950_variant_name", "acc950_last_error", "acc950_mfma_ceiling", "acc950_copy_probe", "acc950_stream_read_probe",
 ]
 
 
@@ -53,6 +53,9 @@ def lib():
     L.acc950_launch_geometry.argtypes = [ci, ci, ci, ci, ci] + [i64] * 6 + [ci, ci, ctypes.POINTER(cu), ctypes.POINTER(cu),
                                                                            ctypes.POINTER(cu), ctypes.POINTER(ci)]
     L.acc950_variant_name.argtypes = [ci, ctypes.c_char_p, ctypes.c_size_t]
+    L.acc950_mfma_ceiling.argtypes = [ci, ci, ci, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double)]
+    L.acc950_copy_probe.argtypes = [vp, vp, ctypes.c_size_t, vp]
+    L.acc950_stream_read_probe.argtypes = [vp, ctypes.c_size_t, vp, vp]
     L.acc950_last_error.restype = ctypes.c_char_p
     for name in EXPORTS:
         if name != "acc950_last_error":
@@ -64,6 +67,14 @@ def lib():
 def check(rc):
     if rc != OK:
         raise Acc950Error(rc, lib().acc950_last_error().decode())
+
+
+def mfma_ceiling(in_type, data_mode=2, iters=20000):
+    """(tera-ops/s, sustained shader clock in GHz) of a pure MFMA loop on this GPU;
+    data_mode 0 zeros, 1 constant, 2 random operands."""
+    t, g = ctypes.c_double(), ctypes.c_double()
+    check(lib().acc950_mfma_ceiling(in_type, data_mode, iters, ctypes.byref(t), ctypes.byref(g)))
+    return t.value, g.value
 
 
 def variant_name(variant):

@@ -110,6 +110,8 @@ bool mfma_can_take(const MfmaVariant& v, const Problem& pb)
     } else {
         if (g.M % v.bm || g.N % v.bn || g.K % bk) return false;
     }
+    // offsets inside one output tile are 32-bit in the write-back
+    if ((int64_t)v.bm * g.c_rs * 4 >= (1ll << 32)) return false;
     // per-lane global offsets of the direct fill are 32-bit
     if ((int64_t)v.bm * lda * es >= (1ll << 31) || (int64_t)(v.b_kc ? v.bn : bk) * ldb * es >= (1ll << 31)) return false;
     return true;

@@ -226,6 +226,8 @@ __device__ __forceinline__ void tile_coords(int pid, int tiles_m, int tiles_n, i
 // Compile-time description of one kernel instantiation.
 template <int IN_, int BM_, int BN_, int WAVES_M_, int WAVES_N_, bool A_KC_, bool B_KC_, bool DIRECT_, bool EDGE_, int KB_, int STAGES_>
 struct MfmaConfig {
+    // workgroups meant to share a CU: as many as the LDS allows, at most 2 waves per SIMD in all
+    static constexpr int WGS_PER_CU = (WAVES_M_ * WAVES_N_ <= 4 && 2 * STAGES_ * (BM_ + BN_) * KB_ <= 160 * 1024 && BM_ * BN_ <= 256 * 128) ? 2 : 1;
     static constexpr int IN = IN_, BM = BM_, BN = BN_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_, KB = KB_, STAGES = STAGES_;
     static constexpr bool A_KC = A_KC_, B_KC = B_KC_, DIRECT = DIRECT_, EDGE = EDGE_;
     static constexpr int NT = WAVES_M * WAVES_N * 64;
@@ -237,7 +239,7 @@ struct MfmaConfig {
 };
 
 template <typename Cfg>
-__global__ void __launch_bounds__(Cfg::NT) gemm_mfma_kernel(GemmArgs p)
+__global__ void __launch_bounds__(Cfg::NT, Cfg::WGS_PER_CU) gemm_mfma_kernel(GemmArgs p)
 {
     constexpr int IN = Cfg::IN, BM = Cfg::BM, BN = Cfg::BN, WAVES_M = Cfg::WAVES_M, WAVES_N = Cfg::WAVES_N;
     constexpr int KB = Cfg::KB, STAGES = Cfg::STAGES, NT = Cfg::NT;
@@ -418,42 +420,55 @@ __global__ void __launch_bounds__(Cfg::NT) gemm_mfma_kernel(GemmArgs p)
     // Write-back: optional "+= C" (no SET prologue), epilogue op, narrowing store.
     // MFMA 32x32 accumulator layout: register r of lane l holds
     //   row = (r/4)*8 + (l/32)*4 + r%4,  column = l%32.
-    const int row_base = m0 + wr0 + (lane >> 5) * 4;
-    const int col_base = n0 + wc0 + (lane & 31);
-    auto for_each_acc = [&](auto&& fn) {
-#pragma unroll
-        for (int i = 0; i < TM; ++i)
-#pragma unroll
-            for (int j = 0; j < TN; ++j)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const int row = row_base + i * 32 + (r >> 2) * 8 + (r & 3);
-                    const int col = col_base + j * 32;
-                    if (EDGE && (row >= p.M || col >= p.N)) continue;
-                    acc[i][j][r] = fn(acc[i][j][r], (int64_t)row * p.c_rs + (int64_t)col * p.c_cs);
-                }
-    };
-    // epilogue as two selects on wave-uniform conditions (no per-element branches)
+    // C is row-major here (the host transposes the problem otherwise).  Addresses are a
+    // workgroup-uniform tile base plus one 32-bit offset per accumulator row, so the
+    // write-back needs no 64-bit address registers next to the live accumulators.
     const bool is_relu = p.epilogue == EPI_RELU, is_nocond = p.epilogue == EPI_RELU_NOCOND;
-    auto epilogue = [&](scalar_t v) -> scalar_t {
+    auto epilogue = [&](scalar_t v) -> scalar_t { // two selects on wave-uniform conditions, no per-element branch
         scalar_t r = v > scalar_t(0) ? v : scalar_t(0);
         scalar_t n = v * (v > scalar_t(0) ? scalar_t(1) : scalar_t(0));
         return is_relu ? r : (is_nocond ? n : v);
     };
-    if constexpr (IN == IN_I8) {
-        int* C = (int*)p.C;
-        if (p.prologue == PRO_NONE) for_each_acc([&](int v, int64_t idx) { return (int)((unsigned)v + (unsigned)C[idx]); });
-        for_each_acc([&](int v, int64_t idx) { C[idx] = epilogue(v); return v; });
-    } else {
-        if (p.prologue == PRO_NONE) {
-            if (p.out_type == T_F32) for_each_acc([&](float v, int64_t idx) { return v + ((const float*)p.C)[idx]; });
-            else if (p.out_type == T_F16) for_each_acc([&](float v, int64_t idx) { return v + f16_bits_to_float(((const uint16_t*)p.C)[idx]); });
-            else for_each_acc([&](float v, int64_t idx) { return v + bf16_bits_to_float(((const uint16_t*)p.C)[idx]); });
-        }
-        if (p.out_type == T_F32) for_each_acc([&](float v, int64_t idx) { ((float*)p.C)[idx] = epilogue(v); return v; });
-        else if (p.out_type == T_F16) for_each_acc([&](float v, int64_t idx) { ((uint16_t*)p.C)[idx] = float_to_f16_bits(epilogue(v)); return v; });
-        else for_each_acc([&](float v, int64_t idx) { ((uint16_t*)p.C)[idx] = float_to_bf16_bits(epilogue(v)); return v; });
-    }
+    const bool accumulate = p.prologue == PRO_NONE;
+    const int row_in_tile = wr0 + (lane >> 5) * 4, col_in_tile = wc0 + (lane & 31);
+    auto write_back = [&](auto out_tag) {
+        using out_t = decltype(out_tag);
+        constexpr unsigned OS = sizeof(out_t);
+        char* tile_base = (char*)p.C + ((int64_t)m0 * p.c_rs + n0) * OS; // uniform
+        const unsigned row_bytes = (unsigned)p.c_rs * OS;
+        const unsigned lane_off = (unsigned)row_in_tile * row_bytes + (unsigned)col_in_tile * OS;
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int row_off = i * 32 + (r >> 2) * 8 + (r & 3);
+                const unsigned off = lane_off + (unsigned)row_off * row_bytes;
+                if (EDGE && m0 + row_in_tile + row_off >= p.M) continue;
+#pragma unroll
+                for (int j = 0; j < TN; ++j) {
+                    if (EDGE && n0 + col_in_tile + j * 32 >= p.N) continue;
+                    out_t* dst = (out_t*)(tile_base + off + j * 32 * OS);
+                    scalar_t v = acc[i][j][r];
+                    if constexpr (std::is_same<out_t, int>::value) {
+                        if (accumulate) v = (int)((unsigned)v + (unsigned)*dst);
+                        *dst = epilogue(v);
+                    } else if constexpr (std::is_same<out_t, float>::value) {
+                        if (accumulate) v += *dst;
+                        *dst = epilogue(v);
+                    } else if constexpr (std::is_same<out_t, _Float16>::value) {
+                        if (accumulate) v += (float)*dst;
+                        *dst = (_Float16)epilogue(v); // v_cvt_f16_f32: round to nearest even
+                    } else { // bf16 bits
+                        if (accumulate) v += bf16_bits_to_float(*dst);
+                        *dst = float_to_bf16_bits(epilogue(v));
+                    }
+                }
+            }
+    };
+    if constexpr (IN == IN_I8) write_back(int{});
+    else if (p.out_type == T_F32) write_back(float{});
+    else if (p.out_type == T_F16) write_back(_Float16{});
+    else write_back(uint16_t{});
 }
 
 // Host launcher for one kernel instantiation.

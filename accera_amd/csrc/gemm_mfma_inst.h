@@ -22,6 +22,8 @@ namespace acc950 {
     V(256, 256, 2, 4, BKC, true, false, 64, 4),     \
     V(256, 256, 2, 4, BKC, true, false, 64, 3),     \
     V(256, 128, 2, 2, BKC, true, false, 128, 3),    \
+    V(256, 128, 2, 2, BKC, true, false, 64, 3),     \
+    V(128, 256, 2, 2, BKC, true, false, 64, 3),     \
     V(128, 128, 2, 2, BKC, true, false, 128, 2),    \
     V(128, 128, 2, 2, BKC, true, false, 64, 4),     \
     V(128, 128, 2, 2, BKC, false, false, 128, 2),   \

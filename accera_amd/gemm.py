@@ -18,6 +18,34 @@ def _mat(t, name):
     return t.data_ptr(), t.stride(0), t.stride(1)
 
 
+class GemmCall:
+    """One matmul+epilogue bound to its tensors, like one function of a package bound to
+    its arrays: everything about the call is fixed at construction, calling it only
+    launches.  Keeps the tensors alive; `stream` is a raw hipStream_t (int) or None for the
+    stream that is current when the object is built."""
+
+    def __init__(self, A, B, C, prologue=_lib.PROLOGUE_SET0, epilogue=_lib.EPILOGUE_RELU, variant=_lib.VARIANT_AUTO,
+                 k_splits=0, stream=None):
+        M, K = A.shape
+        K2, N = B.shape
+        if K2 != K or tuple(C.shape) != (M, N):
+            raise ValueError(f"shape mismatch: A {tuple(A.shape)}, B {tuple(B.shape)}, C {tuple(C.shape)}")
+        if A.dtype != B.dtype or A.dtype not in _TORCH_TYPES or C.dtype not in _TORCH_TYPES:
+            raise ValueError(f"unsupported dtypes {A.dtype}, {B.dtype}, {C.dtype}")
+        if stream is None:
+            stream = torch.cuda.current_stream(C.device).cuda_stream
+        self.tensors = (A, B, C)
+        self._fn = _lib.lib().acc950_gemm_relu_ex
+        self._args = (_TORCH_TYPES[A.dtype], _TORCH_TYPES[C.dtype], M, N, K, *_mat(A, "A"), *_mat(B, "B"), *_mat(C, "C"),
+                      prologue, epilogue, variant, k_splits, stream)
+
+    def __call__(self):
+        rc = self._fn(*self._args)
+        if rc:
+            _lib.check(rc)
+        return self.tensors[2]
+
+
 def gemm_relu(A, B, C, prologue=_lib.PROLOGUE_SET0, epilogue=_lib.EPILOGUE_RELU, variant=_lib.VARIANT_AUTO,
               k_splits=0, stream=None):
     """C = epilogue((prologue == SET0 ? 0 : C) + A @ B), in place on C, asynchronously.

@@ -91,13 +91,17 @@ def run_gpu(c, steps, warmup, variant=-1, k_splits=0):
     sets = make_inputs(c, n_sets, seed=1000)
     stream = torch.cuda.current_stream()
 
+    # one bound call per input set: the timed loop only launches
+    calls = [acc.GemmCall(A, B, C, prologue=acc.PROLOGUE_SET0, epilogue=acc.EPILOGUE_RELU, variant=variant, k_splits=k_splits)
+             for A, B, C in sets]
+
     def step(i):
-        A, B, C = sets[i % n_sets]
-        acc.gemm_relu(A, B, C, prologue=acc.PROLOGUE_SET0, epilogue=acc.EPILOGUE_RELU, variant=variant, k_splits=k_splits)
+        calls[i % n_sets]()
 
     for i in range(warmup):
         step(i)
     torch.cuda.synchronize()
+    run_gpu.rotating_sets = n_sets
     ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
     ev0.record(stream)
@@ -140,6 +144,47 @@ def cpu_baseline(c, threads, budget_rows=None):
                 sample=f"rows 0..{M - 1} of A against all of B ({M}x{N}x{K}), one pass, OpenMP over column tiles")
 
 
+def traffic_bytes(name):
+    """HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE and scaled by the
+    plain copy kernel of known size (written to profiles/traffic.json by accera_amd.profiling)."""
+    path = os.path.join(ROOT, "profiles", "traffic.json")
+    if not os.path.exists(path):
+        return None
+    with open(path) as f:
+        rec = json.load(f).get(name)
+    return None if not rec else int(rec["hbm_bytes_per_launch"])
+
+
+def machine_ceiling(c):
+    """What this GPU sustains, measured now: pure-MFMA rate on random operands (the engine
+    clock under MFMA load is data dependent) or a plain streaming read of the same size."""
+    import torch
+    from accera_amd import _lib
+    if c["bound"] == "mfma" and c["in_type"] in ("f16", "bf16", "i8"):
+        t = getattr(_lib, c["in_type"].upper())
+        rnd, ghz = _lib.mfma_ceiling(t, 2, 20000)
+        cool, ghz0 = _lib.mfma_ceiling(t, 0, 20000)
+        return {"mfma_only_random_operands": round(rnd, 1), "clock_ghz_random": round(ghz, 3),
+                "mfma_only_zero_operands": round(cool, 1), "clock_ghz_zero": round(ghz0, 3), "unit": "TFLOP/s" if t != _lib.I8 else "TOP/s"}
+    if c["bound"] == "hbm":
+        nbytes = c["K"] * c["N"] * ES[c["in_type"]]
+        bufs = [torch.empty(nbytes, dtype=torch.uint8, device="cuda").fill_(i + 1) for i in range(8)]
+        out = torch.zeros(1, dtype=torch.int32, device="cuda")
+        stream = torch.cuda.current_stream()
+        L = _lib.lib()
+        for i in range(8):
+            _lib.check(L.acc950_stream_read_probe(bufs[i].data_ptr(), nbytes, out.data_ptr(), stream.cuda_stream))
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        for i in range(80):
+            _lib.check(L.acc950_stream_read_probe(bufs[i % 8].data_ptr(), nbytes, out.data_ptr(), stream.cuda_stream))
+        e1.record(stream)
+        torch.cuda.synchronize()
+        return {"plain_streaming_read_same_bytes": round(nbytes / (e0.elapsed_time(e1) * 1e-3 / 80) / 1e9, 1), "unit": "GB/s"}
+    return None
+
+
 def measure(name, steps, warmup, variant=-1, k_splits=0):
     c = CONFIGS[name]
     wall, launch_s, _ = run_gpu(c, steps, warmup, variant, k_splits)
@@ -152,7 +197,7 @@ def measure(name, steps, warmup, variant=-1, k_splits=0):
         value, vunit = flops * steps / wall / 1e12, unit
     return dict(config=name, workload=c["workload"], value=round(value, 3), unit=vunit, ms_per_step=round(wall / steps * 1e3, 5),
                 roofline=dict(bound=c["bound"], achieved=round(achieved, 3), peak=peak, unit=unit,
-                              frac=round(achieved / peak, 4), traffic=None),
+                              frac=round(achieved / peak, 4), traffic=traffic_bytes(name)),
                 flops_per_launch=flops, bytes_per_launch=nbytes)
 
 
@@ -179,6 +224,11 @@ def main():
     _lib.check(_lib.lib().acc950_init(0))
 
     c = CONFIGS[args.config]
+    # plain copy of known size: the reference point for scaling profiler byte counters
+    probe = torch.empty(2, 64 << 20, dtype=torch.uint8, device="cuda")
+    _lib.check(_lib.lib().acc950_copy_probe(probe[1].data_ptr(), probe[0].data_ptr(), 64 << 20, torch.cuda.current_stream().cuda_stream))
+    torch.cuda.synchronize()
+    del probe
     m = measure(args.config, args.steps, args.warmup, args.variant, args.k_splits)
     grid, block, lds, chosen = _lib.launch_geometry(
         getattr(_lib, c["in_type"].upper()), getattr(_lib, c["out_type"].upper()), c["M"], c["N"], c["K"],
@@ -190,13 +240,15 @@ def main():
         "dtype": {"f16": "f16", "bf16": "bf16", "i8": "int8", "f32": "f32"}[c["in_type"]], "data": "synthetic",
         "config": {"workload": c["workload"], "M": c["M"], "N": c["N"], "K": c["K"], "kernel": _lib.variant_name(chosen),
                    "grid": grid, "block": block, "dynamic_lds_bytes": lds, "device": torch.cuda.get_device_name(0),
+                   "arch": torch.cuda.get_device_properties(0).gcnArchName,
                    "compute_units": torch.cuda.get_device_properties(0).multi_processor_count},
         "roofline": m["roofline"],
+        "machine_ceiling": machine_ceiling(c),
     }
     if not args.no_cpu:
         threads = min(16, os.cpu_count() or 1)
         # bounded sample: about 10-30 s of single-core work spread over the host cores
-        rows = {"c2": 1024, "c4": 512, "c3": None, "c1": None, "c5": None}[args.config]
+        rows = {"c2": None, "c4": 2048, "c3": None, "c1": None, "c5": None}[args.config]
         out["cpu_baseline"] = cpu_baseline(c, threads, rows)
     if args.all:
         out["other_configs"] = [measure(n, max(20, args.steps // 4) if n == "c4" else args.steps, args.warmup)
