@@ -174,29 +174,37 @@ int auto_skinny_splits(int variant, const GemmArgs& g)
     return splits;
 }
 
-// Preference order of MFMA tiles for the automatic choice: biggest tile that still
-// yields at least ~one workgroup per CU, else smaller tiles, else the edge kernel.
+// Automatic MFMA tile choice.  Cost of a candidate = rounds of workgroups over the 256 CUs
+// x tile area (time per round), with two workgroups sharing a CU for the tiles whose LDS
+// and register budget allows it; ties go to the larger tile (more reuse per byte fetched).
+// Among equal tiles the ping-pong kernel with four 64-byte stages is preferred, then the
+// others in table order; partial tiles only fit the edge kernel.
 int auto_mfma_variant(const Problem& pb)
 {
     int n = 0;
     const MfmaVariant* tab = mfma_table(pb.g.in_type, &n);
     if (!tab) return -1;
-    struct Want { int bm, bn, wm, wn; bool direct, edge; int kb, stages; };
-    const int64_t tiles256 = ((int64_t)pb.g.M / 256) * (pb.g.N / 256);
-    const Want big = {256, 256, 2, 4, true, false, 128, 2}, mid = {256, 128, 2, 2, true, false, 128, 3},
-               small = {128, 128, 2, 2, true, false, 128, 2}, edge = {128, 128, 2, 2, false, true, 128, 2};
-    Want order[4];
-    if (tiles256 >= 200) { order[0] = big; order[1] = mid; order[2] = small; }
-    else { order[0] = small; order[1] = mid; order[2] = big; }
-    order[3] = edge;
-    for (const Want& w : order)
-        for (int i = 0; i < n; ++i) {
-            const MfmaVariant& v = tab[i];
-            if (v.bm == w.bm && v.bn == w.bn && v.waves_m == w.wm && v.waves_n == w.wn && v.direct == w.direct &&
-                v.edge == w.edge && v.kb == w.kb && v.stages == w.stages && mfma_can_take(v, pb))
-                return i;
-        }
-    return -1;
+    int best = -1;
+    double best_cost = 0;
+    int best_rank = 0;
+    for (int i = 0; i < n; ++i) {
+        const MfmaVariant& v = tab[i];
+        if (!mfma_can_take(v, pb)) continue;
+        const int64_t tiles = (((int64_t)pb.g.M + v.bm - 1) / v.bm) * (((int64_t)pb.g.N + v.bn - 1) / v.bn);
+        const int wgs_per_cu = (tiles > 256 && v.waves_m * v.waves_n <= 4 &&
+                                2 * v.stages * (v.bm + v.bn) * v.kb <= 160 * 1024 && v.bm * v.bn <= 256 * 128) ? 2 : 1;
+        const int64_t rounds = (tiles + 256 * wgs_per_cu - 1) / (256 * wgs_per_cu);
+        double cost = (double)rounds * wgs_per_cu * v.bm * v.bn;
+        if (v.edge) cost *= 1.5;                 // register-staged fill, bounds checks
+        if (!v.direct) cost *= 1.2;
+        // rank inside one tile shape: ping-pong kb64 x4 > ping-pong others > 8-wave > rest
+        int rank = v.pingpong ? (v.kb == 64 && v.stages == 4 ? 4 : 3) : (v.waves_m * v.waves_n == 8 ? 2 : 1);
+        const bool better = best < 0 || cost < best_cost * 0.999 ||
+                            (cost <= best_cost * 1.001 && ((int64_t)v.bm * v.bn > (int64_t)tab[best].bm * tab[best].bn ||
+                                                           ((int64_t)v.bm * v.bn == (int64_t)tab[best].bm * tab[best].bn && rank > best_rank)));
+        if (better) { best = i; best_cost = cost; best_rank = rank; }
+    }
+    return best;
 }
 
 struct Choice {
@@ -415,8 +423,9 @@ int acc950_variant_name(int variant, char* buf, size_t buf_len)
     const MfmaVariant* tab = mfma_variants_f16(&n);
     if (variant < 0 || variant >= n) return fail(ACC950_INVALID_ARGUMENT, "unknown kernel variant");
     const MfmaVariant& v = tab[variant];
-    std::snprintf(buf, buf_len, "mfma %dx%d kb%d waves %dx%d B=%s fill=%s stages=%d%s", v.bm, v.bn, v.kb, v.waves_m, v.waves_n,
-                  v.b_kc ? "col-major" : "row-major", v.direct ? "direct" : "registers", v.stages, v.edge ? " edge" : "");
+    std::snprintf(buf, buf_len, "mfma %dx%d kb%d waves %dx%d B=%s fill=%s stages=%d%s%s", v.bm, v.bn, v.kb, v.waves_m, v.waves_n,
+                  v.b_kc ? "col-major" : "row-major", v.direct ? "direct" : "registers", v.stages, v.edge ? " edge" : "",
+                  v.pingpong ? " pingpong" : "");
     return ACC950_OK;
 }
 

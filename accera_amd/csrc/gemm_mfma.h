@@ -224,8 +224,10 @@ __device__ __forceinline__ void tile_coords(int pid, int tiles_m, int tiles_n, i
 }
 
 // Compile-time description of one kernel instantiation.
-template <int IN_, int BM_, int BN_, int WAVES_M_, int WAVES_N_, bool A_KC_, bool B_KC_, bool DIRECT_, bool EDGE_, int KB_, int STAGES_>
+template <int IN_, int BM_, int BN_, int WAVES_M_, int WAVES_N_, bool A_KC_, bool B_KC_, bool DIRECT_, bool EDGE_, int KB_, int STAGES_,
+          bool PINGPONG_ = false>
 struct MfmaConfig {
+    static constexpr bool PINGPONG = PINGPONG_;
     // workgroups meant to share a CU: as many as the LDS allows, at most 2 waves per SIMD in all
     static constexpr int WGS_PER_CU = (WAVES_M_ * WAVES_N_ <= 4 && 2 * STAGES_ * (BM_ + BN_) * KB_ <= 160 * 1024 && BM_ * BN_ <= 256 * 128) ? 2 : 1;
     static constexpr int IN = IN_, BM = BM_, BN = BN_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_, KB = KB_, STAGES = STAGES_;
@@ -236,6 +238,7 @@ struct MfmaConfig {
     static_assert(DIRECT || STAGES == 2, "the register-staged fill is double-buffered");
     static_assert(STAGES >= 2 && STAGES <= 4, "2 to 4 LDS stages");
     static_assert(LDS_BYTES <= 160 * 1024, "LDS budget of one CU");
+    static_assert(!PINGPONG || (DIRECT && WAVES_M * WAVES_N == 8), "ping-pong needs 8 waves and direct fills");
 };
 
 template <typename Cfg>
@@ -353,7 +356,74 @@ __global__ void __launch_bounds__(Cfg::NT, Cfg::WGS_PER_CU) gemm_mfma_kernel(Gem
         }
     };
 
-    if constexpr (DIRECT) {
+    if constexpr (Cfg::PINGPONG) {
+        // Ping-pong schedule for 8 waves (two per SIMD).  Every k-step is split into a
+        // memory cluster (fragment reads from LDS, a share of the fills of tile kt+D) and
+        // a compute cluster (the MFMAs of that step), each closed by a barrier.  Waves
+        // 4..7 run one cluster behind waves 0..3, so on every SIMD one wave is in its
+        // compute cluster while its sibling is in its memory cluster: LDS and fill latency
+        // is hidden by the sibling's MFMAs instead of by software pipelining.
+        constexpr int D = STAGES - 1;
+        const int group = wave >> 2;
+        auto raw_barrier = [&]() {
+            __builtin_amdgcn_sched_barrier(0);
+            asm volatile("s_barrier" ::: "memory");
+            __builtin_amdgcn_sched_barrier(0);
+        };
+#pragma unroll
+        for (int s = 0; s < D; ++s)
+            if (s < KT) {
+#pragma unroll
+                for (int f = 0; f < FILLS; ++f) issue_fill(f, s, s * BK);
+            }
+        if (KT >= D) wait_vmcnt<(D - 1) * FILLS>();
+        else wait_vmcnt<0>();
+        __syncthreads();
+        if (group == 1) raw_barrier(); // one cluster behind
+        // CL k-steps form one cluster: the whole K tile when it has 2 steps, half of it when 4
+        constexpr int CL = 2, CLUSTERS = KSTEPS / CL, FPC = (FILLS + CLUSTERS - 1) / CLUSTERS;
+        auto pp_tile = [&](int kt, auto fill_tag) {
+            constexpr bool fill = decltype(fill_tag)::value;
+            const char* sa = smem + (kt % STAGES) * STAGE_BYTES;
+            const char* sb = sa + TA::TILE_BYTES;
+#pragma unroll
+            for (int c = 0; c < CLUSTERS; ++c) {
+                // ---- memory cluster
+#pragma unroll
+                for (int q = 0; q < CL; ++q) {
+#pragma unroll
+                    for (int j = 0; j < TN; ++j) bf[q][j] = TB::read_frag(sb, wc0 + j * 32, c * CL + q, lane);
+#pragma unroll
+                    for (int i = 0; i < TM; ++i) af[q][i] = TA::read_frag(sa, wr0 + i * 32, c * CL + q, lane);
+                }
+                if constexpr (fill) {
+#pragma unroll
+                    for (int u = 0; u < FPC; ++u)
+                        if (c * FPC + u < FILLS) issue_fill(c * FPC + u, (kt + D) % STAGES, (kt + D) * BK);
+                }
+                if (c + 1 == CLUSTERS) { // own fills of tile kt+1 have landed before the barrier publishes them
+                    if constexpr (fill) wait_vmcnt<(D - 1) * FILLS>();
+                    else wait_vmcnt<0>();
+                }
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); // fragments are in registers: the buffer may be refilled
+                raw_barrier();
+                // ---- compute cluster
+                __builtin_amdgcn_s_setprio(2);
+#pragma unroll
+                for (int q = 0; q < CL; ++q)
+#pragma unroll
+                    for (int i = 0; i < TM; ++i)
+#pragma unroll
+                        for (int j = 0; j < TN; ++j) mfma32<IN>(af[q][i], bf[q][j], acc[i][j]);
+                __builtin_amdgcn_s_setprio(0);
+                raw_barrier();
+            }
+        };
+        int kt = 0;
+        for (; kt + D < KT; ++kt) pp_tile(kt, std::true_type{});
+        for (; kt < KT; ++kt) pp_tile(kt, std::false_type{});
+        if (group == 0) raw_barrier(); // match the extra barrier of the other group
+    } else if constexpr (DIRECT) {
         // D tiles are in flight beyond the one being computed; AHEAD of them are already
         // published (landed and behind a barrier) when a tile starts.
         constexpr int D = STAGES - 1;

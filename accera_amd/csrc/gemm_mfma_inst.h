@@ -12,8 +12,11 @@
 namespace acc950 {
 
 #define V(BM, BN, WM, WN, BKC, DIRECT, EDGE, KB, STAGES)                                               \
-    { BM, BN, WM, WN, /*a_kc=*/true, BKC, DIRECT, EDGE, KB, STAGES,                                    \
+    { BM, BN, WM, WN, /*a_kc=*/true, BKC, DIRECT, EDGE, KB, STAGES, false,                             \
       &launch_mfma<MfmaConfig<ACC950_IN, BM, BN, WM, WN, true, BKC, DIRECT, EDGE, KB, STAGES>> }
+#define VP(BM, BN, WM, WN, BKC, KB, STAGES)                                                             \
+    { BM, BN, WM, WN, /*a_kc=*/true, BKC, true, false, KB, STAGES, true,                               \
+      &launch_mfma<MfmaConfig<ACC950_IN, BM, BN, WM, WN, true, BKC, true, false, KB, STAGES, true>> }
 
 #define LAYOUT(BKC)                                 \
     V(256, 256, 2, 2, BKC, true, false, 128, 2),    \
@@ -27,14 +30,21 @@ namespace acc950 {
     V(128, 128, 2, 2, BKC, true, false, 128, 2),    \
     V(128, 128, 2, 2, BKC, true, false, 64, 4),     \
     V(128, 128, 2, 2, BKC, false, false, 128, 2),   \
-    V(128, 128, 2, 2, BKC, false, true, 128, 2)
+    V(128, 128, 2, 2, BKC, false, true, 128, 2),    \
+    VP(256, 256, 2, 4, BKC, 64, 4),                 \
+    VP(256, 256, 2, 4, BKC, 128, 2),                \
+    VP(256, 256, 2, 4, BKC, 64, 3)
 
 static const MfmaVariant kVariants[] = {
     LAYOUT(false), // B row-major (N contiguous): transpose reads
     LAYOUT(true),  // B column-major (K contiguous)
+    // 192-wide tiles (N = 3072 = 16 x 192 gives one tile per CU); K-contiguous B only
+    VP(256, 192, 4, 2, true, 128, 2),
+    V(256, 192, 4, 2, true, true, false, 128, 2),
 };
 #undef LAYOUT
 #undef V
+#undef VP
 
 const MfmaVariant* ACC950_TABLE_FN(int* count)
 {

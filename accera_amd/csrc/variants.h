@@ -12,6 +12,7 @@ struct MfmaVariant {
     bool edge;           // handles M/N/K that are not tile multiples
     int kb;              // bytes of K per tile (64 or 128)
     int stages;          // LDS buffers
+    bool pingpong;       // sibling waves alternate memory and compute clusters
     LaunchFn launch;
 };
 

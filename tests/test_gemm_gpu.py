@@ -64,8 +64,10 @@ def test_mfma_all_variants(in_type, out_type, b_layout):
         print("variant", v, name, in_type, b_layout, flush=True)
         # two tiles in each direction; K tile counts below, at and above the pipeline depth
         kb = int(re.search(r"kb(\d+)", name).group(1)) // (1 if in_type == "i8" else 2)
+        bm, bn = map(int, re.search(r"mfma (\d+)x(\d+)", name).groups())
+        M, N = max(512, 2 * bm), (max(512, 2 * bn) if 512 % bn == 0 else 3 * bn)
         for k_tiles in (1, 2, 3, 7):
-            run_case(in_type, out_type, 512, 512, k_tiles * kb, b_layout=b_layout, variant=v, seed=v + k_tiles)
+            run_case(in_type, out_type, M, N, k_tiles * kb, b_layout=b_layout, variant=v, seed=v + k_tiles)
         if "edge" in name:
             # ragged M, N (multiple of the 16-byte vector only) and a K tail
             run_case(in_type, out_type, 200, 144, 336 if in_type == "i8" else 176, b_layout=b_layout, variant=v, seed=100 + v)
