@@ -50,10 +50,7 @@ __device__ __forceinline__ float bf16_bits_to_float(uint16_t b) { return __uint_
 // host path and this library's oracle do.)
 __device__ __forceinline__ uint16_t float_to_bf16_bits(float f)
 {
-    uint32_t u = __float_as_uint(f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40u);
-    u += 0x7fffu + ((u >> 16) & 1u);
-    return (uint16_t)(u >> 16);
+    return __builtin_bit_cast(uint16_t, (__bf16)f); // v_cvt_pk_bf16_f32
 }
 
 __device__ __forceinline__ uint16_t float_to_f16_bits(float f)

@@ -67,8 +67,12 @@ struct OperandTile {
     static constexpr int KSTEPS = KB / 32;               // MFMA steps per tile
     static constexpr int TILE_BYTES = R * KB;            // same for KC and MC
     static constexpr int CHUNKS = TILE_BYTES / 16;
-    static constexpr int PER_THREAD = CHUNKS / NT;
-    static_assert(CHUNKS % NT == 0, "tile must split evenly over the workgroup");
+    // Fill instructions per thread.  When the tile does not split evenly over the
+    // workgroup (direct fills only), the waves past the end of the last pass wrap around
+    // and fetch chunks from the start of the tile a second time.
+    static constexpr int PER_THREAD = (CHUNKS + NT - 1) / NT;
+    static constexpr bool EVEN_SPLIT = CHUNKS % NT == 0;
+    static_assert(CHUNKS % 64 == 0, "whole waves");
     // KC: one LDS row is one matrix row (KB bytes); MC: one LDS row is one k (R elements).
     static constexpr int ROW_BYTES = KC ? KB : R * ES;
     static constexpr int CPR = ROW_BYTES / 16;           // 16-byte chunks per LDS row
@@ -145,6 +149,9 @@ struct OperandTile {
         int row = tid / CPR, cpos = tid % CPR;
         return (unsigned)global_off(row, swizzle(row, cpos), 0, 0, ld);
     }
+    // Global byte distance covered by all LDS rows of the tile (for the wrap-around above).
+    __device__ static __forceinline__ int64_t wrap_bytes(int64_t ld) { return global_off(CHUNKS / CPR, 0, 0, 0, ld); }
+    static_assert(EVEN_SPLIT || (CHUNKS / CPR) % SWIZZLE_PERIOD == 0, "wrap-around keeps the swizzle phase");
     // Uniform base of fill i for the tile at (r0, k0).
     __device__ static __forceinline__ const char* direct_base(const char* base, int i, int r0, int k0, int64_t ld)
     {
@@ -294,13 +301,23 @@ __global__ void __launch_bounds__(Cfg::NT, Cfg::WGS_PER_CU) gemm_mfma_kernel(Gem
     }
     constexpr int FILLS_A = TA::PER_THREAD, FILLS_B = TB::PER_THREAD, FILLS = FILLS_A + FILLS_B;
     // fill number f of the tile starting at K element k0 into stage buffer `stage`
+    static_assert(DIRECT || (TA::EVEN_SPLIT && TB::EVEN_SPLIT), "register-staged fills need an even split");
+    auto fill_one = [&](auto tile_tag, int f, unsigned lds_tile, unsigned lane_off, const char* base, int r0, int k0,
+                        int64_t ld) {
+        using T = decltype(tile_tag);
+        unsigned pos = wave_lds + f * NT * 16; // byte position of this wave's 1 KB inside the tile (wave-uniform)
+        const char* src = T::direct_base(base, f, r0, k0, ld);
+        if constexpr (!T::EVEN_SPLIT) {
+            if (pos >= (unsigned)T::TILE_BYTES) {
+                pos -= T::TILE_BYTES;
+                src -= T::wrap_bytes(ld);
+            }
+        }
+        T::direct_issue(lds_tile + pos, lane_off, src);
+    };
     auto issue_fill = [&](int f, int stage, int k0) {
-        if (f < FILLS_A)
-            TA::direct_issue(smem_addr + stage * STAGE_BYTES + wave_lds + f * NT * 16, a_lane_off,
-                             TA::direct_base(Ab, f, m0, k0, lda));
-        else
-            TB::direct_issue(smem_addr + stage * STAGE_BYTES + TA::TILE_BYTES + wave_lds + (f - FILLS_A) * NT * 16,
-                             b_lane_off, TB::direct_base(Bb, f - FILLS_A, n0, k0, ldb));
+        if (f < FILLS_A) fill_one(TA{}, f, smem_addr + stage * STAGE_BYTES, a_lane_off, Ab, m0, k0, lda);
+        else fill_one(TB{}, f - FILLS_A, smem_addr + stage * STAGE_BYTES + TA::TILE_BYTES, b_lane_off, Bb, n0, k0, ldb);
     };
 
     // MFMAs of one K tile.  Fragments are double-buffered across the k-steps: the LDS
@@ -493,15 +510,19 @@ __global__ void __launch_bounds__(Cfg::NT, Cfg::WGS_PER_CU) gemm_mfma_kernel(Gem
     // C is row-major here (the host transposes the problem otherwise).  Addresses are a
     // workgroup-uniform tile base plus one 32-bit offset per accumulator row, so the
     // write-back needs no 64-bit address registers next to the live accumulators.
-    const bool is_relu = p.epilogue == EPI_RELU, is_nocond = p.epilogue == EPI_RELU_NOCOND;
-    auto epilogue = [&](scalar_t v) -> scalar_t { // two selects on wave-uniform conditions, no per-element branch
-        scalar_t r = v > scalar_t(0) ? v : scalar_t(0);
-        scalar_t n = v * (v > scalar_t(0) ? scalar_t(1) : scalar_t(0));
-        return is_relu ? r : (is_nocond ? n : v);
+    // The epilogue kind is wave-uniform: ReLU (the fused path) gets its own copy of the
+    // write-back with a single max per element, the other kinds share one with selects.
+    const bool is_nocond = p.epilogue == EPI_RELU_NOCOND;
+    auto epilogue = [&](scalar_t v, auto relu_tag) -> scalar_t {
+        if constexpr (decltype(relu_tag)::value) return v > scalar_t(0) ? v : scalar_t(0);
+        else {
+            scalar_t n = v * (v > scalar_t(0) ? scalar_t(1) : scalar_t(0));
+            return is_nocond ? n : v;
+        }
     };
     const bool accumulate = p.prologue == PRO_NONE;
     const int row_in_tile = wr0 + (lane >> 5) * 4, col_in_tile = wc0 + (lane & 31);
-    auto write_back = [&](auto out_tag) {
+    auto write_back = [&](auto out_tag, auto relu_tag) {
         using out_t = decltype(out_tag);
         constexpr unsigned OS = sizeof(out_t);
         char* tile_base = (char*)p.C + ((int64_t)m0 * p.c_rs + n0) * OS; // uniform
@@ -521,24 +542,85 @@ __global__ void __launch_bounds__(Cfg::NT, Cfg::WGS_PER_CU) gemm_mfma_kernel(Gem
                     scalar_t v = acc[i][j][r];
                     if constexpr (std::is_same<out_t, int>::value) {
                         if (accumulate) v = (int)((unsigned)v + (unsigned)*dst);
-                        *dst = epilogue(v);
+                        *dst = epilogue(v, relu_tag);
                     } else if constexpr (std::is_same<out_t, float>::value) {
                         if (accumulate) v += *dst;
-                        *dst = epilogue(v);
+                        *dst = epilogue(v, relu_tag);
                     } else if constexpr (std::is_same<out_t, _Float16>::value) {
                         if (accumulate) v += (float)*dst;
-                        *dst = (_Float16)epilogue(v); // v_cvt_f16_f32: round to nearest even
+                        *dst = (_Float16)epilogue(v, relu_tag); // v_cvt_f16_f32: round to nearest even
                     } else { // bf16 bits
                         if (accumulate) v += bf16_bits_to_float(*dst);
-                        *dst = float_to_bf16_bits(epilogue(v));
+                        *dst = float_to_bf16_bits(epilogue(v, relu_tag));
                     }
                 }
             }
     };
-    if constexpr (IN == IN_I8) write_back(int{});
-    else if (p.out_type == T_F32) write_back(float{});
-    else if (p.out_type == T_F16) write_back(_Float16{});
-    else write_back(uint16_t{});
+    // 16-bit outputs: a lane's accumulators are one column wide, so direct stores write
+    // 64-byte pieces of a row per instruction.  Instead each wave stages 32 rows of its
+    // tile in a private slab of the (now idle) LDS tile buffers, two columns packed per
+    // dword after a swap with the neighbouring lane, and streams them out as 16-byte
+    // pieces that cover whole rows of the wave tile.
+    constexpr int PITCH_DW = (WTN / 2) % 32 == 16 ? WTN / 2 : WTN / 2 + 16; // rows r, r+1 in different bank halves
+    constexpr bool CAN_STAGE = !EDGE && IN != IN_I8 && (NT / 64) * 32 * PITCH_DW * 4 <= Cfg::LDS_BYTES;
+    auto write_back_staged = [&](auto out_tag, auto relu_tag) {
+        using out_t = decltype(out_tag);
+        const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+        unsigned* slab = (unsigned*)(smem + wave_u * (32 * PITCH_DW * 4));
+        const int odd = lane & 1;
+        const int wrow = (lane >> 5) * 4 + odd, wcol = (lane & 31) >> 1;
+        char* wave_base = (char*)p.C + ((int64_t)(m0 + (wave_u / WAVES_N) * WTM) * p.c_rs + n0 + (wave_u % WAVES_N) * WTN) * 2;
+        const unsigned row_bytes = (unsigned)p.c_rs * 2;
+        constexpr int CPRW = WTN / 8;             // 16-byte pieces per row of the wave tile
+        constexpr int PIECES = 32 * CPRW / 64;    // per lane and 32-row slab
+        // (lo, hi) = (own row 2t, own row 2t+1) narrowed with round-to-nearest-even
+        auto pack2 = [&](float lo, float hi) -> unsigned {
+            if constexpr (std::is_same<out_t, _Float16>::value) {
+                typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+                return __builtin_bit_cast(unsigned, h2{(_Float16)lo, (_Float16)hi});
+            } else {
+                typedef __bf16 b2 __attribute__((ext_vector_type(2)));
+                return __builtin_bit_cast(unsigned, b2{(__bf16)lo, (__bf16)hi});
+            }
+        };
+        // even lane (column c):   row 2t   <- (own lo, neighbour lo) = columns c, c+1
+        // odd lane  (column c+1): row 2t+1 <- (neighbour hi, own hi)
+        const unsigned sel = odd ? 0x03020706u : 0x05040100u; // v_perm_b32: bytes 0-3 from own, 4-7 from neighbour
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int t = 0; t < 8; ++t) {
+                    const unsigned own = pack2(epilogue(acc[i][j][2 * t], relu_tag), epilogue(acc[i][j][2 * t + 1], relu_tag));
+                    const unsigned nbr = (unsigned)__builtin_amdgcn_update_dpp(0, (int)own, 0xB1, 0xF, 0xF, true); // lane ^ 1
+                    const int row = (t >> 1) * 8 + (t & 1) * 2 + wrow;
+                    slab[row * PITCH_DW + j * 16 + wcol] = __builtin_amdgcn_perm(nbr, own, sel);
+                }
+#pragma unroll
+            for (int it = 0; it < PIECES; ++it) {
+                const int id = it * 64 + lane;
+                const int row = id / CPRW, cc = id % CPRW;
+                const i32x4 v = *(const i32x4*)(slab + row * PITCH_DW + cc * 4);
+                *(i32x4*)(wave_base + (unsigned)(i * 32 + row) * row_bytes + cc * 16) = v;
+            }
+        }
+    };
+    const bool staged = CAN_STAGE && !accumulate && p.c_rs % 8 == 0 && ((size_t)p.C & 15) == 0;
+    auto write_back_any = [&](auto relu_tag) {
+        if constexpr (IN == IN_I8) write_back(int{}, relu_tag);
+        else if (p.out_type == T_F32) write_back(float{}, relu_tag);
+        else if (CAN_STAGE && staged) {
+            if constexpr (CAN_STAGE) {
+                __syncthreads(); // every wave is done reading the tile buffers
+                if (p.out_type == T_F16) write_back_staged(_Float16{}, relu_tag);
+                else write_back_staged(uint16_t{}, relu_tag);
+            }
+        } else if (p.out_type == T_F16) write_back(_Float16{}, relu_tag);
+        else write_back(uint16_t{}, relu_tag);
+    };
+    if (p.epilogue == EPI_RELU) write_back_any(std::true_type{});
+    else write_back_any(std::false_type{});
 }
 
 // Host launcher for one kernel instantiation.

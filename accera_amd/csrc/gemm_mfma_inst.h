@@ -19,9 +19,7 @@ namespace acc950 {
       &launch_mfma<MfmaConfig<ACC950_IN, BM, BN, WM, WN, true, BKC, true, false, KB, STAGES, true>> }
 
 #define LAYOUT(BKC)                                 \
-    V(256, 256, 2, 2, BKC, true, false, 128, 2),    \
     V(256, 256, 2, 4, BKC, true, false, 128, 2),    \
-    V(256, 256, 2, 2, BKC, true, false, 64, 4),     \
     V(256, 256, 2, 4, BKC, true, false, 64, 4),     \
     V(256, 256, 2, 4, BKC, true, false, 64, 3),     \
     V(256, 128, 2, 2, BKC, true, false, 128, 3),    \
@@ -39,7 +37,7 @@ static const MfmaVariant kVariants[] = {
     LAYOUT(false), // B row-major (N contiguous): transpose reads
     LAYOUT(true),  // B column-major (K contiguous)
     // 192-wide tiles (N = 3072 = 16 x 192 gives one tile per CU); K-contiguous B only
-    VP(256, 192, 4, 2, true, 128, 2),
+    VP(256, 192, 4, 2, true, 64, 4),
     V(256, 192, 4, 2, true, true, false, 128, 2),
 };
 #undef LAYOUT

@@ -204,8 +204,9 @@ def measure(name, steps, warmup, variant=-1, k_splits=0):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--steps", type=int, default=500)
+    ap.add_argument("--warmup", type=int, default=500,
+                    help="untimed steps; the engine clock takes some tens of ms of load to settle after idle")
     ap.add_argument("--config", default="c2", choices=sorted(CONFIGS))
     ap.add_argument("--variant", type=int, default=-1)
     ap.add_argument("--k-splits", type=int, default=0)

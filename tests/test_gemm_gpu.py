@@ -270,6 +270,42 @@ def test_relu_special_values(variant, epi):
     assert np.array_equal(np.signbit(got[ok]), np.signbit(want[ok]))
 
 
+@pytest.mark.parametrize("out_type", ["bf16", "f16"])
+@pytest.mark.parametrize("variant,prologue", [(-1, ora.PRO_SET0), (-1, ora.PRO_NONE), (200, ora.PRO_SET0)])
+def test_narrowing_store_rounds_to_nearest_even(out_type, variant, prologue):
+    """x + y is exact in the float accumulator and lands on / next to a rounding tie of the
+    16-bit output type: the store must round to nearest even, overflow to inf and keep NaN
+    (the widen-accumulate-narrow rule, CppPrinterUtils.h:95-118 with LLVM's host rounding).
+    Covers the packed (SET prologue) and the element-wise (accumulating, generic) stores."""
+    import accera_amd as acc
+    import torch
+    in_type = "bf16" if out_type == "bf16" else "f16"
+    mant = 7 if out_type == "bf16" else 10
+    u = 2.0 ** -mant                       # ulp of the output type at 1.0
+    big = (2 - u) * (2.0 ** 127 if out_type == "bf16" else 2.0 ** 15)   # largest finite
+    pairs = [(1.0, u / 2), (1.0 + u, u / 2), (1.0, u / 2 * (1 + u)), (1.0 + u, u / 4), (-1.0, -u / 2), (-1.0 - u, -u / 2),
+             (big, big * u / 4), (big, big), (-big, -big * u / 4), (np.inf, 1.0), (np.nan, 1.0), (3.0, -3.0), (0.375, u * 0.375 / 2),
+             (1024.0, 1024 * 3 * u / 2), (1.0, 0.0), (-2.5, 0.0)]
+    M, N, K = 128, 128, 32
+    x = np.array([p[0] for p in pairs] * (M // len(pairs)), np.float32)
+    y = np.array([p[1] for p in pairs] * (M // len(pairs)), np.float32)
+    Af = np.zeros((M, K), np.float32)
+    Af[:, 3], Af[:, 17] = x, y
+    Bf = np.zeros((K, N), np.float32)
+    Bf[3, :], Bf[17, :] = 1.0, 1.0
+    A, B = ora.narrow(Af, in_type), ora.narrow(Bf, in_type)
+    assert np.array_equal(ora.widen(A, in_type)[:, 3][~np.isnan(x)], x[~np.isnan(x)].astype(np.float64)), "inputs must be exact"
+    C0 = ora.narrow(np.zeros((M, N), np.float32), out_type)
+    dC = to_device(C0, out_type)
+    acc.gemm_relu(to_device(A, in_type), to_device(B, in_type), dC, prologue=prologue, epilogue=acc.EPILOGUE_NONE, variant=variant)
+    torch.cuda.synchronize()
+    got = ora.widen(to_host(dC, out_type), out_type)
+    want = ora.widen(ora.narrow(x + y, out_type), out_type)[:, None].repeat(N, 1)
+    assert np.array_equal(np.isnan(got), np.isnan(want))
+    ok = ~np.isnan(want)
+    assert np.array_equal(got[ok], want[ok]), (got[:16, 0], want[:16, 0])
+
+
 def test_linearity_and_k_split_invariance_full_size_int8():
     """Size-independent property at a large size: for int8, A@[B1|B2] computed as one
     N=2048 problem equals the two N=1024 problems, and equals int64 NumPy on sampled rows."""
