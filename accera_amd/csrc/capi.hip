@@ -117,17 +117,28 @@ bool mfma_can_take(const MfmaVariant& v, const Problem& pb)
     return true;
 }
 
-bool skinny_can_take(const Problem& pb)
+bool skinny_can_take(const Problem& pb, int sv)
 {
     const GemmArgs& g = pb.g;
+    const SkinnyVariant& v = skinny_variant(sv);
     if (g.in_type != T_F16 && g.in_type != T_BF16) return false;
-    if (g.M < 1 || g.M > 8 || g.N < 8 || g.K < 2) return false;
+    if (g.M < 1 || g.M > v.max_m || g.N < 8 || g.K < v.k_step) return false;
     if (g.a_cs != 1 || g.b_cs != 1 || g.c_cs != 1) return false;
-    if (g.N % 8 || g.K % 2 || g.b_rs % 8 || g.a_rs % 2) return false;
+    if (g.N % 8 || g.K % v.k_step || g.b_rs % 8) return false;
+    if (g.a_rs % (v.mfma ? 8 : 2)) return false; // A pieces are fetched 16 (4) bytes at a time
     // per-lane offsets of the direct-to-LDS fills are 32-bit
-    if ((int64_t)g.K * g.b_rs * 2 >= (1ll << 32) || (int64_t)8 * g.a_rs * 2 >= (1ll << 32)) return false;
-    if (pb.have_pointers && (!aligned16(g.B) || (reinterpret_cast<uintptr_t>(g.A) & 3u))) return false;
+    if ((int64_t)g.K * g.b_rs * 2 >= (1ll << 32) || (int64_t)v.max_m * g.a_rs * 2 >= (1ll << 32)) return false;
+    if (pb.have_pointers && (!aligned16(g.B) || (reinterpret_cast<uintptr_t>(g.A) & (v.mfma ? 15u : 3u)))) return false;
     return true;
+}
+
+// First skinny variant that takes the problem (the table lists the MFMA family first, best
+// first), or -1.
+int auto_skinny_variant(const Problem& pb)
+{
+    for (int sv = 0; sv < skinny_num_variants(); ++sv)
+        if (skinny_can_take(pb, sv)) return sv;
+    return -1;
 }
 
 // ---- scratch for the skinny kernels' K split -----------------------------------------
@@ -158,8 +169,6 @@ hipError_t ensure_workspace(size_t floats, size_t counters)
     }
     return hipSuccess;
 }
-
-int auto_skinny_variant(const GemmArgs&) { return 0; }
 
 int auto_skinny_splits(int variant, const GemmArgs& g)
 {
@@ -216,8 +225,8 @@ int choose(const Problem& pb, int variant, int k_splits, Choice* c)
 {
     c->splits = 1;
     if (variant == ACC950_VARIANT_AUTO) {
-        if (skinny_can_take(pb)) {
-            int sv = auto_skinny_variant(pb.g);
+        const int sv = auto_skinny_variant(pb);
+        if (sv >= 0) {
             c->variant = ACC950_VARIANT_SKINNY_BASE + sv;
             c->splits = k_splits > 0 ? k_splits : auto_skinny_splits(sv, pb.g);
             return ACC950_OK;
@@ -234,10 +243,14 @@ int choose(const Problem& pb, int variant, int k_splits, Choice* c)
         return ACC950_OK;
     }
     if (variant >= ACC950_VARIANT_SKINNY_BASE && variant < ACC950_VARIANT_SKINNY_BASE + skinny_num_variants()) {
-        if (!skinny_can_take(pb)) return fail(ACC950_UNSUPPORTED, "skinny kernel needs 16-bit inputs, M <= 8, row-major A/B/C, N % 8 == 0, K % 2 == 0");
+        const int sv = variant - ACC950_VARIANT_SKINNY_BASE;
+        if (!skinny_can_take(pb, sv))
+            return fail(ACC950_UNSUPPORTED, "skinny kernel needs 16-bit inputs, row-major A/B/C, N % 8 == 0, and M <= 32, K % 16 == 0 (MFMA family) "
+                                            "or M <= 8, K % 2 == 0 (dot-product family)");
         c->variant = variant;
-        c->splits = k_splits > 0 ? k_splits : auto_skinny_splits(variant - ACC950_VARIANT_SKINNY_BASE, pb.g);
-        if (c->splits > pb.g.K / 2) c->splits = pb.g.K / 2;
+        c->splits = k_splits > 0 ? k_splits : auto_skinny_splits(sv, pb.g);
+        const int max_splits = pb.g.K / skinny_variant(sv).k_step;
+        if (c->splits > max_splits) c->splits = max_splits;
         return ACC950_OK;
     }
     int n = 0;
@@ -267,8 +280,17 @@ int run(const Problem& pb, const Choice& c, hipStream_t stream, LaunchGeom* geom
         s.a_rs = g.a_rs; s.b_rs = g.b_rs; s.c_rs = g.c_rs;
         s.in_type = g.in_type; s.out_type = g.out_type; s.prologue = g.prologue; s.epilogue = g.epilogue;
         s.splits = c.splits;
-        if (!dry_run && c.splits > 1) {
-            e = ensure_workspace(skinny_scratch_floats(sv, g.N, c.splits), (size_t)skinny_column_blocks(sv, g.N));
+        s.extra_phase = -1;
+        // 64-column MFMA blocks, no K split, dense rows of a multiple of 512 bytes: blocks whose
+        // 128-byte lines have address bits 8:7 = 11 stream ~25 % slower (measured), so they are
+        // shared by two workgroups each; the otherwise idle CUs take the second halves.
+        const SkinnyVariant& skv = skinny_variant(sv);
+        if (skv.mfma && skv.cols == 64 && c.splits == 1 && pb.have_pointers && (g.b_rs * 2) % 512 == 0 &&
+            skinny_column_blocks(sv, g.N) >= 128 && skinny_column_blocks(sv, g.N) <= 200 && g.K >= 512)
+            s.extra_phase = (int)((3u - (unsigned)(reinterpret_cast<uintptr_t>(g.B) >> 7)) & 3u);
+        const int ws_splits = s.extra_phase >= 0 ? 2 : c.splits;
+        if (!dry_run && ws_splits > 1) {
+            e = ensure_workspace(skinny_scratch_floats(sv, g.N, ws_splits), (size_t)skinny_column_blocks(sv, g.N));
             if (e != hipSuccess) return fail_hip(e, "workspace allocation");
             s.scratch = g_scratch;
             s.counters = g_counters;
@@ -416,7 +438,8 @@ int acc950_variant_name(int variant, char* buf, size_t buf_len)
     if (variant >= ACC950_VARIANT_SKINNY_BASE && variant < ACC950_VARIANT_SKINNY_BASE + skinny_num_variants()) {
         int lpr, waves, depth;
         skinny_variant_info(variant - ACC950_VARIANT_SKINNY_BASE, &lpr, &waves, &depth);
-        std::snprintf(buf, buf_len, "skinny cols/wg=%d waves=%d depth=%d", lpr * 8, waves, depth);
+        std::snprintf(buf, buf_len, "skinny %s cols/wg=%d waves=%d depth=%d",
+                      skinny_variant(variant - ACC950_VARIANT_SKINNY_BASE).mfma ? "mfma" : "dot2", lpr * 8, waves, depth);
         return ACC950_OK;
     }
     int n = 0;

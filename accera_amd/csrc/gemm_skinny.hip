@@ -61,7 +61,14 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_skinny_kernel(SkinnyArgs p)
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int kp = lane / LPR, cg = lane % LPR;
-    const int col0 = blockIdx.x * CB + cg * 8;
+    // Workgroup ids are dealt round-robin to the 8 XCDs; column block = (id % 8) * per + id / 8
+    // gives every XCD a contiguous range of blocks, hence all residues of the 128-byte line
+    // index and all channels of its L2 (ids mapped 1:1 to blocks would leave an XCD with
+    // every 8th line of a row only).
+    const int nblocks = (p.N + CB - 1) / CB;
+    const int bx = (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
+    if (bx >= nblocks) return;
+    const int col0 = bx * CB + cg * 8;
     const bool col_ok = col0 < p.N; // N is a multiple of 8
 
     // K range of this workgroup, in k pairs
@@ -198,12 +205,12 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_skinny_kernel(SkinnyArgs p)
     // level of the memory system that all XCDs share), so no cache-wide write-back is
     // needed: the stores only have to be acknowledged (vmcnt = 0) before this workgroup
     // takes its ticket.
-    float* part = p.scratch + ((int64_t)blockIdx.y * gridDim.x + blockIdx.x) * (64 * LPR);
+    float* part = p.scratch + ((int64_t)blockIdx.y * nblocks + bx) * (64 * LPR);
 #pragma unroll
     for (int j = 0; j < VPL; ++j) __hip_atomic_store(part + j * 64 + lane, v[j], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     unsigned ticket = 0;
-    if (lane == 0) ticket = __hip_atomic_fetch_add(p.counters + blockIdx.x, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (lane == 0) ticket = __hip_atomic_fetch_add(p.counters + bx, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     ticket = __shfl(ticket, 0, 64);
     if (ticket != (unsigned)p.splits - 1) return;
     // last arrival: drop any stale copies of the scratch lines from this XCD's caches, then
@@ -213,13 +220,13 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_skinny_kernel(SkinnyArgs p)
 #pragma unroll
     for (int j = 0; j < VPL; ++j) sum[j] = 0.f;
     for (int sp = 0; sp < p.splits; ++sp) {
-        const float* src = p.scratch + ((int64_t)sp * gridDim.x + blockIdx.x) * (64 * LPR) + lane;
+        const float* src = p.scratch + ((int64_t)sp * nblocks + bx) * (64 * LPR) + lane;
 #pragma unroll
         for (int j = 0; j < VPL; ++j) sum[j] += src[j * 64];
     }
 #pragma unroll
     for (int j = 0; j < VPL; ++j) finish((j + VPL * kp) >> 3, (j + VPL * kp) & 7, sum[j]);
-    if (lane == 0) p.counters[blockIdx.x] = 0; // ready for the next launch
+    if (lane == 0) p.counters[bx] = 0; // ready for the next launch
 }
 
 template <bool BF16, int LPR, int WAVES, int DEPTH>
@@ -230,7 +237,7 @@ hipError_t launch_one(const SkinnyArgs& a, hipStream_t stream, LaunchGeom* geom,
     unsigned lds = WAVES * DEPTH * (2048 + 256);
     const unsigned red = (WAVES - 1) * LPR * 64 * 4;
     if (lds < red) lds = red;
-    dim3 grid((a.N + CB - 1) / CB, a.splits, 1), block(WAVES * 64, 1, 1);
+    dim3 grid(((a.N + CB - 1) / CB + 7) / 8 * 8, a.splits, 1), block(WAVES * 64, 1, 1);
     if (geom) {
         geom->grid[0] = grid.x; geom->grid[1] = grid.y; geom->grid[2] = 1;
         geom->block[0] = block.x; geom->block[1] = geom->block[2] = 1;
@@ -248,35 +255,50 @@ hipError_t launch_one(const SkinnyArgs& a, hipStream_t stream, LaunchGeom* geom,
     return hipGetLastError();
 }
 
-struct SkinnyVariant {
-    int lpr, waves, depth;
-    hipError_t (*f16)(const SkinnyArgs&, hipStream_t, LaunchGeom*, bool);
-    hipError_t (*bf16)(const SkinnyArgs&, hipStream_t, LaunchGeom*, bool);
-};
-#define SV(LPR, W, D) { LPR, W, D, &launch_one<false, LPR, W, D>, &launch_one<true, LPR, W, D> }
-const SkinnyVariant kSkinny[] = { SV(8, 4, 8), SV(8, 8, 4), SV(8, 8, 8), SV(8, 4, 4), SV(8, 16, 4), SV(8, 16, 2), SV(16, 4, 8), SV(16, 8, 4), SV(32, 4, 8) };
+#define SV(LPR, W, D) { LPR * 8, W, D, false, 8, 2, 64 * LPR, &launch_one<false, LPR, W, D>, &launch_one<true, LPR, W, D> }
+const SkinnyVariant kSkinny[] = { SV(8, 4, 8), SV(8, 8, 4), SV(16, 4, 8), SV(32, 4, 8) };
 #undef SV
-constexpr int kNumSkinny = (int)(sizeof(kSkinny) / sizeof(kSkinny[0]));
 
 } // namespace
 
-int skinny_num_variants() { return kNumSkinny; }
+const SkinnyVariant* skinny_dot2_table(int* count)
+{
+    *count = (int)(sizeof(kSkinny) / sizeof(kSkinny[0]));
+    return kSkinny;
+}
+
+int skinny_num_variants()
+{
+    int a, b;
+    skinny_mfma_table(&a);
+    skinny_dot2_table(&b);
+    return a + b;
+}
+const SkinnyVariant& skinny_variant(int v)
+{
+    int a, b;
+    const SkinnyVariant* m = skinny_mfma_table(&a);
+    const SkinnyVariant* d = skinny_dot2_table(&b);
+    return v < a ? m[v] : d[v - a];
+}
 void skinny_variant_info(int v, int* lpr, int* waves, int* depth)
 {
-    *lpr = kSkinny[v].lpr;
-    *waves = kSkinny[v].waves;
-    *depth = kSkinny[v].depth;
+    const SkinnyVariant& s = skinny_variant(v);
+    *lpr = s.cols / 8;
+    *waves = s.waves;
+    *depth = s.depth;
 }
-int skinny_column_blocks(int v, int N) { return (N + kSkinny[v].lpr * 8 - 1) / (kSkinny[v].lpr * 8); }
+int skinny_column_blocks(int v, int N) { return (N + skinny_variant(v).cols - 1) / skinny_variant(v).cols; }
 size_t skinny_scratch_floats(int v, int N, int splits)
 {
-    return splits <= 1 ? 0 : (size_t)splits * skinny_column_blocks(v, N) * 64 * kSkinny[v].lpr;
+    return splits <= 1 ? 0 : (size_t)splits * skinny_column_blocks(v, N) * skinny_variant(v).block_floats;
 }
 
 hipError_t launch_skinny(int v, const SkinnyArgs& a, hipStream_t stream, LaunchGeom* geom, bool dry_run)
 {
-    if (v < 0 || v >= kNumSkinny) return hipErrorInvalidValue;
-    return a.in_type == T_BF16 ? kSkinny[v].bf16(a, stream, geom, dry_run) : kSkinny[v].f16(a, stream, geom, dry_run);
+    if (v < 0 || v >= skinny_num_variants()) return hipErrorInvalidValue;
+    const SkinnyVariant& s = skinny_variant(v);
+    return a.in_type == T_BF16 ? s.bf16(a, stream, geom, dry_run) : s.f16(a, stream, geom, dry_run);
 }
 
 } // namespace acc950

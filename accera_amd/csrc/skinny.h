@@ -1,4 +1,4 @@
-// Host-visible interface of the skinny (M <= 8) streaming GEMM kernels.
+// Host-visible interface of the skinny (few rows of A) streaming GEMM kernels.
 #pragma once
 #include "common.h"
 #include <stddef.h>
@@ -14,11 +14,33 @@ struct SkinnyArgs {
     int in_type, out_type;
     int prologue, epilogue;
     int splits;         // K split over grid.y
-    float* scratch;     // splits > 1: [split][column block][64*LPR] partial sums
+    int extra_phase;    // MFMA family, splits == 1: column blocks with index % 4 == extra_phase are split in two
+                        // (second halves run as extra workgroups behind the regular grid); -1: none
+    float* scratch;     // splits > 1: [split][column block][floats per block] partial sums
     unsigned* counters; // splits > 1: one arrival counter per column block, zero between launches
 };
 
+typedef hipError_t (*SkinnyLaunchFn)(const SkinnyArgs&, hipStream_t, LaunchGeom*, bool);
+
+// One kernel instantiation.  Two families: "dot2" (packed dot products on the vector
+// ALU, M <= 8, K even) and "mfma" (B transposed out of LDS into MFMA operands, M <= 32,
+// K a multiple of 16 per split).
+struct SkinnyVariant {
+    int cols;          // columns per workgroup
+    int waves, depth;  // waves per workgroup, ring slots (steps in flight) per wave
+    bool mfma;
+    int max_m;         // rows of A the kernel can take
+    int k_step;        // K rows per wave step; every K split is a whole number of steps
+    int block_floats;  // scratch floats per column block and split
+    SkinnyLaunchFn f16, bf16;
+};
+
+// tables of the two families (gemm_skinny.hip, gemm_skinny_mfma.hip)
+const SkinnyVariant* skinny_dot2_table(int* count);
+const SkinnyVariant* skinny_mfma_table(int* count);
+
 int skinny_num_variants();
+const SkinnyVariant& skinny_variant(int v); // MFMA family first, then dot2
 void skinny_variant_info(int v, int* lanes_per_row, int* waves, int* depth);
 int skinny_column_blocks(int v, int N);
 size_t skinny_scratch_floats(int v, int N, int splits);

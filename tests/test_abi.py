@@ -48,7 +48,7 @@ def test_launch_geometry_of_the_configs():
     g, b, lds, v = _lib.launch_geometry(_lib.I8, _lib.I32, 8192, 8192, 8192, (8192, 1), (8192, 1), (8192, 1))
     assert "mfma" in _lib.variant_name(v)
     g, b, lds, v = _lib.launch_geometry(_lib.F16, _lib.F16, 8, 11008, 4096, (4096, 1), (11008, 1), (11008, 1))
-    assert "skinny" in _lib.variant_name(v) and g[0] == 11008 // 64 and b[0] % 64 == 0
+    assert "skinny" in _lib.variant_name(v) and g[0] * g[1] >= 43 and b[0] % 64 == 0
     g, b, lds, v = _lib.launch_geometry(_lib.F32, _lib.F32, 512, 512, 512, (512, 1), (512, 1), (512, 1))
     assert v == _lib.VARIANT_F32_MFMA and g[:2] == [16, 16]
     # unaligned shapes fall to the thread-bound kernel, explicit variants refuse them

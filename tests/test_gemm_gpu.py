@@ -176,14 +176,26 @@ def test_readme_quickstart_shape_and_data():
 @pytest.mark.parametrize("in_type,out_type", [("f16", "f16"), ("f16", "f32"), ("bf16", "bf16")])
 def test_skinny_all_variants_and_splits(in_type, out_type):
     from accera_amd import _lib
-    for sv in range(_lib.num_skinny_variants()):
+    names = [_lib.variant_name(100 + sv) for sv in range(_lib.num_skinny_variants())]
+    for sv, name in enumerate(names):
         for splits in (1, 3, 8):
-            print("skinny", sv, _lib.variant_name(100 + sv), "splits", splits, flush=True)
+            print("skinny", sv, name, "splits", splits, flush=True)
             run_case(in_type, out_type, 8, 1024 + 64, 1024, variant=100 + sv, splits=splits, seed=sv * 10 + splits, dist="normal")
-    # ragged: M < 8, N not a multiple of the column block, K not a multiple of the k step
-    run_case(in_type, out_type, 5, 1000, 998, variant=100, splits=4, seed=77, dist="normal")
-    run_case(in_type, out_type, 1, 8, 2, variant=100, splits=1, seed=78, dist="normal", epilogue=ora.EPI_NONE)
+    mfma = 100 + next(i for i, n in enumerate(names) if "mfma" in n)
+    dot2 = 100 + next(i for i, n in enumerate(names) if "dot2" in n)
+    # matrix-core family: up to 32 rows of A; ragged M, N not a multiple of the column block,
+    # fewer k steps than waves, more splits than steps allow
+    run_case(in_type, out_type, 32, 1024 + 64, 1024, variant=mfma, splits=2, seed=70, dist="normal")
+    run_case(in_type, out_type, 17, 1000, 1008, variant=mfma, splits=4, seed=71, dist="normal")
+    run_case(in_type, out_type, 1, 8, 16, variant=mfma, splits=1, seed=72, dist="normal", epilogue=ora.EPI_NONE)
+    run_case(in_type, out_type, 3, 72, 48, variant=mfma, splits=8, seed=73, dist="normal")
+    # dot-product family: M < 8, K not a multiple of the k step
+    run_case(in_type, out_type, 5, 1000, 998, variant=dot2, splits=4, seed=77, dist="normal")
+    run_case(in_type, out_type, 1, 8, 2, variant=dot2, splits=1, seed=78, dist="normal", epilogue=ora.EPI_NONE)
+    # automatic choice: K % 16 != 0 falls to the dot-product family; accumulate into C
+    run_case(in_type, out_type, 5, 1000, 998, seed=74, dist="normal")
     run_case(in_type, out_type, 8, 2048, 512, seed=79, dist="normal", prologue=ora.PRO_NONE)
+    run_case(in_type, out_type, 24, 2048, 512, seed=80, dist="normal", prologue=ora.PRO_NONE, epilogue=ora.EPI_RELU_NOCOND)
 
 
 def test_skinny_repeated_launches_reuse_counters():
