@@ -21,7 +21,7 @@ VARIANT_AUTO, VARIANT_SKINNY_BASE, VARIANT_GENERIC, VARIANT_F32_MFMA = -1, 100, 
 EXPORTS = [
     "acc950_init", "acc950_gemm_relu", "acc950_gemm_relu_ex", "acc950_gemm_relu_host",
     "acc950_launch_geometry", "acc950_num_variants", "acc950_num_skinny_variants",
-    "acc950_variant_name", "acc950_last_error", "acc950_mfma_ceiling", "acc950_copy_probe", "acc950_stream_read_probe",
+    "acc950_variant_name", "acc950_last_error", "acc950_mfma_ceiling", "acc950_mfma_phase_probe", "acc950_copy_probe", "acc950_stream_read_probe",
 ]
 
 
@@ -54,6 +54,7 @@ def lib():
                                                                            ctypes.POINTER(cu), ctypes.POINTER(ci)]
     L.acc950_variant_name.argtypes = [ci, ctypes.c_char_p, ctypes.c_size_t]
     L.acc950_mfma_ceiling.argtypes = [ci, ci, ci, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double)]
+    L.acc950_mfma_phase_probe.argtypes = [ci, ci, ci, ci, ci, vp, vp, vp, ctypes.POINTER(ctypes.c_double)]
     L.acc950_copy_probe.argtypes = [vp, vp, ctypes.c_size_t, vp]
     L.acc950_stream_read_probe.argtypes = [vp, ctypes.c_size_t, vp, vp]
     L.acc950_last_error.restype = ctypes.c_char_p
@@ -67,6 +68,15 @@ def lib():
 def check(rc):
     if rc != OK:
         raise Acc950Error(rc, lib().acc950_last_error().decode())
+
+
+def mfma_phase_probe(in_type, out_type, M, N, K, a_ptr, b_ptr, c_ptr):
+    """In-kernel phase times of the 256x256 ping-pong kernel on device operands; returns a dict."""
+    out = (ctypes.c_double * 8)()
+    check(lib().acc950_mfma_phase_probe(in_type, out_type, M, N, K, a_ptr, b_ptr, c_ptr, out))
+    return {"prologue_us": out[0] / 1e3, "main_loop_us": out[1] / 1e3, "write_back_us": out[2] / 1e3,
+            "clock_ghz_prologue": out[3], "clock_ghz_main_loop": out[4], "clock_ghz_write_back": out[5],
+            "kernel_span_us": out[6] / 1e3, "mfma_pipe_busy_main_loop": out[7]}
 
 
 def mfma_ceiling(in_type, data_mode=2, iters=20000):

@@ -3,6 +3,7 @@
 #include "../../include/accera_mi355x_gemm.h"
 #include "common.h"
 #include "skinny.h"
+#include <vector>
 #include "variants.h"
 
 #include <cstdio>
@@ -362,6 +363,55 @@ int acc950_gemm_relu(int in_type, int out_type, int M, int N, int K,
 {
     return acc950_gemm_relu_ex(in_type, out_type, M, N, K, A, a_rs, a_cs, B, b_rs, b_cs, C, c_rs, c_cs, prologue, epilogue,
                                ACC950_VARIANT_AUTO, 0, stream);
+}
+
+int acc950_mfma_phase_probe(int in_type, int out_type, int M, int N, int K, const void* A, const void* B, void* C, double* out)
+{
+    if (!out) return fail(ACC950_INVALID_ARGUMENT, "null output");
+    Problem pb;
+    int rc = make_problem(in_type, out_type, M, N, K, A, K, 1, B, N, 1, C, N, 1, PRO_SET0, EPI_RELU, true, &pb);
+    if (rc) return rc;
+    const MfmaVariant probe = {256, 256, 2, 4, true, false, true, false, 64, 4, true, nullptr};
+    int n_unused = 0;
+    if (M < 256 || N < 256 || K < 1 || !mfma_table(pb.g.in_type, &n_unused) || !mfma_can_take(probe, pb))
+        return fail(ACC950_UNSUPPORTED, "the phase probe runs the 256x256 ping-pong kernel: 8/16-bit inputs, dense row-major A, B, C, M and N multiples of 256, K of 64 bytes");
+    GemmArgs g = pb.g;
+    const int tiles = (M / 256) * (N / 256);
+    hipError_t e = hipMalloc((void**)&g.stamps, (size_t)tiles * 8 * sizeof(unsigned long long));
+    if (e != hipSuccess) return fail_hip(e, "stamp buffer");
+    std::vector<unsigned long long> h((size_t)tiles * 8);
+    const int reps = 20; // the last launch is the one read back; the others settle the clocks
+    for (int i = 0; i < reps && e == hipSuccess; ++i) {
+        e = g.in_type == T_I8 ? launch_mfma_timed_i8(g, nullptr, nullptr, false)
+            : g.in_type == T_BF16 ? launch_mfma_timed_bf16(g, nullptr, nullptr, false) : launch_mfma_timed_f16(g, nullptr, nullptr, false);
+    }
+    if (e == hipSuccess) e = hipDeviceSynchronize();
+    if (e == hipSuccess) e = hipMemcpy(h.data(), g.stamps, h.size() * sizeof(unsigned long long), hipMemcpyDeviceToHost);
+    hipError_t e2 = hipFree(g.stamps);
+    if (e != hipSuccess) return fail_hip(e, "phase probe");
+    if (e2 != hipSuccess) return fail_hip(e2, "phase probe");
+    // per phase: average wall time (100 MHz counter) and average shader cycles over the workgroups
+    unsigned long long first = ~0ull, last = 0;
+    double ns[3] = {0, 0, 0}, cyc[3] = {0, 0, 0};
+    for (int t = 0; t < tiles; ++t) {
+        const unsigned long long* w = &h[(size_t)t * 8];
+        first = w[1] < first ? w[1] : first;
+        last = w[7] > last ? w[7] : last;
+        for (int q = 0; q < 3; ++q) {
+            ns[q] += (double)(w[(q + 1) * 2 + 1] - w[q * 2 + 1]) * 10.0;
+            cyc[q] += (double)(w[(q + 1) * 2] - w[q * 2]);
+        }
+    }
+    for (int q = 0; q < 3; ++q) {
+        out[q] = ns[q] / tiles;                       // prologue, main loop, write-back [ns]
+        out[3 + q] = ns[q] > 0 ? cyc[q] / ns[q] : 0;  // shader clock in that phase [GHz]
+    }
+    out[6] = (double)(last - first) * 10.0;           // first workgroup start to last workgroup end [ns]
+    // MFMA pipe occupancy of the main loop: two waves per SIMD, 8 MFMAs of 32 cycles per k step each
+    const int es = g.in_type == T_I8 ? 1 : 2;
+    const double mfma_cycles = 2.0 * 8.0 * 32.0 * ((double)K * es / 32.0);
+    out[7] = cyc[1] > 0 ? mfma_cycles / (cyc[1] / tiles) : 0;
+    return ACC950_OK;
 }
 
 int acc950_launch_geometry(int in_type, int out_type, int M, int N, int K,

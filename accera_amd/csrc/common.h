@@ -25,6 +25,7 @@ struct GemmArgs {
     int in_type, out_type;
     int prologue, epilogue;
     int tiles_m, tiles_n; // workgroup grid in tiles (MFMA kernels)
+    unsigned long long* stamps; // timed MFMA instantiation only: [workgroup][4 points][shader clock, 100 MHz clock]
 };
 
 typedef int i32x4 __attribute__((ext_vector_type(4)));

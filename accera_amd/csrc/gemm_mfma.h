@@ -232,9 +232,13 @@ __device__ __forceinline__ void tile_coords(int pid, int tiles_m, int tiles_n, i
 
 // Compile-time description of one kernel instantiation.
 template <int IN_, int BM_, int BN_, int WAVES_M_, int WAVES_N_, bool A_KC_, bool B_KC_, bool DIRECT_, bool EDGE_, int KB_, int STAGES_,
-          bool PINGPONG_ = false>
+          bool PINGPONG_ = false, bool TIMED_ = false>
 struct MfmaConfig {
     static constexpr bool PINGPONG = PINGPONG_;
+    // TIMED: wave 0 of every workgroup reads the shader-clock counter and the constant
+    // 100 MHz counter at kernel entry, after the prologue, after the main loop and at the
+    // end, and writes them to GemmArgs::stamps (phase times and the clock the engine ran at).
+    static constexpr bool TIMED = TIMED_;
     // workgroups meant to share a CU: as many as the LDS allows, at most 2 waves per SIMD in all
     static constexpr int WGS_PER_CU = (WAVES_M_ * WAVES_N_ <= 4 && 2 * STAGES_ * (BM_ + BN_) * KB_ <= 160 * 1024 && BM_ * BN_ <= 256 * 128) ? 2 : 1;
     static constexpr int IN = IN_, BM = BM_, BN = BN_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_, KB = KB_, STAGES = STAGES_;
@@ -273,6 +277,17 @@ __global__ void __launch_bounds__(Cfg::NT, Cfg::WGS_PER_CU) gemm_mfma_kernel(Gem
     const int wave = tid >> 6;
     const int wr0 = (wave / WAVES_N) * WTM;
     const int wc0 = (wave % WAVES_N) * WTN;
+
+    unsigned long long stamp_clk[4], stamp_ref[4];
+    auto stamp = [&](int i) {
+        if constexpr (Cfg::TIMED) {
+            __builtin_amdgcn_sched_barrier(0);
+            stamp_clk[i] = __builtin_amdgcn_s_memtime();
+            stamp_ref[i] = __builtin_amdgcn_s_memrealtime();
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    stamp(0);
 
     int tile_m, tile_n;
     tile_coords(blockIdx.x, p.tiles_m, p.tiles_n, tile_m, tile_n);
@@ -396,6 +411,7 @@ __global__ void __launch_bounds__(Cfg::NT, Cfg::WGS_PER_CU) gemm_mfma_kernel(Gem
         if (KT >= D) wait_vmcnt<(D - 1) * FILLS>();
         else wait_vmcnt<0>();
         __syncthreads();
+        stamp(1);
         if (group == 1) raw_barrier(); // one cluster behind
         // CL k-steps form one cluster: the whole K tile when it has 2 steps, half of it when 4
         constexpr int CL = 2, CLUSTERS = KSTEPS / CL, FPC = (FILLS + CLUSTERS - 1) / CLUSTERS;
@@ -457,6 +473,7 @@ __global__ void __launch_bounds__(Cfg::NT, Cfg::WGS_PER_CU) gemm_mfma_kernel(Gem
         if (KT >= D) wait_vmcnt<YOUNGER>();
         else wait_vmcnt<0>();
         __syncthreads();
+        stamp(1);
         if constexpr (CROSS) load_first_frags(smem, smem + TA::TILE_BYTES);
         int kt = 0;
         // steady state: tile kt+D exists and is fetched now
@@ -504,6 +521,7 @@ __global__ void __launch_bounds__(Cfg::NT, Cfg::WGS_PER_CU) gemm_mfma_kernel(Gem
         }
     }
 
+    stamp(2);
     // Write-back: optional "+= C" (no SET prologue), epilogue op, narrowing store.
     // MFMA 32x32 accumulator layout: register r of lane l holds
     //   row = (r/4)*8 + (l/32)*4 + r%4,  column = l%32.
@@ -621,6 +639,17 @@ __global__ void __launch_bounds__(Cfg::NT, Cfg::WGS_PER_CU) gemm_mfma_kernel(Gem
     };
     if (p.epilogue == EPI_RELU) write_back_any(std::true_type{});
     else write_back_any(std::false_type{});
+    if constexpr (Cfg::TIMED) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // stores acknowledged
+        stamp(3);
+        if (threadIdx.x == 0 && p.stamps) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                p.stamps[(blockIdx.x * 4 + i) * 2] = stamp_clk[i];
+                p.stamps[(blockIdx.x * 4 + i) * 2 + 1] = stamp_ref[i];
+            }
+        }
+    }
 }
 
 // Host launcher for one kernel instantiation.

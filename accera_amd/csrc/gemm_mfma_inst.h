@@ -44,6 +44,13 @@ static const MfmaVariant kVariants[] = {
 #undef V
 #undef VP
 
+// Timed build of the kernel the automatic choice takes for large aligned problems
+// (256x256 ping-pong, row-major B): same code plus four clock stamps per workgroup.
+hipError_t ACC950_TIMED_FN(const GemmArgs& a, hipStream_t stream, LaunchGeom* geom, bool dry_run)
+{
+    return launch_mfma<MfmaConfig<ACC950_IN, 256, 256, 2, 4, true, false, true, false, 64, 4, true, true>>(a, stream, geom, dry_run);
+}
+
 const MfmaVariant* ACC950_TABLE_FN(int* count)
 {
     *count = (int)(sizeof(kVariants) / sizeof(kVariants[0]));

@@ -20,6 +20,11 @@ const MfmaVariant* mfma_variants_f16(int* count);
 const MfmaVariant* mfma_variants_bf16(int* count);
 const MfmaVariant* mfma_variants_i8(int* count);
 
+// timed build of the 256x256 ping-pong kernel (row-major B, full tiles only)
+hipError_t launch_mfma_timed_f16(const GemmArgs& a, hipStream_t stream, LaunchGeom* geom, bool dry_run);
+hipError_t launch_mfma_timed_bf16(const GemmArgs& a, hipStream_t stream, LaunchGeom* geom, bool dry_run);
+hipError_t launch_mfma_timed_i8(const GemmArgs& a, hipStream_t stream, LaunchGeom* geom, bool dry_run);
+
 bool f32_can_take(const GemmArgs& g);
 hipError_t launch_f32(const GemmArgs& a, hipStream_t stream, LaunchGeom* geom, bool dry_run);
 hipError_t launch_generic(const GemmArgs& a, hipStream_t stream, LaunchGeom* geom, bool dry_run);

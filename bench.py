@@ -187,7 +187,17 @@ def machine_ceiling(c):
 
 def measure(name, steps, warmup, variant=-1, k_splits=0):
     c = CONFIGS[name]
-    wall, launch_s, _ = run_gpu(c, steps, warmup, variant, k_splits)
+    wall, launch_s, first_set = run_gpu(c, steps, warmup, variant, k_splits)
+    in_kernel = None
+    if c["bound"] == "mfma" and c["in_type"] in ("f16", "bf16", "i8") and c["b"] == "row" and c["M"] % 256 == 0 and c["N"] % 256 == 0 \
+            and variant < 0:
+        # clock stamps inside the 256x256 ping-pong kernel on the same operands: phase times, the
+        # engine clock in each phase, and how busy the MFMA pipe is at that clock
+        from accera_amd import _lib
+        A, B, C = first_set
+        in_kernel = {k: round(v, 4) for k, v in _lib.mfma_phase_probe(
+            getattr(_lib, c["in_type"].upper()), getattr(_lib, c["out_type"].upper()), c["M"], c["N"], c["K"],
+            A.data_ptr(), B.data_ptr(), C.data_ptr()).items()}
     flops, nbytes = algorithmic_flops(c), algorithmic_bytes(c)
     if c["bound"] == "hbm":
         achieved, peak, unit = nbytes / launch_s / 1e9, HBM_PEAK_GBS, "GB/s"
@@ -198,7 +208,7 @@ def measure(name, steps, warmup, variant=-1, k_splits=0):
     return dict(config=name, workload=c["workload"], value=round(value, 3), unit=vunit, ms_per_step=round(wall / steps * 1e3, 5),
                 roofline=dict(bound=c["bound"], achieved=round(achieved, 3), peak=peak, unit=unit,
                               frac=round(achieved / peak, 4), traffic=traffic_bytes(name)),
-                flops_per_launch=flops, bytes_per_launch=nbytes)
+                flops_per_launch=flops, bytes_per_launch=nbytes, in_kernel=in_kernel)
 
 
 def main():
@@ -245,6 +255,7 @@ def main():
                    "compute_units": torch.cuda.get_device_properties(0).multi_processor_count},
         "roofline": m["roofline"],
         "machine_ceiling": machine_ceiling(c),
+        "in_kernel": m["in_kernel"],
     }
     if not args.no_cpu:
         threads = min(16, os.cpu_count() or 1)
