@@ -9,8 +9,8 @@ Sub-modules
             (Array, Nest, fuse, Plan.tensorize/cache/bind, Package.add/build)
 """
 from . import _lib  # noqa: F401
-from ._lib import (Acc950Error, EPILOGUE_NONE, EPILOGUE_RELU, EPILOGUE_RELU_NOCOND, PROLOGUE_NONE,  # noqa: F401
-                   PROLOGUE_SET0, VARIANT_AUTO, VARIANT_F32_MFMA, VARIANT_GENERIC, VARIANT_SKINNY_BASE)
+from ._lib import (Acc950Error, EPILOGUE_NONE, EPILOGUE_RELU, EPILOGUE_RELU_NOCOND, EPILOGUE_SCALE, EPILOGUE_SET,  # noqa: F401
+                   PROLOGUE_NONE, PROLOGUE_SCALE, PROLOGUE_SET, PROLOGUE_SET0, VARIANT_AUTO, VARIANT_F32_MFMA, VARIANT_GENERIC, VARIANT_SKINNY_BASE)
 
 __all__ = ["gemm_relu", "GemmCall", "hat"]
 

@@ -13,13 +13,13 @@ INCLUDE_DIR = os.path.join(os.path.dirname(_HERE), "include")
 
 # element types / ops / status codes / variant ids (accera_mi355x_gemm.h)
 F32, F16, BF16, I8, I32 = 0, 1, 2, 3, 4
-PROLOGUE_NONE, PROLOGUE_SET0 = 0, 1
-EPILOGUE_NONE, EPILOGUE_RELU, EPILOGUE_RELU_NOCOND = 0, 1, 2
+PROLOGUE_NONE, PROLOGUE_SET0, PROLOGUE_SET, PROLOGUE_SCALE = 0, 1, 1, 2
+EPILOGUE_NONE, EPILOGUE_RELU, EPILOGUE_RELU_NOCOND, EPILOGUE_SCALE, EPILOGUE_SET = 0, 1, 2, 3, 4
 OK, INVALID_ARGUMENT, UNSUPPORTED, HIP_ERROR = 0, 1, 2, 3
 VARIANT_AUTO, VARIANT_SKINNY_BASE, VARIANT_GENERIC, VARIANT_F32_MFMA = -1, 100, 200, 201
 
 EXPORTS = [
-    "acc950_init", "acc950_gemm_relu", "acc950_gemm_relu_ex", "acc950_gemm_relu_host",
+    "acc950_init", "acc950_gemm_relu", "acc950_gemm_relu_ex", "acc950_gemm_relu_host", "acc950_gemm_ops", "acc950_gemm_ops_host",
     "acc950_launch_geometry", "acc950_num_variants", "acc950_num_skinny_variants",
     "acc950_variant_name", "acc950_last_error", "acc950_mfma_ceiling", "acc950_mfma_phase_probe", "acc950_copy_probe", "acc950_stream_read_probe",
 ]
@@ -50,6 +50,9 @@ def lib():
     L.acc950_gemm_relu.argtypes = [ci, ci, ci, ci, ci] + mat * 3 + [ci, ci, vp]
     L.acc950_gemm_relu_ex.argtypes = [ci, ci, ci, ci, ci] + mat * 3 + [ci, ci, ci, ci, vp]
     L.acc950_gemm_relu_host.argtypes = [ci, ci, ci, ci, ci] + mat * 3 + [ci, ci]
+    cd = ctypes.c_double
+    L.acc950_gemm_ops.argtypes = [ci, ci, ci, ci, ci] + mat * 3 + [ci, cd, ci, cd, ci, ci, vp]
+    L.acc950_gemm_ops_host.argtypes = [ci, ci, ci, ci, ci] + mat * 3 + [ci, cd, ci, cd]
     L.acc950_launch_geometry.argtypes = [ci, ci, ci, ci, ci] + [i64] * 6 + [ci, ci, ctypes.POINTER(cu), ctypes.POINTER(cu),
                                                                            ctypes.POINTER(cu), ctypes.POINTER(ci)]
     L.acc950_variant_name.argtypes = [ci, ctypes.c_char_p, ctypes.c_size_t]

@@ -66,20 +66,24 @@ struct Problem {
 
 int make_problem(int in_type, int out_type, int M, int N, int K,
                  const void* A, int64_t a_rs, int64_t a_cs, const void* B, int64_t b_rs, int64_t b_cs,
-                 void* C, int64_t c_rs, int64_t c_cs, int prologue, int epilogue, bool need_pointers, Problem* out)
+                 void* C, int64_t c_rs, int64_t c_cs, int prologue, int epilogue, bool need_pointers, Problem* out,
+                 double prologue_arg = 0.0, double epilogue_arg = 0.0)
 {
     if (!type_pair_ok(in_type, out_type)) return fail(ACC950_INVALID_ARGUMENT, "unsupported input/output element type pair");
     if (M < 0 || N < 0 || K < 0) return fail(ACC950_INVALID_ARGUMENT, "negative matrix dimension");
     if (a_rs < 0 || a_cs < 0 || b_rs < 0 || b_cs < 0 || c_rs < 0 || c_cs < 0)
         return fail(ACC950_INVALID_ARGUMENT, "negative strides are not supported");
-    if (prologue != PRO_NONE && prologue != PRO_SET0) return fail(ACC950_INVALID_ARGUMENT, "unknown prologue op");
-    if (epilogue != EPI_NONE && epilogue != EPI_RELU && epilogue != EPI_RELU_NOCOND)
+    if (prologue != PRO_NONE && prologue != PRO_SET && prologue != PRO_SCALE) return fail(ACC950_INVALID_ARGUMENT, "unknown prologue op");
+    if (epilogue != EPI_NONE && epilogue != EPI_RELU && epilogue != EPI_RELU_NOCOND && epilogue != EPI_SCALE && epilogue != EPI_SET)
         return fail(ACC950_INVALID_ARGUMENT, "unknown epilogue op");
+    if (prologue_arg != prologue_arg || epilogue_arg != epilogue_arg) return fail(ACC950_INVALID_ARGUMENT, "NaN op argument");
     if (need_pointers && M > 0 && N > 0 && (!C || (K > 0 && (!A || !B))))
         return fail(ACC950_INVALID_ARGUMENT, "null matrix pointer");
     GemmArgs g{};
     g.in_type = in_type; g.out_type = out_type;
     g.prologue = prologue; g.epilogue = epilogue;
+    g.prologue_arg = prologue == PRO_NONE ? 0.f : (float)prologue_arg;
+    g.epilogue_arg = (epilogue == EPI_SCALE || epilogue == EPI_SET) ? (float)epilogue_arg : 0.f;
     const bool transpose = c_cs != 1 && c_rs == 1 && N > 1;
     if (!transpose) {
         g.A = A; g.B = B; g.C = C; g.M = M; g.N = N; g.K = K;
@@ -280,6 +284,7 @@ int run(const Problem& pb, const Choice& c, hipStream_t stream, LaunchGeom* geom
         s.A = g.A; s.B = g.B; s.C = g.C; s.M = g.M; s.N = g.N; s.K = g.K;
         s.a_rs = g.a_rs; s.b_rs = g.b_rs; s.c_rs = g.c_rs;
         s.in_type = g.in_type; s.out_type = g.out_type; s.prologue = g.prologue; s.epilogue = g.epilogue;
+        s.prologue_arg = g.prologue_arg; s.epilogue_arg = g.epilogue_arg;
         s.splits = c.splits;
         s.extra_phase = -1;
         // 64-column MFMA blocks, no K split, dense rows of a multiple of 512 bytes: blocks whose
@@ -343,18 +348,28 @@ int acc950_init(int device_id)
     return ACC950_OK;
 }
 
-int acc950_gemm_relu_ex(int in_type, int out_type, int M, int N, int K,
-                        const void* A, int64_t a_rs, int64_t a_cs, const void* B, int64_t b_rs, int64_t b_cs,
-                        void* C, int64_t c_rs, int64_t c_cs, int prologue, int epilogue, int variant, int k_splits,
-                        void* stream)
+int acc950_gemm_ops(int in_type, int out_type, int M, int N, int K,
+                    const void* A, int64_t a_rs, int64_t a_cs, const void* B, int64_t b_rs, int64_t b_cs,
+                    void* C, int64_t c_rs, int64_t c_cs, int prologue, double prologue_arg, int epilogue, double epilogue_arg,
+                    int variant, int k_splits, void* stream)
 {
     Problem pb;
-    int rc = make_problem(in_type, out_type, M, N, K, A, a_rs, a_cs, B, b_rs, b_cs, C, c_rs, c_cs, prologue, epilogue, true, &pb);
+    int rc = make_problem(in_type, out_type, M, N, K, A, a_rs, a_cs, B, b_rs, b_cs, C, c_rs, c_cs, prologue, epilogue, true, &pb,
+                          prologue_arg, epilogue_arg);
     if (rc) return rc;
     Choice c;
     rc = choose(pb, variant, k_splits, &c);
     if (rc) return rc;
     return run(pb, c, (hipStream_t)stream, nullptr, false);
+}
+
+int acc950_gemm_relu_ex(int in_type, int out_type, int M, int N, int K,
+                        const void* A, int64_t a_rs, int64_t a_cs, const void* B, int64_t b_rs, int64_t b_cs,
+                        void* C, int64_t c_rs, int64_t c_cs, int prologue, int epilogue, int variant, int k_splits,
+                        void* stream)
+{
+    return acc950_gemm_ops(in_type, out_type, M, N, K, A, a_rs, a_cs, B, b_rs, b_cs, C, c_rs, c_cs, prologue, 0.0, epilogue, 0.0,
+                           variant, k_splits, stream);
 }
 
 int acc950_gemm_relu(int in_type, int out_type, int M, int N, int K,
@@ -438,8 +453,16 @@ int acc950_gemm_relu_host(int in_type, int out_type, int M, int N, int K,
                           const void* A, int64_t a_rs, int64_t a_cs, const void* B, int64_t b_rs, int64_t b_cs,
                           void* C, int64_t c_rs, int64_t c_cs, int prologue, int epilogue)
 {
+    return acc950_gemm_ops_host(in_type, out_type, M, N, K, A, a_rs, a_cs, B, b_rs, b_cs, C, c_rs, c_cs, prologue, 0.0, epilogue, 0.0);
+}
+
+int acc950_gemm_ops_host(int in_type, int out_type, int M, int N, int K,
+                         const void* A, int64_t a_rs, int64_t a_cs, const void* B, int64_t b_rs, int64_t b_cs,
+                         void* C, int64_t c_rs, int64_t c_cs, int prologue, double prologue_arg, int epilogue, double epilogue_arg)
+{
     Problem check;
-    int rc = make_problem(in_type, out_type, M, N, K, A, a_rs, a_cs, B, b_rs, b_cs, C, c_rs, c_cs, prologue, epilogue, true, &check);
+    int rc = make_problem(in_type, out_type, M, N, K, A, a_rs, a_cs, B, b_rs, b_cs, C, c_rs, c_cs, prologue, epilogue, true, &check,
+                          prologue_arg, epilogue_arg);
     if (rc) return rc;
     if (M == 0 || N == 0) return ACC950_OK;
     const size_t a_bytes = extent_elems(M, K, a_rs, a_cs) * elem_size(in_type);
@@ -456,10 +479,10 @@ int acc950_gemm_relu_host(int in_type, int out_type, int M, int N, int K,
     if (b_bytes && (e = hipMemcpy(g_dB.p, B, b_bytes, hipMemcpyHostToDevice)) != hipSuccess) return fail_hip(e, "copy B to device");
     // C travels to the device when it is accumulated into, or when its extent has gaps
     // that the copy back must not clobber
-    if (prologue == PRO_NONE || !c_dense)
+    if (prologue != PRO_SET || !c_dense)
         if ((e = hipMemcpy(g_dC.p, C, c_bytes, hipMemcpyHostToDevice)) != hipSuccess) return fail_hip(e, "copy C to device");
-    rc = acc950_gemm_relu(in_type, out_type, M, N, K, g_dA.p, a_rs, a_cs, g_dB.p, b_rs, b_cs, g_dC.p, c_rs, c_cs,
-                          prologue, epilogue, nullptr);
+    rc = acc950_gemm_ops(in_type, out_type, M, N, K, g_dA.p, a_rs, a_cs, g_dB.p, b_rs, b_cs, g_dC.p, c_rs, c_cs,
+                         prologue, prologue_arg, epilogue, epilogue_arg, ACC950_VARIANT_AUTO, 0, nullptr);
     if (rc) return rc;
     if ((e = hipMemcpy(C, g_dC.p, c_bytes, hipMemcpyDeviceToHost)) != hipSuccess) return fail_hip(e, "copy C to host");
     return ACC950_OK;

@@ -10,8 +10,11 @@ enum : int { T_F32 = 0, T_F16 = 1, T_BF16 = 2, T_I8 = 3, T_I32 = 4 };
 // Prologue / epilogue ops of the tensorized plan
 // (/root/reference/accera/python/accera/lang/Plan.py:208-379, fragment ops
 //  /root/reference/accera/acc-translate/src/Target/Cpp/CppPrinterUtils.h:630-655).
-enum : int { PRO_NONE = 0, PRO_SET0 = 1 };
-enum : int { EPI_NONE = 0, EPI_RELU = 1, EPI_RELU_NOCOND = 2 };
+// Prologue acts on the C fragment before the products are added (NONE: keep C, SET: C = arg,
+// SCALE: C *= arg); epilogue acts on the finished sum.  Arguments are cast to the
+// accumulator type (float or int), as the reference's fragment helpers do.
+enum : int { PRO_NONE = 0, PRO_SET = 1, PRO_SET0 = 1, PRO_SCALE = 2 };
+enum : int { EPI_NONE = 0, EPI_RELU = 1, EPI_RELU_NOCOND = 2, EPI_SCALE = 3, EPI_SET = 4 };
 
 // Arguments of one GEMM launch.  Strides are in elements.
 struct GemmArgs {
@@ -24,6 +27,7 @@ struct GemmArgs {
     int64_t c_rs, c_cs; // C[i,j] at i*c_rs + j*c_cs
     int in_type, out_type;
     int prologue, epilogue;
+    float prologue_arg, epilogue_arg; // SET / SCALE operand (0 for the other ops)
     int tiles_m, tiles_n; // workgroup grid in tiles (MFMA kernels)
     unsigned long long* stamps; // timed MFMA instantiation only: [workgroup][4 points][shader clock, 100 MHz clock]
 };
@@ -62,15 +66,32 @@ __device__ __forceinline__ uint16_t float_to_f16_bits(float f)
 
 __device__ __forceinline__ float f16_bits_to_float(uint16_t b) { return (float)__builtin_bit_cast(_Float16, b); }
 
-// ---- fragment epilogue ops (CppPrinterUtils.h:630-643) ---------------------------
+// ---- fragment ops (CppPrinterUtils.h:630-655) ------------------------------------
 // relu:                v > 0 ? v : 0     (NaN -> 0, -0 -> +0)
 // relu_no_conditional: v *= (v > 0)      (NaN stays NaN, negatives -> -0)
+// scale:               v *= arg          set: v = arg
+__device__ __forceinline__ int wrap_mul(int a, int b) { return (int)((unsigned)a * (unsigned)b); }
+__device__ __forceinline__ float wrap_mul(float a, float b) { return a * b; }
+__device__ __forceinline__ int wrap_add(int a, int b) { return (int)((unsigned)a + (unsigned)b); }
+__device__ __forceinline__ float wrap_add(float a, float b) { return a + b; }
+
 template <typename T>
-__device__ __forceinline__ T apply_epilogue(T v, int epi)
+__device__ __forceinline__ T apply_epilogue(T v, int epi, float arg = 0.f)
 {
     if (epi == EPI_RELU) return v > T(0) ? v : T(0);
     if (epi == EPI_RELU_NOCOND) return v * T(v > T(0) ? 1 : 0);
+    if (epi == EPI_SCALE) return wrap_mul(v, (T)arg);
+    if (epi == EPI_SET) return (T)arg;
     return v;
+}
+
+// Sum of products + the prologue'd C element (c_old is only read when the op keeps C).
+template <typename T, typename LoadC>
+__device__ __forceinline__ T apply_prologue(T sum, int pro, float arg, LoadC&& load_c)
+{
+    if (pro == PRO_SET) return wrap_add(sum, (T)arg);
+    if (pro == PRO_SCALE) return wrap_add(sum, wrap_mul(load_c(), (T)arg));
+    return wrap_add(sum, load_c());
 }
 
 // Store one float accumulator as the output element type.

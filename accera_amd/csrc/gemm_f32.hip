@@ -92,8 +92,8 @@ __global__ void __launch_bounds__(256) gemm_f32_kernel(GemmArgs p)
         if (orow >= p.M || ocol >= p.N) continue;
         float* C = (float*)p.C;
         const int64_t idx = (int64_t)orow * p.c_rs + (int64_t)ocol * p.c_cs;
-        if (p.prologue == PRO_NONE) v += C[idx];
-        C[idx] = apply_epilogue<float>(v, p.epilogue);
+        v = apply_prologue<float>(v, p.prologue, p.prologue_arg, [&]() { return C[idx]; });
+        C[idx] = apply_epilogue<float>(v, p.epilogue, p.epilogue_arg);
     }
 }
 

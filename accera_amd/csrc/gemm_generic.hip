@@ -79,11 +79,11 @@ __global__ void __launch_bounds__(256) gemm_generic_kernel(GemmArgs p)
             AccT v = acc[i][j];
             if constexpr (std::is_same<AccT, int>::value) {
                 int* C = (int*)p.C;
-                if (p.prologue == PRO_NONE) v = (int)((unsigned)v + (unsigned)C[idx]);
-                C[idx] = apply_epilogue<int>(v, p.epilogue);
+                v = apply_prologue<int>(v, p.prologue, p.prologue_arg, [&]() { return C[idx]; });
+                C[idx] = apply_epilogue<int>(v, p.epilogue, p.epilogue_arg);
             } else {
-                if (p.prologue == PRO_NONE) v += load_out(p.C, p.out_type, idx);
-                store_out(p.C, p.out_type, idx, apply_epilogue<float>(v, p.epilogue));
+                v = apply_prologue<float>(v, p.prologue, p.prologue_arg, [&]() { return load_out(p.C, p.out_type, idx); });
+                store_out(p.C, p.out_type, idx, apply_epilogue<float>(v, p.epilogue, p.epilogue_arg));
             }
         }
 }

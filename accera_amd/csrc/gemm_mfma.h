@@ -522,25 +522,19 @@ __global__ void __launch_bounds__(Cfg::NT, Cfg::WGS_PER_CU) gemm_mfma_kernel(Gem
     }
 
     stamp(2);
-    // Write-back: optional "+= C" (no SET prologue), epilogue op, narrowing store.
+    // Write-back in three passes over the accumulator registers, so that every piece of
+    // code exists once per thing it depends on (element type or op), not once per combination:
+    //   A. prologue NONE / SCALE: acc += (arg *) C        (one copy per output type)
+    //   B. prologue SET constant and the epilogue op, in place   (one copy per op)
+    //   C. narrowing store                                 (one copy per output type)
     // MFMA 32x32 accumulator layout: register r of lane l holds
     //   row = (r/4)*8 + (l/32)*4 + r%4,  column = l%32.
     // C is row-major here (the host transposes the problem otherwise).  Addresses are a
     // workgroup-uniform tile base plus one 32-bit offset per accumulator row, so the
     // write-back needs no 64-bit address registers next to the live accumulators.
-    // The epilogue kind is wave-uniform: ReLU (the fused path) gets its own copy of the
-    // write-back with a single max per element, the other kinds share one with selects.
-    const bool is_nocond = p.epilogue == EPI_RELU_NOCOND;
-    auto epilogue = [&](scalar_t v, auto relu_tag) -> scalar_t {
-        if constexpr (decltype(relu_tag)::value) return v > scalar_t(0) ? v : scalar_t(0);
-        else {
-            scalar_t n = v * (v > scalar_t(0) ? scalar_t(1) : scalar_t(0));
-            return is_nocond ? n : v;
-        }
-    };
-    const bool accumulate = p.prologue == PRO_NONE;
     const int row_in_tile = wr0 + (lane >> 5) * 4, col_in_tile = wc0 + (lane & 31);
-    auto write_back = [&](auto out_tag, auto relu_tag) {
+    // acc element = fn(pointer to the output element, acc element) for every element of the wave tile
+    auto for_each_element = [&](auto out_tag, auto&& fn) {
         using out_t = decltype(out_tag);
         constexpr unsigned OS = sizeof(out_t);
         char* tile_base = (char*)p.C + ((int64_t)m0 * p.c_rs + n0) * OS; // uniform
@@ -556,24 +550,47 @@ __global__ void __launch_bounds__(Cfg::NT, Cfg::WGS_PER_CU) gemm_mfma_kernel(Gem
 #pragma unroll
                 for (int j = 0; j < TN; ++j) {
                     if (EDGE && n0 + col_in_tile + j * 32 >= p.N) continue;
-                    out_t* dst = (out_t*)(tile_base + off + j * 32 * OS);
-                    scalar_t v = acc[i][j][r];
-                    if constexpr (std::is_same<out_t, int>::value) {
-                        if (accumulate) v = (int)((unsigned)v + (unsigned)*dst);
-                        *dst = epilogue(v, relu_tag);
-                    } else if constexpr (std::is_same<out_t, float>::value) {
-                        if (accumulate) v += *dst;
-                        *dst = epilogue(v, relu_tag);
-                    } else if constexpr (std::is_same<out_t, _Float16>::value) {
-                        if (accumulate) v += (float)*dst;
-                        *dst = (_Float16)epilogue(v, relu_tag); // v_cvt_f16_f32: round to nearest even
-                    } else { // bf16 bits
-                        if (accumulate) v += bf16_bits_to_float(*dst);
-                        *dst = float_to_bf16_bits(epilogue(v, relu_tag));
-                    }
+                    acc[i][j][r] = fn((out_t*)(tile_base + off + j * 32 * OS), acc[i][j][r]);
                 }
+                if ((r & 3) == 3) __builtin_amdgcn_sched_barrier(0); // keep loads of pass A near their use: no second copy of the tile in registers
             }
     };
+    auto for_each_acc = [&](auto&& fn) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[i][j][r] = fn(acc[i][j][r]);
+    };
+
+    auto general_ops = [&]() {
+    // ---- pass A
+    const bool accumulate = p.prologue != PRO_SET; // NONE, SCALE: C is read
+    if (accumulate) {
+        const scalar_t c_mul = p.prologue == PRO_SCALE ? (scalar_t)p.prologue_arg : scalar_t(1); // x1 is exact
+        if constexpr (IN == IN_I8) for_each_element(int{}, [&](int* c, int v) { return wrap_add(v, wrap_mul(*c, c_mul)); });
+        else if (p.out_type == T_F32) for_each_element(float{}, [&](float* c, float v) { return v + *c * c_mul; });
+        else if (p.out_type == T_F16) for_each_element(_Float16{}, [&](_Float16* c, float v) { return v + (float)*c * c_mul; });
+        else for_each_element(uint16_t{}, [&](uint16_t* c, float v) { return v + bf16_bits_to_float(*c) * c_mul; });
+    }
+
+    // ---- pass B (wave-uniform switches; ReLU after a SET-0 prologue is the fused hot path: one max per element)
+    if (p.prologue == PRO_SET && p.prologue_arg != 0.f) {
+        const scalar_t set_value = (scalar_t)p.prologue_arg;
+        for_each_acc([&](scalar_t v) { return wrap_add(v, set_value); });
+    }
+    {
+        const scalar_t epi_arg = (scalar_t)p.epilogue_arg;
+        if (p.epilogue == EPI_RELU) for_each_acc([&](scalar_t v) { return v > scalar_t(0) ? v : scalar_t(0); });
+        else if (p.epilogue == EPI_RELU_NOCOND) for_each_acc([&](scalar_t v) { return v * (v > scalar_t(0) ? scalar_t(1) : scalar_t(0)); });
+        else if (p.epilogue == EPI_SCALE) for_each_acc([&](scalar_t v) { return wrap_mul(v, epi_arg); });
+        else if (p.epilogue == EPI_SET) for_each_acc([&](scalar_t) { return epi_arg; });
+    }
+
+    };
+
+    // ---- pass C
     // 16-bit outputs: a lane's accumulators are one column wide, so direct stores write
     // 64-byte pieces of a row per instruction.  Instead each wave stages 32 rows of its
     // tile in a private slab of the (now idle) LDS tile buffers, two columns packed per
@@ -581,7 +598,8 @@ __global__ void __launch_bounds__(Cfg::NT, Cfg::WGS_PER_CU) gemm_mfma_kernel(Gem
     // pieces that cover whole rows of the wave tile.
     constexpr int PITCH_DW = (WTN / 2) % 32 == 16 ? WTN / 2 : WTN / 2 + 16; // rows r, r+1 in different bank halves
     constexpr bool CAN_STAGE = !EDGE && IN != IN_I8 && (NT / 64) * 32 * PITCH_DW * 4 <= Cfg::LDS_BYTES;
-    auto write_back_staged = [&](auto out_tag, auto relu_tag) {
+    auto store_staged = [&](auto out_tag, auto relu_tag) {
+        auto fin = [&](float v) { return decltype(relu_tag)::value ? (v > 0.f ? v : 0.f) : v; };
         using out_t = decltype(out_tag);
         const int wave_u = __builtin_amdgcn_readfirstlane(wave);
         unsigned* slab = (unsigned*)(smem + wave_u * (32 * PITCH_DW * 4));
@@ -610,7 +628,7 @@ __global__ void __launch_bounds__(Cfg::NT, Cfg::WGS_PER_CU) gemm_mfma_kernel(Gem
             for (int j = 0; j < TN; ++j)
 #pragma unroll
                 for (int t = 0; t < 8; ++t) {
-                    const unsigned own = pack2(epilogue(acc[i][j][2 * t], relu_tag), epilogue(acc[i][j][2 * t + 1], relu_tag));
+                    const unsigned own = pack2(fin(acc[i][j][2 * t]), fin(acc[i][j][2 * t + 1]));
                     const unsigned nbr = (unsigned)__builtin_amdgcn_update_dpp(0, (int)own, 0xB1, 0xF, 0xF, true); // lane ^ 1
                     const int row = (t >> 1) * 8 + (t & 1) * 2 + wrow;
                     slab[row * PITCH_DW + j * 16 + wcol] = __builtin_amdgcn_perm(nbr, own, sel);
@@ -624,21 +642,24 @@ __global__ void __launch_bounds__(Cfg::NT, Cfg::WGS_PER_CU) gemm_mfma_kernel(Gem
             }
         }
     };
-    const bool staged = CAN_STAGE && !accumulate && p.c_rs % 8 == 0 && ((size_t)p.C & 15) == 0;
-    auto write_back_any = [&](auto relu_tag) {
-        if constexpr (IN == IN_I8) write_back(int{}, relu_tag);
-        else if (p.out_type == T_F32) write_back(float{}, relu_tag);
-        else if (CAN_STAGE && staged) {
-            if constexpr (CAN_STAGE) {
-                __syncthreads(); // every wave is done reading the tile buffers
-                if (p.out_type == T_F16) write_back_staged(_Float16{}, relu_tag);
-                else write_back_staged(uint16_t{}, relu_tag);
-            }
-        } else if (p.out_type == T_F16) write_back(_Float16{}, relu_tag);
-        else write_back(uint16_t{}, relu_tag);
+    auto store_all = [&](auto relu_tag) {
+        auto fin = [&](scalar_t v) { return decltype(relu_tag)::value ? (v > scalar_t(0) ? v : scalar_t(0)) : v; };
+    const bool staged = CAN_STAGE && p.c_rs % 8 == 0 && ((size_t)p.C & 15) == 0;
+    if constexpr (IN == IN_I8) for_each_element(int{}, [&](int* c, int v) { *c = fin(v); return v; });
+    else if (p.out_type == T_F32) for_each_element(float{}, [&](float* c, float v) { *c = fin(v); return v; });
+    else if (CAN_STAGE && staged) {
+        if constexpr (CAN_STAGE) {
+            __syncthreads(); // every wave is done reading the tile buffers
+            if (p.out_type == T_F16) store_staged(_Float16{}, relu_tag);
+            else store_staged(uint16_t{}, relu_tag);
+        }
+    } else if (p.out_type == T_F16) for_each_element(_Float16{}, [&](_Float16* c, float v) { *c = (_Float16)fin(v); return v; }); // RNE
+    else for_each_element(uint16_t{}, [&](uint16_t* c, float v) { *c = float_to_bf16_bits(fin(v)); return v; });
     };
-    if (p.epilogue == EPI_RELU) write_back_any(std::true_type{});
-    else write_back_any(std::false_type{});
+    // One straight line through the passes: splitting the fused matmul + ReLU case off into a
+    // branch of its own makes the register allocator spill hundreds of accumulators.
+    general_ops();
+    store_all(std::false_type{});
     if constexpr (Cfg::TIMED) {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // stores acknowledged
         stamp(3);

@@ -190,8 +190,8 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_skinny_kernel(SkinnyArgs p)
     auto finish = [&](int m, int n, float s) {
         if (!col_ok || m >= p.M) return;
         const int64_t idx = (int64_t)m * p.c_rs + (col0 + n);
-        if (p.prologue == PRO_NONE) s += load_out(p.C, p.out_type, idx);
-        store_out(p.C, p.out_type, idx, apply_epilogue<float>(s, p.epilogue));
+        s = apply_prologue<float>(s, p.prologue, p.prologue_arg, [&]() { return load_out(p.C, p.out_type, idx); });
+        store_out(p.C, p.out_type, idx, apply_epilogue<float>(s, p.epilogue, p.epilogue_arg));
     };
 
     if (p.splits == 1) {

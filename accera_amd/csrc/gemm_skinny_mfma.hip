@@ -209,7 +209,7 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_skinny_mfma_kernel(SkinnyArgs
 
     const int groups = p.M * (CB / 4); // float4 groups of the workgroup's block
     // four adjacent columns of one row: one 8- or 16-byte store when C allows it
-    const bool vec_ok = p.prologue == PRO_NONE ? false
+    const bool vec_ok = p.prologue != PRO_SET ? false
                         : (p.out_type == T_F32 ? (p.c_rs % 4 == 0 && ((size_t)p.C & 15) == 0) : (p.c_rs % 4 == 0 && ((size_t)p.C & 7) == 0));
     auto finish4 = [&](int grp, f32x4 s) {
         const int row = grp / (CB / 4), n = col_base + (grp % (CB / 4)) * 4;
@@ -218,7 +218,7 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_skinny_mfma_kernel(SkinnyArgs
         if (vec_ok) {
             f32x4 r;
 #pragma unroll
-            for (int e = 0; e < 4; ++e) r[e] = apply_epilogue<float>(s[e], p.epilogue);
+            for (int e = 0; e < 4; ++e) r[e] = apply_epilogue<float>(s[e] + p.prologue_arg, p.epilogue, p.epilogue_arg);
             if (p.out_type == T_F32) {
                 *(f32x4*)((float*)p.C + idx) = r;
             } else if (p.out_type == T_F16) {
@@ -233,8 +233,8 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_skinny_mfma_kernel(SkinnyArgs
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
             float v = s[e];
-            if (p.prologue == PRO_NONE) v += load_out(p.C, p.out_type, idx + e);
-            store_out(p.C, p.out_type, idx + e, apply_epilogue<float>(v, p.epilogue));
+            v = apply_prologue<float>(v, p.prologue, p.prologue_arg, [&]() { return load_out(p.C, p.out_type, idx + e); });
+            store_out(p.C, p.out_type, idx + e, apply_epilogue<float>(v, p.epilogue, p.epilogue_arg));
         }
     };
 

@@ -13,6 +13,7 @@ struct SkinnyArgs {
     int64_t a_rs, b_rs, c_rs; // row strides in elements
     int in_type, out_type;
     int prologue, epilogue;
+    float prologue_arg, epilogue_arg;
     int splits;         // K split over grid.y
     int extra_phase;    // MFMA family, splits == 1: column blocks with index % 4 == extra_phase are split in two
                         // (second halves run as extra workgroups behind the regular grid); -1: none

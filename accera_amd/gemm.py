@@ -25,7 +25,7 @@ class GemmCall:
     stream that is current when the object is built."""
 
     def __init__(self, A, B, C, prologue=_lib.PROLOGUE_SET0, epilogue=_lib.EPILOGUE_RELU, variant=_lib.VARIANT_AUTO,
-                 k_splits=0, stream=None):
+                 k_splits=0, stream=None, prologue_arg=0.0, epilogue_arg=0.0):
         M, K = A.shape
         K2, N = B.shape
         if K2 != K or tuple(C.shape) != (M, N):
@@ -35,9 +35,9 @@ class GemmCall:
         if stream is None:
             stream = torch.cuda.current_stream(C.device).cuda_stream
         self.tensors = (A, B, C)
-        self._fn = _lib.lib().acc950_gemm_relu_ex
+        self._fn = _lib.lib().acc950_gemm_ops
         self._args = (_TORCH_TYPES[A.dtype], _TORCH_TYPES[C.dtype], M, N, K, *_mat(A, "A"), *_mat(B, "B"), *_mat(C, "C"),
-                      prologue, epilogue, variant, k_splits, stream)
+                      prologue, float(prologue_arg), epilogue, float(epilogue_arg), variant, k_splits, stream)
 
     def __call__(self):
         rc = self._fn(*self._args)
@@ -47,8 +47,13 @@ class GemmCall:
 
 
 def gemm_relu(A, B, C, prologue=_lib.PROLOGUE_SET0, epilogue=_lib.EPILOGUE_RELU, variant=_lib.VARIANT_AUTO,
-              k_splits=0, stream=None):
-    """C = epilogue((prologue == SET0 ? 0 : C) + A @ B), in place on C, asynchronously.
+              k_splits=0, stream=None, prologue_arg=0.0, epilogue_arg=0.0):
+    """C = epilogue(prologue(C) + A @ B), in place on C, asynchronously.
+
+    prologue: NONE keeps C, SET replaces it by ``prologue_arg`` (0: the fused matmul+ReLU),
+    SCALE multiplies it by ``prologue_arg`` (GEMM beta); epilogue: NONE, RELU, RELU_NOCOND,
+    SCALE by ``epilogue_arg`` (GEMM alpha), SET
+    (/root/reference/docs/Tutorials/GPU/Tensor_MatMul_ElementWiseOps_GPU.md:85-99).
 
     A (M,K), B (K,N), C (M,N) are CUDA/HIP tensors; strides are honoured (a
     column-major B is ``B_storage.t()`` of an (N,K) tensor).  Types: fp16/bf16 in ->
@@ -63,8 +68,8 @@ def gemm_relu(A, B, C, prologue=_lib.PROLOGUE_SET0, epilogue=_lib.EPILOGUE_RELU,
         raise ValueError(f"unsupported dtypes {A.dtype}, {B.dtype}, {C.dtype}")
     if stream is None:
         stream = torch.cuda.current_stream(C.device).cuda_stream
-    rc = _lib.lib().acc950_gemm_relu_ex(_TORCH_TYPES[A.dtype], _TORCH_TYPES[C.dtype], M, N, K,
-                                        *_mat(A, "A"), *_mat(B, "B"), *_mat(C, "C"),
-                                        prologue, epilogue, variant, k_splits, stream)
+    rc = _lib.lib().acc950_gemm_ops(_TORCH_TYPES[A.dtype], _TORCH_TYPES[C.dtype], M, N, K,
+                                    *_mat(A, "A"), *_mat(B, "B"), *_mat(C, "C"),
+                                    prologue, float(prologue_arg), epilogue, float(epilogue_arg), variant, k_splits, stream)
     _lib.check(rc)
     return C

@@ -351,10 +351,11 @@ class Plan:
     def tensorize(self, indices, mma_shape=None, use_static_offsets=False, num_total_passes=1, num_fused_passes=None,
                   scheduling_policy=MMASchedulingPolicy.PASS_ORDER, prologue_op=MMAFragmentOp.NONE, prologue_arg=0,
                   epilogue_op=MMAFragmentOp.NONE, epilogue_arg=0, **_):
-        if prologue_op not in (MMAFragmentOp.NONE, MMAFragmentOp.SET) or (prologue_op == MMAFragmentOp.SET and prologue_arg != 0):
-            raise NotImplementedError("prologue must be NONE or SET 0")
-        if epilogue_op not in (MMAFragmentOp.NONE, MMAFragmentOp.ReLU, MMAFragmentOp.ReLU_NoConditional):
-            raise NotImplementedError("epilogue must be NONE, ReLU or ReLU_NoConditional")
+        if prologue_op not in (MMAFragmentOp.NONE, MMAFragmentOp.SET, MMAFragmentOp.SCALE):
+            raise NotImplementedError("prologue must be NONE, SET or SCALE")
+        if epilogue_op not in (MMAFragmentOp.NONE, MMAFragmentOp.ReLU, MMAFragmentOp.ReLU_NoConditional, MMAFragmentOp.SET,
+                               MMAFragmentOp.SCALE):
+            raise NotImplementedError("unknown epilogue op")
         self.prologue_op, self.prologue_arg = prologue_op, prologue_arg
         self.epilogue_op, self.epilogue_arg = epilogue_op, epilogue_arg
         self.commands.append(("tensorize", mma_shape, num_total_passes))
@@ -377,9 +378,10 @@ class Plan:
 # ---- pattern match to the GEMM (+ReLU) hot path -------------------------------------------------
 
 class _GemmSpec:
-    def __init__(self, A, B, C, M, N, K, prologue, epilogue):
+    def __init__(self, A, B, C, M, N, K, prologue, epilogue, prologue_arg=0.0, epilogue_arg=0.0):
         self.A, self.B, self.C, self.M, self.N, self.K = A, B, C, M, N, K
         self.prologue, self.epilogue = prologue, epilogue
+        self.prologue_arg, self.epilogue_arg = float(prologue_arg), float(epilogue_arg)
 
 
 def _match(source):
@@ -429,15 +431,23 @@ def _match(source):
         if not ok:
             raise unsupported
         epilogue = _lib.EPILOGUE_RELU
-    prologue = _lib.PROLOGUE_NONE
+    prologue, prologue_arg, epilogue_arg = _lib.PROLOGUE_NONE, 0.0, 0.0
     if plan:
         if plan.prologue_op == MMAFragmentOp.SET:
-            prologue = _lib.PROLOGUE_SET0
+            prologue, prologue_arg = _lib.PROLOGUE_SET, plan.prologue_arg
+        elif plan.prologue_op == MMAFragmentOp.SCALE:
+            prologue, prologue_arg = _lib.PROLOGUE_SCALE, plan.prologue_arg
+        if plan.epilogue_op != MMAFragmentOp.NONE and epilogue != _lib.EPILOGUE_NONE:
+            raise NotImplementedError("a fused ReLU nest and a tensorize epilogue op at the same time")
         if plan.epilogue_op == MMAFragmentOp.ReLU:
             epilogue = _lib.EPILOGUE_RELU
         elif plan.epilogue_op == MMAFragmentOp.ReLU_NoConditional:
             epilogue = _lib.EPILOGUE_RELU_NOCOND
-    return _GemmSpec(A, B, C, M, N, K, prologue, epilogue)
+        elif plan.epilogue_op == MMAFragmentOp.SCALE:
+            epilogue, epilogue_arg = _lib.EPILOGUE_SCALE, plan.epilogue_arg
+        elif plan.epilogue_op == MMAFragmentOp.SET:
+            epilogue, epilogue_arg = _lib.EPILOGUE_SET, plan.epilogue_arg
+    return _GemmSpec(A, B, C, M, N, K, prologue, epilogue, prologue_arg, epilogue_arg)
 
 
 # ---- package -------------------------------------------------------------------------------------
@@ -471,7 +481,7 @@ class Package:
         if spec.A.element_type != spec.B.element_type:
             raise ValueError("A and B must have the same element type")
         sig = repr((base_name, [(a.role.value, a.element_type.c_name, a.shape, a.layout.name) for a in args],
-                    spec.prologue, spec.epilogue, sorted((parameters or {}).items())))
+                    spec.prologue, spec.prologue_arg, spec.epilogue, spec.epilogue_arg, sorted((parameters or {}).items())))
         name = f"{base_name}_{hashlib.md5(sig.encode()).hexdigest()[:16]}"
         self._functions.append(dict(name=name, base_name=base_name, spec=spec, args=args, auxiliary=auxiliary or {},
                                     parameters=parameters or {}))
@@ -490,14 +500,14 @@ class Package:
             pa, pb, pc = order[id(s.A)], order[id(s.B)], order[id(s.C)]
             call_args = (f"{s.A.element_type.lib_id}, {s.C.element_type.lib_id}, {s.M}, {s.N}, {s.K}, "
                          f"{pa}, {s.A.strides[0]}, {s.A.strides[1]}, {pb}, {s.B.strides[0]}, {s.B.strides[1]}, "
-                         f"{pc}, {s.C.strides[0]}, {s.C.strides[1]}, {s.prologue}, {s.epilogue}")
+                         f"{pc}, {s.C.strides[0]}, {s.C.strides[1]}, {s.prologue}, {s.prologue_arg!r}, {s.epilogue}, {s.epilogue_arg!r}")
             lines += [
                 f"void {f['name']}(void* a0, void* a1, void* a2)", "{",
-                f"    if (acc950_gemm_relu_host({call_args}) != ACC950_OK)",
+                f"    if (acc950_gemm_ops_host({call_args}) != ACC950_OK)",
                 f"        fprintf(stderr, \"{f['name']}: %s\\n\", acc950_last_error());", "}",
                 "/* same function on device pointers, asynchronous on `stream` (hipStream_t or NULL) */",
                 f"int {f['name']}__device(void* a0, void* a1, void* a2, void* stream)", "{",
-                f"    return acc950_gemm_relu({call_args}, stream);", "}", ""]
+                f"    return acc950_gemm_ops({call_args}, ACC950_VARIANT_AUTO, 0, stream);", "}", ""]
         return "\n".join(lines)
 
     def build(self, name, format=None, mode=None, platform=None, tolerance=1e-5, output_dir=None, **_):
@@ -535,7 +545,8 @@ class Package:
                    # (Package.py:714-743): launch geometry of the kernel behind this entry point
                    "accera_mi355x": {"device_entry": f"{f['name']}__device", "kernel": _lib.variant_name(variant),
                                      "launch_parameters": grid + block, "dynamic_shared_mem_bytes": lds,
-                                     "prologue": s.prologue, "epilogue": s.epilogue}}
+                                     "prologue": s.prologue, "prologue_arg": s.prologue_arg, "epilogue": s.epilogue,
+                                     "epilogue_arg": s.epilogue_arg}}
             aux.update(f["auxiliary"])
             functions.append(_hat.Function(name=f["name"], base_name=f["base_name"], arguments=arguments, auxiliary=aux))
         _hat.write_hat(hat_path, name, functions, link_target=f"{name}.so",

@@ -32,11 +32,15 @@ extern "C" {
 /* prologue / epilogue ops of plan.tensorize
  * (/root/reference/accera/python/accera/lang/Plan.py:208-379;
  *  device helpers /root/reference/accera/acc-translate/src/Target/Cpp/CppPrinterUtils.h:630-655) */
-#define ACC950_PROLOGUE_NONE 0 /* C = epilogue(C + A*B) */
-#define ACC950_PROLOGUE_SET0 1 /* C = epilogue(A*B)     (MMAFragmentOp.SET with 0) */
+#define ACC950_PROLOGUE_NONE 0  /* C = epilogue(C + A*B) */
+#define ACC950_PROLOGUE_SET0 1  /* C = epilogue(A*B)           (MMAFragmentOp.SET with 0) */
+#define ACC950_PROLOGUE_SET 1   /* C = epilogue(arg + A*B)     (MMAFragmentOp.SET, acc950_gemm_ops) */
+#define ACC950_PROLOGUE_SCALE 2 /* C = epilogue(arg*C + A*B)   (MMAFragmentOp.SCALE: the beta of a GEMM) */
 #define ACC950_EPILOGUE_NONE 0
 #define ACC950_EPILOGUE_RELU 1           /* v > 0 ? v : 0 */
 #define ACC950_EPILOGUE_RELU_NOCOND 2    /* v *= (v > 0)  */
+#define ACC950_EPILOGUE_SCALE 3          /* v *= arg      (the alpha of a GEMM) */
+#define ACC950_EPILOGUE_SET 4            /* v = arg */
 
 /* status codes */
 #define ACC950_OK 0
@@ -88,6 +92,28 @@ int acc950_gemm_relu_ex(int in_type, int out_type, int M, int N, int K,
                         const void* B, int64_t b_row_stride, int64_t b_col_stride,
                         void* C, int64_t c_row_stride, int64_t c_col_stride,
                         int prologue, int epilogue, int variant, int k_splits, void* stream);
+
+/*
+ * General form with the operands of the fragment ops: every prologue / epilogue op of
+ * the reference's tensorized plan (/root/reference/accera/python/accera/lang/Plan.py:208-379;
+ * helpers set / scale / relu / relu_no_conditional,
+ * /root/reference/accera/acc-translate/src/Target/Cpp/CppPrinterUtils.h:630-655; GEMM alpha / beta table,
+ * /root/reference/docs/Tutorials/GPU/Tensor_MatMul_ElementWiseOps_GPU.md:85-99).  The operands are cast to
+ * the accumulator type (float, or int for int8 inputs) as the reference's helpers do; an
+ * operand of an op that takes none is ignored.  acc950_gemm_relu_ex is this call with both
+ * operands 0.  acc950_gemm_ops_host is the same on HOST pointers (see below).
+ */
+int acc950_gemm_ops(int in_type, int out_type, int M, int N, int K,
+                    const void* A, int64_t a_row_stride, int64_t a_col_stride,
+                    const void* B, int64_t b_row_stride, int64_t b_col_stride,
+                    void* C, int64_t c_row_stride, int64_t c_col_stride,
+                    int prologue, double prologue_arg, int epilogue, double epilogue_arg,
+                    int variant, int k_splits, void* stream);
+int acc950_gemm_ops_host(int in_type, int out_type, int M, int N, int K,
+                         const void* A, int64_t a_row_stride, int64_t a_col_stride,
+                         const void* B, int64_t b_row_stride, int64_t b_col_stride,
+                         void* C, int64_t c_row_stride, int64_t c_col_stride,
+                         int prologue, double prologue_arg, int epilogue, double epilogue_arg);
 
 /*
  * Same computation on HOST pointers, synchronous: copies A, B (and C when it is

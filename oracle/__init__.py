@@ -33,8 +33,8 @@ _LIB_PATH = os.path.join(_HERE, "liboracle.so")
 F32, F16, BF16, I8, I32 = 0, 1, 2, 3, 4
 TYPE_IDS = {"f32": F32, "f16": F16, "bf16": BF16, "i8": I8, "i32": I32}
 NP_STORAGE = {"f32": np.float32, "f16": np.float16, "bf16": np.uint16, "i8": np.int8, "i32": np.int32}
-PRO_NONE, PRO_SET0 = 0, 1
-EPI_NONE, EPI_RELU, EPI_RELU_NOCOND = 0, 1, 2
+PRO_NONE, PRO_SET0, PRO_SET, PRO_SCALE = 0, 1, 1, 2
+EPI_NONE, EPI_RELU, EPI_RELU_NOCOND, EPI_SCALE, EPI_SET = 0, 1, 2, 3, 4
 SCHED_NAIVE, SCHED_TRANSFORMED = 0, 1
 
 _lib = None
@@ -129,23 +129,40 @@ def gemm_relu(A, B, C, in_type, out_type, prologue=PRO_SET0, epilogue=EPI_RELU,
     return C
 
 
-def gemm_relu_exact(A, B, C0, in_type, out_type, prologue=PRO_SET0, epilogue=EPI_RELU, narrow_out=True):
+def _op_arg(arg, in_type):
+    """Operand of a SET / SCALE fragment op cast to the accumulator type, as the reference's
+    helpers do (`const _Ty arg`, /root/reference/accera/acc-translate/src/Target/Cpp/CppPrinterUtils.h:644-655)."""
+    return int(arg) if in_type == "i8" else float(np.float32(arg))
+
+
+def gemm_relu_exact(A, B, C0, in_type, out_type, prologue=PRO_SET0, epilogue=EPI_RELU, narrow_out=True,
+                    prologue_arg=0.0, epilogue_arg=0.0):
     """NumPy restatement: exact widened product summed in float64 / int64.
+
+    prologue: NONE keeps C0, SET replaces it by ``prologue_arg``, SCALE multiplies it by
+    ``prologue_arg``; epilogue: NONE, RELU, RELU_NOCOND, SCALE by ``epilogue_arg``, SET
+    (/root/reference/docs/Tutorials/GPU/Tensor_MatMul_ElementWiseOps_GPU.md:85-99).  The C
+    nests in gemm_relu_oracle.c cover NONE / SET 0 and the two ReLUs only.
 
     Returns the result narrowed to ``out_type`` storage (or the float64 / int64
     pre-narrowing values when ``narrow_out`` is False).
     """
     Aw, Bw = widen(A, in_type), widen(B, in_type)
     S = Aw @ Bw
-    if prologue != PRO_SET0:
-        S = S + widen(C0, out_type)
-    if in_type == "i8":
-        S = ((S + 2**31) % 2**32) - 2**31  # int32 wrap-around
-        if epilogue in (EPI_RELU, EPI_RELU_NOCOND):
-            S = np.maximum(S, 0)
+    if prologue == PRO_SET:
+        S = S + _op_arg(prologue_arg, in_type)
+    elif prologue == PRO_SCALE:
+        S = S + widen(C0, out_type) * _op_arg(prologue_arg, in_type)
     else:
-        if epilogue == EPI_RELU:
-            S = np.where(S > 0, S, 0.0)
-        elif epilogue == EPI_RELU_NOCOND:
-            S = S * (S > 0)
+        S = S + widen(C0, out_type)
+    wrap = (lambda x: ((x + 2**31) % 2**32) - 2**31) if in_type == "i8" else (lambda x: x)
+    S = wrap(S)
+    if epilogue == EPI_RELU:
+        S = np.maximum(S, 0) if in_type == "i8" else np.where(S > 0, S, 0.0)
+    elif epilogue == EPI_RELU_NOCOND:
+        S = np.maximum(S, 0) if in_type == "i8" else S * (S > 0)
+    elif epilogue == EPI_SCALE:
+        S = wrap(S * _op_arg(epilogue_arg, in_type))
+    elif epilogue == EPI_SET:
+        S = np.full_like(S, _op_arg(epilogue_arg, in_type))
     return narrow(S, out_type) if narrow_out else S

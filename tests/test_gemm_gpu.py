@@ -318,6 +318,34 @@ def test_narrowing_store_rounds_to_nearest_even(out_type, variant, prologue):
     assert np.array_equal(got[ok], want[ok]), (got[:16, 0], want[:16, 0])
 
 
+# ---- SET / SCALE fragment ops (GEMM alpha / beta table) through every kernel family ---------------------
+OPS = [(ora.PRO_SET, 0.0, ora.EPI_SCALE, 5.0), (ora.PRO_SCALE, 0.5, ora.EPI_NONE, 0.0), (ora.PRO_SCALE, -2.0, ora.EPI_SCALE, 3.0),
+       (ora.PRO_SET, -7.0, ora.EPI_RELU, 0.0), (ora.PRO_SET, 3.0, ora.EPI_RELU_NOCOND, 0.0), (ora.PRO_NONE, 0.0, ora.EPI_SET, 1.25),
+       (ora.PRO_SCALE, 2.9, ora.EPI_SCALE, -3.7)]
+
+
+@pytest.mark.parametrize("case", [("f16", "f32", 256, 512, 256, -1), ("bf16", "bf16", 256, 384, 128, -1), ("i8", "i32", 256, 256, 512, -1),
+                                  ("f16", "f16", 200, 144, 176, -1), ("f32", "f32", 96, 80, 72, -1), ("f16", "f32", 33, 47, 29, 200),
+                                  ("f16", "f16", 8, 1088, 512, -1), ("bf16", "f32", 24, 1024, 256, -1), ("f16", "f16", 5, 1000, 998, -1)])
+def test_fragment_ops_alpha_beta(case):
+    """C = epilogue(prologue(C) + A@B) for the SET / SCALE ops of the reference's tensorized plan
+    (Tensor_MatMul_ElementWiseOps_GPU.md:85-99; helpers CppPrinterUtils.h:630-655), on the MFMA,
+    edge, fp32, generic and both skinny kernels."""
+    import accera_amd as acc
+    import torch
+    in_type, out_type, M, N, K, variant = case
+    for n, (pro, pa, epi, ea) in enumerate(OPS):
+        rng = np.random.default_rng(300 + n)
+        A, B = make_input(rng, (M, K), in_type), make_input(rng, (K, N), in_type)
+        C0 = make_input(rng, (M, N), "i8").astype(np.int32) * 1000 if out_type == "i32" else make_input(rng, (M, N), out_type)
+        dC = to_device(C0, out_type)
+        acc.gemm_relu(to_device(A, in_type), to_device(B, in_type), dC, prologue=pro, prologue_arg=pa, epilogue=epi, epilogue_arg=ea,
+                      variant=variant)
+        torch.cuda.synchronize()
+        want = ora.gemm_relu_exact(A, B, C0, in_type, out_type, pro, epi, prologue_arg=pa, epilogue_arg=ea)
+        assert_matches(to_host(dC, out_type), want, out_type, K)
+
+
 def test_linearity_and_k_split_invariance_full_size_int8():
     """Size-independent property at a large size: for int8, A@[B1|B2] computed as one
     N=2048 problem equals the two N=1024 problems, and equals int64 NumPy on sampled rows."""

@@ -236,3 +236,38 @@ def test_bad_type_combination_is_rejected():
     C = np.zeros((4, 4), np.float32)
     with pytest.raises(ValueError):
         ora.gemm_relu(A, A, C, "i8", "f32")
+
+
+# ---- SET / SCALE fragment ops of the NumPy restatement, pinned by closed forms ------------------
+def test_alpha_beta_table_constant_fill_known_answers():
+    """The reference's GEMM table C = alpha*(A@B) + beta*C
+    (docs/Tutorials/GPU/Tensor_MatMul_ElementWiseOps_GPU.md:85-99) on its own constant fills
+    A = 2, B = 3, C = 0.42 (docs/Tutorials/Hello_MatMul.md:165-237): every entry is a closed form."""
+    M, N, K = 8, 16, 256
+    A = np.full((M, K), 2, np.float32)
+    B = np.full((K, N), 3, np.float32)
+    C = np.full((M, N), 0.42, np.float32)
+    e = lambda **kw: ora.gemm_relu_exact(A, B, C, "f32", "f32", narrow_out=False, **kw)
+    assert np.all(e(prologue=ora.PRO_SET, prologue_arg=0, epilogue=ora.EPI_NONE) == 6.0 * K)                       # C = A@B
+    assert np.allclose(e(prologue=ora.PRO_NONE, epilogue=ora.EPI_NONE), 6.0 * K + np.float32(0.42))                # C += A@B
+    assert np.allclose(e(prologue=ora.PRO_SCALE, prologue_arg=0.5, epilogue=ora.EPI_NONE), 6.0 * K + 0.5 * np.float32(0.42))
+    assert np.all(e(prologue=ora.PRO_SET, prologue_arg=0, epilogue=ora.EPI_SCALE, epilogue_arg=5.0) == 30.0 * K)   # alpha = 5
+    assert np.all(e(prologue=ora.PRO_SET, prologue_arg=-7.0, epilogue=ora.EPI_NONE) == 6.0 * K - 7.0)
+    assert np.all(e(prologue=ora.PRO_NONE, epilogue=ora.EPI_SET, epilogue_arg=1.25) == 1.25)
+    # epilogue SCALE acts on the whole fragment, prologue'd C included: (beta*C + A@B) * alpha
+    got = e(prologue=ora.PRO_SCALE, prologue_arg=2.0, epilogue=ora.EPI_SCALE, epilogue_arg=-3.0)
+    assert np.allclose(got, -3.0 * (6.0 * K + 2.0 * np.float32(0.42)))
+
+
+def test_int_ops_cast_operands_and_wrap():
+    """Operands are cast to the accumulator type (int for int8 inputs: 2.9 -> 2) and int32 sums wrap."""
+    rng = np.random.default_rng(5)
+    A = rng.integers(-128, 128, (16, 32), dtype=np.int8)
+    B = rng.integers(-128, 128, (32, 16), dtype=np.int8)
+    C = rng.integers(-1000, 1000, (16, 16)).astype(np.int32)
+    P = A.astype(np.int64) @ B.astype(np.int64)
+    wrap = lambda x: ((x + 2**31) % 2**32) - 2**31
+    got = ora.gemm_relu_exact(A, B, C, "i8", "i32", ora.PRO_SCALE, ora.EPI_SCALE, prologue_arg=2.9, epilogue_arg=-3.7)
+    assert np.array_equal(got, wrap((P + 2 * C.astype(np.int64)) * -3).astype(np.int32))
+    got = ora.gemm_relu_exact(A, B, C, "i8", "i32", ora.PRO_SET, ora.EPI_SCALE, prologue_arg=11, epilogue_arg=2**20)
+    assert np.array_equal(got, wrap((P + 11) * 2**20).astype(np.int32)) and (np.abs((P + 11) * 2**20) >= 2**31).any()
