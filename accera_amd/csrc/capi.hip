@@ -104,21 +104,23 @@ bool mfma_can_take(const MfmaVariant& v, const Problem& pb)
     const GemmArgs& g = pb.g;
     if (g.M <= 0 || g.N <= 0 || g.K <= 0) return false;
     const int es = elem_size(g.in_type), vec = 16 / es, bk = v.kb / es;
-    if (g.a_cs != 1 || g.c_cs != 1) return false; // A row-major (K contiguous), C row-major
+    if (g.c_cs != 1) return false;                          // C row-major
+    if (v.a_kc ? g.a_cs != 1 : g.a_rs != 1) return false;   // A with K contiguous (row-major) or M contiguous
     if (v.b_kc ? g.b_rs != 1 : g.b_cs != 1) return false;
-    const int64_t lda = g.a_rs, ldb = v.b_kc ? g.b_cs : g.b_rs;
+    const int64_t lda = v.a_kc ? g.a_rs : g.a_cs, ldb = v.b_kc ? g.b_cs : g.b_rs;
     if (lda % vec || ldb % vec) return false;
     if (pb.have_pointers && (!aligned16(g.A) || !aligned16(g.B))) return false;
     if (v.edge) {
         if (g.K % vec) return false;
         if (!v.b_kc && g.N % vec) return false;
+        if (!v.a_kc && g.M % vec) return false;
     } else {
         if (g.M % v.bm || g.N % v.bn || g.K % bk) return false;
     }
     // offsets inside one output tile are 32-bit in the write-back
     if ((int64_t)v.bm * g.c_rs * 4 >= (1ll << 32)) return false;
     // per-lane global offsets of the direct fill are 32-bit
-    if ((int64_t)v.bm * lda * es >= (1ll << 31) || (int64_t)(v.b_kc ? v.bn : bk) * ldb * es >= (1ll << 31)) return false;
+    if ((int64_t)(v.a_kc ? v.bm : bk) * lda * es >= (1ll << 31) || (int64_t)(v.b_kc ? v.bn : bk) * ldb * es >= (1ll << 31)) return false;
     return true;
 }
 
@@ -519,9 +521,9 @@ int acc950_variant_name(int variant, char* buf, size_t buf_len)
     const MfmaVariant* tab = mfma_variants_f16(&n);
     if (variant < 0 || variant >= n) return fail(ACC950_INVALID_ARGUMENT, "unknown kernel variant");
     const MfmaVariant& v = tab[variant];
-    std::snprintf(buf, buf_len, "mfma %dx%d kb%d waves %dx%d B=%s fill=%s stages=%d%s%s", v.bm, v.bn, v.kb, v.waves_m, v.waves_n,
-                  v.b_kc ? "col-major" : "row-major", v.direct ? "direct" : "registers", v.stages, v.edge ? " edge" : "",
-                  v.pingpong ? " pingpong" : "");
+    std::snprintf(buf, buf_len, "mfma %dx%d kb%d waves %dx%d %sB=%s fill=%s stages=%d%s%s", v.bm, v.bn, v.kb, v.waves_m, v.waves_n,
+                  v.a_kc ? "" : "A=col-major ", v.b_kc ? "col-major" : "row-major", v.direct ? "direct" : "registers", v.stages,
+                  v.edge ? " edge" : "", v.pingpong ? " pingpong" : "");
     return ACC950_OK;
 }
 

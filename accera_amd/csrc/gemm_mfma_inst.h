@@ -11,12 +11,21 @@
 
 namespace acc950 {
 
-#define V(BM, BN, WM, WN, BKC, DIRECT, EDGE, KB, STAGES)                                               \
-    { BM, BN, WM, WN, /*a_kc=*/true, BKC, DIRECT, EDGE, KB, STAGES, false,                             \
-      &launch_mfma<MfmaConfig<ACC950_IN, BM, BN, WM, WN, true, BKC, DIRECT, EDGE, KB, STAGES>> }
-#define VP(BM, BN, WM, WN, BKC, KB, STAGES)                                                             \
-    { BM, BN, WM, WN, /*a_kc=*/true, BKC, true, false, KB, STAGES, true,                               \
-      &launch_mfma<MfmaConfig<ACC950_IN, BM, BN, WM, WN, true, BKC, true, false, KB, STAGES, true>> }
+#define VA(AKC, BM, BN, WM, WN, BKC, DIRECT, EDGE, KB, STAGES)                                         \
+    { BM, BN, WM, WN, AKC, BKC, DIRECT, EDGE, KB, STAGES, false,                                       \
+      &launch_mfma<MfmaConfig<ACC950_IN, BM, BN, WM, WN, AKC, BKC, DIRECT, EDGE, KB, STAGES>> }
+#define VPA(AKC, BM, BN, WM, WN, BKC, KB, STAGES)                                                       \
+    { BM, BN, WM, WN, AKC, BKC, true, false, KB, STAGES, true,                                         \
+      &launch_mfma<MfmaConfig<ACC950_IN, BM, BN, WM, WN, AKC, BKC, true, false, KB, STAGES, true>> }
+#define V(BM, BN, WM, WN, BKC, DIRECT, EDGE, KB, STAGES) VA(true, BM, BN, WM, WN, BKC, DIRECT, EDGE, KB, STAGES)
+#define VP(BM, BN, WM, WN, BKC, KB, STAGES) VPA(true, BM, BN, WM, WN, BKC, KB, STAGES)
+// column-major A (M contiguous; the "transA" shapes of the reference's sweep lists,
+// /root/reference/tools/benchmarkers/gemm_*.csv): staged as it lies in memory and read with the
+// transposing LDS loads, like a row-major B
+#define LAYOUT_AT(BKC)                                    \
+    VPA(false, 256, 256, 2, 4, BKC, 64, 4),               \
+    VA(false, 128, 128, 2, 2, BKC, true, false, 128, 2),  \
+    VA(false, 128, 128, 2, 2, BKC, false, true, 128, 2)
 
 #define LAYOUT(BKC)                                 \
     V(256, 256, 2, 4, BKC, true, false, 128, 2),    \
@@ -39,7 +48,12 @@ static const MfmaVariant kVariants[] = {
     // 192-wide tiles (N = 3072 = 16 x 192 gives one tile per CU); K-contiguous B only
     VP(256, 192, 4, 2, true, 64, 4),
     V(256, 192, 4, 2, true, true, false, 128, 2),
+    LAYOUT_AT(false),
+    LAYOUT_AT(true),
 };
+#undef LAYOUT_AT
+#undef VA
+#undef VPA
 #undef LAYOUT
 #undef V
 #undef VP

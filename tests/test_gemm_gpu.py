@@ -20,7 +20,7 @@ PAIRS = [("f16", "f32"), ("f16", "f16"), ("bf16", "f32"), ("bf16", "bf16"), ("i8
 
 
 def run_case(in_type, out_type, M, N, K, b_layout="row", c_layout="row", variant=-1, splits=0,
-             prologue=ora.PRO_SET0, epilogue=ora.EPI_RELU, seed=0, dist="uniform", expect_variant=None):
+             prologue=ora.PRO_SET0, epilogue=ora.EPI_RELU, seed=0, dist="uniform", expect_variant=None, a_layout="row"):
     import accera_amd as acc
     import torch
     rng = np.random.default_rng(seed)
@@ -28,6 +28,8 @@ def run_case(in_type, out_type, M, N, K, b_layout="row", c_layout="row", variant
     B = make_input(rng, (K, N), in_type, dist)
     if b_layout == "col":
         B = np.asfortranarray(B)
+    if a_layout == "col":
+        A = np.asfortranarray(A)
     if prologue == ora.PRO_NONE:
         C0 = make_input(rng, (M, N), "i8", dist).astype(np.int32) * 1000 if out_type == "i32" else \
             make_input(rng, (M, N), out_type, dist)
@@ -52,7 +54,7 @@ def run_case(in_type, out_type, M, N, K, b_layout="row", c_layout="row", variant
 def _variants(b_layout):
     from accera_amd import _lib
     names = [(v, _lib.variant_name(v)) for v in range(_lib.num_variants())]
-    key = "B=col-major" if b_layout == "col" else "B=row-major"
+    key = " B=col-major" if b_layout == "col" else " B=row-major"
     return [(v, n) for v, n in names if key in n]
 
 
@@ -64,13 +66,15 @@ def test_mfma_all_variants(in_type, out_type, b_layout):
         print("variant", v, name, in_type, b_layout, flush=True)
         # two tiles in each direction; K tile counts below, at and above the pipeline depth
         kb = int(re.search(r"kb(\d+)", name).group(1)) // (1 if in_type == "i8" else 2)
+        a_layout = "col" if "A=col-major" in name else "row"
         bm, bn = map(int, re.search(r"mfma (\d+)x(\d+)", name).groups())
         M, N = max(512, 2 * bm), (max(512, 2 * bn) if 512 % bn == 0 else 3 * bn)
         for k_tiles in (1, 2, 3, 7):
-            run_case(in_type, out_type, M, N, k_tiles * kb, b_layout=b_layout, variant=v, seed=v + k_tiles)
+            run_case(in_type, out_type, M, N, k_tiles * kb, b_layout=b_layout, variant=v, seed=v + k_tiles, a_layout=a_layout)
         if "edge" in name:
             # ragged M, N (multiple of the 16-byte vector only) and a K tail
-            run_case(in_type, out_type, 200, 144, 336 if in_type == "i8" else 176, b_layout=b_layout, variant=v, seed=100 + v)
+            run_case(in_type, out_type, 208 if a_layout == "col" else 200, 144, 336 if in_type == "i8" else 176, b_layout=b_layout,
+                     variant=v, seed=100 + v, a_layout=a_layout)
 
 
 @pytest.mark.parametrize("in_type,out_type", PAIRS)
@@ -79,6 +83,18 @@ def test_mfma_auto_output_types(in_type, out_type):
     run_case(in_type, out_type, 256, 384, 512, seed=4, prologue=ora.PRO_NONE)
     run_case(in_type, out_type, 256, 384, 512, seed=5, epilogue=ora.EPI_RELU_NOCOND, b_layout="col")
     run_case(in_type, out_type, 256, 384, 512, seed=6, epilogue=ora.EPI_NONE, prologue=ora.PRO_NONE)
+
+
+def test_column_major_a_takes_the_mfma_kernels():
+    """Column-major A (the transA rows of the reference's sweep lists, tools/benchmarkers/gemm_*.csv)
+    is chosen automatically and matches; so is a transposed view of a row-major tensor."""
+    from accera_amd import _lib
+    for in_type, out_type in [("f16", "f32"), ("bf16", "bf16"), ("i8", "i32")]:
+        for b_layout in ("row", "col"):
+            run_case(in_type, out_type, 512, 768, 1024, a_layout="col", b_layout=b_layout, seed=11)
+            run_case(in_type, out_type, 384, 128, 256, a_layout="col", b_layout=b_layout, seed=12, prologue=ora.PRO_NONE)
+    g, b, lds, v = _lib.launch_geometry(_lib.F16, _lib.F32, 4096, 4096, 4096, (1, 4096), (4096, 1), (4096, 1))
+    assert "A=col-major" in _lib.variant_name(v) and "pingpong" in _lib.variant_name(v)
 
 
 def test_mfma_single_k_tile_and_many_tiles():
