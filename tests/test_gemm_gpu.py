@@ -384,6 +384,43 @@ def test_linearity_and_k_split_invariance_full_size_int8():
     assert np.array_equal(C.astype(np.int64).sum(axis=1), A.astype(np.int64) @ B.astype(np.int64).sum(axis=1))
 
 
+# ---- the benchmark configurations at their full sizes --------------------------------------------------
+@pytest.mark.parametrize("cfg", [("f16", "f32", 4096, 4096, 4096, "row", "uniform"), ("bf16", "bf16", 4096, 3072, 768, "col", "normal"),
+                                 ("i8", "i32", 8192, 8192, 8192, "row", "uniform"), ("f16", "f16", 8, 11008, 4096, "row", "normal")])
+def test_benchmark_configurations_at_full_size(cfg):
+    """Automatic kernel choice at the sizes the benchmark quotes: sampled rows and columns of the
+    result against the exact restatement (float64 matmul of the exactly widened inputs; for int8 every
+    partial sum stays below 2^53, so float64 BLAS is exact there too), plus the row-checksum identity
+    sum_j (A@B)[i,j] = A[i,:] . (B 1) on the pre-ReLU product for the integer case."""
+    import accera_amd as acc
+    import torch
+    in_type, out_type, M, N, K, b_layout, dist = cfg
+    rng = np.random.default_rng(M + N + K)
+    A, B = make_input(rng, (M, K), in_type, dist), make_input(rng, (K, N), in_type, dist)
+    if b_layout == "col":
+        B = np.asfortranarray(B)
+    dA, dB = to_device(A, in_type), to_device(B, in_type)
+    dC = to_device(out_zeros(M, N, out_type) + (1 if out_type == "i32" else 0), out_type)  # poisoned: SET must overwrite
+    acc.gemm_relu(dA, dB, dC)
+    torch.cuda.synchronize()
+    got = ora.widen(to_host(dC, out_type), out_type)
+    Aw, Bw = ora.widen(A, in_type).astype(np.float64), ora.widen(B, in_type).astype(np.float64)
+    rows = np.arange(M) if M <= 64 else rng.choice(M, 48, replace=False)
+    cols = rng.choice(N, 48, replace=False)
+    want_rows = np.maximum(Aw[rows] @ Bw, 0)
+    want_cols = np.maximum(Aw @ Bw[:, cols], 0)
+    if out_type == "i32":
+        assert np.array_equal(got[rows], want_rows) and np.array_equal(got[:, cols], want_cols)
+        dC2 = to_device(out_zeros(M, N, out_type), out_type)
+        acc.gemm_relu(dA, dB, dC2, epilogue=acc.EPILOGUE_NONE)
+        torch.cuda.synchronize()
+        assert np.array_equal(to_host(dC2, "i32").astype(np.int64).sum(axis=1), (Aw @ Bw.sum(axis=1)).astype(np.int64))
+    else:
+        assert_matches(ora.narrow(got[rows], out_type), ora.narrow(want_rows, out_type), out_type, K)
+        assert_matches(ora.narrow(got[:, cols], out_type), ora.narrow(want_cols, out_type), out_type, K)
+    assert (got[rows] == 0).any() and (got[rows] > 0).any()
+
+
 # ---- error behaviour of the C ABI ---------------------------------------------------------------
 def test_errors_are_reported_not_thrown():
     import accera_amd as acc
