@@ -213,8 +213,12 @@ int auto_mfma_variant(const Problem& pb)
         double cost = (double)rounds * wgs_per_cu * v.bm * v.bn;
         if (v.edge) cost *= 1.5;                 // register-staged fill, bounds checks
         if (!v.direct) cost *= 1.2;
-        // rank inside one tile shape: ping-pong kb64 x4 > ping-pong others > 8-wave > rest
-        int rank = v.pingpong ? (v.kb == 64 && v.stages == 4 ? 4 : 3) : (v.waves_m * v.waves_n == 8 ? 2 : 1);
+        // measured on sweeps: 4-wave tiles reach about 85 % of the ping-pong kernel's rate when two
+        // workgroups share a CU and about 70 % when a workgroup has the CU to itself
+        if (v.waves_m * v.waves_n <= 4) cost /= wgs_per_cu == 2 ? 0.85 : 0.7;
+        // rank inside one tile shape: ping-pong kb64 x4 > ping-pong others > 8-wave > 4-wave (kb64 x4 first)
+        int rank = v.pingpong ? (v.kb == 64 && v.stages == 4 ? 8 : 6) : (v.waves_m * v.waves_n == 8 ? 4 : 2);
+        if (!v.pingpong && v.kb == 64 && v.stages == 4) rank += 1;
         const bool better = best < 0 || cost < best_cost * 0.999 ||
                             (cost <= best_cost * 1.001 && ((int64_t)v.bm * v.bn > (int64_t)tab[best].bm * tab[best].bn ||
                                                            ((int64_t)v.bm * v.bn == (int64_t)tab[best].bm * tab[best].bn && rank > best_rank)));

@@ -1,0 +1,170 @@
+"""Variant sweep over a list of GEMM shapes: the counterpart of the reference's benchmark driver
+(/root/reference/tools/benchmarkers/accera_gemm.py:187-348 builds one package per point of its
+tuning space, :584-657 checks each against NumPy and times it with hatlib's min-of-means).
+
+Here the points of the space are the prebuilt kernel variants of libaccera_mi355x.so.  For every
+row of a shape list (columns m,n,k,transA,transB,alpha,beta,lda,ldb,ldc as in the reference's
+tools/benchmarkers/gemm_*.csv; transX = 1 means the operand is stored column-major) the tool
+
+  * asks the library which variants can take the problem (acc950_launch_geometry),
+  * runs each on device-resident random inputs, optionally checks it against a float64 / int64
+    NumPy product on sampled rows (rtol 1e-2 as the reference's driver),
+  * times it with HIP events (min over batches of the mean time per launch),
+  * writes one CSV row per (shape, variant) and prints the best variant per shape.
+
+    python -m accera_amd.tune --input accera_amd/shapes/transformer_gemm.csv --type f16 --check --relu
+
+alpha / beta map to the fragment ops: beta 0 -> prologue SET 0, beta 1 -> none, else SCALE beta;
+alpha != 1 -> epilogue SCALE alpha (a ReLU epilogue and alpha != 1 exclude each other, as in the
+reference's table docs/Tutorials/GPU/Tensor_MatMul_ElementWiseOps_GPU.md:85-99).
+"""
+import argparse
+import csv
+import sys
+
+import numpy as np
+
+from . import _lib
+
+_OUT_FOR = {"f32": "f32", "f16": "f32", "bf16": "bf16", "i8": "i32"}
+
+
+def _torch_dtype(torch, t):
+    return {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16, "i8": torch.int8, "i32": torch.int32}[t]
+
+
+def _make(torch, rows, cols, t, col_major, gen):
+    """Random (rows x cols) matrix on the device, stored row- or column-major."""
+    shape = (cols, rows) if col_major else (rows, cols)
+    if t == "i8":
+        x = torch.randint(-128, 128, shape, device="cuda", dtype=torch.int8, generator=gen)
+    else:
+        x = (torch.rand(shape, device="cuda", generator=gen) * 2 - 1).to(_torch_dtype(torch, t))
+    return x.t() if col_major else x
+
+
+def candidates(in_id, out_id, M, N, K, sa, sb, sc, splits_for_skinny=(0, 2, 4, 8)):
+    """(variant, k_splits) pairs the library accepts for this problem."""
+    L = _lib.lib()
+    ids = list(range(_lib.num_variants())) + [_lib.VARIANT_SKINNY_BASE + i for i in range(_lib.num_skinny_variants())]
+    ids += [_lib.VARIANT_F32_MFMA, _lib.VARIANT_GENERIC]
+    out = []
+    for v in ids:
+        for sp in (splits_for_skinny if v >= _lib.VARIANT_SKINNY_BASE and v < _lib.VARIANT_GENERIC else (0,)):
+            try:
+                _lib.launch_geometry(in_id, out_id, M, N, K, sa, sb, sc, v, sp)
+            except _lib.Acc950Error:
+                continue
+            out.append((v, sp))
+    return out
+
+
+def time_call(torch, call, min_time_s=0.05, batches=5):
+    """Min over batches of the mean time per launch, HIP events on the launch stream."""
+    for _ in range(3):
+        call()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record(); call(); e1.record(); torch.cuda.synchronize()
+    one = max(e0.elapsed_time(e1) * 1e-3, 1e-6)
+    n = int(min(max(min_time_s / batches / one, 5), 2000))
+    best = float("inf")
+    for _ in range(batches):
+        e0.record()
+        for _ in range(n):
+            call()
+        e1.record()
+        torch.cuda.synchronize()
+        best = min(best, e0.elapsed_time(e1) * 1e-3 / n)
+    return best
+
+
+def sweep(rows, in_type, relu, check, out_type=None, min_time_s=0.05, log=print):
+    import torch
+    from .gemm import GemmCall
+    if not torch.cuda.is_available():
+        raise RuntimeError("no GPU visible; the HIP kernels have no CPU fallback")
+    out_type = out_type or _OUT_FOR[in_type]
+    in_id, out_id = getattr(_lib, in_type.upper()), getattr(_lib, out_type.upper())
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(7)
+    results = []
+    for r in rows:
+        M, N, K = int(r["m"]), int(r["n"]), int(r["k"])
+        ta, tb = bool(int(r.get("transA", 0))), bool(int(r.get("transB", 0)))
+        alpha, beta = float(r.get("alpha", 1.0)), float(r.get("beta", 0.0))
+        A, B = _make(torch, M, K, in_type, ta, gen), _make(torch, K, N, in_type, tb, gen)
+        C0 = _make(torch, M, N, "i8" if out_type == "i32" else out_type, False, gen).to(_torch_dtype(torch, out_type))
+        pro, parg = (_lib.PROLOGUE_SET0, 0.0) if beta == 0 else (_lib.PROLOGUE_NONE, 0.0) if beta == 1 else (_lib.PROLOGUE_SCALE, beta)
+        if alpha != 1 and relu:
+            log(f"{M}x{N}x{K}: skipped (alpha != 1 and a fused ReLU are two epilogue ops; one kernel carries one)")
+            continue
+        epi, earg = (_lib.EPILOGUE_SCALE, alpha) if alpha != 1 else (_lib.EPILOGUE_RELU if relu else _lib.EPILOGUE_NONE, 0.0)
+        want = sample = None
+        if check:
+            idx = np.arange(M) if M <= 64 else np.random.default_rng(M + N).choice(M, 32, replace=False)
+            Ah, Bh = A[torch.as_tensor(idx, device="cuda")].double().cpu().numpy(), B.double().cpu().numpy()
+            parg_c, earg_c = (int(parg), int(earg)) if in_type == "i8" else (np.float32(parg), np.float32(earg))
+            want = Ah @ Bh + (0 if beta == 0 else C0[torch.as_tensor(idx, device="cuda")].double().cpu().numpy() * (1 if beta == 1 else parg_c))
+            want = want * earg_c if alpha != 1 else (np.maximum(want, 0) if relu else want)
+            sample = torch.as_tensor(idx, device="cuda")
+        sa, sb, sc = (A.stride(0), A.stride(1)), (B.stride(0), B.stride(1)), (N, 1)
+        best = None
+        for v, sp in candidates(in_id, out_id, M, N, K, sa, sb, sc):
+            C = C0.clone()
+            call = GemmCall(A, B, C, prologue=pro, epilogue=epi, variant=v, k_splits=sp, prologue_arg=parg, epilogue_arg=earg)
+            try:
+                call()
+            except _lib.Acc950Error:
+                continue  # refused with the actual pointers (alignment)
+            ok = ""
+            if check:
+                C.copy_(C0)
+                call()
+                torch.cuda.synchronize()
+                got = C[sample].double().cpu().numpy()
+                tol = 0 if out_type == "i32" else 1e-2
+                ok = bool(np.allclose(got, want, rtol=tol, atol=tol * max(1.0, float(np.abs(want).max())) * 1e-1))
+            if beta != 0:
+                t = time_call(torch, lambda: (C.copy_(C0), call()), min_time_s) - time_call(torch, lambda: C.copy_(C0), min_time_s)
+            else:
+                t = time_call(torch, call, min_time_s)
+            row = dict(m=M, n=N, k=K, transA=int(ta), transB=int(tb), alpha=alpha, beta=beta, type=in_type, out_type=out_type,
+                       variant=v, k_splits=sp, kernel=_lib.variant_name(v), time_ms=round(t * 1e3, 5),
+                       TFlops=round(2.0 * M * N * K / t / 1e12, 3), correct=ok)
+            results.append(row)
+            if ok is not False and (best is None or row["time_ms"] < best["time_ms"]):
+                best = row
+        if best:
+            log(f"{M}x{N}x{K} tA={int(ta)} tB={int(tb)} a={alpha} b={beta}: best {best['TFlops']} TFlops {best['time_ms']} ms  "
+                f"variant {best['variant']} splits {best['k_splits']} ({best['kernel']})")
+    return results
+
+
+def main(argv=None):
+    ap = argparse.ArgumentParser(description=__doc__.split("\n")[0])
+    ap.add_argument("--input", required=True, help="shape list (csv: m,n,k,transA,transB,alpha,beta,...)")
+    ap.add_argument("--type", default="f16", choices=sorted(_OUT_FOR))
+    ap.add_argument("--out-type", default=None, choices=["f32", "f16", "bf16", "i32"])
+    ap.add_argument("--relu", action="store_true", help="fused ReLU epilogue (rows with alpha != 1 are rejected)")
+    ap.add_argument("--check", action="store_true", help="verify every variant against a NumPy product on sampled rows")
+    ap.add_argument("--output", default=None, help="csv of all (shape, variant) results")
+    ap.add_argument("--min-time", type=float, default=0.05, help="seconds of timed launches per variant")
+    args = ap.parse_args(argv)
+    with open(args.input) as f:
+        rows = [r for r in csv.DictReader(f) if r.get("m")]
+    _lib.check(_lib.lib().acc950_init(0))
+    results = sweep(rows, args.type, args.relu, args.check, args.out_type, args.min_time)
+    if args.output and results:
+        with open(args.output, "w", newline="") as f:
+            w = csv.DictWriter(f, fieldnames=list(results[0]))
+            w.writeheader()
+            w.writerows(results)
+    bad = [r for r in results if r["correct"] is False]
+    for r in bad:
+        print(f"MISMATCH {r['m']}x{r['n']}x{r['k']} variant {r['variant']} ({r['kernel']})", file=sys.stderr)
+    return 1 if bad else 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -72,3 +72,21 @@ def test_argument_checking_on_the_host():
     assert rc == _lib.INVALID_ARGUMENT and b"null" in _lib.lib().acc950_last_error()
     # empty problems are a no-op
     assert _lib.lib().acc950_gemm_relu(_lib.F16, _lib.F32, 0, 64, 64, None, 64, 1, None, 64, 1, None, 64, 1, 1, 1, None) == 0
+
+
+def test_sweep_tool_lists_the_variants_that_take_a_problem():
+    """accera_amd.tune enumerates the points of the variant space for a shape (counterpart of
+    get_variants, tools/benchmarkers/accera_gemm.py:187-348) without touching the GPU."""
+    from accera_amd import tune
+    c = tune.candidates(_lib.F16, _lib.F32, 4096, 4096, 4096, (4096, 1), (4096, 1), (4096, 1))
+    names = [_lib.variant_name(v) for v, _ in c]
+    assert any("pingpong" in n for n in names) and any("generic" in n for n in names)
+    assert not any("skinny" in n or "A=col-major" in n or " B=col-major" in n for n in names)
+    c = tune.candidates(_lib.F16, _lib.F16, 8, 11008, 4096, (4096, 1), (11008, 1), (11008, 1))
+    assert any("skinny mfma" in _lib.variant_name(v) and sp == 4 for v, sp in c)
+    c = tune.candidates(_lib.F16, _lib.F32, 1024, 1024, 1024, (1, 1024), (1024, 1), (1024, 1))
+    assert all("A=col-major" in _lib.variant_name(v) or "generic" in _lib.variant_name(v) for v, _ in c)
+    import csv, os
+    with open(os.path.join(os.path.dirname(tune.__file__), "shapes", "transformer_gemm.csv")) as f:
+        rows = list(csv.DictReader(f))
+    assert len(rows) >= 10 and {"m", "n", "k", "transA", "transB", "alpha", "beta"} <= set(rows[0])

@@ -421,6 +421,18 @@ def test_benchmark_configurations_at_full_size(cfg):
     assert (got[rows] == 0).any() and (got[rows] > 0).any()
 
 
+def test_sweep_tool_checks_and_times_every_variant():
+    """accera_amd.tune on two small rows (one with alpha / beta, one transposed): every variant the
+    library accepts must pass the NumPy check (rtol 1e-2 as accera_gemm.py:632)."""
+    from accera_amd import tune
+    rows = [dict(m=512, n=768, k=256, transA=0, transB=1, alpha=1.0, beta=0.0), dict(m=256, n=256, k=512, transA=1, transB=0, alpha=2.0, beta=0.5),
+            dict(m=8, n=1088, k=512, transA=0, transB=0, alpha=1.0, beta=1.0)]
+    res = tune.sweep(rows, "f16", relu=False, check=True, min_time_s=0.002, log=lambda *_: None)
+    assert len(res) >= 8 and all(r["correct"] is True for r in res), [r for r in res if r["correct"] is not True]
+    res = tune.sweep(rows[:1], "i8", relu=True, check=True, min_time_s=0.002, log=lambda *_: None)
+    assert res and all(r["correct"] is True for r in res)
+
+
 # ---- error behaviour of the C ABI ---------------------------------------------------------------
 def test_errors_are_reported_not_thrown():
     import accera_amd as acc
