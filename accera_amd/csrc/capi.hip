@@ -64,11 +64,19 @@ struct Problem {
     bool have_pointers;
 };
 
+// Batch of independent problems: count and element distance between consecutive A, B, C.
+struct Batch {
+    int count = 1;
+    int64_t a_bs = 0, b_bs = 0, c_bs = 0;
+};
+
 int make_problem(int in_type, int out_type, int M, int N, int K,
                  const void* A, int64_t a_rs, int64_t a_cs, const void* B, int64_t b_rs, int64_t b_cs,
                  void* C, int64_t c_rs, int64_t c_cs, int prologue, int epilogue, bool need_pointers, Problem* out,
-                 double prologue_arg = 0.0, double epilogue_arg = 0.0)
+                 double prologue_arg = 0.0, double epilogue_arg = 0.0, Batch batch = Batch())
 {
+    if (batch.count < 0 || batch.a_bs < 0 || batch.b_bs < 0 || batch.c_bs < 0) return fail(ACC950_INVALID_ARGUMENT, "negative batch count or stride");
+    if (batch.count > 65535) return fail(ACC950_INVALID_ARGUMENT, "at most 65535 problems per batch");
     if (!type_pair_ok(in_type, out_type)) return fail(ACC950_INVALID_ARGUMENT, "unsupported input/output element type pair");
     if (M < 0 || N < 0 || K < 0) return fail(ACC950_INVALID_ARGUMENT, "negative matrix dimension");
     if (a_rs < 0 || a_cs < 0 || b_rs < 0 || b_cs < 0 || c_rs < 0 || c_cs < 0)
@@ -92,6 +100,11 @@ int make_problem(int in_type, int out_type, int M, int N, int K,
         g.A = B; g.B = A; g.C = C; g.M = N; g.N = M; g.K = K;
         g.a_rs = b_cs; g.a_cs = b_rs; g.b_rs = a_cs; g.b_cs = a_rs; g.c_rs = c_cs; g.c_cs = c_rs;
     }
+    g.batch = batch.count;
+    g.a_bs = transpose ? batch.b_bs : batch.a_bs;
+    g.b_bs = transpose ? batch.a_bs : batch.b_bs;
+    g.c_bs = batch.c_bs;
+    if (batch.count == 0) g.M = 0; // nothing to do
     out->g = g;
     out->have_pointers = need_pointers;
     return ACC950_OK;
@@ -110,6 +123,7 @@ bool mfma_can_take(const MfmaVariant& v, const Problem& pb)
     const int64_t lda = v.a_kc ? g.a_rs : g.a_cs, ldb = v.b_kc ? g.b_cs : g.b_rs;
     if (lda % vec || ldb % vec) return false;
     if (pb.have_pointers && (!aligned16(g.A) || !aligned16(g.B))) return false;
+    if (g.batch > 1 && (g.a_bs % vec || g.b_bs % vec)) return false; // every problem of the batch 16-byte aligned
     if (v.edge) {
         if (g.K % vec) return false;
         if (!v.b_kc && g.N % vec) return false;
@@ -136,6 +150,7 @@ bool skinny_can_take(const Problem& pb, int sv)
     // per-lane offsets of the direct-to-LDS fills are 32-bit
     if ((int64_t)g.K * g.b_rs * 2 >= (1ll << 32) || (int64_t)v.max_m * g.a_rs * 2 >= (1ll << 32)) return false;
     if (pb.have_pointers && (!aligned16(g.B) || (reinterpret_cast<uintptr_t>(g.A) & (v.mfma ? 15u : 3u)))) return false;
+    if (g.batch > 1 && (g.b_bs % 8 || g.a_bs % (v.mfma ? 8 : 2))) return false;
     return true;
 }
 
@@ -292,17 +307,22 @@ int run(const Problem& pb, const Choice& c, hipStream_t stream, LaunchGeom* geom
         s.in_type = g.in_type; s.out_type = g.out_type; s.prologue = g.prologue; s.epilogue = g.epilogue;
         s.prologue_arg = g.prologue_arg; s.epilogue_arg = g.epilogue_arg;
         s.splits = c.splits;
+        s.batch = g.batch; s.a_bs = g.a_bs; s.b_bs = g.b_bs; s.c_bs = g.c_bs;
         s.extra_phase = -1;
         // 64-column MFMA blocks, no K split, dense rows of a multiple of 512 bytes: blocks whose
         // 128-byte lines have address bits 8:7 = 11 stream ~25 % slower (measured), so they are
         // shared by two workgroups each; the otherwise idle CUs take the second halves.
         const SkinnyVariant& skv = skinny_variant(sv);
         if (skv.mfma && skv.cols == 64 && c.splits == 1 && pb.have_pointers && (g.b_rs * 2) % 512 == 0 &&
-            skinny_column_blocks(sv, g.N) >= 128 && skinny_column_blocks(sv, g.N) <= 200 && g.K >= 512)
+            skinny_column_blocks(sv, g.N) >= 128 && skinny_column_blocks(sv, g.N) <= 200 && g.K >= 512 &&
+            (g.batch <= 1 || (g.b_bs * 2) % 512 == 0))
             s.extra_phase = (int)((3u - (unsigned)(reinterpret_cast<uintptr_t>(g.B) >> 7)) & 3u);
         const int ws_splits = s.extra_phase >= 0 ? 2 : c.splits;
         if (!dry_run && ws_splits > 1) {
-            e = ensure_workspace(skinny_scratch_floats(sv, g.N, ws_splits), (size_t)skinny_column_blocks(sv, g.N));
+            const size_t nb = g.batch > 1 ? (size_t)g.batch : 1;
+            s.scratch_bs = (int64_t)skinny_scratch_floats(sv, g.N, ws_splits);
+            s.counter_bs = skinny_column_blocks(sv, g.N);
+            e = ensure_workspace(nb * (size_t)s.scratch_bs, nb * (size_t)s.counter_bs);
             if (e != hipSuccess) return fail_hip(e, "workspace allocation");
             s.scratch = g_scratch;
             s.counters = g_counters;
@@ -362,6 +382,23 @@ int acc950_gemm_ops(int in_type, int out_type, int M, int N, int K,
     Problem pb;
     int rc = make_problem(in_type, out_type, M, N, K, A, a_rs, a_cs, B, b_rs, b_cs, C, c_rs, c_cs, prologue, epilogue, true, &pb,
                           prologue_arg, epilogue_arg);
+    if (rc) return rc;
+    Choice c;
+    rc = choose(pb, variant, k_splits, &c);
+    if (rc) return rc;
+    return run(pb, c, (hipStream_t)stream, nullptr, false);
+}
+
+int acc950_gemm_batched(int in_type, int out_type, int batch, int M, int N, int K,
+                        const void* A, int64_t a_bs, int64_t a_rs, int64_t a_cs, const void* B, int64_t b_bs, int64_t b_rs, int64_t b_cs,
+                        void* C, int64_t c_bs, int64_t c_rs, int64_t c_cs, int prologue, double prologue_arg, int epilogue,
+                        double epilogue_arg, int variant, int k_splits, void* stream)
+{
+    Problem pb;
+    Batch bt;
+    bt.count = batch; bt.a_bs = a_bs; bt.b_bs = b_bs; bt.c_bs = c_bs;
+    int rc = make_problem(in_type, out_type, M, N, K, A, a_rs, a_cs, B, b_rs, b_cs, C, c_rs, c_cs, prologue, epilogue, true, &pb,
+                          prologue_arg, epilogue_arg, bt);
     if (rc) return rc;
     Choice c;
     rc = choose(pb, variant, k_splits, &c);
@@ -466,15 +503,28 @@ int acc950_gemm_ops_host(int in_type, int out_type, int M, int N, int K,
                          const void* A, int64_t a_rs, int64_t a_cs, const void* B, int64_t b_rs, int64_t b_cs,
                          void* C, int64_t c_rs, int64_t c_cs, int prologue, double prologue_arg, int epilogue, double epilogue_arg)
 {
+    return acc950_gemm_batched_host(in_type, out_type, 1, M, N, K, A, 0, a_rs, a_cs, B, 0, b_rs, b_cs, C, 0, c_rs, c_cs, prologue,
+                                    prologue_arg, epilogue, epilogue_arg);
+}
+
+int acc950_gemm_batched_host(int in_type, int out_type, int batch, int M, int N, int K,
+                             const void* A, int64_t a_bs, int64_t a_rs, int64_t a_cs, const void* B, int64_t b_bs, int64_t b_rs,
+                             int64_t b_cs, void* C, int64_t c_bs, int64_t c_rs, int64_t c_cs, int prologue, double prologue_arg,
+                             int epilogue, double epilogue_arg)
+{
     Problem check;
+    Batch bt;
+    bt.count = batch; bt.a_bs = a_bs; bt.b_bs = b_bs; bt.c_bs = c_bs;
     int rc = make_problem(in_type, out_type, M, N, K, A, a_rs, a_cs, B, b_rs, b_cs, C, c_rs, c_cs, prologue, epilogue, true, &check,
-                          prologue_arg, epilogue_arg);
+                          prologue_arg, epilogue_arg, bt);
     if (rc) return rc;
-    if (M == 0 || N == 0) return ACC950_OK;
-    const size_t a_bytes = extent_elems(M, K, a_rs, a_cs) * elem_size(in_type);
-    const size_t b_bytes = extent_elems(K, N, b_rs, b_cs) * elem_size(in_type);
-    const size_t c_bytes = extent_elems(M, N, c_rs, c_cs) * elem_size(out_type);
-    const bool c_dense = extent_elems(M, N, c_rs, c_cs) == (size_t)M * (size_t)N;
+    if (M == 0 || N == 0 || batch == 0) return ACC950_OK;
+    const size_t nb = (size_t)(batch - 1);
+    const size_t a_elems = extent_elems(M, K, a_rs, a_cs), b_elems = extent_elems(K, N, b_rs, b_cs), c_elems = extent_elems(M, N, c_rs, c_cs);
+    const size_t a_bytes = (a_elems ? nb * a_bs + a_elems : 0) * elem_size(in_type);
+    const size_t b_bytes = (b_elems ? nb * b_bs + b_elems : 0) * elem_size(in_type);
+    const size_t c_bytes = (nb * c_bs + c_elems) * elem_size(out_type);
+    const bool c_dense = c_elems == (size_t)M * (size_t)N && (batch == 1 || (size_t)c_bs == c_elems);
 
     std::lock_guard<std::mutex> lock(g_host_mutex);
     hipError_t e;
@@ -483,12 +533,12 @@ int acc950_gemm_ops_host(int in_type, int out_type, int M, int N, int K,
     if ((e = reserve(g_dC, c_bytes)) != hipSuccess) return fail_hip(e, "hipMalloc(C)");
     if (a_bytes && (e = hipMemcpy(g_dA.p, A, a_bytes, hipMemcpyHostToDevice)) != hipSuccess) return fail_hip(e, "copy A to device");
     if (b_bytes && (e = hipMemcpy(g_dB.p, B, b_bytes, hipMemcpyHostToDevice)) != hipSuccess) return fail_hip(e, "copy B to device");
-    // C travels to the device when it is accumulated into, or when its extent has gaps
-    // that the copy back must not clobber
+    // C travels to the device when it is read (prologue NONE / SCALE), or when its extent has
+    // gaps that the copy back must not clobber
     if (prologue != PRO_SET || !c_dense)
         if ((e = hipMemcpy(g_dC.p, C, c_bytes, hipMemcpyHostToDevice)) != hipSuccess) return fail_hip(e, "copy C to device");
-    rc = acc950_gemm_ops(in_type, out_type, M, N, K, g_dA.p, a_rs, a_cs, g_dB.p, b_rs, b_cs, g_dC.p, c_rs, c_cs,
-                         prologue, prologue_arg, epilogue, epilogue_arg, ACC950_VARIANT_AUTO, 0, nullptr);
+    rc = acc950_gemm_batched(in_type, out_type, batch, M, N, K, g_dA.p, a_bs, a_rs, a_cs, g_dB.p, b_bs, b_rs, b_cs, g_dC.p, c_bs, c_rs,
+                             c_cs, prologue, prologue_arg, epilogue, epilogue_arg, ACC950_VARIANT_AUTO, 0, nullptr);
     if (rc) return rc;
     if ((e = hipMemcpy(C, g_dC.p, c_bytes, hipMemcpyDeviceToHost)) != hipSuccess) return fail_hip(e, "copy C to host");
     return ACC950_OK;

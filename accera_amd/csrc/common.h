@@ -29,6 +29,8 @@ struct GemmArgs {
     int prologue, epilogue;
     float prologue_arg, epilogue_arg; // SET / SCALE operand (0 for the other ops)
     int tiles_m, tiles_n; // workgroup grid in tiles (MFMA kernels)
+    int batch;                  // independent problems, one per blockIdx.z (1 for a plain GEMM)
+    int64_t a_bs, b_bs, c_bs;   // element distance between consecutive problems of a batch
     unsigned long long* stamps; // timed MFMA instantiation only: [workgroup][4 points][shader clock, 100 MHz clock]
 };
 
@@ -106,6 +108,16 @@ __device__ __forceinline__ float load_out(const void* C, int out_type, int64_t i
     if (out_type == T_F32) return ((const float*)C)[idx];
     if (out_type == T_F16) return f16_bits_to_float(((const uint16_t*)C)[idx]);
     return bf16_bits_to_float(((const uint16_t*)C)[idx]);
+}
+
+// Batched launch: blockIdx.z picks the problem; the kernel then sees one plain GEMM.
+__device__ __forceinline__ int elem_bytes(int type) { return type == T_I8 ? 1 : (type == T_F16 || type == T_BF16) ? 2 : 4; }
+__device__ __forceinline__ void select_batch(GemmArgs& p)
+{
+    const int64_t z = blockIdx.z;
+    p.A = (const char*)p.A + z * p.a_bs * elem_bytes(p.in_type);
+    p.B = (const char*)p.B + z * p.b_bs * elem_bytes(p.in_type);
+    p.C = (char*)p.C + z * p.c_bs * elem_bytes(p.out_type);
 }
 
 // ---- host-side launch record -------------------------------------------------------

@@ -37,6 +37,7 @@ template <bool A_KC, bool B_KC>
 __global__ void __launch_bounds__(256) gemm_f32_kernel(GemmArgs p)
 {
     __shared__ float red[3][16][64];
+    select_batch(p);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int r = lane & 31, kh = lane >> 5;
     const int row = blockIdx.y * 32 + r, col = blockIdx.x * 32 + r;
@@ -110,9 +111,9 @@ bool f32_can_take(const GemmArgs& g) { return g.in_type == T_F32 && g.M > 0 && g
 
 hipError_t launch_f32(const GemmArgs& g, hipStream_t stream, LaunchGeom* geom, bool dry_run)
 {
-    dim3 grid((g.N + 31) / 32, (g.M + 31) / 32, 1), block(256, 1, 1);
+    dim3 grid((g.N + 31) / 32, (g.M + 31) / 32, g.batch > 1 ? g.batch : 1), block(256, 1, 1);
     if (geom) {
-        geom->grid[0] = grid.x; geom->grid[1] = grid.y; geom->grid[2] = 1;
+        geom->grid[0] = grid.x; geom->grid[1] = grid.y; geom->grid[2] = grid.z;
         geom->block[0] = 256; geom->block[1] = geom->block[2] = 1;
         geom->dyn_lds = 0;
     }

@@ -32,6 +32,7 @@ __global__ void __launch_bounds__(256) gemm_generic_kernel(GemmArgs p)
 {
     __shared__ AccT sA[GK][GT + 1]; // [k][m]
     __shared__ AccT sB[GK][GT + 1]; // [k][n]
+    select_batch(p);
     const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
     const int m0 = blockIdx.y * GT, n0 = blockIdx.x * GT;
 
@@ -92,9 +93,9 @@ __global__ void __launch_bounds__(256) gemm_generic_kernel(GemmArgs p)
 
 hipError_t launch_generic(const GemmArgs& a, hipStream_t stream, LaunchGeom* geom, bool dry_run)
 {
-    dim3 grid((a.N + GT - 1) / GT, (a.M + GT - 1) / GT, 1), block(256, 1, 1);
+    dim3 grid((a.N + GT - 1) / GT, (a.M + GT - 1) / GT, a.batch > 1 ? a.batch : 1), block(256, 1, 1);
     if (geom) {
-        geom->grid[0] = grid.x; geom->grid[1] = grid.y; geom->grid[2] = 1;
+        geom->grid[0] = grid.x; geom->grid[1] = grid.y; geom->grid[2] = grid.z;
         geom->block[0] = 256; geom->block[1] = geom->block[2] = 1;
         geom->dyn_lds = 0;
     }

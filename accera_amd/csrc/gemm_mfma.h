@@ -271,6 +271,7 @@ __global__ void __launch_bounds__(Cfg::NT, Cfg::WGS_PER_CU) gemm_mfma_kernel(Gem
     constexpr int STAGE_BYTES = TA::TILE_BYTES + TB::TILE_BYTES;
 
     extern __shared__ __attribute__((aligned(1024))) char smem[];
+    select_batch(p);
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -666,7 +667,7 @@ __global__ void __launch_bounds__(Cfg::NT, Cfg::WGS_PER_CU) gemm_mfma_kernel(Gem
         if (threadIdx.x == 0 && p.stamps) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                p.stamps[(blockIdx.x * 4 + i) * 2] = stamp_clk[i];
+                p.stamps[(blockIdx.x * 4 + i) * 2] = stamp_clk[i]; // (probe runs unbatched)
                 p.stamps[(blockIdx.x * 4 + i) * 2 + 1] = stamp_ref[i];
             }
         }
@@ -683,7 +684,8 @@ hipError_t launch_mfma(const GemmArgs& a, hipStream_t stream, LaunchGeom* geom, 
     args.tiles_n = (a.N + Cfg::BN - 1) / Cfg::BN;
     if (geom) {
         geom->grid[0] = (unsigned)(args.tiles_m * args.tiles_n);
-        geom->grid[1] = geom->grid[2] = 1;
+        geom->grid[1] = 1;
+        geom->grid[2] = a.batch > 1 ? a.batch : 1;
         geom->block[0] = Cfg::NT;
         geom->block[1] = geom->block[2] = 1;
         geom->dyn_lds = Cfg::LDS_BYTES;
@@ -695,7 +697,7 @@ hipError_t launch_mfma(const GemmArgs& a, hipStream_t stream, LaunchGeom* geom, 
         if (e != hipSuccess) return e;
         attr_set = true;
     }
-    hipLaunchKernelGGL(kern, dim3(args.tiles_m * args.tiles_n), dim3(Cfg::NT), Cfg::LDS_BYTES, stream, args);
+    hipLaunchKernelGGL(kern, dim3(args.tiles_m * args.tiles_n, 1, a.batch > 1 ? a.batch : 1), dim3(Cfg::NT), Cfg::LDS_BYTES, stream, args);
     return hipGetLastError();
 }
 

@@ -63,6 +63,14 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_skinny_mfma_kernel(SkinnyArgs
     constexpr int NT = WAVES * 64;
     static_assert(LOADS * (DEPTH - 1) < 64, "vmcnt is a 6-bit counter");
     extern __shared__ __attribute__((aligned(1024))) char smem[];
+    { // batched launch: blockIdx.z picks the problem (and its slice of the K-split workspace)
+        const int64_t z = blockIdx.z;
+        p.A = (const char*)p.A + z * p.a_bs * 2;
+        p.B = (const char*)p.B + z * p.b_bs * 2;
+        p.C = (char*)p.C + z * p.c_bs * (p.out_type == T_F32 ? 4 : 2);
+        p.scratch += z * p.scratch_bs;
+        p.counters += z * p.counter_bs;
+    }
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -291,9 +299,9 @@ hipError_t launch_one(const SkinnyArgs& a, hipStream_t stream, LaunchGeom* geom,
     if (lds < red) lds = red;
     const int nblocks = (a.N + CB - 1) / CB;
     const int extra = a.extra_phase >= 0 && a.splits == 1 ? (nblocks - a.extra_phase + 3) / 4 : 0;
-    dim3 grid((nblocks + 7) / 8 * 8 + extra, a.splits, 1), block(WAVES * 64, 1, 1);
+    dim3 grid((nblocks + 7) / 8 * 8 + extra, a.splits, a.batch > 1 ? a.batch : 1), block(WAVES * 64, 1, 1);
     if (geom) {
-        geom->grid[0] = grid.x; geom->grid[1] = grid.y; geom->grid[2] = 1;
+        geom->grid[0] = grid.x; geom->grid[1] = grid.y; geom->grid[2] = grid.z;
         geom->block[0] = block.x; geom->block[1] = geom->block[2] = 1;
         geom->dyn_lds = lds;
     }

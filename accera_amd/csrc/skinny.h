@@ -17,6 +17,9 @@ struct SkinnyArgs {
     int splits;         // K split over grid.y
     int extra_phase;    // MFMA family, splits == 1: column blocks with index % 4 == extra_phase are split in two
                         // (second halves run as extra workgroups behind the regular grid); -1: none
+    int batch;                       // independent problems, one per blockIdx.z
+    int64_t a_bs, b_bs, c_bs;        // element distance between consecutive problems
+    int64_t scratch_bs, counter_bs;  // same for the K-split workspace (floats, counters)
     float* scratch;     // splits > 1: [split][column block][floats per block] partial sums
     unsigned* counters; // splits > 1: one arrival counter per column block, zero between launches
 };

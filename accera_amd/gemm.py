@@ -11,11 +11,31 @@ _TORCH_TYPES = {
 
 
 def _mat(t, name):
-    if t.dim() != 2:
-        raise ValueError(f"{name} must be 2-D")
+    if t.dim() not in (2, 3):
+        raise ValueError(f"{name} must be 2-D, or 3-D for a batch")
     if not t.is_cuda:
         raise ValueError(f"{name} must live on the GPU (there is no CPU path)")
-    return t.data_ptr(), t.stride(0), t.stride(1)
+    if t.dim() == 3:
+        return t.data_ptr(), t.stride(0), t.stride(1), t.stride(2)
+    return t.data_ptr(), 0, t.stride(0), t.stride(1)
+
+
+def _problem(A, B, C):
+    """(in type, out type, batch, M, N, K, A ptr + strides, B ..., C ...) of a 2-D call or of a batch
+    (3-D tensors (batch, rows, cols); a 2-D A or B is shared by every problem of the batch)."""
+    batch = C.shape[0] if C.dim() == 3 else 1
+    if C.dim() == 2 and (A.dim() == 3 or B.dim() == 3):
+        raise ValueError("a batched A or B needs a 3-D C")
+    for t, name in ((A, "A"), (B, "B")):
+        if t.dim() == 3 and t.shape[0] != batch:
+            raise ValueError(f"{name} has {t.shape[0]} matrices, C has {batch}")
+    M, K = A.shape[-2:]
+    K2, N = B.shape[-2:]
+    if K2 != K or tuple(C.shape[-2:]) != (M, N):
+        raise ValueError(f"shape mismatch: A {tuple(A.shape)}, B {tuple(B.shape)}, C {tuple(C.shape)}")
+    if A.dtype != B.dtype or A.dtype not in _TORCH_TYPES or C.dtype not in _TORCH_TYPES:
+        raise ValueError(f"unsupported dtypes {A.dtype}, {B.dtype}, {C.dtype}")
+    return (_TORCH_TYPES[A.dtype], _TORCH_TYPES[C.dtype], batch, M, N, K, *_mat(A, "A"), *_mat(B, "B"), *_mat(C, "C"))
 
 
 class GemmCall:
@@ -26,18 +46,12 @@ class GemmCall:
 
     def __init__(self, A, B, C, prologue=_lib.PROLOGUE_SET0, epilogue=_lib.EPILOGUE_RELU, variant=_lib.VARIANT_AUTO,
                  k_splits=0, stream=None, prologue_arg=0.0, epilogue_arg=0.0):
-        M, K = A.shape
-        K2, N = B.shape
-        if K2 != K or tuple(C.shape) != (M, N):
-            raise ValueError(f"shape mismatch: A {tuple(A.shape)}, B {tuple(B.shape)}, C {tuple(C.shape)}")
-        if A.dtype != B.dtype or A.dtype not in _TORCH_TYPES or C.dtype not in _TORCH_TYPES:
-            raise ValueError(f"unsupported dtypes {A.dtype}, {B.dtype}, {C.dtype}")
+        problem = _problem(A, B, C)
         if stream is None:
             stream = torch.cuda.current_stream(C.device).cuda_stream
         self.tensors = (A, B, C)
-        self._fn = _lib.lib().acc950_gemm_ops
-        self._args = (_TORCH_TYPES[A.dtype], _TORCH_TYPES[C.dtype], M, N, K, *_mat(A, "A"), *_mat(B, "B"), *_mat(C, "C"),
-                      prologue, float(prologue_arg), epilogue, float(epilogue_arg), variant, k_splits, stream)
+        self._fn = _lib.lib().acc950_gemm_batched
+        self._args = (*problem, prologue, float(prologue_arg), epilogue, float(epilogue_arg), variant, k_splits, stream)
 
     def __call__(self):
         rc = self._fn(*self._args)
@@ -56,20 +70,12 @@ def gemm_relu(A, B, C, prologue=_lib.PROLOGUE_SET0, epilogue=_lib.EPILOGUE_RELU,
     (/root/reference/docs/Tutorials/GPU/Tensor_MatMul_ElementWiseOps_GPU.md:85-99).
 
     A (M,K), B (K,N), C (M,N) are CUDA/HIP tensors; strides are honoured (a
-    column-major B is ``B_storage.t()`` of an (N,K) tensor).  Types: fp16/bf16 in ->
-    fp32/fp16/bf16 out, int8 -> int32, fp32 -> fp32.  Mirrors calling one function of
-    an Accera package on (A, B, C) (/root/reference/README.md:124-130), on device memory.
+    column-major B is ``B_storage.t()`` of an (N,K) tensor).  With a 3-D C (batch, M, N) the
+    call is a batch of independent problems in one launch (the reference's batch matmul nest,
+    /root/reference/accera/python/accera/test/mfma_tests.py:435-549); A and B are 3-D, or 2-D to be
+    shared by the whole batch.  Types: fp16/bf16 in -> fp32/fp16/bf16 out, int8 -> int32,
+    fp32 -> fp32.  Mirrors calling one function of an Accera package on (A, B, C)
+    (/root/reference/README.md:124-130), on device memory.
     """
-    M, K = A.shape
-    K2, N = B.shape
-    if K2 != K or tuple(C.shape) != (M, N):
-        raise ValueError(f"shape mismatch: A {tuple(A.shape)}, B {tuple(B.shape)}, C {tuple(C.shape)}")
-    if A.dtype != B.dtype or A.dtype not in _TORCH_TYPES or C.dtype not in _TORCH_TYPES:
-        raise ValueError(f"unsupported dtypes {A.dtype}, {B.dtype}, {C.dtype}")
-    if stream is None:
-        stream = torch.cuda.current_stream(C.device).cuda_stream
-    rc = _lib.lib().acc950_gemm_ops(_TORCH_TYPES[A.dtype], _TORCH_TYPES[C.dtype], M, N, K,
-                                    *_mat(A, "A"), *_mat(B, "B"), *_mat(C, "C"),
-                                    prologue, float(prologue_arg), epilogue, float(epilogue_arg), variant, k_splits, stream)
-    _lib.check(rc)
+    GemmCall(A, B, C, prologue, epilogue, variant, k_splits, stream, prologue_arg, epilogue_arg)()
     return C

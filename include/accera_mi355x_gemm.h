@@ -116,6 +116,26 @@ int acc950_gemm_ops_host(int in_type, int out_type, int M, int N, int K,
                          int prologue, double prologue_arg, int epilogue, double epilogue_arg);
 
 /*
+ * Batch of `batch` independent problems of one shape, one launch (grid.z = batch):
+ * C[b] = epilogue(prologue(C[b]) + A[b] * B[b]); x_batch_stride is the element distance
+ * between consecutive matrices (0 broadcasts one matrix to every problem).  Counterpart of
+ * the reference's batch matmul nest C[b,i,j] += A[b,i,k] * B[b,k,j] with the batch index
+ * bound to the grid (/root/reference/accera/python/accera/test/mfma_tests.py:435-549, 2519-2549).
+ * acc950_gemm_batched_host is the same on HOST pointers.
+ */
+int acc950_gemm_batched(int in_type, int out_type, int batch, int M, int N, int K,
+                        const void* A, int64_t a_batch_stride, int64_t a_row_stride, int64_t a_col_stride,
+                        const void* B, int64_t b_batch_stride, int64_t b_row_stride, int64_t b_col_stride,
+                        void* C, int64_t c_batch_stride, int64_t c_row_stride, int64_t c_col_stride,
+                        int prologue, double prologue_arg, int epilogue, double epilogue_arg,
+                        int variant, int k_splits, void* stream);
+int acc950_gemm_batched_host(int in_type, int out_type, int batch, int M, int N, int K,
+                             const void* A, int64_t a_batch_stride, int64_t a_row_stride, int64_t a_col_stride,
+                             const void* B, int64_t b_batch_stride, int64_t b_row_stride, int64_t b_col_stride,
+                             void* C, int64_t c_batch_stride, int64_t c_row_stride, int64_t c_col_stride,
+                             int prologue, double prologue_arg, int epilogue, double epilogue_arg);
+
+/*
  * Same computation on HOST pointers, synchronous: copies A, B (and C when it is
  * accumulated into) to the device, runs the kernel, copies C back.  This is the
  * calling convention of a HAT_DYNAMIC package function `void f(T* A, T* B, T* C)` as

@@ -421,6 +421,36 @@ def test_benchmark_configurations_at_full_size(cfg):
     assert (got[rows] == 0).any() and (got[rows] > 0).any()
 
 
+@pytest.mark.parametrize("case", [("f16", "f32", 3, 1280, 768, 1024, -1), ("bf16", "bf16", 8, 256, 384, 128, -1), ("i8", "i32", 4, 256, 256, 512, -1),
+                                  ("f32", "f32", 32, 128, 128, 128, -1), ("f16", "f16", 5, 100, 72, 40, -1), ("f16", "f16", 6, 8, 1088, 512, -1),
+                                  ("f16", "f16", 3, 8, 1088, 512, 100), ("bf16", "f32", 2, 5, 1000, 998, -1), ("f16", "f32", 1, 64, 64, 64, -1)])
+def test_batched_gemm(case):
+    """C[b] = relu(A[b] @ B[b]) in one launch: the reference's batch matmul nest
+    (mfma_tests.py:435-549; shapes 3 x 1280x768x1024, 8 x ..., 32 x 128^3, 1 x 64^3 from :2519-2549) on
+    every kernel family; then with one B shared by the batch (batch stride 0) and accumulation into C."""
+    import accera_amd as acc
+    import torch
+    in_type, out_type, batch, M, N, K, variant = case
+    rng = np.random.default_rng(batch * 1000 + M)
+    A = np.stack([make_input(rng, (M, K), in_type, "normal") for _ in range(batch)])
+    B = np.stack([make_input(rng, (K, N), in_type, "normal") for _ in range(batch)])
+    C0 = np.stack([(make_input(rng, (M, N), "i8").astype(np.int32) if out_type == "i32" else make_input(rng, (M, N), out_type)) for _ in range(batch)])
+    up = lambda x, t: torch.stack([to_device(m, t) for m in x])
+    dA, dB, dC = up(A, in_type), up(B, in_type), up(C0, out_type)
+    acc.gemm_relu(dA, dB, dC, variant=variant, k_splits=3 if variant >= 100 else 0)
+    torch.cuda.synchronize()
+    got = [to_host(dC[b], out_type) for b in range(batch)]
+    for b in range(batch):
+        assert_matches(got[b], ora.gemm_relu_exact(A[b], B[b], None, in_type, out_type), out_type, K)
+    # shared B (2-D) and accumulate
+    dC = up(C0, out_type)
+    acc.gemm_relu(dA, dB[0], dC, prologue=acc.PROLOGUE_NONE, epilogue=acc.EPILOGUE_NONE, variant=variant)
+    torch.cuda.synchronize()
+    for b in range(batch):
+        want = ora.gemm_relu_exact(A[b], B[0], C0[b], in_type, out_type, ora.PRO_NONE, ora.EPI_NONE)
+        assert_matches(to_host(dC[b], out_type), want, out_type, K)
+
+
 def test_sweep_tool_checks_and_times_every_variant():
     """accera_amd.tune on two small rows (one with alpha / beta, one transposed): every variant the
     library accepts must pass the NumPy check (rtol 1e-2 as accera_gemm.py:632)."""
