@@ -240,8 +240,8 @@ class Array:
         DEFERRED = 2
 
     def __init__(self, role, element_type=ScalarType.float32, layout=None, shape=None, name="", **_):
-        if shape is None or len(shape) != 2:
-            raise NotImplementedError("this build handles 2-D arrays (matrices) only")
+        if shape is None or len(shape) not in (2, 3):
+            raise NotImplementedError("this build handles matrices and batches of matrices (2-D / 3-D arrays) only")
         self.role = role
         self.element_type = element_type
         self.layout = layout or Array.Layout.FIRST_MAJOR
@@ -250,8 +250,15 @@ class Array:
 
     @property
     def strides(self):
-        r, c = self.shape
-        return (c, 1) if self.layout == Array.Layout.FIRST_MAJOR else (1, r)
+        """Element strides: FIRST_MAJOR has the last dimension contiguous, LAST_MAJOR the first
+        (/root/reference/accera/python/accera/lang/Layout.py:36-58)."""
+        dims = self.shape if self.layout == Array.Layout.FIRST_MAJOR else self.shape[::-1]
+        out, step = [], 1
+        for d in reversed(dims):
+            out.append(step)
+            step *= d
+        out = out[::-1]
+        return tuple(out if self.layout == Array.Layout.FIRST_MAJOR else out[::-1])
 
     def __getitem__(self, idx):
         return _Ref(self, idx)
@@ -378,8 +385,9 @@ class Plan:
 # ---- pattern match to the GEMM (+ReLU) hot path -------------------------------------------------
 
 class _GemmSpec:
-    def __init__(self, A, B, C, M, N, K, prologue, epilogue, prologue_arg=0.0, epilogue_arg=0.0):
+    def __init__(self, A, B, C, M, N, K, prologue, epilogue, prologue_arg=0.0, epilogue_arg=0.0, batch=None):
         self.A, self.B, self.C, self.M, self.N, self.K = A, B, C, M, N, K
+        self.batch = batch  # None: plain GEMM; n: C[b,i,j] += A[b,i,k] * B[b,k,j] for b < n
         self.prologue, self.epilogue = prologue, epilogue
         self.prologue_arg, self.epilogue_arg = float(prologue_arg), float(epilogue_arg)
 
@@ -389,45 +397,49 @@ def _match(source):
     sched = plan.schedule if plan else (source if isinstance(source, Schedule) else source.create_schedule())
     nests = sched.nests
     unsupported = NotImplementedError(
-        "this build compiles exactly one pattern: C[i,j] += A[i,k] * B[k,j], optionally fused with C[i,j] = max(C[i,j], 0)")
-    if len(nests) not in (1, 2) or len(nests[0].shape) != 3 or len(nests[0].statements) != 1:
+        "this build compiles exactly one pattern: C[i,j] += A[i,k] * B[k,j] (or its batched form C[b,i,j] += A[b,i,k] * B[b,k,j]), "
+        "optionally fused with C[i,j] = max(C[i,j], 0)")
+    if len(nests) not in (1, 2) or len(nests[0].shape) not in (3, 4) or len(nests[0].statements) != 1:
         raise unsupported
     mm = nests[0]
-    i, j, k = mm.indices
+    batched = len(mm.shape) == 4
+    bidx = mm.indices[:1] if batched else ()
+    i, j, k = mm.indices[-3:]
     dst, val = mm.statements[0]
     val = _strip_cast(val)
     if not (isinstance(val, _Bin) and val.op == "add"):
         raise unsupported
     acc_ref, prod = _strip_cast(val.a), _strip_cast(val.b)
-    if not (isinstance(acc_ref, _Ref) and acc_ref.array is dst.array and acc_ref.idx == (i, j) and dst.idx == (i, j)):
+    if not (isinstance(acc_ref, _Ref) and acc_ref.array is dst.array and acc_ref.idx == (*bidx, i, j) and dst.idx == (*bidx, i, j)):
         raise unsupported
     if not (isinstance(prod, _Bin) and prod.op == "mul"):
         raise unsupported
     a, b = _strip_cast(prod.a), _strip_cast(prod.b)
     if not (isinstance(a, _Ref) and isinstance(b, _Ref)):
         raise unsupported
-    if a.idx == (k, j) and b.idx == (i, k):
+    if a.idx == (*bidx, k, j) and b.idx == (*bidx, i, k):
         a, b = b, a
-    if a.idx != (i, k) or b.idx != (k, j):
+    if a.idx != (*bidx, i, k) or b.idx != (*bidx, k, j):
         raise unsupported
-    M, N, K = mm.shape
+    M, N, K = mm.shape[-3:]
+    nb = (mm.shape[0],) if batched else ()
     A, B, C = a.array, b.array, dst.array
-    if A.shape != (M, K) or B.shape != (K, N) or C.shape != (M, N):
+    if A.shape != (*nb, M, K) or B.shape != (*nb, K, N) or C.shape != (*nb, M, N):
         raise ValueError(f"array shapes {A.shape}, {B.shape}, {C.shape} do not match the nest {mm.shape}")
     epilogue = _lib.EPILOGUE_NONE
     if len(nests) == 2:
         relu = nests[1]
-        if not (sched.fused and sched.partial == 2 and relu.shape == (M, N) and len(relu.statements) == 1):
+        if not (sched.fused and sched.partial == len(nb) + 2 and relu.shape == (*nb, M, N) and len(relu.statements) == 1):
             raise unsupported
-        i2, j2 = relu.indices
+        ridx = tuple(relu.indices)
         rdst, rval = relu.statements[0]
         rval = _strip_cast(rval)
-        ok = (rdst.array is C and rdst.idx == (i2, j2) and isinstance(rval, _Bin) and rval.op == "max")
+        ok = (rdst.array is C and rdst.idx == ridx and isinstance(rval, _Bin) and rval.op == "max")
         if ok:
             x, z = _strip_cast(rval.a), _strip_cast(rval.b)
             if isinstance(x, _Const):
                 x, z = z, x
-            ok = isinstance(x, _Ref) and x.array is C and x.idx == (i2, j2) and isinstance(z, _Const) and z.v == 0
+            ok = isinstance(x, _Ref) and x.array is C and x.idx == ridx and isinstance(z, _Const) and z.v == 0
         if not ok:
             raise unsupported
         epilogue = _lib.EPILOGUE_RELU
@@ -447,7 +459,7 @@ def _match(source):
             epilogue, epilogue_arg = _lib.EPILOGUE_SCALE, plan.epilogue_arg
         elif plan.epilogue_op == MMAFragmentOp.SET:
             epilogue, epilogue_arg = _lib.EPILOGUE_SET, plan.epilogue_arg
-    return _GemmSpec(A, B, C, M, N, K, prologue, epilogue, prologue_arg, epilogue_arg)
+    return _GemmSpec(A, B, C, M, N, K, prologue, epilogue, prologue_arg, epilogue_arg, batch=mm.shape[0] if batched else None)
 
 
 # ---- package -------------------------------------------------------------------------------------
@@ -498,16 +510,19 @@ class Package:
             s = f["spec"]
             order = {id(a): n for a, n in zip(f["args"], ("a0", "a1", "a2"))}
             pa, pb, pc = order[id(s.A)], order[id(s.B)], order[id(s.C)]
-            call_args = (f"{s.A.element_type.lib_id}, {s.C.element_type.lib_id}, {s.M}, {s.N}, {s.K}, "
-                         f"{pa}, {s.A.strides[0]}, {s.A.strides[1]}, {pb}, {s.B.strides[0]}, {s.B.strides[1]}, "
-                         f"{pc}, {s.C.strides[0]}, {s.C.strides[1]}, {s.prologue}, {s.prologue_arg!r}, {s.epilogue}, {s.epilogue_arg!r}")
+            nb = s.batch if s.batch is not None else 1
+            st = lambda arr: ((0,) + tuple(arr.strides))[-3:] if len(arr.strides) == 2 else tuple(arr.strides)
+            (abs_, ars, acs), (bbs, brs, bcs), (cbs, crs, ccs) = st(s.A), st(s.B), st(s.C)
+            call_args = (f"{s.A.element_type.lib_id}, {s.C.element_type.lib_id}, {nb}, {s.M}, {s.N}, {s.K}, "
+                         f"{pa}, {abs_}, {ars}, {acs}, {pb}, {bbs}, {brs}, {bcs}, {pc}, {cbs}, {crs}, {ccs}, "
+                         f"{s.prologue}, {s.prologue_arg!r}, {s.epilogue}, {s.epilogue_arg!r}")
             lines += [
                 f"void {f['name']}(void* a0, void* a1, void* a2)", "{",
-                f"    if (acc950_gemm_ops_host({call_args}) != ACC950_OK)",
+                f"    if (acc950_gemm_batched_host({call_args}) != ACC950_OK)",
                 f"        fprintf(stderr, \"{f['name']}: %s\\n\", acc950_last_error());", "}",
                 "/* same function on device pointers, asynchronous on `stream` (hipStream_t or NULL) */",
                 f"int {f['name']}__device(void* a0, void* a1, void* a2, void* stream)", "{",
-                f"    return acc950_gemm_ops({call_args}, ACC950_VARIANT_AUTO, 0, stream);", "}", ""]
+                f"    return acc950_gemm_batched({call_args}, ACC950_VARIANT_AUTO, 0, stream);", "}", ""]
         return "\n".join(lines)
 
     def build(self, name, format=None, mode=None, platform=None, tolerance=1e-5, output_dir=None, **_):
@@ -539,7 +554,9 @@ class Package:
                 arguments.append(_hat.Argument(name=a.name, declared_type=f"{ct}*", element_type=ct, usage=a.role.value,
                                                shape=list(a.shape), affine_map=list(a.strides)))
             grid, block, lds, variant = _lib.launch_geometry(s.A.element_type.lib_id, s.C.element_type.lib_id, s.M, s.N, s.K,
-                                                             s.A.strides, s.B.strides, s.C.strides)
+                                                             s.A.strides[-2:], s.B.strides[-2:], s.C.strides[-2:])
+            if s.batch is not None:
+                grid = grid[:2] + [s.batch]  # the batch index is bound to grid.z
             aux = {"accera": {"base_name": f["base_name"], "parameters": {k: str(v) for k, v in f["parameters"].items()}},
                    # structural counterpart of the device-function record of the reference's GPU packages
                    # (Package.py:714-743): launch geometry of the kernel behind this entry point

@@ -217,6 +217,67 @@ def test_tensorized_plan_package_on_numpy_arrays(tmp_path, in_t, out_t, shape, b
     assert_matches(C, ora.gemm_relu_exact(A, B, None, it, ot), ot, K)
 
 
+def _batched_package(tmp, batch, M, N, K, in_t=acc.ScalarType.float16, out_t=acc.ScalarType.float32, alpha=None):
+    """The reference's batch matmul nest (mfma_tests.py:435-470) fused with ReLU, or with an alpha epilogue."""
+    A = acc.Array(role=acc.Role.INPUT, element_type=in_t, shape=(batch, M, K))
+    B = acc.Array(role=acc.Role.INPUT, element_type=in_t, shape=(batch, K, N))
+    C = acc.Array(role=acc.Role.INPUT_OUTPUT, element_type=out_t, shape=(batch, M, N))
+    nest = acc.Nest(shape=(batch, M, N, K))
+    b, i, j, k = nest.get_indices()
+
+    @nest.iteration_logic
+    def _():
+        C[b, i, j] += A[b, i, k] * B[b, k, j]
+
+    target = acc.Target(acc.Target.Model.AMD_MI355X)
+    if alpha is None:
+        relu = acc.Nest(shape=(batch, M, N))
+        b2, i2, j2 = relu.get_indices()
+
+        @relu.iteration_logic
+        def _():
+            C[b2, i2, j2] = acc.max(C[b2, i2, j2], 0.0)
+
+        plan = acc.fuse(nest.create_schedule(), relu.create_schedule(), partial=3).create_plan(target)
+        plan.tensorize(indices=plan.schedule.get_indices()[1:4], mma_shape=acc.MMAShape.M32xN32xK16_B1,
+                       prologue_op=acc.MMAFragmentOp.SET, prologue_arg=0)
+    else:
+        plan = nest.create_schedule().create_plan(target)
+        plan.tensorize(indices=(i, j, k), mma_shape=acc.MMAShape.M32xN32xK16_B1, prologue_op=acc.MMAFragmentOp.SCALE, prologue_arg=0.5,
+                       epilogue_op=acc.MMAFragmentOp.SCALE, epilogue_arg=alpha)
+    package = acc.Package()
+    name = package.add(plan, args=(A, B, C), base_name="batch_matmul")
+    return package.build(name="batch_pkg", format=acc.Package.Format.HAT_DYNAMIC, output_dir=str(tmp)), name
+
+
+def test_batched_nest_is_recorded_with_three_dimensional_arguments(tmp_path):
+    files, name = _batched_package(tmp_path, 3, 128, 256, 64)
+    pkg = hat.parse(files[0])
+    fn = pkg["functions"][name]
+    assert [a["shape"] for a in fn["arguments"]] == [[3, 128, 64], [3, 64, 256], [3, 128, 256]]
+    assert [a["affine_map"] for a in fn["arguments"]] == [[8192, 64, 1], [16384, 256, 1], [32768, 256, 1]]
+    assert fn["auxiliary"]["accera_mi355x"]["launch_parameters"][2] == 3  # batch index on grid.z
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("alpha", [None, 2.0])
+def test_batched_package_on_numpy_arrays(tmp_path, alpha):
+    batch, M, N, K = 3, 256, 384, 128
+    files, name = _batched_package(tmp_path, batch, M, N, K, alpha=alpha)
+    _, functions = hat.load(files[0])
+    from tests.util import assert_matches, make_input
+    rng = np.random.default_rng(9)
+    A = np.stack([make_input(rng, (M, K), "f16") for _ in range(batch)])
+    B = np.stack([make_input(rng, (K, N), "f16") for _ in range(batch)])
+    C0 = rng.standard_normal((batch, M, N)).astype(np.float32)
+    C = C0.copy()
+    functions[name](A, B, C)
+    for b in range(batch):
+        want = (ora.gemm_relu_exact(A[b], B[b], None, "f16", "f32") if alpha is None else
+                ora.gemm_relu_exact(A[b], B[b], C0[b], "f16", "f32", ora.PRO_SCALE, ora.EPI_SCALE, prologue_arg=0.5, epilogue_arg=alpha))
+        assert_matches(C[b], want, "f32", K)
+
+
 @pytest.mark.gpu
 def test_run_benchmark_reports_hatlib_style_rows(tmp_path):
     hat_path, _ = _quickstart_package(tmp_path, 256, 256, 256)
