@@ -20,7 +20,7 @@ VARIANT_AUTO, VARIANT_SKINNY_BASE, VARIANT_GENERIC, VARIANT_F32_MFMA = -1, 100, 
 
 EXPORTS = [
     "acc950_init", "acc950_gemm_relu", "acc950_gemm_relu_ex", "acc950_gemm_relu_host", "acc950_gemm_ops", "acc950_gemm_ops_host",
-    "acc950_gemm_batched", "acc950_gemm_batched_host",
+    "acc950_gemm_batched", "acc950_gemm_batched_host", "acc950_bind", "acc950_launch", "acc950_unbind",
     "acc950_launch_geometry", "acc950_num_variants", "acc950_num_skinny_variants",
     "acc950_variant_name", "acc950_last_error", "acc950_mfma_ceiling", "acc950_mfma_phase_probe", "acc950_copy_probe", "acc950_stream_read_probe",
 ]
@@ -57,6 +57,9 @@ def lib():
     bmat = [vp, i64, i64, i64]
     L.acc950_gemm_batched.argtypes = [ci, ci, ci, ci, ci, ci] + bmat * 3 + [ci, cd, ci, cd, ci, ci, vp]
     L.acc950_gemm_batched_host.argtypes = [ci, ci, ci, ci, ci, ci] + bmat * 3 + [ci, cd, ci, cd]
+    L.acc950_bind.argtypes = [ci, ci, ci, ci, ci, ci] + bmat * 3 + [ci, cd, ci, cd, ci, ci, vp, ctypes.POINTER(ci)]
+    L.acc950_launch.argtypes = [ci]
+    L.acc950_unbind.argtypes = [ci]
     L.acc950_launch_geometry.argtypes = [ci, ci, ci, ci, ci] + [i64] * 6 + [ci, ci, ctypes.POINTER(cu), ctypes.POINTER(cu),
                                                                            ctypes.POINTER(cu), ctypes.POINTER(ci)]
     L.acc950_variant_name.argtypes = [ci, ctypes.c_char_p, ctypes.c_size_t]

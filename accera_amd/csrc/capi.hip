@@ -406,6 +406,59 @@ int acc950_gemm_batched(int in_type, int out_type, int batch, int M, int N, int 
     return run(pb, c, (hipStream_t)stream, nullptr, false);
 }
 
+// ---- bound calls: validate and choose once, launch many times -------------------------
+struct BoundCall {
+    Problem pb;
+    Choice choice;
+    hipStream_t stream;
+    bool live;
+};
+std::mutex g_bound_mutex;
+std::vector<BoundCall> g_bound;
+
+int acc950_bind(int in_type, int out_type, int batch, int M, int N, int K,
+                const void* A, int64_t a_bs, int64_t a_rs, int64_t a_cs, const void* B, int64_t b_bs, int64_t b_rs, int64_t b_cs,
+                void* C, int64_t c_bs, int64_t c_rs, int64_t c_cs, int prologue, double prologue_arg, int epilogue,
+                double epilogue_arg, int variant, int k_splits, void* stream, int* handle)
+{
+    if (!handle) return fail(ACC950_INVALID_ARGUMENT, "null handle pointer");
+    BoundCall bc{};
+    Batch bt;
+    bt.count = batch; bt.a_bs = a_bs; bt.b_bs = b_bs; bt.c_bs = c_bs;
+    int rc = make_problem(in_type, out_type, M, N, K, A, a_rs, a_cs, B, b_rs, b_cs, C, c_rs, c_cs, prologue, epilogue, true, &bc.pb,
+                          prologue_arg, epilogue_arg, bt);
+    if (rc) return rc;
+    rc = choose(bc.pb, variant, k_splits, &bc.choice);
+    if (rc) return rc;
+    bc.stream = (hipStream_t)stream;
+    bc.live = true;
+    std::lock_guard<std::mutex> lock(g_bound_mutex);
+    for (size_t i = 0; i < g_bound.size(); ++i)
+        if (!g_bound[i].live) { g_bound[i] = bc; *handle = (int)i; return ACC950_OK; }
+    g_bound.push_back(bc);
+    *handle = (int)g_bound.size() - 1;
+    return ACC950_OK;
+}
+
+int acc950_launch(int handle)
+{
+    BoundCall bc;
+    {
+        std::lock_guard<std::mutex> lock(g_bound_mutex);
+        if (handle < 0 || (size_t)handle >= g_bound.size() || !g_bound[handle].live) return fail(ACC950_INVALID_ARGUMENT, "unknown call handle");
+        bc = g_bound[handle];
+    }
+    return run(bc.pb, bc.choice, bc.stream, nullptr, false);
+}
+
+int acc950_unbind(int handle)
+{
+    std::lock_guard<std::mutex> lock(g_bound_mutex);
+    if (handle < 0 || (size_t)handle >= g_bound.size() || !g_bound[handle].live) return fail(ACC950_INVALID_ARGUMENT, "unknown call handle");
+    g_bound[handle].live = false;
+    return ACC950_OK;
+}
+
 int acc950_gemm_relu_ex(int in_type, int out_type, int M, int N, int K,
                         const void* A, int64_t a_rs, int64_t a_cs, const void* B, int64_t b_rs, int64_t b_cs,
                         void* C, int64_t c_rs, int64_t c_cs, int prologue, int epilogue, int variant, int k_splits,

@@ -44,39 +44,25 @@ __global__ void __launch_bounds__(256) gemm_f32_kernel(GemmArgs p)
     const float* A = (const float*)p.A;
     const float* B = (const float*)p.B;
 
-    // Sets of U k chunks (512 k per workgroup pass), double-buffered: all loads of a set are
-    // issued at once, the loads of the next set are queued behind them before the 4*U MFMAs
-    // of the current one run.  The quick-start size is one set per wave; its time is the
-    // L2 -> L1 fill of the 128 KB every workgroup needs (measured: 3.7 us for the loads, 2.2 us
-    // for the MFMAs, 1.7 us for the stores to be acknowledged; interleaving loads and MFMAs
-    // chunk by chunk was measured slower, fewer loads stay in flight).
+    // Sets of U k chunks: load a set, run its 4*U MFMAs.  The quick-start size is bound by the
+    // L2 -> L1 fill of the 128 KB every workgroup needs (clock stamps: 3.7 us for the loads,
+    // 2.2 us of MFMAs, 1.7 us until the stores are acknowledged).  Deeper prefetch (double-buffered
+    // sets of 8 or 16 chunks, or chunk-by-chunk interleaving) was measured 10-15 % slower: with
+    // every workgroup's loads queued at once the memory pipeline only gets slower.
     f32x16 acc = {};
-    constexpr int U = 16;
-    float a[2][U][4], b[2][U][4];
-    auto load_set = [&](int buf, int k0) {
+    constexpr int U = 4;
+    for (int k0 = wave * 8; k0 < p.K; k0 += 32 * U) {
+        float a[U][4], b[U][4];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             const int k = k0 + u * 32 + kh * 4;
-            load_frag<A_KC>(a[buf][u], A, p.a_rs, p.a_cs, row, p.M, k, p.K);
-            load_frag<B_KC>(b[buf][u], B, p.b_cs, p.b_rs, col, p.N, k, p.K);
+            load_frag<A_KC>(a[u], A, p.a_rs, p.a_cs, row, p.M, k, p.K);
+            load_frag<B_KC>(b[u], B, p.b_cs, p.b_rs, col, p.N, k, p.K);
         }
-    };
-    auto mma_set = [&](int buf) {
 #pragma unroll
         for (int u = 0; u < U; ++u)
 #pragma unroll
-            for (int j = 0; j < 4; ++j) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[buf][u][j], b[buf][u][j], acc, 0, 0, 0);
-    };
-    int k0 = wave * 8;
-    if (k0 < p.K) load_set(0, k0);
-    for (; k0 < p.K; k0 += 64 * U) {
-        // sets alternate between the two buffers; out-of-range chunks load zeros
-        if (k0 + 32 * U < p.K) load_set(1, k0 + 32 * U);
-        mma_set(0);
-        if (k0 + 32 * U < p.K) {
-            if (k0 + 64 * U < p.K) load_set(0, k0 + 64 * U);
-            mma_set(1);
-        }
+            for (int j = 0; j < 4; ++j) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u][j], b[u][j], acc, 0, 0, 0);
     }
 
     if (wave > 0) {

@@ -560,9 +560,11 @@ __global__ void __launch_bounds__(Cfg::NT, Cfg::WGS_PER_CU) gemm_mfma_kernel(Gem
 #pragma unroll
         for (int i = 0; i < TM; ++i)
 #pragma unroll
-            for (int j = 0; j < TN; ++j)
+            for (int j = 0; j < TN; ++j) {
 #pragma unroll
                 for (int r = 0; r < 16; ++r) acc[i][j][r] = fn(acc[i][j][r]);
+                __builtin_amdgcn_sched_barrier(0); // block by block, in place
+            }
     };
 
     auto general_ops = [&]() {
@@ -576,19 +578,23 @@ __global__ void __launch_bounds__(Cfg::NT, Cfg::WGS_PER_CU) gemm_mfma_kernel(Gem
         else for_each_element(uint16_t{}, [&](uint16_t* c, float v) { return v + bf16_bits_to_float(*c) * c_mul; });
     }
 
-    // ---- pass B (wave-uniform switches; ReLU after a SET-0 prologue is the fused hot path: one max per element)
-    if (p.prologue == PRO_SET && p.prologue_arg != 0.f) {
-        const scalar_t set_value = (scalar_t)p.prologue_arg;
-        for_each_acc([&](scalar_t v) { return wrap_add(v, set_value); });
-    }
-    {
+    // ---- pass B (ReLU after a SET-0 prologue is the fused hot path: one max per element; every other
+    // combination shares one copy with wave-uniform selects)
+    if (p.epilogue == EPI_RELU && !(p.prologue == PRO_SET && p.prologue_arg != 0.f)) {
+        for_each_acc([&](scalar_t v) { return v > scalar_t(0) ? v : scalar_t(0); });
+    } else if (p.epilogue != EPI_NONE || (p.prologue == PRO_SET && p.prologue_arg != 0.f)) {
+        const scalar_t set_value = p.prologue == PRO_SET ? (scalar_t)p.prologue_arg : scalar_t(0);
         const scalar_t epi_arg = (scalar_t)p.epilogue_arg;
-        if (p.epilogue == EPI_RELU) for_each_acc([&](scalar_t v) { return v > scalar_t(0) ? v : scalar_t(0); });
-        else if (p.epilogue == EPI_RELU_NOCOND) for_each_acc([&](scalar_t v) { return v * (v > scalar_t(0) ? scalar_t(1) : scalar_t(0)); });
-        else if (p.epilogue == EPI_SCALE) for_each_acc([&](scalar_t v) { return wrap_mul(v, epi_arg); });
-        else if (p.epilogue == EPI_SET) for_each_acc([&](scalar_t) { return epi_arg; });
+        const bool is_relu = p.epilogue == EPI_RELU, is_nocond = p.epilogue == EPI_RELU_NOCOND, is_scale = p.epilogue == EPI_SCALE,
+                   is_set = p.epilogue == EPI_SET;
+        for_each_acc([&](scalar_t v) {
+            v = wrap_add(v, set_value);
+            const scalar_t r = v > scalar_t(0) ? v : scalar_t(0);
+            const scalar_t n = v * (v > scalar_t(0) ? scalar_t(1) : scalar_t(0));
+            const scalar_t m = wrap_mul(v, epi_arg);
+            return is_relu ? r : (is_nocond ? n : (is_scale ? m : (is_set ? epi_arg : v)));
+        });
     }
-
     };
 
     // ---- pass C
@@ -660,6 +666,7 @@ __global__ void __launch_bounds__(Cfg::NT, Cfg::WGS_PER_CU) gemm_mfma_kernel(Gem
     // One straight line through the passes: splitting the fused matmul + ReLU case off into a
     // branch of its own makes the register allocator spill hundreds of accumulators.
     general_ops();
+    __builtin_amdgcn_sched_barrier(0);
     store_all(std::false_type{});
     if constexpr (Cfg::TIMED) {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // stores acknowledged

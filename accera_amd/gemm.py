@@ -1,5 +1,7 @@
 """Device-tensor front end of the C ABI: torch supplies device memory and streams,
 every computation happens in the HIP kernels of libaccera_mi355x.so."""
+import ctypes
+
 import torch
 
 from . import _lib
@@ -50,14 +52,23 @@ class GemmCall:
         if stream is None:
             stream = torch.cuda.current_stream(C.device).cuda_stream
         self.tensors = (A, B, C)
-        self._fn = _lib.lib().acc950_gemm_batched
-        self._args = (*problem, prologue, float(prologue_arg), epilogue, float(epilogue_arg), variant, k_splits, stream)
+        L = _lib.lib()
+        handle = ctypes.c_int(-1)
+        _lib.check(L.acc950_bind(*problem, prologue, float(prologue_arg), epilogue, float(epilogue_arg), variant, k_splits, stream,
+                                 ctypes.byref(handle)))
+        self._handle = handle.value
+        self._launch, self._unbind = L.acc950_launch, L.acc950_unbind
 
     def __call__(self):
-        rc = self._fn(*self._args)
+        rc = self._launch(self._handle)
         if rc:
             _lib.check(rc)
         return self.tensors[2]
+
+    def __del__(self):
+        if getattr(self, "_handle", -1) >= 0:
+            self._unbind(self._handle)
+            self._handle = -1
 
 
 def gemm_relu(A, B, C, prologue=_lib.PROLOGUE_SET0, epilogue=_lib.EPILOGUE_RELU, variant=_lib.VARIANT_AUTO,

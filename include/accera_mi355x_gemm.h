@@ -136,6 +136,25 @@ int acc950_gemm_batched_host(int in_type, int out_type, int batch, int M, int N,
                              int prologue, double prologue_arg, int epilogue, double epilogue_arg);
 
 /*
+ * Bound call: validates the problem and chooses the kernel once, then acc950_launch(handle)
+ * only launches (asynchronously on the stream given at bind time).  This is what a function
+ * of a package is to its caller, a fixed kernel for fixed shapes, with the arrays fixed too;
+ * it keeps per-launch host time at a few hundred nanoseconds, which matters for the
+ * quick-start sized problems whose kernels run for a few microseconds
+ * (hatlib times packages by calling the same function on the same arrays in a loop,
+ * /root/reference/tools/benchmarkers/accera_gemm.py:640-648).  Arguments as acc950_gemm_batched.
+ * The caller keeps A, B, C alive until acc950_unbind.
+ */
+int acc950_bind(int in_type, int out_type, int batch, int M, int N, int K,
+                const void* A, int64_t a_batch_stride, int64_t a_row_stride, int64_t a_col_stride,
+                const void* B, int64_t b_batch_stride, int64_t b_row_stride, int64_t b_col_stride,
+                void* C, int64_t c_batch_stride, int64_t c_row_stride, int64_t c_col_stride,
+                int prologue, double prologue_arg, int epilogue, double epilogue_arg,
+                int variant, int k_splits, void* stream, int* handle);
+int acc950_launch(int handle);
+int acc950_unbind(int handle);
+
+/*
  * Same computation on HOST pointers, synchronous: copies A, B (and C when it is
  * accumulated into) to the device, runs the kernel, copies C back.  This is the
  * calling convention of a HAT_DYNAMIC package function `void f(T* A, T* B, T* C)` as

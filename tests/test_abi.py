@@ -90,3 +90,25 @@ def test_sweep_tool_lists_the_variants_that_take_a_problem():
     with open(os.path.join(os.path.dirname(tune.__file__), "shapes", "transformer_gemm.csv")) as f:
         rows = list(csv.DictReader(f))
     assert len(rows) >= 10 and {"m", "n", "k", "transA", "transB", "alpha", "beta"} <= set(rows[0])
+
+
+def test_bound_call_handles_without_launching():
+    """acc950_bind validates and chooses once; handles are reused after acc950_unbind; unknown handles
+    are reported.  (No launch here: there is no GPU on the CPU test tier.)"""
+    import ctypes
+    L = _lib.lib()
+    h = ctypes.c_int(-1)
+    args = (_lib.F16, _lib.F32, 1, 256, 256, 256, 0x10000, 0, 256, 1, 0x20000, 0, 256, 1, 0x30000, 0, 256, 1,
+            _lib.PROLOGUE_SET0, 0.0, _lib.EPILOGUE_RELU, 0.0, _lib.VARIANT_AUTO, 0, None)
+    assert L.acc950_bind(*args, ctypes.byref(h)) == _lib.OK and h.value >= 0
+    first = h.value
+    assert L.acc950_unbind(first) == _lib.OK
+    assert L.acc950_unbind(first) == _lib.INVALID_ARGUMENT and L.acc950_launch(first) == _lib.INVALID_ARGUMENT
+    assert L.acc950_bind(*args, ctypes.byref(h)) == _lib.OK and h.value == first   # slot reused
+    assert L.acc950_unbind(first) == _lib.OK
+    bad = list(args)
+    bad[6] = 0   # null A
+    assert L.acc950_bind(*bad, ctypes.byref(h)) == _lib.INVALID_ARGUMENT
+    bad = list(args)
+    bad[22] = 57 + 1000   # unknown variant
+    assert L.acc950_bind(*bad, ctypes.byref(h)) == _lib.INVALID_ARGUMENT
