@@ -119,7 +119,9 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_skinny_mfma_kernel(SkinnyArgs
     }
     const int am = lane >> 1;
     const bool a_active = am < p.M;
-    const unsigned aoff = (unsigned)((int64_t)(a_active ? am : 0) * p.a_rs * 2 + (lane & 1) * 16);
+    // the two 16-byte halves of a row swap places in rows 8-15 and 24-31, so that the 16 lanes of one
+    // read phase (32-byte row pitch) spread over all banks
+    const unsigned aoff = (unsigned)((int64_t)(a_active ? am : 0) * p.a_rs * 2 + ((lane & 1) ^ ((am >> 3) & 1)) * 16);
 
     auto issue = [&](int it, int slot) { // it < my_steps
         const int s = s_begin + wave + it * WAVES;
@@ -148,7 +150,7 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_skinny_mfma_kernel(SkinnyArgs
             const int chunk = j * 4 + g * 2 + ((i16 & 3) >> 1);
             roff[j][q] = (unsigned)(k * RB + ((chunk ^ ((k & 3) << 1)) << 4) + (i16 & 1) * 8);
         }
-    const unsigned aread = B_BYTES + (lane & 31) * 32 + h * 16;
+    const unsigned aread = B_BYTES + (lane & 31) * 32 + (h ^ (((lane & 31) >> 3) & 1)) * 16;
 
     f32x16 acc[JB];
 #pragma unroll
