@@ -56,7 +56,7 @@ def lib():
     L.acc950_gemm_ops_host.argtypes = [ci, ci, ci, ci, ci] + mat * 3 + [ci, cd, ci, cd]
     bmat = [vp, i64, i64, i64]
     L.acc950_gemm_batched.argtypes = [ci, ci, ci, ci, ci, ci] + bmat * 3 + [ci, cd, ci, cd, ci, ci, vp]
-    L.acc950_gemm_batched_host.argtypes = [ci, ci, ci, ci, ci, ci] + bmat * 3 + [ci, cd, ci, cd]
+    L.acc950_gemm_batched_host.argtypes = [ci, ci, ci, ci, ci, ci] + bmat * 3 + [ci, cd, ci, cd, ci, ci]
     L.acc950_bind.argtypes = [ci, ci, ci, ci, ci, ci] + bmat * 3 + [ci, cd, ci, cd, ci, ci, vp, ctypes.POINTER(ci)]
     L.acc950_launch.argtypes = [ci]
     L.acc950_unbind.argtypes = [ci]

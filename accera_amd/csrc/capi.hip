@@ -557,13 +557,13 @@ int acc950_gemm_ops_host(int in_type, int out_type, int M, int N, int K,
                          void* C, int64_t c_rs, int64_t c_cs, int prologue, double prologue_arg, int epilogue, double epilogue_arg)
 {
     return acc950_gemm_batched_host(in_type, out_type, 1, M, N, K, A, 0, a_rs, a_cs, B, 0, b_rs, b_cs, C, 0, c_rs, c_cs, prologue,
-                                    prologue_arg, epilogue, epilogue_arg);
+                                    prologue_arg, epilogue, epilogue_arg, ACC950_VARIANT_AUTO, 0);
 }
 
 int acc950_gemm_batched_host(int in_type, int out_type, int batch, int M, int N, int K,
                              const void* A, int64_t a_bs, int64_t a_rs, int64_t a_cs, const void* B, int64_t b_bs, int64_t b_rs,
                              int64_t b_cs, void* C, int64_t c_bs, int64_t c_rs, int64_t c_cs, int prologue, double prologue_arg,
-                             int epilogue, double epilogue_arg)
+                             int epilogue, double epilogue_arg, int variant, int k_splits)
 {
     Problem check;
     Batch bt;
@@ -591,7 +591,7 @@ int acc950_gemm_batched_host(int in_type, int out_type, int batch, int M, int N,
     if (prologue != PRO_SET || !c_dense)
         if ((e = hipMemcpy(g_dC.p, C, c_bytes, hipMemcpyHostToDevice)) != hipSuccess) return fail_hip(e, "copy C to device");
     rc = acc950_gemm_batched(in_type, out_type, batch, M, N, K, g_dA.p, a_bs, a_rs, a_cs, g_dB.p, b_bs, b_rs, b_cs, g_dC.p, c_bs, c_rs,
-                             c_cs, prologue, prologue_arg, epilogue, epilogue_arg, ACC950_VARIANT_AUTO, 0, nullptr);
+                             c_cs, prologue, prologue_arg, epilogue, epilogue_arg, variant, k_splits, nullptr);
     if (rc) return rc;
     if ((e = hipMemcpy(C, g_dC.p, c_bytes, hipMemcpyDeviceToHost)) != hipSuccess) return fail_hip(e, "copy C to host");
     return ACC950_OK;

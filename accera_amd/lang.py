@@ -390,6 +390,8 @@ class _GemmSpec:
         self.batch = batch  # None: plain GEMM; n: C[b,i,j] += A[b,i,k] * B[b,k,j] for b < n
         self.prologue, self.epilogue = prologue, epilogue
         self.prologue_arg, self.epilogue_arg = float(prologue_arg), float(epilogue_arg)
+        self.block_tile = None               # (bm, bn) when a GPU plan's outermost splits of i and j name one
+        self.variant = _lib.VARIANT_AUTO     # kernel instantiation picked from the block tile, else automatic
 
 
 def _match(source):
@@ -459,7 +461,37 @@ def _match(source):
             epilogue, epilogue_arg = _lib.EPILOGUE_SCALE, plan.epilogue_arg
         elif plan.epilogue_op == MMAFragmentOp.SET:
             epilogue, epilogue_arg = _lib.EPILOGUE_SET, plan.epilogue_arg
-    return _GemmSpec(A, B, C, M, N, K, prologue, epilogue, prologue_arg, epilogue_arg, batch=mm.shape[0] if batched else None)
+    spec = _GemmSpec(A, B, C, M, N, K, prologue, epilogue, prologue_arg, epilogue_arg, batch=mm.shape[0] if batched else None)
+    if plan and plan.target.category == Target.Category.GPU:
+        # The outermost split of i and of j is the block tile of a GPU plan (the reference binds the
+        # resulting outer indices to BLOCK_Y / BLOCK_X: lang/Plan.py:793-825, mfma_tests.py:89-97).  If
+        # the library has an MFMA instantiation with that tile which takes this problem, the package
+        # function is bound to it; otherwise the library chooses.
+        first = {}
+        for cmd in sched.commands:
+            if cmd[0] == "split" and cmd[1] in (i, j) and cmd[1] not in first:
+                first[cmd[1]] = int(cmd[2])
+        if i in first and j in first:
+            spec.block_tile = (first[i], first[j])
+            spec.variant = _variant_for_tile(spec, *spec.block_tile)
+    return spec
+
+
+def _variant_for_tile(spec, bm, bn):
+    """Best-ranked MFMA variant with block tile bm x bn that accepts the problem, else VARIANT_AUTO."""
+    best = _lib.VARIANT_AUTO
+    for v in range(_lib.num_variants()):
+        name = _lib.variant_name(v)
+        if f"mfma {bm}x{bn} " not in name:
+            continue
+        try:
+            _lib.launch_geometry(spec.A.element_type.lib_id, spec.C.element_type.lib_id, spec.M, spec.N, spec.K,
+                                 spec.A.strides[-2:], spec.B.strides[-2:], spec.C.strides[-2:], v, 0)
+        except _lib.Acc950Error:
+            continue
+        if best == _lib.VARIANT_AUTO or ("pingpong" in name and "pingpong" not in _lib.variant_name(best)):
+            best = v
+    return best
 
 
 # ---- package -------------------------------------------------------------------------------------
@@ -518,11 +550,11 @@ class Package:
                          f"{s.prologue}, {s.prologue_arg!r}, {s.epilogue}, {s.epilogue_arg!r}")
             lines += [
                 f"void {f['name']}(void* a0, void* a1, void* a2)", "{",
-                f"    if (acc950_gemm_batched_host({call_args}) != ACC950_OK)",
+                f"    if (acc950_gemm_batched_host({call_args}, {s.variant}, 0) != ACC950_OK)",
                 f"        fprintf(stderr, \"{f['name']}: %s\\n\", acc950_last_error());", "}",
                 "/* same function on device pointers, asynchronous on `stream` (hipStream_t or NULL) */",
                 f"int {f['name']}__device(void* a0, void* a1, void* a2, void* stream)", "{",
-                f"    return acc950_gemm_batched({call_args}, ACC950_VARIANT_AUTO, 0, stream);", "}", ""]
+                f"    return acc950_gemm_batched({call_args}, {s.variant}, 0, stream);", "}", ""]
         return "\n".join(lines)
 
     def build(self, name, format=None, mode=None, platform=None, tolerance=1e-5, output_dir=None, **_):
@@ -554,7 +586,7 @@ class Package:
                 arguments.append(_hat.Argument(name=a.name, declared_type=f"{ct}*", element_type=ct, usage=a.role.value,
                                                shape=list(a.shape), affine_map=list(a.strides)))
             grid, block, lds, variant = _lib.launch_geometry(s.A.element_type.lib_id, s.C.element_type.lib_id, s.M, s.N, s.K,
-                                                             s.A.strides[-2:], s.B.strides[-2:], s.C.strides[-2:])
+                                                             s.A.strides[-2:], s.B.strides[-2:], s.C.strides[-2:], s.variant)
             if s.batch is not None:
                 grid = grid[:2] + [s.batch]  # the batch index is bound to grid.z
             aux = {"accera": {"base_name": f["base_name"], "parameters": {k: str(v) for k, v in f["parameters"].items()}},

@@ -133,7 +133,8 @@ int acc950_gemm_batched_host(int in_type, int out_type, int batch, int M, int N,
                              const void* A, int64_t a_batch_stride, int64_t a_row_stride, int64_t a_col_stride,
                              const void* B, int64_t b_batch_stride, int64_t b_row_stride, int64_t b_col_stride,
                              void* C, int64_t c_batch_stride, int64_t c_row_stride, int64_t c_col_stride,
-                             int prologue, double prologue_arg, int epilogue, double epilogue_arg);
+                             int prologue, double prologue_arg, int epilogue, double epilogue_arg,
+                             int variant, int k_splits);
 
 /*
  * Bound call: validates the problem and chooses the kernel once, then acc950_launch(handle)

@@ -124,6 +124,44 @@ def test_column_major_and_types_are_recorded(tmp_path):
     assert aux["dynamic_shared_mem_bytes"] > 0 and aux["device_entry"] == name + "__device"
 
 
+def test_block_tile_of_a_gpu_plan_selects_the_kernel(tmp_path):
+    """The outermost splits of i and j of a GPU plan are its block tile (mfma_tests.py:89-97 tiles, binds the
+    outer indices to BLOCK_Y / BLOCK_X); a tile the library has a kernel for binds the package function to it."""
+    M = N = K = 1024
+    A = acc.Array(role=acc.Role.INPUT, element_type=acc.ScalarType.float16, shape=(M, K))
+    B = acc.Array(role=acc.Role.INPUT, element_type=acc.ScalarType.float16, shape=(K, N))
+    C = acc.Array(role=acc.Role.INPUT_OUTPUT, element_type=acc.ScalarType.float32, shape=(M, N))
+
+    def plan_with(tile):
+        nest = acc.Nest(shape=(M, N, K))
+        i, j, k = nest.get_indices()
+
+        @nest.iteration_logic
+        def _():
+            C[i, j] += A[i, k] * B[k, j]
+
+        schedule = nest.create_schedule()
+        target = acc.Target(acc.Target.Model.AMD_MI355X)
+        ii, jj, kk = schedule.tile({i: tile[0], j: tile[1], k: 64})
+        schedule.reorder(i, j, k, ii, jj, kk)
+        plan = schedule.create_plan(target)
+        plan.bind({i: target.GridUnit.BLOCK_Y, j: target.GridUnit.BLOCK_X})
+        plan.tensorize(indices=(ii, jj, kk), mma_shape=acc.MMAShape.M32xN32xK16_B1, prologue_op=acc.MMAFragmentOp.SET, prologue_arg=0,
+                       epilogue_op=acc.MMAFragmentOp.ReLU)
+        return plan
+
+    package = acc.Package()
+    n256 = package.add(plan_with((256, 256)), args=(A, B, C), base_name="tile256")
+    n128 = package.add(plan_with((128, 128)), args=(A, B, C), base_name="tile128")
+    n48 = package.add(plan_with((48, 80)), args=(A, B, C), base_name="tile_other")   # no such kernel: automatic choice
+    files = package.build(name="tiles", format=acc.Package.Format.HAT_DYNAMIC, output_dir=str(tmp_path))
+    fns = hat.parse(files[0])["functions"]
+    rec = lambda n: fns[n]["auxiliary"]["accera_mi355x"]
+    assert "mfma 256x256" in rec(n256)["kernel"] and rec(n256)["launch_parameters"][:3] == [16, 1, 1]
+    assert "mfma 128x128" in rec(n128)["kernel"] and rec(n128)["launch_parameters"][:3] == [64, 1, 1]
+    assert "mfma" in rec(n48)["kernel"]
+
+
 def test_only_the_matmul_pattern_is_accepted():
     A = acc.Array(role=acc.Role.INPUT, shape=(8, 8))
     B = acc.Array(role=acc.Role.INPUT, shape=(8, 8))
