@@ -12,7 +12,7 @@ LIB_PATH = os.path.join(LIB_DIR, "libaccera_mi355x.so")
 INCLUDE_DIR = os.path.join(os.path.dirname(_HERE), "include")
 
 # element types / ops / status codes / variant ids (accera_mi355x_gemm.h)
-F32, F16, BF16, I8, I32 = 0, 1, 2, 3, 4
+F32, F16, BF16, I8, I32, I16 = 0, 1, 2, 3, 4, 5
 PROLOGUE_NONE, PROLOGUE_SET0, PROLOGUE_SET, PROLOGUE_SCALE = 0, 1, 1, 2
 EPILOGUE_NONE, EPILOGUE_RELU, EPILOGUE_RELU_NOCOND, EPILOGUE_SCALE, EPILOGUE_SET = 0, 1, 2, 3, 4
 OK, INVALID_ARGUMENT, UNSUPPORTED, HIP_ERROR = 0, 1, 2, 3

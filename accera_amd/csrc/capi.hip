@@ -31,7 +31,7 @@ int elem_size(int t)
 {
     switch (t) {
     case T_F32: case T_I32: return 4;
-    case T_F16: case T_BF16: return 2;
+    case T_F16: case T_BF16: case T_I16: return 2;
     case T_I8: return 1;
     default: return 0;
     }
@@ -39,7 +39,7 @@ int elem_size(int t)
 
 bool type_pair_ok(int in, int out)
 {
-    if (in == T_I8) return out == T_I32;
+    if (in == T_I8) return out == T_I32 || out == T_I16 || out == T_I8;
     if (in == T_F32) return out == T_F32;
     if (in == T_F16 || in == T_BF16) return out == T_F32 || out == T_F16 || out == T_BF16;
     return false;

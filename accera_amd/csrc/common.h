@@ -6,7 +6,7 @@
 namespace acc950 {
 
 // Element types (values match include/accera_mi355x_gemm.h).
-enum : int { T_F32 = 0, T_F16 = 1, T_BF16 = 2, T_I8 = 3, T_I32 = 4 };
+enum : int { T_F32 = 0, T_F16 = 1, T_BF16 = 2, T_I8 = 3, T_I32 = 4, T_I16 = 5 };
 // Prologue / epilogue ops of the tensorized plan
 // (/root/reference/accera/python/accera/lang/Plan.py:208-379, fragment ops
 //  /root/reference/accera/acc-translate/src/Target/Cpp/CppPrinterUtils.h:630-655).
@@ -110,8 +110,24 @@ __device__ __forceinline__ float load_out(const void* C, int out_type, int64_t i
     return bf16_bits_to_float(((const uint16_t*)C)[idx]);
 }
 
+// Integer outputs: int8 / int16 elements widen with their sign on the way in and keep the
+// low bits of the int32 sum on the way out, as the reference's accumulator fragment load / store
+// does with plain C conversions (/root/reference/accera/acc-translate/src/Target/Cpp/CppPrinterUtils.h:277-293).
+__device__ __forceinline__ void store_out_int(void* C, int out_type, int64_t idx, int v)
+{
+    if (out_type == T_I32) ((int*)C)[idx] = v;
+    else if (out_type == T_I16) ((int16_t*)C)[idx] = (int16_t)v;
+    else ((int8_t*)C)[idx] = (int8_t)v;
+}
+__device__ __forceinline__ int load_out_int(const void* C, int out_type, int64_t idx)
+{
+    if (out_type == T_I32) return ((const int*)C)[idx];
+    if (out_type == T_I16) return ((const int16_t*)C)[idx];
+    return ((const int8_t*)C)[idx];
+}
+
 // Batched launch: blockIdx.z picks the problem; the kernel then sees one plain GEMM.
-__device__ __forceinline__ int elem_bytes(int type) { return type == T_I8 ? 1 : (type == T_F16 || type == T_BF16) ? 2 : 4; }
+__device__ __forceinline__ int elem_bytes(int type) { return type == T_I8 ? 1 : (type == T_F16 || type == T_BF16 || type == T_I16) ? 2 : 4; }
 __device__ __forceinline__ void select_batch(GemmArgs& p)
 {
     const int64_t z = blockIdx.z;

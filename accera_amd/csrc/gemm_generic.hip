@@ -79,9 +79,8 @@ __global__ void __launch_bounds__(256) gemm_generic_kernel(GemmArgs p)
             int64_t idx = m * p.c_rs + n * p.c_cs;
             AccT v = acc[i][j];
             if constexpr (std::is_same<AccT, int>::value) {
-                int* C = (int*)p.C;
-                v = apply_prologue<int>(v, p.prologue, p.prologue_arg, [&]() { return C[idx]; });
-                C[idx] = apply_epilogue<int>(v, p.epilogue, p.epilogue_arg);
+                v = apply_prologue<int>(v, p.prologue, p.prologue_arg, [&]() { return load_out_int(p.C, p.out_type, idx); });
+                store_out_int(p.C, p.out_type, idx, apply_epilogue<int>(v, p.epilogue, p.epilogue_arg));
             } else {
                 v = apply_prologue<float>(v, p.prologue, p.prologue_arg, [&]() { return load_out(p.C, p.out_type, idx); });
                 store_out(p.C, p.out_type, idx, apply_epilogue<float>(v, p.epilogue, p.epilogue_arg));

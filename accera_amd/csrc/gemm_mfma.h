@@ -572,8 +572,11 @@ __global__ void __launch_bounds__(Cfg::NT, Cfg::WGS_PER_CU) gemm_mfma_kernel(Gem
     const bool accumulate = p.prologue != PRO_SET; // NONE, SCALE: C is read
     if (accumulate) {
         const scalar_t c_mul = p.prologue == PRO_SCALE ? (scalar_t)p.prologue_arg : scalar_t(1); // x1 is exact
-        if constexpr (IN == IN_I8) for_each_element(int{}, [&](int* c, int v) { return wrap_add(v, wrap_mul(*c, c_mul)); });
-        else if (p.out_type == T_F32) for_each_element(float{}, [&](float* c, float v) { return v + *c * c_mul; });
+        if constexpr (IN == IN_I8) { // narrow integer outputs widen with their sign
+            if (p.out_type == T_I32) for_each_element(int{}, [&](int* c, int v) { return wrap_add(v, wrap_mul(*c, c_mul)); });
+            else if (p.out_type == T_I16) for_each_element(int16_t{}, [&](int16_t* c, int v) { return wrap_add(v, wrap_mul((int)*c, c_mul)); });
+            else for_each_element(int8_t{}, [&](int8_t* c, int v) { return wrap_add(v, wrap_mul((int)*c, c_mul)); });
+        } else if (p.out_type == T_F32) for_each_element(float{}, [&](float* c, float v) { return v + *c * c_mul; });
         else if (p.out_type == T_F16) for_each_element(_Float16{}, [&](_Float16* c, float v) { return v + (float)*c * c_mul; });
         else for_each_element(uint16_t{}, [&](uint16_t* c, float v) { return v + bf16_bits_to_float(*c) * c_mul; });
     }
@@ -649,11 +652,53 @@ __global__ void __launch_bounds__(Cfg::NT, Cfg::WGS_PER_CU) gemm_mfma_kernel(Gem
             }
         }
     };
+    // int8 / int16 outputs keep the low bits of the int32 sums.  Each lane writes its elements
+    // into the wave's slab at their row-major place; the slab then leaves as 16-byte pieces.
+    constexpr bool CAN_STAGE_INT = !EDGE && IN == IN_I8 && (NT / 64) * 32 * PITCH_DW * 4 <= Cfg::LDS_BYTES && WTN % 32 == 0;
+    auto store_staged_int = [&](auto out_tag) {
+        using out_t = decltype(out_tag);
+        constexpr int OS = sizeof(out_t);
+        constexpr int PITCH_B = PITCH_DW * 4;
+        const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+        char* slab = smem + wave_u * (32 * PITCH_B);
+        char* wave_base = (char*)p.C + ((int64_t)(m0 + (wave_u / WAVES_N) * WTM) * p.c_rs + n0 + (wave_u % WAVES_N) * WTN) * OS;
+        const unsigned row_bytes = (unsigned)p.c_rs * OS;
+        constexpr int CPRW = WTN * OS / 16;       // 16-byte pieces per row of the wave tile
+        constexpr int PIECES = 32 * CPRW / 64;    // per lane and 32-row slab
+        const int srow = (lane >> 5) * 4, scol = lane & 31;
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int row = (r >> 2) * 8 + (r & 3) + srow;
+                    *(out_t*)(slab + row * PITCH_B + (j * 32 + scol) * OS) = (out_t)acc[i][j][r];
+                }
+#pragma unroll
+            for (int it = 0; it < PIECES; ++it) {
+                const int id = it * 64 + lane;
+                const int row = id / CPRW, cc = id % CPRW;
+                const i32x4 v = *(const i32x4*)(slab + row * PITCH_B + cc * 16);
+                *(i32x4*)(wave_base + (unsigned)(i * 32 + row) * row_bytes + cc * 16) = v;
+            }
+        }
+    };
     auto store_all = [&](auto relu_tag) {
         auto fin = [&](scalar_t v) { return decltype(relu_tag)::value ? (v > scalar_t(0) ? v : scalar_t(0)) : v; };
     const bool staged = CAN_STAGE && p.c_rs % 8 == 0 && ((size_t)p.C & 15) == 0;
-    if constexpr (IN == IN_I8) for_each_element(int{}, [&](int* c, int v) { *c = fin(v); return v; });
-    else if (p.out_type == T_F32) for_each_element(float{}, [&](float* c, float v) { *c = fin(v); return v; });
+    if constexpr (IN == IN_I8) {
+        const bool aligned = (p.c_rs * (p.out_type == T_I16 ? 2 : 1)) % 16 == 0 && ((size_t)p.C & 15) == 0;
+        if (p.out_type == T_I32) for_each_element(int{}, [&](int* c, int v) { *c = fin(v); return v; });
+        else if (CAN_STAGE_INT && aligned) {
+            if constexpr (CAN_STAGE_INT) {
+                __syncthreads(); // every wave is done reading the tile buffers
+                if (p.out_type == T_I16) store_staged_int(int16_t{});
+                else store_staged_int(int8_t{});
+            }
+        } else if (p.out_type == T_I16) for_each_element(int16_t{}, [&](int16_t* c, int v) { *c = (int16_t)fin(v); return v; });
+        else for_each_element(int8_t{}, [&](int8_t* c, int v) { *c = (int8_t)fin(v); return v; });
+    } else if (p.out_type == T_F32) for_each_element(float{}, [&](float* c, float v) { *c = fin(v); return v; });
     else if (CAN_STAGE && staged) {
         if constexpr (CAN_STAGE) {
             __syncthreads(); // every wave is done reading the tile buffers

@@ -8,7 +8,7 @@ from . import _lib
 
 _TORCH_TYPES = {
     torch.float32: _lib.F32, torch.float16: _lib.F16, torch.bfloat16: _lib.BF16,
-    torch.int8: _lib.I8, torch.int32: _lib.I32,
+    torch.int8: _lib.I8, torch.int32: _lib.I32, torch.int16: _lib.I16,
 }
 
 
@@ -84,7 +84,7 @@ def gemm_relu(A, B, C, prologue=_lib.PROLOGUE_SET0, epilogue=_lib.EPILOGUE_RELU,
     column-major B is ``B_storage.t()`` of an (N,K) tensor).  With a 3-D C (batch, M, N) the
     call is a batch of independent problems in one launch (the reference's batch matmul nest,
     /root/reference/accera/python/accera/test/mfma_tests.py:435-549); A and B are 3-D, or 2-D to be
-    shared by the whole batch.  Types: fp16/bf16 in -> fp32/fp16/bf16 out, int8 -> int32,
+    shared by the whole batch.  Types: fp16/bf16 in -> fp32/fp16/bf16 out, int8 -> int32/int16/int8,
     fp32 -> fp32.  Mirrors calling one function of an Accera package on (A, B, C)
     (/root/reference/README.md:124-130), on device memory.
     """

@@ -47,6 +47,7 @@ class ScalarType(enum.Enum):
     bfloat16 = ("bfloat16_t", _lib.BF16)
     int8 = ("int8_t", _lib.I8)
     int32 = ("int32_t", _lib.I32)
+    int16 = ("int16_t", _lib.I16)
 
     @property
     def c_name(self):
@@ -138,6 +139,8 @@ class Target:
         (ScalarType.float16, ScalarType.float32): [MMAShape.M32xN32xK16_B1],
         (ScalarType.bfloat16, ScalarType.float32): [MMAShape.M32xN32xK16_B1],
         (ScalarType.int8, ScalarType.int32): [MMAShape.M32xN32xK32_B1],
+        (ScalarType.int8, ScalarType.int16): [MMAShape.M32xN32xK32_B1],
+        (ScalarType.int8, ScalarType.int8): [MMAShape.M32xN32xK32_B1],
         (ScalarType.float32, ScalarType.float32): [MMAShape.M32xN32xK2_B1],
     }
 

@@ -30,7 +30,7 @@ _OUT_FOR = {"f32": "f32", "f16": "f32", "bf16": "bf16", "i8": "i32"}
 
 
 def _torch_dtype(torch, t):
-    return {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16, "i8": torch.int8, "i32": torch.int32}[t]
+    return {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16, "i8": torch.int8, "i32": torch.int32, "i16": torch.int16}[t]
 
 
 def _make(torch, rows, cols, t, col_major, gen):

@@ -22,12 +22,16 @@ extern "C" {
 #endif
 
 /* element types; the .hat element_type names are float, float16_t, bfloat16_t,
- * int8_t, int32_t (TranslateToHeader.cpp:165-192, 329-400) */
+ * int8_t, int16_t, int32_t (TranslateToHeader.cpp:165-192, 329-400).  Pairs taken:
+ * f32 -> f32; f16 / bf16 -> f32, f16, bf16; i8 -> i32, i16, i8 (the output pairs of the reference's
+ * MI100 tensor-core table, /root/reference/accera/python/accera/Targets.py:796-821).  int16 / int8
+ * outputs widen with their sign when C is read and keep the low bits of the int32 result. */
 #define ACC950_F32 0
 #define ACC950_F16 1
 #define ACC950_BF16 2
 #define ACC950_I8 3
 #define ACC950_I32 4
+#define ACC950_I16 5
 
 /* prologue / epilogue ops of plan.tensorize
  * (/root/reference/accera/python/accera/lang/Plan.py:208-379;

@@ -30,9 +30,9 @@ import numpy as np
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB_PATH = os.path.join(_HERE, "liboracle.so")
 
-F32, F16, BF16, I8, I32 = 0, 1, 2, 3, 4
-TYPE_IDS = {"f32": F32, "f16": F16, "bf16": BF16, "i8": I8, "i32": I32}
-NP_STORAGE = {"f32": np.float32, "f16": np.float16, "bf16": np.uint16, "i8": np.int8, "i32": np.int32}
+F32, F16, BF16, I8, I32, I16 = 0, 1, 2, 3, 4, 5
+TYPE_IDS = {"f32": F32, "f16": F16, "bf16": BF16, "i8": I8, "i32": I32, "i16": I16}
+NP_STORAGE = {"f32": np.float32, "f16": np.float16, "bf16": np.uint16, "i8": np.int8, "i32": np.int32, "i16": np.int16}
 PRO_NONE, PRO_SET0, PRO_SET, PRO_SCALE = 0, 1, 1, 2
 EPI_NONE, EPI_RELU, EPI_RELU_NOCOND, EPI_SCALE, EPI_SET = 0, 1, 2, 3, 4
 SCHED_NAIVE, SCHED_TRANSFORMED = 0, 1
@@ -83,7 +83,7 @@ def widen(x, type_name):
     """Array of a storage type -> float64 (float family) or int64 (int family), exactly."""
     if type_name == "bf16":
         return from_bf16(x).astype(np.float64)
-    if type_name in ("i8", "i32"):
+    if type_name in ("i8", "i16", "i32"):
         return np.asarray(x).astype(np.int64)
     return np.asarray(x).astype(np.float64)
 
@@ -96,7 +96,11 @@ def narrow(x, type_name):
         return x.astype(np.float32).astype(np.float16)
     if type_name == "f32":
         return x.astype(np.float32)
-    return x.astype(np.int64).astype(np.int32)
+    # integer outputs keep the low bits of the int32 sum, like the plain C conversion in the
+    # reference's accumulator store (/root/reference/accera/acc-translate/src/Target/Cpp/CppPrinterUtils.h:289-293)
+    bits = {"i32": 32, "i16": 16, "i8": 8}[type_name]
+    x = x.astype(np.int64)
+    return (((x + 2 ** (bits - 1)) % 2 ** bits) - 2 ** (bits - 1)).astype(NP_STORAGE[type_name])
 
 
 def _strides_elems(a):

@@ -55,7 +55,7 @@
 #include <stdlib.h>
 #include <string.h>
 
-enum { ORA_F32 = 0, ORA_F16 = 1, ORA_BF16 = 2, ORA_I8 = 3, ORA_I32 = 4 };
+enum { ORA_F32 = 0, ORA_F16 = 1, ORA_BF16 = 2, ORA_I8 = 3, ORA_I32 = 4, ORA_I16 = 5 };
 enum { ORA_PRO_NONE = 0, ORA_PRO_SET0 = 1 };
 enum { ORA_EPI_NONE = 0, ORA_EPI_RELU = 1, ORA_EPI_RELU_NOCOND = 2 };
 enum { ORA_SCHED_NAIVE = 0, ORA_SCHED_TRANSFORMED = 1 };
@@ -280,7 +280,9 @@ static int gemm_i(int M, int N, int K,
  * the same numbers a .hat file carries as affine_map
  * (/root/reference/accera/ir/src/TranslateToHeader.cpp:726-753).
  * in_type: ORA_F32 | ORA_F16 | ORA_BF16 (out_type any float type), or ORA_I8
- * (out_type ORA_I32).  Returns 0, -1 on a bad type combination, -2 on
+ * (out_type ORA_I32, or ORA_I16 / ORA_I8: C widens with its sign on the way in and
+ * keeps the low bits of the int32 result on the way out, the plain C conversions of
+ * /root/reference/accera/acc-translate/src/Target/Cpp/CppPrinterUtils.h:277-293).  Returns 0, -1 on a bad type combination, -2 on
  * allocation failure.  Threads are set by the caller through OMP_NUM_THREADS /
  * oracle_set_threads().
  */
@@ -292,6 +294,26 @@ int oracle_gemm_relu(int in_type, int out_type, int M, int N, int K,
 {
     if (M < 0 || N < 0 || K < 0) return -1;
     if (in_type == ORA_I8) {
+        if (out_type == ORA_I16 || out_type == ORA_I8) {
+            /* through an int32 copy of C */
+            int32_t* T = (int32_t*)malloc(sizeof(int32_t) * (size_t)(M > 0 ? M : 1) * (size_t)(N > 0 ? N : 1));
+            if (!T) return -2;
+            for (int i = 0; i < M; ++i)
+                for (int j = 0; j < N; ++j) {
+                    const int64_t idx = i * c_rs + j * c_cs;
+                    T[(int64_t)i * N + j] = out_type == ORA_I16 ? (int32_t)((const int16_t*)C)[idx] : (int32_t)((const int8_t*)C)[idx];
+                }
+            int rc = gemm_i(M, N, K, (const int8_t*)A, a_rs, a_cs, (const int8_t*)B, b_rs, b_cs, T, N, 1, prologue, epilogue, schedule);
+            for (int i = 0; i < M && rc == 0; ++i)
+                for (int j = 0; j < N; ++j) {
+                    const int64_t idx = i * c_rs + j * c_cs;
+                    const uint32_t u = (uint32_t)T[(int64_t)i * N + j];
+                    if (out_type == ORA_I16) ((uint16_t*)C)[idx] = (uint16_t)u; /* same bits as the int16_t conversion */
+                    else ((uint8_t*)C)[idx] = (uint8_t)u;
+                }
+            free(T);
+            return rc;
+        }
         if (out_type != ORA_I32) return -1;
         return gemm_i(M, N, K, (const int8_t*)A, a_rs, a_cs, (const int8_t*)B, b_rs, b_cs,
                       (int32_t*)C, c_rs, c_cs, prologue, epilogue, schedule);

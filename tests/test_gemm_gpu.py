@@ -12,11 +12,11 @@ import numpy as np
 import pytest
 
 import oracle as ora
-from tests.util import assert_matches, make_input, out_zeros, to_device, to_host
+from tests.util import INT_OUT, assert_matches, make_c0, make_input, out_zeros, to_device, to_host
 
 pytestmark = pytest.mark.gpu
 
-PAIRS = [("f16", "f32"), ("f16", "f16"), ("bf16", "f32"), ("bf16", "bf16"), ("i8", "i32")]
+PAIRS = [("f16", "f32"), ("f16", "f16"), ("bf16", "f32"), ("bf16", "bf16"), ("i8", "i32"), ("i8", "i16"), ("i8", "i8")]
 
 
 def run_case(in_type, out_type, M, N, K, b_layout="row", c_layout="row", variant=-1, splits=0,
@@ -31,11 +31,10 @@ def run_case(in_type, out_type, M, N, K, b_layout="row", c_layout="row", variant
     if a_layout == "col":
         A = np.asfortranarray(A)
     if prologue == ora.PRO_NONE:
-        C0 = make_input(rng, (M, N), "i8", dist).astype(np.int32) * 1000 if out_type == "i32" else \
-            make_input(rng, (M, N), out_type, dist)
+        C0 = make_c0(rng, (M, N), out_type, dist)
     else:
         # poison C so that a kernel that wrongly reads it cannot pass
-        C0 = np.full((M, N), 77, np.int32) if out_type == "i32" else make_input(rng, (M, N), out_type, dist)
+        C0 = np.full((M, N), 77, ora.NP_STORAGE[out_type]) if out_type in INT_OUT else make_input(rng, (M, N), out_type, dist)
     if c_layout == "col":
         C0 = np.asfortranarray(C0)
     dA, dB, dC = to_device(A, in_type), to_device(B, in_type), to_device(C0, out_type)
@@ -75,6 +74,47 @@ def test_mfma_all_variants(in_type, out_type, b_layout):
             # ragged M, N (multiple of the 16-byte vector only) and a K tail
             run_case(in_type, out_type, 208 if a_layout == "col" else 200, 144, 336 if in_type == "i8" else 176, b_layout=b_layout,
                      variant=v, seed=100 + v, a_layout=a_layout)
+
+
+@pytest.mark.parametrize("out_type", ["i16", "i8"])
+def test_mfma_all_variants_narrow_integer_outputs(out_type):
+    """int8 -> int16 / int8 (pairs of the reference's tensor-core table, Targets.py:814-821; its tests
+    mfma_tests.py:2117-2141): every tile geometry's write-back, overwriting and accumulating, with
+    full-range data so that the kept low bits differ from the int32 sums."""
+    for b_layout in ("row", "col"):
+        for v, name in _variants(b_layout):
+            print("variant", v, name, out_type, b_layout, flush=True)
+            kb = int(re.search(r"kb(\d+)", name).group(1))
+            a_layout = "col" if "A=col-major" in name else "row"
+            bm, bn = map(int, re.search(r"mfma (\d+)x(\d+)", name).groups())
+            M, N = max(512, 2 * bm), (max(512, 2 * bn) if 512 % bn == 0 else 3 * bn)
+            run_case("i8", out_type, M, N, 2 * kb, b_layout=b_layout, variant=v, seed=v, a_layout=a_layout)
+            run_case("i8", out_type, M, N, 3 * kb, b_layout=b_layout, variant=v, seed=v + 1, a_layout=a_layout, prologue=ora.PRO_NONE)
+            if "edge" in name:
+                run_case("i8", out_type, 208 if a_layout == "col" else 200, 144, 336, b_layout=b_layout, variant=v, seed=50 + v,
+                         a_layout=a_layout, prologue=ora.PRO_NONE)
+
+
+def test_narrow_integer_outputs_known_answers():
+    """Closed forms: sums past the output range keep their low bits; C widens with its sign."""
+    import accera_amd as acc
+    import torch
+    M = N = 256
+    K = 512
+    ones = np.ones((M, K), np.int8)
+    for out_type, np_t, bits in (("i16", np.int16, 16), ("i8", np.int8, 8)):
+        # K * 127 = 65024: 0xFE00 -> -512 as int16, 0x00 -> 0 as int8
+        dC = to_device(np.zeros((M, N), np_t), out_type)
+        acc.gemm_relu(to_device(ones, "i8"), to_device(np.full((K, N), 127, np.int8), "i8"), dC, epilogue=acc.EPILOGUE_NONE)
+        torch.cuda.synchronize()
+        want = ((K * 127 + 2 ** (bits - 1)) % 2 ** bits) - 2 ** (bits - 1)
+        assert np.all(to_host(dC, out_type) == want), (out_type, want)
+        # C = -1 everywhere (all bits set) must count as -1, not 255 / 65535: -1 + K*1 = 511
+        dC = to_device(np.full((M, N), -1, np_t), out_type)
+        acc.gemm_relu(to_device(ones, "i8"), to_device(np.ones((K, N), np.int8), "i8"), dC, prologue=acc.PROLOGUE_NONE)
+        torch.cuda.synchronize()
+        want = ((511 + 2 ** (bits - 1)) % 2 ** bits) - 2 ** (bits - 1)
+        assert np.all(to_host(dC, out_type) == want), (out_type, want)
 
 
 @pytest.mark.parametrize("in_type,out_type", PAIRS)
@@ -341,6 +381,7 @@ OPS = [(ora.PRO_SET, 0.0, ora.EPI_SCALE, 5.0), (ora.PRO_SCALE, 0.5, ora.EPI_NONE
 
 
 @pytest.mark.parametrize("case", [("f16", "f32", 256, 512, 256, -1), ("bf16", "bf16", 256, 384, 128, -1), ("i8", "i32", 256, 256, 512, -1),
+                                  ("i8", "i16", 256, 256, 512, -1), ("i8", "i8", 256, 512, 256, -1), ("i8", "i8", 33, 47, 29, -1),
                                   ("f16", "f16", 200, 144, 176, -1), ("f32", "f32", 96, 80, 72, -1), ("f16", "f32", 33, 47, 29, 200),
                                   ("f16", "f16", 8, 1088, 512, -1), ("bf16", "f32", 24, 1024, 256, -1), ("f16", "f16", 5, 1000, 998, -1)])
 def test_fragment_ops_alpha_beta(case):
@@ -353,7 +394,7 @@ def test_fragment_ops_alpha_beta(case):
     for n, (pro, pa, epi, ea) in enumerate(OPS):
         rng = np.random.default_rng(300 + n)
         A, B = make_input(rng, (M, K), in_type), make_input(rng, (K, N), in_type)
-        C0 = make_input(rng, (M, N), "i8").astype(np.int32) * 1000 if out_type == "i32" else make_input(rng, (M, N), out_type)
+        C0 = make_c0(rng, (M, N), out_type)
         dC = to_device(C0, out_type)
         acc.gemm_relu(to_device(A, in_type), to_device(B, in_type), dC, prologue=pro, prologue_arg=pa, epilogue=epi, epilogue_arg=ea,
                       variant=variant)
@@ -422,6 +463,7 @@ def test_benchmark_configurations_at_full_size(cfg):
 
 
 @pytest.mark.parametrize("case", [("f16", "f32", 3, 1280, 768, 1024, -1), ("bf16", "bf16", 8, 256, 384, 128, -1), ("i8", "i32", 4, 256, 256, 512, -1),
+                                  ("i8", "i16", 3, 256, 256, 512, -1), ("i8", "i8", 5, 128, 384, 256, -1),
                                   ("f32", "f32", 32, 128, 128, 128, -1), ("f16", "f16", 5, 100, 72, 40, -1), ("f16", "f16", 6, 8, 1088, 512, -1),
                                   ("f16", "f16", 3, 8, 1088, 512, 100), ("bf16", "f32", 2, 5, 1000, 998, -1), ("f16", "f32", 1, 64, 64, 64, -1)])
 def test_batched_gemm(case):
@@ -434,7 +476,7 @@ def test_batched_gemm(case):
     rng = np.random.default_rng(batch * 1000 + M)
     A = np.stack([make_input(rng, (M, K), in_type, "normal") for _ in range(batch)])
     B = np.stack([make_input(rng, (K, N), in_type, "normal") for _ in range(batch)])
-    C0 = np.stack([(make_input(rng, (M, N), "i8").astype(np.int32) if out_type == "i32" else make_input(rng, (M, N), out_type)) for _ in range(batch)])
+    C0 = np.stack([make_c0(rng, (M, N), out_type, scale=1) for _ in range(batch)])
     up = lambda x, t: torch.stack([to_device(m, t) for m in x])
     dA, dB, dC = up(A, in_type), up(B, in_type), up(C0, out_type)
     acc.gemm_relu(dA, dB, dC, variant=variant, k_splits=3 if variant >= 100 else 0)

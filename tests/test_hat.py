@@ -234,6 +234,8 @@ def test_readme_quickstart_end_to_end(tmp_path):
     (acc.ScalarType.float16, acc.ScalarType.float32, (256, 384, 512), None),
     (acc.ScalarType.bfloat16, acc.ScalarType.bfloat16, (256, 256, 192), acc.Array.Layout.LAST_MAJOR),
     (acc.ScalarType.int8, acc.ScalarType.int32, (256, 256, 256), None),
+    (acc.ScalarType.int8, acc.ScalarType.int16, (256, 128, 128), None),       # mfma_tests.py:2141 sizes
+    (acc.ScalarType.int8, acc.ScalarType.int8, (128, 256, 512), acc.Array.Layout.LAST_MAJOR),  # mfma_tests.py:2123 sizes
     (acc.ScalarType.float16, acc.ScalarType.float16, (8, 1024, 512), None),
     (acc.ScalarType.float32, acc.ScalarType.float32, (16, 16, 16), None),     # mfma_tests.py:2579-2602 sizes
     (acc.ScalarType.float32, acc.ScalarType.float32, (128, 128, 16), None),
@@ -243,7 +245,7 @@ def test_tensorized_plan_package_on_numpy_arrays(tmp_path, in_t, out_t, shape, b
     (hat_path, _), name = _gpu_plan_package(tmp_path, in_t, out_t, M, N, K, b_layout)
     _, functions = hat.load(hat_path)
     tn = {acc.ScalarType.float16: "f16", acc.ScalarType.bfloat16: "bf16", acc.ScalarType.int8: "i8",
-          acc.ScalarType.float32: "f32", acc.ScalarType.int32: "i32"}
+          acc.ScalarType.float32: "f32", acc.ScalarType.int32: "i32", acc.ScalarType.int16: "i16"}
     it, ot = tn[in_t], tn[out_t]
     from tests.util import assert_matches, make_input
     rng = np.random.default_rng(5)

@@ -271,3 +271,37 @@ def test_int_ops_cast_operands_and_wrap():
     assert np.array_equal(got, wrap((P + 2 * C.astype(np.int64)) * -3).astype(np.int32))
     got = ora.gemm_relu_exact(A, B, C, "i8", "i32", ora.PRO_SET, ora.EPI_SCALE, prologue_arg=11, epilogue_arg=2**20)
     assert np.array_equal(got, wrap((P + 11) * 2**20).astype(np.int32)) and (np.abs((P + 11) * 2**20) >= 2**31).any()
+
+
+@pytest.mark.parametrize("out_type,np_t,bits", [("i16", np.int16, 16), ("i8", np.int8, 8)])
+def test_narrow_integer_outputs_keep_low_bits_and_widen_with_sign(out_type, np_t, bits):
+    """int8 -> int16 / int8 (pairs of /root/reference/accera/python/accera/Targets.py:814-821): the
+    accumulator fragment is int32; C converts to it like a C integer conversion (sign kept) and
+    back by dropping the high bits (CppPrinterUtils.h:277-293).  Pinned by known answers worked by
+    hand and by a brute-force Python loop, on both restatements."""
+    K = 512
+    ones = np.ones((4, K), np.int8)
+    # 512 * 127 = 65024 = 0xFE00: int16 -> -512, int8 -> 0x00 = 0
+    by_hand = {"i16": -512, "i8": 0}[out_type]
+    for f in (lambda A, B, C, *a: ora.gemm_relu(A, B, C.copy(), "i8", out_type, *a),
+              lambda A, B, C, *a: ora.gemm_relu_exact(A, B, C, "i8", out_type, *a)):
+        got = f(ones, np.full((K, 4), 127, np.int8), np.zeros((4, 4), np_t), ora.PRO_SET0, ora.EPI_NONE)
+        assert got.dtype == np_t and np.all(got == by_hand)
+        # C = -1 (all bits set) counts as -1: -1 + 512 = 511 = 0x1FF: int16 -> 511, int8 -> 0xFF = -1
+        got = f(ones, np.ones((K, 4), np.int8), np.full((4, 4), -1, np_t), ora.PRO_NONE, ora.EPI_RELU)
+        assert np.all(got == {"i16": 511, "i8": -1}[out_type])
+        # ReLU acts on the int32 sum, before the narrowing: -65024 -> 0
+        got = f(ones, np.full((K, 4), -127, np.int8), np.zeros((4, 4), np_t), ora.PRO_SET0, ora.EPI_RELU)
+        assert np.all(got == 0)
+    rng = np.random.default_rng(bits)
+    A = rng.integers(-128, 128, (5, 37), dtype=np.int8)
+    B = rng.integers(-128, 128, (37, 6), dtype=np.int8)
+    C = rng.integers(-2 ** (bits - 1), 2 ** (bits - 1), (5, 6)).astype(np_t)
+    want = np.zeros((5, 6), np_t)
+    for i in range(5):
+        for j in range(6):
+            s = int(C[i, j]) + sum(int(A[i, k]) * int(B[k, j]) for k in range(37))
+            s = max(s, 0) & (2 ** bits - 1)
+            want[i, j] = s - 2 ** bits if s >= 2 ** (bits - 1) else s
+    assert np.array_equal(ora.gemm_relu(A, B, C.copy(), "i8", out_type, ora.PRO_NONE, ora.EPI_RELU), want)
+    assert np.array_equal(ora.gemm_relu_exact(A, B, C, "i8", out_type, ora.PRO_NONE, ora.EPI_RELU), want)

@@ -27,6 +27,19 @@ def make_input(rng, shape, t, dist="uniform"):
     return ora.to_bf16(x)
 
 
+INT_OUT = ("i32", "i16", "i8")
+
+
+def make_c0(rng, shape, out_type, dist="uniform", scale=1000):
+    """Initial C of an accumulating call.  int32: int8 draws times ``scale``; int16 / int8: the
+    full range of the type (so that widening must honour the sign); float: like the inputs."""
+    if out_type == "i32":
+        return make_input(rng, shape, "i8", dist).astype(np.int32) * scale
+    if out_type == "i16":
+        return rng.integers(-2**15, 2**15, shape, dtype=np.int16)
+    return make_input(rng, shape, out_type, dist)
+
+
 def to_device(x, t):
     torch = _torch()
     x = np.ascontiguousarray(x) if not (x.flags.c_contiguous or x.flags.f_contiguous) else x
@@ -53,7 +66,7 @@ def assert_matches(got, want, out_type, K, exact=False, rtol=None):
     """got/want in storage dtype.  Integer: bit-exact.  Float: rtol by type
     (1e-3 for fp32 output of an fp32-accumulated sum, 1e-2 for fp16/bf16 output) plus an
     absolute term for near-cancelling sums that scales with sqrt(K)."""
-    if out_type == "i32" or exact:
+    if out_type in INT_OUT or exact:
         assert np.array_equal(got, want), f"{(got != want).sum()} of {got.size} elements differ"
         return
     g, w = ora.widen(got, out_type), ora.widen(want, out_type)
