@@ -113,9 +113,9 @@ int acc950_mfma_ceiling(int in_type, int data_mode, int iters, double* tera_ops,
         if (clock_ghz) *clock_ghz = c[1] > 0 ? (double)c[0] / (c[1] * 10.0) : 0.0; // wall clock ticks at 100 MHz
         rc = ACC950_OK;
     } while (false);
-    if (e0) hipEventDestroy(e0);
-    if (e1) hipEventDestroy(e1);
-    hipFree(src); hipFree(out); hipFree(clk);
+    if (e0) (void)hipEventDestroy(e0);
+    if (e1) (void)hipEventDestroy(e1);
+    (void)hipFree(src); (void)hipFree(out); (void)hipFree(clk);
     return rc;
 }
 

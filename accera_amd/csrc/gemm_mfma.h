@@ -252,6 +252,34 @@ struct MfmaConfig {
     static_assert(!PINGPONG || (DIRECT && WAVES_M * WAVES_N == 8), "ping-pong needs 8 waves and direct fills");
 };
 
+// ---- buffer access to the output tile ---------------------------------------------------
+// A raw buffer descriptor (base in scalar registers, 32-bit offsets) over the part of C a
+// workgroup or wave writes; reads and writes name an element by a per-lane offset, a scalar
+// offset and an immediate.
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+struct CTile {
+    __amdgpu_buffer_rsrc_t rsrc;
+};
+__device__ __forceinline__ CTile c_tile(void* base)
+{
+    // no range check by the hardware: the kernels test the edges themselves
+    return CTile{__builtin_amdgcn_make_buffer_rsrc(base, 0, -1, 0x00020000)};
+}
+template <typename T>
+__device__ __forceinline__ T c_load(CTile t, unsigned voff, unsigned soff)
+{
+    if constexpr (sizeof(T) == 4) return __builtin_bit_cast(T, __builtin_amdgcn_raw_buffer_load_b32(t.rsrc, voff, soff, 0));
+    else if constexpr (sizeof(T) == 2) return __builtin_bit_cast(T, __builtin_amdgcn_raw_buffer_load_b16(t.rsrc, voff, soff, 0));
+    else return __builtin_bit_cast(T, __builtin_amdgcn_raw_buffer_load_b8(t.rsrc, voff, soff, 0));
+}
+template <typename T>
+__device__ __forceinline__ void c_store(CTile t, unsigned voff, unsigned soff, T v)
+{
+    if constexpr (sizeof(T) == 4) __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v), t.rsrc, voff, soff, 0);
+    else if constexpr (sizeof(T) == 2) __builtin_amdgcn_raw_buffer_store_b16(__builtin_bit_cast(unsigned short, v), t.rsrc, voff, soff, 0);
+    else __builtin_amdgcn_raw_buffer_store_b8(__builtin_bit_cast(unsigned char, v), t.rsrc, voff, soff, 0);
+}
+
 template <typename Cfg>
 __global__ void __launch_bounds__(Cfg::NT, Cfg::WGS_PER_CU) gemm_mfma_kernel(GemmArgs p)
 {
@@ -530,15 +558,16 @@ __global__ void __launch_bounds__(Cfg::NT, Cfg::WGS_PER_CU) gemm_mfma_kernel(Gem
     //   C. narrowing store                                 (one copy per output type)
     // MFMA 32x32 accumulator layout: register r of lane l holds
     //   row = (r/4)*8 + (l/32)*4 + r%4,  column = l%32.
-    // C is row-major here (the host transposes the problem otherwise).  Addresses are a
-    // workgroup-uniform tile base plus one 32-bit offset per accumulator row, so the
-    // write-back needs no 64-bit address registers next to the live accumulators.
+    // C is row-major here (the host transposes the problem otherwise).  All accesses to C are
+    // buffer instructions on a descriptor of the workgroup's tile: the lane's place in the tile
+    // is one 32-bit register, the row of the access a scalar offset and the column block an
+    // immediate, so no address registers compete with the live accumulators.
     const int row_in_tile = wr0 + (lane >> 5) * 4, col_in_tile = wc0 + (lane & 31);
-    // acc element = fn(pointer to the output element, acc element) for every element of the wave tile
+    // fn(descriptor, lane offset, row offset, acc element) -> acc element, for every element of the wave tile
     auto for_each_element = [&](auto out_tag, auto&& fn) {
         using out_t = decltype(out_tag);
         constexpr unsigned OS = sizeof(out_t);
-        char* tile_base = (char*)p.C + ((int64_t)m0 * p.c_rs + n0) * OS; // uniform
+        const CTile tile = c_tile((char*)p.C + ((int64_t)m0 * p.c_rs + n0) * OS); // uniform
         const unsigned row_bytes = (unsigned)p.c_rs * OS;
         const unsigned lane_off = (unsigned)row_in_tile * row_bytes + (unsigned)col_in_tile * OS;
 #pragma unroll
@@ -546,12 +575,12 @@ __global__ void __launch_bounds__(Cfg::NT, Cfg::WGS_PER_CU) gemm_mfma_kernel(Gem
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int row_off = i * 32 + (r >> 2) * 8 + (r & 3);
-                const unsigned off = lane_off + (unsigned)row_off * row_bytes;
+                const unsigned soff = (unsigned)row_off * row_bytes; // scalar
                 if (EDGE && m0 + row_in_tile + row_off >= p.M) continue;
 #pragma unroll
                 for (int j = 0; j < TN; ++j) {
                     if (EDGE && n0 + col_in_tile + j * 32 >= p.N) continue;
-                    acc[i][j][r] = fn((out_t*)(tile_base + off + j * 32 * OS), acc[i][j][r]);
+                    acc[i][j][r] = fn(tile, lane_off + j * 32 * OS, soff, acc[i][j][r]);
                 }
                 if ((r & 3) == 3) __builtin_amdgcn_sched_barrier(0); // keep loads of pass A near their use: no second copy of the tile in registers
             }
@@ -572,13 +601,42 @@ __global__ void __launch_bounds__(Cfg::NT, Cfg::WGS_PER_CU) gemm_mfma_kernel(Gem
     const bool accumulate = p.prologue != PRO_SET; // NONE, SCALE: C is read
     if (accumulate) {
         const scalar_t c_mul = p.prologue == PRO_SCALE ? (scalar_t)p.prologue_arg : scalar_t(1); // x1 is exact
-        if constexpr (IN == IN_I8) { // narrow integer outputs widen with their sign
-            if (p.out_type == T_I32) for_each_element(int{}, [&](int* c, int v) { return wrap_add(v, wrap_mul(*c, c_mul)); });
-            else if (p.out_type == T_I16) for_each_element(int16_t{}, [&](int16_t* c, int v) { return wrap_add(v, wrap_mul((int)*c, c_mul)); });
-            else for_each_element(int8_t{}, [&](int8_t* c, int v) { return wrap_add(v, wrap_mul((int)*c, c_mul)); });
-        } else if (p.out_type == T_F32) for_each_element(float{}, [&](float* c, float v) { return v + *c * c_mul; });
-        else if (p.out_type == T_F16) for_each_element(_Float16{}, [&](_Float16* c, float v) { return v + (float)*c * c_mul; });
-        else for_each_element(uint16_t{}, [&](uint16_t* c, float v) { return v + bf16_bits_to_float(*c) * c_mul; });
+        // One copy for all output types of the kernel (a switch over the load widths would hand the
+        // register allocator one version of every accumulator per type to merge): the aligned dword
+        // that holds the element is read and the element cut out of it.
+        const unsigned sh = (p.out_type == T_I32 || p.out_type == T_F32) ? 2 : (p.out_type == T_I8 ? 0 : 1);
+        const unsigned m_f32 = p.out_type == T_F32 ? ~0u : 0u, m_f16 = p.out_type == T_F16 ? ~0u : 0u, m_bf16 = p.out_type == T_BF16 ? ~0u : 0u;
+        char* tile_base = (char*)p.C + (((int64_t)m0 * p.c_rs + n0) << sh);
+        const unsigned base_mis = (unsigned)(size_t)tile_base & 3u;  // the descriptor starts at the dword that holds the tile's first element
+        const CTile tile = c_tile(tile_base - base_mis);
+        const unsigned row_bytes = (unsigned)p.c_rs << sh;
+        const unsigned lane_off = base_mis + (unsigned)row_in_tile * row_bytes + ((unsigned)col_in_tile << sh);
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int row_off = i * 32 + (r >> 2) * 8 + (r & 3);
+                if (EDGE && m0 + row_in_tile + row_off >= p.M) continue;
+#pragma unroll
+                for (int j = 0; j < TN; ++j) {
+                    if (EDGE && n0 + col_in_tile + j * 32 >= p.N) continue;
+                    const unsigned off = lane_off + ((unsigned)row_off * row_bytes + ((unsigned)(j * 32) << sh));
+                    const unsigned mis = off & 3u; // byte of the element inside its dword
+                    const unsigned word = __builtin_amdgcn_raw_buffer_load_b32(tile.rsrc, off - mis, 0, 0);
+                    if constexpr (IN == IN_I8) { // int16 / int8 widen with their sign
+                        const int c = sh == 2 ? (int)word : __builtin_amdgcn_sbfe((int)word, mis * 8, 8u << sh);
+                        acc[i][j][r] = wrap_add(acc[i][j][r], wrap_mul(c, c_mul));
+                    } else {
+                        // the three readings of the word, blended with wave-uniform masks (selects on a
+                        // uniform condition come back as one branch per element)
+                        const unsigned half = word >> (mis * 8);
+                        const unsigned as_f16 = __float_as_uint((float)__builtin_bit_cast(_Float16, (unsigned short)half));
+                        const unsigned bits = (word & m_f32) | (as_f16 & m_f16) | ((half << 16) & m_bf16);
+                        acc[i][j][r] += __uint_as_float(bits) * c_mul;
+                    }
+                }
+                if ((r & 3) == 3) __builtin_amdgcn_sched_barrier(0); // keep the loads near their use: no second copy of the tile in registers
+            }
     }
 
     // ---- pass B (ReLU after a SET-0 prologue is the fused hot path: one max per element; every other
@@ -601,24 +659,39 @@ __global__ void __launch_bounds__(Cfg::NT, Cfg::WGS_PER_CU) gemm_mfma_kernel(Gem
     };
 
     // ---- pass C
-    // 16-bit outputs: a lane's accumulators are one column wide, so direct stores write
-    // 64-byte pieces of a row per instruction.  Instead each wave stages 32 rows of its
-    // tile in a private slab of the (now idle) LDS tile buffers, two columns packed per
-    // dword after a swap with the neighbouring lane, and streams them out as 16-byte
-    // pieces that cover whole rows of the wave tile.
+    // Narrow outputs: a lane's accumulators are one column wide, so direct stores write
+    // 64- or 32-byte pieces of a row per instruction.  Instead each wave stages 32 rows of its
+    // tile in a private slab of the (now idle) LDS tile buffers and streams them out as
+    // 16-byte pieces that cover whole rows of the wave tile.
     constexpr int PITCH_DW = (WTN / 2) % 32 == 16 ? WTN / 2 : WTN / 2 + 16; // rows r, r+1 in different bank halves
-    constexpr bool CAN_STAGE = !EDGE && IN != IN_I8 && (NT / 64) * 32 * PITCH_DW * 4 <= Cfg::LDS_BYTES;
+    constexpr int PITCH_B = PITCH_DW * 4;
+    constexpr bool CAN_STAGE = !EDGE && (NT / 64) * 32 * PITCH_B <= Cfg::LDS_BYTES;
+    // the wave's slab of 32 rows leaves as 16-byte pieces: rows i*32 .. i*32+31 of the wave tile
+    auto stream_slab = [&](auto out_tag, const char* slab, int i) {
+        constexpr int OS = sizeof(decltype(out_tag));
+        const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+        const CTile tile = c_tile((char*)p.C + ((int64_t)(m0 + (wave_u / WAVES_N) * WTM) * p.c_rs + n0 + (wave_u % WAVES_N) * WTN) * OS);
+        const unsigned row_bytes = (unsigned)p.c_rs * OS;
+        constexpr int CPRW = WTN * OS / 16;       // 16-byte pieces per row of the wave tile
+        constexpr int PIECES = 32 * CPRW / 64;    // per lane and 32-row slab
+        static_assert((32 * CPRW) % 64 == 0, "pieces divide evenly over the lanes");
+#pragma unroll
+        for (int it = 0; it < PIECES; ++it) {
+            const int id = it * 64 + lane;
+            const int row = id / CPRW, cc = id % CPRW;
+            const i32x4 v = *(const i32x4*)(slab + row * PITCH_B + cc * 16);
+            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), tile.rsrc, (unsigned)row * row_bytes + cc * 16,
+                                                   (unsigned)(i * 32) * row_bytes, 0);
+        }
+    };
+    // fp16 / bf16: two columns packed per dword after a swap with the neighbouring lane
     auto store_staged = [&](auto out_tag, auto relu_tag) {
         auto fin = [&](float v) { return decltype(relu_tag)::value ? (v > 0.f ? v : 0.f) : v; };
         using out_t = decltype(out_tag);
         const int wave_u = __builtin_amdgcn_readfirstlane(wave);
-        unsigned* slab = (unsigned*)(smem + wave_u * (32 * PITCH_DW * 4));
+        unsigned* slab = (unsigned*)(smem + wave_u * (32 * PITCH_B));
         const int odd = lane & 1;
         const int wrow = (lane >> 5) * 4 + odd, wcol = (lane & 31) >> 1;
-        char* wave_base = (char*)p.C + ((int64_t)(m0 + (wave_u / WAVES_N) * WTM) * p.c_rs + n0 + (wave_u % WAVES_N) * WTN) * 2;
-        const unsigned row_bytes = (unsigned)p.c_rs * 2;
-        constexpr int CPRW = WTN / 8;             // 16-byte pieces per row of the wave tile
-        constexpr int PIECES = 32 * CPRW / 64;    // per lane and 32-row slab
         // (lo, hi) = (own row 2t, own row 2t+1) narrowed with round-to-nearest-even
         auto pack2 = [&](float lo, float hi) -> unsigned {
             if constexpr (std::is_same<out_t, _Float16>::value) {
@@ -643,28 +716,15 @@ __global__ void __launch_bounds__(Cfg::NT, Cfg::WGS_PER_CU) gemm_mfma_kernel(Gem
                     const int row = (t >> 1) * 8 + (t & 1) * 2 + wrow;
                     slab[row * PITCH_DW + j * 16 + wcol] = __builtin_amdgcn_perm(nbr, own, sel);
                 }
-#pragma unroll
-            for (int it = 0; it < PIECES; ++it) {
-                const int id = it * 64 + lane;
-                const int row = id / CPRW, cc = id % CPRW;
-                const i32x4 v = *(const i32x4*)(slab + row * PITCH_DW + cc * 4);
-                *(i32x4*)(wave_base + (unsigned)(i * 32 + row) * row_bytes + cc * 16) = v;
-            }
+            stream_slab(uint16_t{}, (const char*)slab, i);
         }
     };
-    // int8 / int16 outputs keep the low bits of the int32 sums.  Each lane writes its elements
-    // into the wave's slab at their row-major place; the slab then leaves as 16-byte pieces.
-    constexpr bool CAN_STAGE_INT = !EDGE && IN == IN_I8 && (NT / 64) * 32 * PITCH_DW * 4 <= Cfg::LDS_BYTES && WTN % 32 == 0;
+    // int16 / int8: the low bits of the int32 sums, written into the slab at their row-major place
     auto store_staged_int = [&](auto out_tag) {
         using out_t = decltype(out_tag);
         constexpr int OS = sizeof(out_t);
-        constexpr int PITCH_B = PITCH_DW * 4;
         const int wave_u = __builtin_amdgcn_readfirstlane(wave);
         char* slab = smem + wave_u * (32 * PITCH_B);
-        char* wave_base = (char*)p.C + ((int64_t)(m0 + (wave_u / WAVES_N) * WTM) * p.c_rs + n0 + (wave_u % WAVES_N) * WTN) * OS;
-        const unsigned row_bytes = (unsigned)p.c_rs * OS;
-        constexpr int CPRW = WTN * OS / 16;       // 16-byte pieces per row of the wave tile
-        constexpr int PIECES = 32 * CPRW / 64;    // per lane and 32-row slab
         const int srow = (lane >> 5) * 4, scol = lane & 31;
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
@@ -675,38 +735,32 @@ __global__ void __launch_bounds__(Cfg::NT, Cfg::WGS_PER_CU) gemm_mfma_kernel(Gem
                     const int row = (r >> 2) * 8 + (r & 3) + srow;
                     *(out_t*)(slab + row * PITCH_B + (j * 32 + scol) * OS) = (out_t)acc[i][j][r];
                 }
-#pragma unroll
-            for (int it = 0; it < PIECES; ++it) {
-                const int id = it * 64 + lane;
-                const int row = id / CPRW, cc = id % CPRW;
-                const i32x4 v = *(const i32x4*)(slab + row * PITCH_B + cc * 16);
-                *(i32x4*)(wave_base + (unsigned)(i * 32 + row) * row_bytes + cc * 16) = v;
-            }
+            stream_slab(out_tag, slab, i);
         }
     };
     auto store_all = [&](auto relu_tag) {
         auto fin = [&](scalar_t v) { return decltype(relu_tag)::value ? (v > scalar_t(0) ? v : scalar_t(0)) : v; };
-    const bool staged = CAN_STAGE && p.c_rs % 8 == 0 && ((size_t)p.C & 15) == 0;
-    if constexpr (IN == IN_I8) {
-        const bool aligned = (p.c_rs * (p.out_type == T_I16 ? 2 : 1)) % 16 == 0 && ((size_t)p.C & 15) == 0;
-        if (p.out_type == T_I32) for_each_element(int{}, [&](int* c, int v) { *c = fin(v); return v; });
-        else if (CAN_STAGE_INT && aligned) {
-            if constexpr (CAN_STAGE_INT) {
+        const unsigned os = p.out_type == T_I8 ? 1 : (p.out_type == T_F32 || p.out_type == T_I32) ? 4 : 2;
+        const bool staged = CAN_STAGE && (p.c_rs * os) % 16 == 0 && ((size_t)p.C & 15) == 0;
+        if constexpr (IN == IN_I8) {
+            if (p.out_type == T_I32) for_each_element(int{}, [&](CTile t, unsigned vo, unsigned so, int v) { c_store<int>(t, vo, so, fin(v)); return v; });
+            else if (CAN_STAGE && staged) {
+                if constexpr (CAN_STAGE) {
+                    __syncthreads(); // every wave is done reading the tile buffers
+                    if (p.out_type == T_I16) store_staged_int(int16_t{});
+                    else store_staged_int(int8_t{});
+                }
+            } else if (p.out_type == T_I16) for_each_element(int16_t{}, [&](CTile t, unsigned vo, unsigned so, int v) { c_store<int16_t>(t, vo, so, (int16_t)fin(v)); return v; });
+            else for_each_element(int8_t{}, [&](CTile t, unsigned vo, unsigned so, int v) { c_store<int8_t>(t, vo, so, (int8_t)fin(v)); return v; });
+        } else if (p.out_type == T_F32) for_each_element(float{}, [&](CTile t, unsigned vo, unsigned so, float v) { c_store<float>(t, vo, so, fin(v)); return v; });
+        else if (CAN_STAGE && staged) {
+            if constexpr (CAN_STAGE) {
                 __syncthreads(); // every wave is done reading the tile buffers
-                if (p.out_type == T_I16) store_staged_int(int16_t{});
-                else store_staged_int(int8_t{});
+                if (p.out_type == T_F16) store_staged(_Float16{}, relu_tag);
+                else store_staged(uint16_t{}, relu_tag);
             }
-        } else if (p.out_type == T_I16) for_each_element(int16_t{}, [&](int16_t* c, int v) { *c = (int16_t)fin(v); return v; });
-        else for_each_element(int8_t{}, [&](int8_t* c, int v) { *c = (int8_t)fin(v); return v; });
-    } else if (p.out_type == T_F32) for_each_element(float{}, [&](float* c, float v) { *c = fin(v); return v; });
-    else if (CAN_STAGE && staged) {
-        if constexpr (CAN_STAGE) {
-            __syncthreads(); // every wave is done reading the tile buffers
-            if (p.out_type == T_F16) store_staged(_Float16{}, relu_tag);
-            else store_staged(uint16_t{}, relu_tag);
-        }
-    } else if (p.out_type == T_F16) for_each_element(_Float16{}, [&](_Float16* c, float v) { *c = (_Float16)fin(v); return v; }); // RNE
-    else for_each_element(uint16_t{}, [&](uint16_t* c, float v) { *c = float_to_bf16_bits(fin(v)); return v; });
+        } else if (p.out_type == T_F16) for_each_element(_Float16{}, [&](CTile t, unsigned vo, unsigned so, float v) { c_store<_Float16>(t, vo, so, (_Float16)fin(v)); return v; }); // RNE
+        else for_each_element(uint16_t{}, [&](CTile t, unsigned vo, unsigned so, float v) { c_store<uint16_t>(t, vo, so, float_to_bf16_bits(fin(v))); return v; });
     };
     // One straight line through the passes: splitting the fused matmul + ReLU case off into a
     // branch of its own makes the register allocator spill hundreds of accumulators.
