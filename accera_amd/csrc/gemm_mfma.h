@@ -59,7 +59,8 @@ __device__ __forceinline__ void wait_vmcnt()
 
 // Staging and fragment access for one operand tile of R rows (M or N extent) and KB
 // bytes of K (64 or 128), i.e. BK = KB / element-size K elements.
-template <int IN, int R, bool KC, int NT, int KB>
+// MI16: fragments are read for the 16x16 MFMA shapes (16 rows, 64 bytes of K per step).
+template <int IN, int R, bool KC, int NT, int KB, bool MI16 = false>
 struct OperandTile {
     static_assert(KB == 64 || KB == 128, "K tile is 64 or 128 bytes");
     static constexpr int ES = InTraits<IN>::ES;
@@ -86,10 +87,17 @@ struct OperandTile {
     __device__ static __forceinline__ int swizzle(int row, int c)
     {
         if constexpr (KC) return KB == 128 ? c ^ ((row >> 1) & 7) : c ^ ((row >> 2) & 3);
-        else if constexpr (ES == 2) return c ^ (((row & 3) << 2) & (CPR - 1));
-        else return c ^ (((row & 7) << 1) & (CPR - 1));
+        else if constexpr (!MI16) {
+            if constexpr (ES == 2) return c ^ (((row & 3) << 2) & (CPR - 1));
+            else return c ^ (((row & 7) << 1) & (CPR - 1));
+        } else {
+            // 16-row fragments: neighbouring groups of 16 lanes read the same columns 8 (16-bit) or
+            // 16 (8-bit) k rows apart; that bit of k moves them to the other half of the group
+            if constexpr (ES == 2) return c ^ ((((row & 3) << 2) | (((row >> 3) & 1) << 1)) & (CPR - 1));
+            else return c ^ ((((row & 7) << 1) | ((row >> 4) & 1)) & (CPR - 1));
+        }
     }
-    static constexpr int SWIZZLE_PERIOD = KC ? 16 : (ES == 2 ? 4 : 8); // rows after which it repeats
+    static constexpr int SWIZZLE_PERIOD = KC ? 16 : (ES == 2 ? (MI16 ? 16 : 4) : (MI16 ? 32 : 8)); // rows after which it repeats
 
     // Byte offset in global memory of logical chunk (row, c) of the tile whose first
     // row is r0 (M/N index) and first K element is k0.  ld = leading dimension in elements.
@@ -202,6 +210,47 @@ struct OperandTile {
 #pragma unroll
             for (int q = 0; q < 2; ++q) {
                 int k = ks * 32 + h * 16 + q * 8 + (i >> 1);
+                const char* p = lds + k * ROW_BYTES + swizzle(k, c) * 16 + within;
+                i32x2 w = __builtin_amdgcn_ds_read_tr8_b64_v2i32((ACC950_LDS i32x2*)p);
+                out[q * 2] = w[0];
+                out[q * 2 + 1] = w[1];
+            }
+            return out;
+        }
+    }
+
+    // ---- fragment read for the 16x16 shapes: 16 rows starting at row0, k-step ks (64 bytes of K).
+    // Lane l gets row (l % 16) and the 16 bytes of K number (l / 16) of the step.
+    __device__ static __forceinline__ i32x4 read_frag16(const char* lds, int row0, int ks, int lane)
+    {
+        static_assert(MI16, "tile staged for the 32x32 shapes");
+        const int kg = lane >> 4, i = lane & 15;
+        if constexpr (KC) {
+            int row = row0 + i;
+            int c = ks * 4 + kg;
+            return *(const i32x4*)(lds + row * ROW_BYTES + swizzle(row, c) * 16);
+        } else if constexpr (ES == 2) {
+            // ds_read_b64_tr_b16 (see read_frag): all four groups of 16 lanes read the same 16 columns
+            int col_byte = (row0 + (i & 3) * 4) * 2;
+            int c = col_byte >> 4, within = col_byte & 15;
+            i32x4 out;
+#pragma unroll
+            for (int q = 0; q < 2; ++q) {
+                int k = ks * 32 + kg * 8 + q * 4 + (i >> 2);
+                const char* p = lds + k * ROW_BYTES + swizzle(k, c) * 16 + within;
+                s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((ACC950_LDS s16x4*)p);
+                i32x2 w = __builtin_bit_cast(i32x2, v);
+                out[q * 2] = w[0];
+                out[q * 2 + 1] = w[1];
+            }
+            return out;
+        } else {
+            int col_byte = row0 + (i & 1) * 8;
+            int c = col_byte >> 4, within = col_byte & 15;
+            i32x4 out;
+#pragma unroll
+            for (int q = 0; q < 2; ++q) {
+                int k = ks * 64 + kg * 16 + q * 8 + (i >> 1);
                 const char* p = lds + k * ROW_BYTES + swizzle(k, c) * 16 + within;
                 i32x2 w = __builtin_amdgcn_ds_read_tr8_b64_v2i32((ACC950_LDS i32x2*)p);
                 out[q * 2] = w[0];

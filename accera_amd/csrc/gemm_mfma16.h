@@ -1,0 +1,394 @@
+// Ping-pong MFMA GEMM on the 16x16 instruction shapes of gfx950:
+// v_mfma_f32_16x16x32_{f16,bf16} and v_mfma_i32_16x16x64_i8.
+//
+// Same tiling, staging and schedule as the 8-wave ping-pong form of gemm_mfma.h (the
+// replacement for the reference's tensorized plan,
+// /root/reference/accera/transforms/src/exec/ExecutionPlanToAffineLoweringPass.cpp:5986-6533);
+// what differs is the matrix instruction.  One 16x16 instruction sums 64 bytes of K per output
+// element before it touches the accumulator, twice the run of the 32x32 shapes, and the matrix
+// cores draw measurably less power for the same arithmetic: with random operands and nothing
+// but MFMAs in flight the part sustains about 12 % more throughput on this shape.  Large
+// GEMMs run at the power limit, so that difference carries over.
+//
+// The operands are passed swapped (matrix B's fragment as the instruction's first operand), so
+// a lane ends up with one row and four neighbouring columns of C per 16x16 block: outputs leave
+// as 16-byte (fp32 / int32), 8-byte (16-bit) or 4-byte (int8) pieces with no lane exchange.
+#pragma once
+#include "gemm_mfma.h"
+
+namespace acc950 {
+
+template <int IN> struct In16Traits { using acc_t = f32x4; using scalar_t = float; };
+template <> struct In16Traits<IN_I8> { using acc_t = i32x4; using scalar_t = int; };
+
+// c (16x16, lane: row l%16 of `rows`, columns (l/16)*4..+3 of `cols`) += rows x cols^T over one k-step
+template <int IN>
+__device__ __forceinline__ void mfma16(const i32x4& cols, const i32x4& rows, typename In16Traits<IN>::acc_t& c)
+{
+    if constexpr (IN == IN_F16)
+        c = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, cols), __builtin_bit_cast(f16x8, rows), c, 0, 0, 0);
+    else if constexpr (IN == IN_BF16)
+        c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, cols), __builtin_bit_cast(bf16x8, rows), c, 0, 0, 0);
+    else
+        c = __builtin_amdgcn_mfma_i32_16x16x64_i8(cols, rows, c, 0, 0, 0);
+}
+
+template <int IN_, int BM_, int BN_, int WAVES_M_, int WAVES_N_, bool A_KC_, bool B_KC_, int KB_, int STAGES_, bool TIMED_ = false>
+struct Mfma16Config {
+    static constexpr bool TIMED = TIMED_;
+    static constexpr int IN = IN_, BM = BM_, BN = BN_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_, KB = KB_, STAGES = STAGES_;
+    static constexpr bool A_KC = A_KC_, B_KC = B_KC_;
+    static constexpr int NT = WAVES_M * WAVES_N * 64;
+    static constexpr int LDS_BYTES = STAGES * (BM + BN) * KB;
+    static_assert(WAVES_M * WAVES_N == 8, "two waves per SIMD take turns");
+    static_assert(STAGES >= 2 && STAGES <= 4, "2 to 4 LDS stages (a fifth, 160 KB in all, measured slower)");
+    static_assert(LDS_BYTES <= 160 * 1024, "LDS budget of one CU");
+};
+
+template <typename Cfg>
+__global__ void __launch_bounds__(Cfg::NT, 1) gemm_mfma16_kernel(GemmArgs p)
+{
+    constexpr int IN = Cfg::IN, BM = Cfg::BM, BN = Cfg::BN, WAVES_M = Cfg::WAVES_M, WAVES_N = Cfg::WAVES_N;
+    constexpr int KB = Cfg::KB, STAGES = Cfg::STAGES, NT = Cfg::NT;
+    constexpr bool A_KC = Cfg::A_KC, B_KC = Cfg::B_KC;
+    constexpr int ES = InTraits<IN>::ES;
+    constexpr int BK = KB / ES;
+    constexpr int KSTEPS = KB / 64;
+    constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
+    constexpr int TM = WTM / 16, TN = WTN / 16;
+    static_assert(WTM % 16 == 0 && WTN % 16 == 0, "wave tile is made of 16x16 MFMA blocks");
+    using TA = OperandTile<IN, BM, A_KC, NT, KB, true>;
+    using TB = OperandTile<IN, BN, B_KC, NT, KB, true>;
+    using acc_t = typename In16Traits<IN>::acc_t;
+    using scalar_t = typename In16Traits<IN>::scalar_t;
+    constexpr int STAGE_BYTES = TA::TILE_BYTES + TB::TILE_BYTES;
+
+    extern __shared__ __attribute__((aligned(1024))) char smem[];
+    select_batch(p);
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int wr0 = (wave / WAVES_N) * WTM;
+    const int wc0 = (wave % WAVES_N) * WTN;
+
+    unsigned long long stamp_clk[4], stamp_ref[4];
+    auto stamp = [&](int i) {
+        if constexpr (Cfg::TIMED) {
+            __builtin_amdgcn_sched_barrier(0);
+            stamp_clk[i] = __builtin_amdgcn_s_memtime();
+            stamp_ref[i] = __builtin_amdgcn_s_memrealtime();
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    stamp(0);
+
+    int tile_m, tile_n;
+    tile_coords(blockIdx.x, p.tiles_m, p.tiles_n, tile_m, tile_n);
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+
+    const char* Ab = (const char*)p.A;
+    const char* Bb = (const char*)p.B;
+    const int64_t lda = A_KC ? p.a_rs : p.a_cs; // KC: stride between rows; MC: stride between k
+    const int64_t ldb = B_KC ? p.b_cs : p.b_rs;
+
+    acc_t acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) acc[i][j] = acc_t{};
+
+    const int KT = (p.K + BK - 1) / BK;
+
+    // ---- tile fills, straight from global memory into LDS
+    const unsigned smem_addr = (unsigned)(size_t)(ACC950_LDS char*)smem;
+    const unsigned wave_lds = __builtin_amdgcn_readfirstlane((unsigned)(wave * 1024));
+    const unsigned a_lane_off = TA::direct_lane_offset(lda, tid), b_lane_off = TB::direct_lane_offset(ldb, tid);
+    constexpr int FILLS_A = TA::PER_THREAD, FILLS_B = TB::PER_THREAD, FILLS = FILLS_A + FILLS_B;
+    auto fill_one = [&](auto tile_tag, int f, unsigned lds_tile, unsigned lane_off, const char* base, int r0, int k0, int64_t ld) {
+        using T = decltype(tile_tag);
+        unsigned pos = wave_lds + f * NT * 16; // byte position of this wave's 1 KB inside the tile (wave-uniform)
+        const char* src = T::direct_base(base, f, r0, k0, ld);
+        if constexpr (!T::EVEN_SPLIT) {
+            if (pos >= (unsigned)T::TILE_BYTES) {
+                pos -= T::TILE_BYTES;
+                src -= T::wrap_bytes(ld);
+            }
+        }
+        T::direct_issue(lds_tile + pos, lane_off, src);
+    };
+    auto issue_fill = [&](int f, int stage, int k0) {
+        if (f < FILLS_A) fill_one(TA{}, f, smem_addr + stage * STAGE_BYTES, a_lane_off, Ab, m0, k0, lda);
+        else fill_one(TB{}, f - FILLS_A, smem_addr + stage * STAGE_BYTES + TA::TILE_BYTES, b_lane_off, Bb, n0, k0, ldb);
+    };
+
+    // ---- main loop.  Every k-step (64 bytes of K) is a memory cluster (fragment reads, a share
+    // of the fills of tile kt+D) and a compute cluster (its TM x TN MFMAs), each closed by a
+    // barrier.  Waves 4..7 run one cluster behind waves 0..3, so on every SIMD one wave computes
+    // while its sibling reads.
+    constexpr int D = STAGES - 1;
+    const int group = wave >> 2;
+    auto raw_barrier = [&]() {
+        __builtin_amdgcn_sched_barrier(0);
+        asm volatile("s_barrier" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);
+    };
+#pragma unroll
+    for (int s = 0; s < D; ++s)
+        if (s < KT) {
+#pragma unroll
+            for (int f = 0; f < FILLS; ++f) issue_fill(f, s, s * BK);
+        }
+    if (KT >= D) wait_vmcnt<(D - 1) * FILLS>();
+    else wait_vmcnt<0>();
+    __syncthreads();
+    stamp(1);
+    if (group == 1) raw_barrier(); // one cluster behind
+    constexpr int FPC = (FILLS + KSTEPS - 1) / KSTEPS; // fills issued per cluster
+    i32x4 af[TM], bf[TN];
+    auto pp_tile = [&](int kt, auto fill_tag) {
+        constexpr bool fill = decltype(fill_tag)::value;
+        const char* sa = smem + (kt % STAGES) * STAGE_BYTES;
+        const char* sb = sa + TA::TILE_BYTES;
+#pragma unroll
+        for (int c = 0; c < KSTEPS; ++c) {
+            // ---- memory cluster
+#pragma unroll
+            for (int j = 0; j < TN; ++j) bf[j] = TB::read_frag16(sb, wc0 + j * 16, c, lane);
+#pragma unroll
+            for (int i = 0; i < TM; ++i) af[i] = TA::read_frag16(sa, wr0 + i * 16, c, lane);
+            if constexpr (fill) {
+#pragma unroll
+                for (int u = 0; u < FPC; ++u)
+                    if (c * FPC + u < FILLS) issue_fill(c * FPC + u, (kt + D) % STAGES, (kt + D) * BK);
+            }
+            if (c + 1 == KSTEPS) { // own fills of tile kt+1 have landed before the barrier publishes them
+                if constexpr (fill) wait_vmcnt<(D - 1) * FILLS>();
+                else wait_vmcnt<0>();
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); // fragments are in registers: the buffer may be refilled
+            raw_barrier();
+            // ---- compute cluster
+            __builtin_amdgcn_s_setprio(2);
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j) mfma16<IN>(bf[j], af[i], acc[i][j]);
+            __builtin_amdgcn_s_setprio(0);
+            raw_barrier();
+        }
+    };
+    {
+        int kt = 0;
+        for (; kt + D < KT; ++kt) pp_tile(kt, std::true_type{});
+        for (; kt < KT; ++kt) pp_tile(kt, std::false_type{});
+    }
+    if (group == 0) raw_barrier(); // match the extra barrier of the other group
+
+    stamp(2);
+    // ---- write-back: A. acc += (beta *) C, B. SET constant and epilogue op, C. store.
+    // In block (i, j) lane l holds row i*16 + l%16 and columns j*16 + (l/16)*4 .. +3 of the wave tile.
+    const int lrow = wr0 + (lane & 15), lcol = wc0 + (lane >> 4) * 4;
+    if (p.prologue != PRO_SET) {
+        // One copy for all output types: the aligned dword that holds the element is read and the
+        // element cut out of it (a switch over the load widths would leave the register
+        // allocator one version of every accumulator per type to merge).
+        const scalar_t c_mul = p.prologue == PRO_SCALE ? (scalar_t)p.prologue_arg : scalar_t(1); // x1 is exact
+        const unsigned sh = (p.out_type == T_I32 || p.out_type == T_F32) ? 2 : (p.out_type == T_I8 ? 0 : 1);
+        const unsigned m_f32 = p.out_type == T_F32 ? ~0u : 0u, m_f16 = p.out_type == T_F16 ? ~0u : 0u, m_bf16 = p.out_type == T_BF16 ? ~0u : 0u;
+        char* tile_base = (char*)p.C + (((int64_t)m0 * p.c_rs + n0) << sh);
+        const unsigned base_mis = (unsigned)(size_t)tile_base & 3u; // the descriptor starts at the dword that holds the tile's first element
+        const CTile tile = c_tile(tile_base - base_mis);
+        const unsigned row_bytes = (unsigned)p.c_rs << sh;
+        const unsigned lane_off = base_mis + (unsigned)lrow * row_bytes + ((unsigned)lcol << sh);
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const unsigned off = lane_off + ((unsigned)(i * 16) * row_bytes + ((unsigned)(j * 16 + e) << sh));
+                    const unsigned mis = off & 3u; // byte of the element inside its dword
+                    const unsigned word = __builtin_amdgcn_raw_buffer_load_b32(tile.rsrc, off - mis, 0, 0);
+                    if constexpr (IN == IN_I8) { // int16 / int8 widen with their sign
+                        const int c = sh == 2 ? (int)word : __builtin_amdgcn_sbfe((int)word, mis * 8, 8u << sh);
+                        acc[i][j][e] = wrap_add(acc[i][j][e], wrap_mul(c, c_mul));
+                    } else {
+                        const unsigned half = word >> (mis * 8);
+                        const unsigned as_f16 = __float_as_uint((float)__builtin_bit_cast(_Float16, (unsigned short)half));
+                        const unsigned bits = (word & m_f32) | (as_f16 & m_f16) | ((half << 16) & m_bf16);
+                        acc[i][j][e] += __uint_as_float(bits) * c_mul;
+                    }
+                }
+            __builtin_amdgcn_sched_barrier(0); // block row by block row: loads stay near their use
+        }
+    }
+
+    auto for_each_acc = [&](auto&& fn) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) acc[i][j][e] = fn(acc[i][j][e]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    if (p.epilogue == EPI_RELU && !(p.prologue == PRO_SET && p.prologue_arg != 0.f)) {
+        for_each_acc([&](scalar_t v) { return v > scalar_t(0) ? v : scalar_t(0); }); // the fused hot path: one max per element
+    } else if (p.epilogue != EPI_NONE || (p.prologue == PRO_SET && p.prologue_arg != 0.f)) {
+        const scalar_t set_value = p.prologue == PRO_SET ? (scalar_t)p.prologue_arg : scalar_t(0);
+        const scalar_t epi_arg = (scalar_t)p.epilogue_arg;
+        const bool is_relu = p.epilogue == EPI_RELU, is_nocond = p.epilogue == EPI_RELU_NOCOND, is_scale = p.epilogue == EPI_SCALE,
+                   is_set = p.epilogue == EPI_SET;
+        for_each_acc([&](scalar_t v) {
+            v = wrap_add(v, set_value);
+            const scalar_t r = v > scalar_t(0) ? v : scalar_t(0);
+            const scalar_t n = v * (v > scalar_t(0) ? scalar_t(1) : scalar_t(0));
+            const scalar_t m = wrap_mul(v, epi_arg);
+            return is_relu ? r : (is_nocond ? n : (is_scale ? m : (is_set ? epi_arg : v)));
+        });
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
+    // ---- pass C
+    const unsigned os = p.out_type == T_I8 ? 1 : (p.out_type == T_F32 || p.out_type == T_I32) ? 4 : 2;
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+    // the four values of a block narrowed to the output type, packed in column order
+    auto pack_f16 = [](const acc_t& v) -> i32x2 {
+        typedef _Float16 h4 __attribute__((ext_vector_type(4)));
+        return __builtin_bit_cast(i32x2, h4{(_Float16)v[0], (_Float16)v[1], (_Float16)v[2], (_Float16)v[3]}); // RNE
+    };
+    auto pack_bf16 = [](const acc_t& v) -> i32x2 {
+        typedef __bf16 b4 __attribute__((ext_vector_type(4)));
+        return __builtin_bit_cast(i32x2, b4{(__bf16)v[0], (__bf16)v[1], (__bf16)v[2], (__bf16)v[3]}); // RNE
+    };
+    auto pack_i16 = [](const acc_t& v) -> i32x2 { // low bits of the int32 sums
+        return i32x2{(int)(((unsigned)v[0] & 0xffffu) | ((unsigned)v[1] << 16)), (int)(((unsigned)v[2] & 0xffffu) | ((unsigned)v[3] << 16))};
+    };
+    auto pack_i8 = [](const acc_t& v) -> int {
+        return (int)(((unsigned)v[0] & 0xffu) | (((unsigned)v[1] & 0xffu) << 8) | (((unsigned)v[2] & 0xffu) << 16) | ((unsigned)v[3] << 24));
+    };
+    if (os == 4) {
+        // one 16-byte store per block and lane
+        const CTile tile = c_tile((char*)p.C + ((int64_t)m0 * p.c_rs + n0) * 4);
+        const unsigned row_bytes = (unsigned)p.c_rs * 4;
+        const unsigned lane_off = (unsigned)lrow * row_bytes + (unsigned)lcol * 4;
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, acc[i][j]), tile.rsrc, lane_off + j * 64,
+                                                       (unsigned)(i * 16) * row_bytes, 0);
+    } else if ((p.c_rs * os) % 16 == 0 && ((size_t)p.C & 15) == 0) {
+        // narrow outputs: 16 rows of the wave tile are put together in a wave-private slab of the
+        // (now idle) tile buffers and leave as 16-byte pieces that cover whole rows
+        __syncthreads(); // every wave is done reading the tile buffers
+        auto staged = [&](auto os_tag, auto&& pack) {
+            constexpr int OS = decltype(os_tag)::value;
+            constexpr int ROW = WTN * OS;
+            constexpr int PITCH = (ROW / 32) % 2 == 0 ? ROW + 32 : ROW; // an odd number of 32-byte units: rows spread over the banks
+            static_assert(NT / 64 * 16 * PITCH <= Cfg::LDS_BYTES, "slabs fit the tile buffers");
+            char* slab = smem + wave_u * (16 * PITCH);
+            const CTile tile = c_tile((char*)p.C + ((int64_t)(m0 + (wave_u / WAVES_N) * WTM) * p.c_rs + n0 + (wave_u % WAVES_N) * WTN) * OS);
+            const unsigned row_bytes = (unsigned)p.c_rs * OS;
+            constexpr int CPRW = ROW / 16;                    // 16-byte pieces per row of the wave tile
+            constexpr int PIECES = (16 * CPRW + 63) / 64;     // per lane and 16-row slab
+            char* mine = slab + (lane & 15) * PITCH + ((lane >> 4) * 4) * OS;
+#pragma unroll
+            for (int i = 0; i < TM; ++i) {
+#pragma unroll
+                for (int j = 0; j < TN; ++j) {
+                    auto w = pack(acc[i][j]);
+                    *(decltype(w)*)(mine + j * 16 * OS) = w;
+                }
+#pragma unroll
+                for (int it = 0; it < PIECES; ++it) {
+                    const int id = it * 64 + lane;
+                    if ((16 * CPRW) % 64 != 0 && id >= 16 * CPRW) break;
+                    const int row = id / CPRW, cc = id % CPRW;
+                    const i32x4 v = *(const i32x4*)(slab + row * PITCH + cc * 16);
+                    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), tile.rsrc, (unsigned)row * row_bytes + cc * 16,
+                                                           (unsigned)(i * 16) * row_bytes, 0);
+                }
+            }
+        };
+        if constexpr (IN == IN_I8) {
+            if (os == 2) staged(std::integral_constant<int, 2>{}, pack_i16);
+            else staged(std::integral_constant<int, 1>{}, pack_i8);
+        } else {
+            if (p.out_type == T_F16) staged(std::integral_constant<int, 2>{}, pack_f16);
+            else staged(std::integral_constant<int, 2>{}, pack_bf16);
+        }
+    } else {
+        // rows of C that are not 16-byte aligned: single elements
+        const CTile tile = c_tile((char*)p.C + ((int64_t)m0 * p.c_rs + n0) * os);
+        const unsigned row_bytes = (unsigned)p.c_rs * os;
+        const unsigned lane_off = (unsigned)lrow * row_bytes + (unsigned)lcol * os;
+        auto by_element = [&](auto os_tag, auto&& pack) {
+            constexpr int OS = decltype(os_tag)::value;
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j) {
+                    const unsigned so = (unsigned)(i * 16) * row_bytes + (unsigned)(j * 16) * OS;
+                    auto w = pack(acc[i][j]);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        if constexpr (OS == 2)
+                            __builtin_amdgcn_raw_buffer_store_b16((unsigned short)((unsigned)w[e >> 1] >> ((e & 1) * 16)), tile.rsrc, lane_off + e * 2, so, 0);
+                        else
+                            __builtin_amdgcn_raw_buffer_store_b8((unsigned char)((unsigned)w >> (e * 8)), tile.rsrc, lane_off + e, so, 0);
+                    }
+                }
+        };
+        if constexpr (IN == IN_I8) {
+            if (os == 2) by_element(std::integral_constant<int, 2>{}, pack_i16);
+            else by_element(std::integral_constant<int, 1>{}, pack_i8);
+        } else {
+            if (p.out_type == T_F16) by_element(std::integral_constant<int, 2>{}, pack_f16);
+            else by_element(std::integral_constant<int, 2>{}, pack_bf16);
+        }
+    }
+
+    if constexpr (Cfg::TIMED) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // stores acknowledged
+        stamp(3);
+        if (threadIdx.x == 0 && p.stamps) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                p.stamps[(blockIdx.x * 4 + i) * 2] = stamp_clk[i]; // (probe runs unbatched)
+                p.stamps[(blockIdx.x * 4 + i) * 2 + 1] = stamp_ref[i];
+            }
+        }
+    }
+}
+
+// Host launcher for one kernel instantiation.
+template <typename Cfg>
+hipError_t launch_mfma16(const GemmArgs& a, hipStream_t stream, LaunchGeom* geom, bool dry_run)
+{
+    auto kern = gemm_mfma16_kernel<Cfg>;
+    GemmArgs args = a;
+    args.tiles_m = (a.M + Cfg::BM - 1) / Cfg::BM;
+    args.tiles_n = (a.N + Cfg::BN - 1) / Cfg::BN;
+    if (geom) {
+        geom->grid[0] = (unsigned)(args.tiles_m * args.tiles_n);
+        geom->grid[1] = 1;
+        geom->grid[2] = a.batch > 1 ? a.batch : 1;
+        geom->block[0] = Cfg::NT;
+        geom->block[1] = geom->block[2] = 1;
+        geom->dyn_lds = Cfg::LDS_BYTES;
+    }
+    if (dry_run) return hipSuccess;
+    static bool attr_set = false; // per instantiation; benign if set twice
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES);
+        if (e != hipSuccess) return e;
+        attr_set = true;
+    }
+    hipLaunchKernelGGL(kern, dim3(args.tiles_m * args.tiles_n, 1, a.batch > 1 ? a.batch : 1), dim3(Cfg::NT), Cfg::LDS_BYTES, stream, args);
+    return hipGetLastError();
+}
+
+} // namespace acc950

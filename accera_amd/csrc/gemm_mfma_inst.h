@@ -6,17 +6,21 @@
 //  /root/reference/tools/benchmarkers/accera_gemm.py:187-348): block tile BMxBN, K tile
 // of KB bytes, waves laid out WAVES_M x WAVES_N, the tile fill either direct-to-LDS
 // (STAGES buffers deep) or register-staged, and whether partial edge tiles are handled.
-#include "gemm_mfma.h"
+#include "gemm_mfma16.h"
 #include "variants.h"
 
 namespace acc950 {
 
 #define VA(AKC, BM, BN, WM, WN, BKC, DIRECT, EDGE, KB, STAGES)                                         \
-    { BM, BN, WM, WN, AKC, BKC, DIRECT, EDGE, KB, STAGES, false,                                       \
+    { BM, BN, WM, WN, AKC, BKC, DIRECT, EDGE, KB, STAGES, false, false,                                \
       &launch_mfma<MfmaConfig<ACC950_IN, BM, BN, WM, WN, AKC, BKC, DIRECT, EDGE, KB, STAGES>> }
 #define VPA(AKC, BM, BN, WM, WN, BKC, KB, STAGES)                                                       \
-    { BM, BN, WM, WN, AKC, BKC, true, false, KB, STAGES, true,                                         \
+    { BM, BN, WM, WN, AKC, BKC, true, false, KB, STAGES, true, false,                                  \
       &launch_mfma<MfmaConfig<ACC950_IN, BM, BN, WM, WN, AKC, BKC, true, false, KB, STAGES, true>> }
+// ping-pong on the 16x16 MFMA shapes
+#define V16(AKC, BM, BN, WM, WN, BKC, KB, STAGES)                                                       \
+    { BM, BN, WM, WN, AKC, BKC, true, false, KB, STAGES, true, true,                                   \
+      &launch_mfma16<Mfma16Config<ACC950_IN, BM, BN, WM, WN, AKC, BKC, KB, STAGES>> }
 #define V(BM, BN, WM, WN, BKC, DIRECT, EDGE, KB, STAGES) VA(true, BM, BN, WM, WN, BKC, DIRECT, EDGE, KB, STAGES)
 #define VP(BM, BN, WM, WN, BKC, KB, STAGES) VPA(true, BM, BN, WM, WN, BKC, KB, STAGES)
 // column-major A (M contiguous; the "transA" shapes of the reference's sweep lists,
@@ -50,19 +54,28 @@ static const MfmaVariant kVariants[] = {
     V(256, 192, 4, 2, true, true, false, 128, 2),
     LAYOUT_AT(false),
     LAYOUT_AT(true),
+    // 16x16 MFMA shapes: A row-major x B row- / column-major, A column-major, 192-wide tiles
+    V16(true, 256, 256, 2, 4, false, 64, 4),
+    V16(true, 256, 256, 2, 4, false, 128, 2),
+    V16(true, 256, 256, 2, 4, true, 64, 4),
+    V16(true, 256, 256, 2, 4, true, 128, 2),
+    V16(false, 256, 256, 2, 4, false, 64, 4),
+    V16(false, 256, 256, 2, 4, true, 64, 4),
+    V16(true, 256, 192, 4, 2, true, 64, 4),
 };
 #undef LAYOUT_AT
 #undef VA
 #undef VPA
+#undef V16
 #undef LAYOUT
 #undef V
 #undef VP
 
 // Timed build of the kernel the automatic choice takes for large aligned problems
-// (256x256 ping-pong, row-major B): same code plus four clock stamps per workgroup.
+// (256x256 ping-pong on the 16x16 MFMA shapes, row-major B): same code plus four clock stamps per workgroup.
 hipError_t ACC950_TIMED_FN(const GemmArgs& a, hipStream_t stream, LaunchGeom* geom, bool dry_run)
 {
-    return launch_mfma<MfmaConfig<ACC950_IN, 256, 256, 2, 4, true, false, true, false, 64, 4, true, true>>(a, stream, geom, dry_run);
+    return launch_mfma16<Mfma16Config<ACC950_IN, 256, 256, 2, 4, true, false, 64, 4, true>>(a, stream, geom, dry_run);
 }
 
 const MfmaVariant* ACC950_TABLE_FN(int* count)

@@ -13,6 +13,7 @@ struct MfmaVariant {
     int kb;              // bytes of K per tile (64 or 128)
     int stages;          // LDS buffers
     bool pingpong;       // sibling waves alternate memory and compute clusters
+    bool mi16;           // 16x16 MFMA shapes (else 32x32)
     LaunchFn launch;
 };
 
