@@ -1,8 +1,8 @@
 // Measurement aids used by the benchmark: what this particular GPU can sustain, so that
 // a kernel's distance from the nominal peak can be split into "kernel" and "machine".
 //
-//   * MFMA ceiling: a register-resident loop of independent MFMAs (no memory traffic at
-//     all) on operands that are zero, constant, or random.  On MI355X the sustained
+//   * MFMA ceiling: a register-resident loop of independent MFMAs of the 16x16 shapes the
+//     large-tile kernels use (no memory traffic at all) on operands that are zero, constant, or random.  On MI355X the sustained
 //     engine clock under MFMA load depends strongly on the operand data (power), so the
 //     random-data figure -- not the nominal peak -- is the practical compute roof for
 //     random GEMM inputs.
@@ -18,30 +18,29 @@ using namespace acc950;
 
 namespace {
 
+// 8 waves per workgroup (two per SIMD, as in the GEMM kernels), 16 independent 16x16 accumulators
+// per wave, the instruction written out so that every MFMA accumulates in place.
 template <int IN>
-__global__ void __launch_bounds__(256) mfma_ceiling_kernel(const i32x4* src, float* out, long long* clk, int iters)
+__global__ void __launch_bounds__(512) mfma_ceiling_kernel(const i32x4* src, float* out, long long* clk, int iters)
 {
-    i32x4 a[4], b[2];
+    i32x4 a[4], b[4];
     for (int j = 0; j < 4; ++j) a[j] = src[(threadIdx.x + 64 * j) & 1023];
-    for (int j = 0; j < 2; ++j) b[j] = src[(threadIdx.x + 512 + 64 * j) & 1023];
-    f32x16 accf[8];
-    i32x16 acci[8];
-    for (int j = 0; j < 8; ++j) { accf[j] = f32x16{}; acci[j] = i32x16{}; }
+    for (int j = 0; j < 4; ++j) b[j] = src[(threadIdx.x + 512 + 64 * j) & 1023];
+    f32x4 acc[16];
+    for (int j = 0; j < 16; ++j) acc[j] = f32x4{};
     const long long c0 = clock64(), w0 = wall_clock64();
     for (int it = 0; it < iters; ++it) {
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            if constexpr (IN == T_I8) acci[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[j >> 1], b[j & 1], acci[j], 0, 0, 0);
-            else if constexpr (IN == T_BF16)
-                accf[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a[j >> 1]), __builtin_bit_cast(bf16x8, b[j & 1]), accf[j], 0, 0, 0);
-            else
-                accf[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a[j >> 1]), __builtin_bit_cast(f16x8, b[j & 1]), accf[j], 0, 0, 0);
+        for (int j = 0; j < 16; ++j) {
+            if constexpr (IN == T_I8) asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+v"(acc[j]) : "v"(a[j >> 2]), "v"(b[j & 3]));
+            else if constexpr (IN == T_BF16) asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+v"(acc[j]) : "v"(a[j >> 2]), "v"(b[j & 3]));
+            else asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+v"(acc[j]) : "v"(a[j >> 2]), "v"(b[j & 3]));
         }
     }
     const long long c1 = clock64(), w1 = wall_clock64();
     float s = 0;
-    for (int j = 0; j < 8; ++j)
-        for (int r = 0; r < 16; ++r) s += IN == T_I8 ? (float)acci[j][r] : accf[j][r];
+    for (int j = 0; j < 16; ++j)
+        for (int r = 0; r < 4; ++r) s += IN == T_I8 ? (float)__builtin_bit_cast(int, acc[j][r]) : acc[j][r];
     out[blockIdx.x * blockDim.x + threadIdx.x] = s;
     if (threadIdx.x == 0 && blockIdx.x == 0) { clk[0] = c1 - c0; clk[1] = w1 - w0; }
 }
@@ -89,14 +88,14 @@ int acc950_mfma_ceiling(int in_type, int data_mode, int iters, double* tera_ops,
     hipEvent_t e0 = nullptr, e1 = nullptr;
     int rc = ACC950_HIP_ERROR;
     do {
-        if (hipMalloc((void**)&src, 16384) != hipSuccess || hipMalloc((void**)&out, 256 * 256 * 4) != hipSuccess ||
+        if (hipMalloc((void**)&src, 16384) != hipSuccess || hipMalloc((void**)&out, 256 * 512 * 4) != hipSuccess ||
             hipMalloc((void**)&clk, 16) != hipSuccess) break;
         if (hipMemcpy(src, h.data(), 16384, hipMemcpyHostToDevice) != hipSuccess) break;
         if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) break;
         auto launch = [&](int n) {
-            if (in_type == T_I8) hipLaunchKernelGGL(mfma_ceiling_kernel<T_I8>, dim3(256), dim3(256), 0, 0, src, out, clk, n);
-            else if (in_type == T_BF16) hipLaunchKernelGGL(mfma_ceiling_kernel<T_BF16>, dim3(256), dim3(256), 0, 0, src, out, clk, n);
-            else hipLaunchKernelGGL(mfma_ceiling_kernel<T_F16>, dim3(256), dim3(256), 0, 0, src, out, clk, n);
+            if (in_type == T_I8) hipLaunchKernelGGL(mfma_ceiling_kernel<T_I8>, dim3(256), dim3(512), 0, 0, src, out, clk, n);
+            else if (in_type == T_BF16) hipLaunchKernelGGL(mfma_ceiling_kernel<T_BF16>, dim3(256), dim3(512), 0, 0, src, out, clk, n);
+            else hipLaunchKernelGGL(mfma_ceiling_kernel<T_F16>, dim3(256), dim3(512), 0, 0, src, out, clk, n);
         };
         launch(200);
         if (hipDeviceSynchronize() != hipSuccess) break;
@@ -108,7 +107,7 @@ int acc950_mfma_ceiling(int in_type, int data_mode, int iters, double* tera_ops,
         hipEventElapsedTime(&ms, e0, e1);
         long long c[2];
         if (hipMemcpy(c, clk, 16, hipMemcpyDeviceToHost) != hipSuccess) break;
-        const double ops = 256.0 * 4 * iters * 8 * (in_type == T_I8 ? 65536.0 : 32768.0);
+        const double ops = 256.0 * 8 * iters * 16 * (in_type == T_I8 ? 32768.0 : 16384.0);
         if (tera_ops) *tera_ops = ops / (ms * 1e-3) / 1e12;
         if (clock_ghz) *clock_ghz = c[1] > 0 ? (double)c[0] / (c[1] * 10.0) : 0.0; // wall clock ticks at 100 MHz
         rc = ACC950_OK;

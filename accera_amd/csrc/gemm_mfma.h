@@ -81,7 +81,9 @@ struct OperandTile {
     // LDS chunk position <-> logical chunk of the same row (an involution).
     //  KC, 128-byte rows: a 16-lane read phase touches rows r..r+15 at one chunk; rows
     //      two apart are 256 bytes (all banks) apart, so the row pair index picks the chunk.
-    //  KC,  64-byte rows: four rows fill the 256-byte bank span, so row/4 picks the chunk.
+    //  KC,  64-byte rows: four rows fill the 256-byte bank span, so row/4 picks the chunk.  (For the
+    //      16-row fragments this leaves two-way conflicts; a conflict-free map exists and measured
+    //      2 % slower in the ping-pong kernel, where the reads hide behind the sibling's MFMAs.)
     //  MC: a transpose read touches 4 (16-bit) or 8 (8-bit) consecutive k rows, which are
     //      a multiple of 256 bytes apart; k picks a 64- / 32-byte group inside the row.
     __device__ static __forceinline__ int swizzle(int row, int c)

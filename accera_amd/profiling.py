@@ -38,7 +38,7 @@ def _dominant(acc, counter):
     for k, cs in acc.items():
         if "acc950_copy_kernel" in k or "acc950_stream_read_kernel" in k or "mfma_ceiling" in k or counter not in cs:
             continue
-        if not any(s in k for s in ("gemm_mfma_kernel", "gemm_skinny", "gemm_f32_kernel", "gemm_generic_kernel")):
+        if not any(s in k for s in ("gemm_mfma_kernel", "gemm_mfma16_kernel", "gemm_skinny", "gemm_f32_kernel", "gemm_generic_kernel")):
             continue
         tot = sum(cs[counter])
         if best is None or tot > best[1]:
