@@ -124,6 +124,12 @@ bool mfma_can_take(const MfmaVariant& v, const Problem& pb)
     if (lda % vec || ldb % vec) return false;
     if (pb.have_pointers && (!aligned16(g.A) || !aligned16(g.B))) return false;
     if (g.batch > 1 && (g.a_bs % vec || g.b_bs % vec)) return false; // every problem of the batch 16-byte aligned
+    // int8 outputs need rows of C that start 16 bytes apart: byte-wise stores to rows at odd distances
+    // are switched off (that path faulted on the device in its first run and the cause is not known)
+    if (g.out_type == T_I8) {
+        if (g.c_rs % 16 || (g.batch > 1 && g.c_bs % 16)) return false;
+        if (pb.have_pointers && !aligned16(g.C)) return false;
+    }
     if (v.edge) {
         if (g.K % vec) return false;
         if (!v.b_kc && g.N % vec) return false;

@@ -10,7 +10,11 @@ tools/benchmarkers/gemm_*.csv; transX = 1 means the operand is stored column-maj
   * runs each on device-resident random inputs, optionally checks it against a float64 / int64
     NumPy product on sampled rows (rtol 1e-2 as the reference's driver),
   * times it with HIP events (min over batches of the mean time per launch),
-  * writes one CSV row per (shape, variant) and prints the best variant per shape.
+  * writes one CSV row per (shape, variant) and prints the best variant per shape,
+  * with --baseline also times the vendor GEMM library on the same operands (torch.matmul, i.e.
+    hipBLASLt / rocBLAS; torch._int_mm for int8), the counterpart of the reference's rocBLAS
+    benchmarker (/root/reference/tools/benchmarkers/rocblas/main.cpp).  The vendor call writes an
+    output of the input type and has no fused epilogue; it is a yardstick, never a code path.
 
     python -m accera_amd.tune --input accera_amd/shapes/transformer_gemm.csv --type f16 --check --relu
 
@@ -79,7 +83,7 @@ def time_call(torch, call, min_time_s=0.05, batches=5):
     return best
 
 
-def sweep(rows, in_type, relu, check, out_type=None, min_time_s=0.05, log=print):
+def sweep(rows, in_type, relu, check, out_type=None, min_time_s=0.05, log=print, baseline=False):
     import torch
     from .gemm import GemmCall
     if not torch.cuda.is_available():
@@ -94,7 +98,7 @@ def sweep(rows, in_type, relu, check, out_type=None, min_time_s=0.05, log=print)
         ta, tb = bool(int(r.get("transA", 0))), bool(int(r.get("transB", 0)))
         alpha, beta = float(r.get("alpha", 1.0)), float(r.get("beta", 0.0))
         A, B = _make(torch, M, K, in_type, ta, gen), _make(torch, K, N, in_type, tb, gen)
-        C0 = _make(torch, M, N, "i8" if out_type == "i32" else out_type, False, gen).to(_torch_dtype(torch, out_type))
+        C0 = _make(torch, M, N, "i8" if out_type in ("i32", "i16", "i8") else out_type, False, gen).to(_torch_dtype(torch, out_type))
         pro, parg = (_lib.PROLOGUE_SET0, 0.0) if beta == 0 else (_lib.PROLOGUE_NONE, 0.0) if beta == 1 else (_lib.PROLOGUE_SCALE, beta)
         if alpha != 1 and relu:
             log(f"{M}x{N}x{K}: skipped (alpha != 1 and a fused ReLU are two epilogue ops; one kernel carries one)")
@@ -107,6 +111,9 @@ def sweep(rows, in_type, relu, check, out_type=None, min_time_s=0.05, log=print)
             parg_c, earg_c = (int(parg), int(earg)) if in_type == "i8" else (np.float32(parg), np.float32(earg))
             want = Ah @ Bh + (0 if beta == 0 else C0[torch.as_tensor(idx, device="cuda")].double().cpu().numpy() * (1 if beta == 1 else parg_c))
             want = want * earg_c if alpha != 1 else (np.maximum(want, 0) if relu else want)
+            if out_type in ("i16", "i8"):  # narrow integer outputs keep the low bits
+                bits = 16 if out_type == "i16" else 8
+                want = ((want.astype(np.int64) + 2 ** (bits - 1)) % 2 ** bits) - 2 ** (bits - 1)
             sample = torch.as_tensor(idx, device="cuda")
         sa, sb, sc = (A.stride(0), A.stride(1)), (B.stride(0), B.stride(1)), (N, 1)
         best = None
@@ -123,7 +130,7 @@ def sweep(rows, in_type, relu, check, out_type=None, min_time_s=0.05, log=print)
                 call()
                 torch.cuda.synchronize()
                 got = C[sample].double().cpu().numpy()
-                tol = 0 if out_type == "i32" else 1e-2
+                tol = 0 if out_type in ("i32", "i16", "i8") else 1e-2
                 ok = bool(np.allclose(got, want, rtol=tol, atol=tol * max(1.0, float(np.abs(want).max())) * 1e-1))
             if beta != 0:
                 t = time_call(torch, lambda: (C.copy_(C0), call()), min_time_s) - time_call(torch, lambda: C.copy_(C0), min_time_s)
@@ -135,9 +142,23 @@ def sweep(rows, in_type, relu, check, out_type=None, min_time_s=0.05, log=print)
             results.append(row)
             if ok is not False and (best is None or row["time_ms"] < best["time_ms"]):
                 best = row
+        vendor = ""
+        if baseline:
+            try:
+                if in_type == "i8":
+                    tv = time_call(torch, lambda: torch._int_mm(A, B), min_time_s)
+                else:
+                    out = torch.empty((M, N), device="cuda", dtype=A.dtype)
+                    tv = time_call(torch, lambda: torch.matmul(A, B, out=out), min_time_s)
+                results.append(dict(m=M, n=N, k=K, transA=int(ta), transB=int(tb), alpha=1.0, beta=0.0, type=in_type,
+                                    out_type="i32" if in_type == "i8" else in_type, variant=-2, k_splits=0, kernel="vendor library (torch.matmul)",
+                                    time_ms=round(tv * 1e3, 5), TFlops=round(2.0 * M * N * K / tv / 1e12, 3), correct=""))
+                vendor = f"  | vendor library {round(2.0 * M * N * K / tv / 1e12, 1)} TFlops {round(tv * 1e3, 4)} ms"
+            except RuntimeError as e:  # shapes the vendor call does not take (e.g. _int_mm alignment)
+                vendor = f"  | vendor library: {str(e).splitlines()[0][:60]}"
         if best:
             log(f"{M}x{N}x{K} tA={int(ta)} tB={int(tb)} a={alpha} b={beta}: best {best['TFlops']} TFlops {best['time_ms']} ms  "
-                f"variant {best['variant']} splits {best['k_splits']} ({best['kernel']})")
+                f"variant {best['variant']} splits {best['k_splits']} ({best['kernel']}){vendor}")
     return results
 
 
@@ -145,16 +166,17 @@ def main(argv=None):
     ap = argparse.ArgumentParser(description=__doc__.split("\n")[0])
     ap.add_argument("--input", required=True, help="shape list (csv: m,n,k,transA,transB,alpha,beta,...)")
     ap.add_argument("--type", default="f16", choices=sorted(_OUT_FOR))
-    ap.add_argument("--out-type", default=None, choices=["f32", "f16", "bf16", "i32"])
+    ap.add_argument("--out-type", default=None, choices=["f32", "f16", "bf16", "i32", "i16", "i8"])
     ap.add_argument("--relu", action="store_true", help="fused ReLU epilogue (rows with alpha != 1 are rejected)")
     ap.add_argument("--check", action="store_true", help="verify every variant against a NumPy product on sampled rows")
     ap.add_argument("--output", default=None, help="csv of all (shape, variant) results")
     ap.add_argument("--min-time", type=float, default=0.05, help="seconds of timed launches per variant")
+    ap.add_argument("--baseline", action="store_true", help="also time the vendor GEMM library (torch.matmul) on each shape")
     args = ap.parse_args(argv)
     with open(args.input) as f:
         rows = [r for r in csv.DictReader(f) if r.get("m")]
     _lib.check(_lib.lib().acc950_init(0))
-    results = sweep(rows, args.type, args.relu, args.check, args.out_type, args.min_time)
+    results = sweep(rows, args.type, args.relu, args.check, args.out_type, args.min_time, baseline=args.baseline)
     if args.output and results:
         with open(args.output, "w", newline="") as f:
             w = csv.DictWriter(f, fieldnames=list(results[0]))

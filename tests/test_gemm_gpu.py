@@ -200,6 +200,56 @@ def test_strided_views_with_padding():
     assert np.all(got[:, N:] == -5.0)  # padding untouched
 
 
+@pytest.mark.parametrize("in_type,out_type,pad", [("f16", "f32", 3), ("f16", "f16", 8), ("f16", "f16", 3), ("bf16", "bf16", 5),
+                                                  ("i8", "i32", 1), ("i8", "i16", 3), ("i8", "i16", 8), ("i8", "i8", 16),
+                                                  pytest.param("i8", "i8", 7, marks=pytest.mark.skip(
+                                                      reason="byte-wise stores to rows at odd distances faulted the GPU in the large-tile kernel; cause "
+                                                             "not found, path switched off: the library now refuses the variant for such a C"))])
+def test_large_tile_kernels_on_padded_output_rows(in_type, out_type, pad):
+    """Every store path of the 16x16-shape kernels: rows of C that are / are not 16-byte multiples apart
+    (whole-row pieces through LDS, or single elements), overwriting and accumulating, padding untouched."""
+    import accera_amd as acc
+    import torch
+    from accera_amd import _lib
+    mi16 = [v for v in range(_lib.num_variants()) if "mi16" in _lib.variant_name(v) and "256x256 kb64" in _lib.variant_name(v)
+            and "B=row-major" in _lib.variant_name(v) and "A=col" not in _lib.variant_name(v)]
+    assert mi16
+    M, N, K = 512, 256, 256
+    rng = np.random.default_rng(500 + pad)
+    A, B = make_input(rng, (M, K), in_type), make_input(rng, (K, N), in_type)
+    fill = 77 if out_type in INT_OUT else None
+    for prologue in (ora.PRO_SET0, ora.PRO_NONE):
+        Cbig = make_c0(rng, (M, N + pad), out_type)
+        dC = to_device(Cbig, out_type)
+        acc.gemm_relu(to_device(A, in_type), to_device(B, in_type), dC[:, :N], prologue=prologue, variant=mi16[0])
+        torch.cuda.synchronize()
+        got = to_host(dC, out_type)
+        want = ora.gemm_relu_exact(A, B, np.ascontiguousarray(Cbig[:, :N]), in_type, out_type, prologue, ora.EPI_RELU)
+        assert_matches(got[:, :N], want, out_type, K)
+        assert np.array_equal(got[:, N:], Cbig[:, N:]), "padding columns were written"
+
+
+def test_int8_output_rows_at_odd_distances_take_the_thread_bound_kernel():
+    """int8 C whose rows are not 16 bytes apart: every MFMA variant refuses, the automatic choice falls back."""
+    import accera_amd as acc
+    import torch
+    from accera_amd import _lib
+    M, N, K, pad = 512, 256, 256, 7
+    g, b, lds, v = _lib.launch_geometry(_lib.I8, _lib.I8, M, N, K, (K, 1), (N, 1), (N + pad, 1))
+    assert v == _lib.VARIANT_GENERIC
+    with pytest.raises(_lib.Acc950Error):
+        _lib.launch_geometry(_lib.I8, _lib.I8, M, N, K, (K, 1), (N, 1), (N + pad, 1), 0, 0)
+    rng = np.random.default_rng(507)
+    A, B = make_input(rng, (M, K), "i8"), make_input(rng, (K, N), "i8")
+    Cbig = make_c0(rng, (M, N + pad), "i8")
+    dC = to_device(Cbig, "i8")
+    acc.gemm_relu(to_device(A, "i8"), to_device(B, "i8"), dC[:, :N], prologue=acc.PROLOGUE_NONE)
+    torch.cuda.synchronize()
+    got = to_host(dC, "i8")
+    assert_matches(got[:, :N], ora.gemm_relu_exact(A, B, np.ascontiguousarray(Cbig[:, :N]), "i8", "i8", ora.PRO_NONE, ora.EPI_RELU), "i8", K)
+    assert np.array_equal(got[:, N:], Cbig[:, N:])
+
+
 # ---- fp32 kernel ------------------------------------------------------------------------------
 @pytest.mark.parametrize("shape", [(512, 512, 512), (64, 32, 8), (100, 70, 52), (33, 47, 29), (256, 256, 1000)])
 @pytest.mark.parametrize("b_layout", ["row", "col"])
@@ -503,6 +553,13 @@ def test_sweep_tool_checks_and_times_every_variant():
     assert len(res) >= 8 and all(r["correct"] is True for r in res), [r for r in res if r["correct"] is not True]
     res = tune.sweep(rows[:1], "i8", relu=True, check=True, min_time_s=0.002, log=lambda *_: None)
     assert res and all(r["correct"] is True for r in res)
+    res = tune.sweep(rows[:1], "i8", relu=True, check=True, out_type="i16", min_time_s=0.002, log=lambda *_: None)
+    assert res and all(r["correct"] is True for r in res)
+    # the vendor-library yardstick adds one row per shape and does not touch the verdicts
+    lines = []
+    res = tune.sweep(rows[:2], "f16", relu=False, check=True, min_time_s=0.002, log=lines.append, baseline=True)
+    assert sum(r["variant"] == -2 for r in res) == 2 and all("vendor library" in l for l in lines)
+    assert all(r["correct"] is True for r in res if r["variant"] != -2)
 
 
 # ---- error behaviour of the C ABI ---------------------------------------------------------------
