@@ -338,7 +338,10 @@ int run(const Problem& pb, const Choice& c, hipStream_t stream, LaunchGeom* geom
     } else {
         int n = 0;
         const MfmaVariant* tab = mfma_table(g.in_type, &n);
-        e = tab[c.variant].launch(g, stream, geom, dry_run);
+        // kernels with a lean build take C = A*B and C = relu(A*B) there, everything else in the full build
+        const MfmaVariant& mv = tab[c.variant];
+        const bool lean = g.prologue == PRO_SET && g.prologue_arg == 0.f && (g.epilogue == EPI_RELU || g.epilogue == EPI_NONE);
+        e = (mv.launch_general && !lean ? mv.launch_general : mv.launch)(g, stream, geom, dry_run);
     }
     if (e != hipSuccess) return fail_hip(e, "kernel launch");
     return ACC950_OK;
@@ -489,7 +492,7 @@ int acc950_mfma_phase_probe(int in_type, int out_type, int M, int N, int K, cons
     Problem pb;
     int rc = make_problem(in_type, out_type, M, N, K, A, K, 1, B, N, 1, C, N, 1, PRO_SET0, EPI_RELU, true, &pb);
     if (rc) return rc;
-    const MfmaVariant probe = {256, 256, 2, 4, true, false, true, false, 64, 4, true, false, nullptr};
+    const MfmaVariant probe = {256, 256, 2, 4, true, false, true, false, 64, 4, true, false, nullptr, nullptr};
     int n_unused = 0;
     if (M < 256 || N < 256 || K < 1 || !mfma_table(pb.g.in_type, &n_unused) || !mfma_can_take(probe, pb))
         return fail(ACC950_UNSUPPORTED, "the phase probe runs the 256x256 ping-pong kernel: 8/16-bit inputs, dense row-major A, B, C, M and N multiples of 256, K of 64 bytes");

@@ -33,9 +33,11 @@ __device__ __forceinline__ void mfma16(const i32x4& cols, const i32x4& rows, typ
         c = __builtin_amdgcn_mfma_i32_16x16x64_i8(cols, rows, c, 0, 0, 0);
 }
 
-template <int IN_, int BM_, int BN_, int WAVES_M_, int WAVES_N_, bool A_KC_, bool B_KC_, int KB_, int STAGES_, bool TIMED_ = false>
+// GENERAL: the build that carries every prologue / epilogue op; the other build takes only C = A*B
+// and C = relu(A*B) (SET 0 prologue) and is kept free of scratch use, which costs 4-20 us per dispatch.
+template <int IN_, int BM_, int BN_, int WAVES_M_, int WAVES_N_, bool A_KC_, bool B_KC_, int KB_, int STAGES_, bool GENERAL_ = false, bool TIMED_ = false>
 struct Mfma16Config {
-    static constexpr bool TIMED = TIMED_;
+    static constexpr bool TIMED = TIMED_, GENERAL = GENERAL_;
     static constexpr int IN = IN_, BM = BM_, BN = BN_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_, KB = KB_, STAGES = STAGES_;
     static constexpr bool A_KC = A_KC_, B_KC = B_KC_;
     static constexpr int NT = WAVES_M * WAVES_N * 64;
@@ -186,72 +188,14 @@ __global__ void __launch_bounds__(Cfg::NT, 1) gemm_mfma16_kernel(GemmArgs p)
     if (group == 0) raw_barrier(); // match the extra barrier of the other group
 
     stamp(2);
-    // ---- write-back: A. acc += (beta *) C, B. SET constant and epilogue op, C. store.
+    // ---- write-back.  Two leaves, chosen once: the fused matmul + ReLU (SET 0 prologue: C is not
+    // read, one max per element on the way out) and everything else (acc += (beta *) C, SET constant,
+    // epilogue op, then the same stores).  No accumulator changes on one side of a branch and is
+    // used after it, so the register allocator never has two versions of the tile to merge -- that
+    // merging used to push a few registers into scratch, and a kernel that uses scratch at all
+    // pays 4 us (256 workgroups) to 20 us (1024) more per dispatch on this device.
     // In block (i, j) lane l holds row i*16 + l%16 and columns j*16 + (l/16)*4 .. +3 of the wave tile.
     const int lrow = wr0 + (lane & 15), lcol = wc0 + (lane >> 4) * 4;
-    if (p.prologue != PRO_SET) {
-        // One copy for all output types: the aligned dword that holds the element is read and the
-        // element cut out of it (a switch over the load widths would leave the register
-        // allocator one version of every accumulator per type to merge).
-        const scalar_t c_mul = p.prologue == PRO_SCALE ? (scalar_t)p.prologue_arg : scalar_t(1); // x1 is exact
-        const unsigned sh = (p.out_type == T_I32 || p.out_type == T_F32) ? 2 : (p.out_type == T_I8 ? 0 : 1);
-        const unsigned m_f32 = p.out_type == T_F32 ? ~0u : 0u, m_f16 = p.out_type == T_F16 ? ~0u : 0u, m_bf16 = p.out_type == T_BF16 ? ~0u : 0u;
-        char* tile_base = (char*)p.C + (((int64_t)m0 * p.c_rs + n0) << sh);
-        const unsigned base_mis = (unsigned)(size_t)tile_base & 3u; // the descriptor starts at the dword that holds the tile's first element
-        const CTile tile = c_tile(tile_base - base_mis);
-        const unsigned row_bytes = (unsigned)p.c_rs << sh;
-        const unsigned lane_off = base_mis + (unsigned)lrow * row_bytes + ((unsigned)lcol << sh);
-#pragma unroll
-        for (int i = 0; i < TM; ++i) {
-#pragma unroll
-            for (int j = 0; j < TN; ++j)
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const unsigned off = lane_off + ((unsigned)(i * 16) * row_bytes + ((unsigned)(j * 16 + e) << sh));
-                    const unsigned mis = off & 3u; // byte of the element inside its dword
-                    const unsigned word = __builtin_amdgcn_raw_buffer_load_b32(tile.rsrc, off - mis, 0, 0);
-                    if constexpr (IN == IN_I8) { // int16 / int8 widen with their sign
-                        const int c = sh == 2 ? (int)word : __builtin_amdgcn_sbfe((int)word, mis * 8, 8u << sh);
-                        acc[i][j][e] = wrap_add(acc[i][j][e], wrap_mul(c, c_mul));
-                    } else {
-                        const unsigned half = word >> (mis * 8);
-                        const unsigned as_f16 = __float_as_uint((float)__builtin_bit_cast(_Float16, (unsigned short)half));
-                        const unsigned bits = (word & m_f32) | (as_f16 & m_f16) | ((half << 16) & m_bf16);
-                        acc[i][j][e] += __uint_as_float(bits) * c_mul;
-                    }
-                }
-            __builtin_amdgcn_sched_barrier(0); // block row by block row: loads stay near their use
-        }
-    }
-
-    auto for_each_acc = [&](auto&& fn) {
-#pragma unroll
-        for (int i = 0; i < TM; ++i) {
-#pragma unroll
-            for (int j = 0; j < TN; ++j)
-#pragma unroll
-                for (int e = 0; e < 4; ++e) acc[i][j][e] = fn(acc[i][j][e]);
-            __builtin_amdgcn_sched_barrier(0);
-        }
-    };
-    if (p.epilogue == EPI_RELU && !(p.prologue == PRO_SET && p.prologue_arg != 0.f)) {
-        for_each_acc([&](scalar_t v) { return v > scalar_t(0) ? v : scalar_t(0); }); // the fused hot path: one max per element
-    } else if (p.epilogue != EPI_NONE || (p.prologue == PRO_SET && p.prologue_arg != 0.f)) {
-        const scalar_t set_value = p.prologue == PRO_SET ? (scalar_t)p.prologue_arg : scalar_t(0);
-        const scalar_t epi_arg = (scalar_t)p.epilogue_arg;
-        const bool is_relu = p.epilogue == EPI_RELU, is_nocond = p.epilogue == EPI_RELU_NOCOND, is_scale = p.epilogue == EPI_SCALE,
-                   is_set = p.epilogue == EPI_SET;
-        for_each_acc([&](scalar_t v) {
-            v = wrap_add(v, set_value);
-            const scalar_t r = v > scalar_t(0) ? v : scalar_t(0);
-            const scalar_t n = v * (v > scalar_t(0) ? scalar_t(1) : scalar_t(0));
-            const scalar_t m = wrap_mul(v, epi_arg);
-            return is_relu ? r : (is_nocond ? n : (is_scale ? m : (is_set ? epi_arg : v)));
-        });
-    }
-    __builtin_amdgcn_sched_barrier(0);
-
-    // ---- pass C
     const unsigned os = p.out_type == T_I8 ? 1 : (p.out_type == T_F32 || p.out_type == T_I32) ? 4 : 2;
     const int wave_u = __builtin_amdgcn_readfirstlane(wave);
     // the four values of a block narrowed to the output type, packed in column order
@@ -269,6 +213,9 @@ __global__ void __launch_bounds__(Cfg::NT, 1) gemm_mfma16_kernel(GemmArgs p)
     auto pack_i8 = [](const acc_t& v) -> int {
         return (int)(((unsigned)v[0] & 0xffu) | (((unsigned)v[1] & 0xffu) << 8) | (((unsigned)v[2] & 0xffu) << 16) | ((unsigned)v[3] << 24));
     };
+    // pass C: fin(v) is the last elementwise step (ReLU in the fused leaf, identity otherwise)
+    auto store_tile = [&](auto&& fin) {
+        auto fin4 = [&](const acc_t& v) { return acc_t{fin(v[0]), fin(v[1]), fin(v[2]), fin(v[3])}; };
     if (os == 4) {
         // one 16-byte store per block and lane
         const CTile tile = c_tile((char*)p.C + ((int64_t)m0 * p.c_rs + n0) * 4);
@@ -278,7 +225,7 @@ __global__ void __launch_bounds__(Cfg::NT, 1) gemm_mfma16_kernel(GemmArgs p)
         for (int i = 0; i < TM; ++i)
 #pragma unroll
             for (int j = 0; j < TN; ++j)
-                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, acc[i][j]), tile.rsrc, lane_off + j * 64,
+                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, fin4(acc[i][j])), tile.rsrc, lane_off + j * 64,
                                                        (unsigned)(i * 16) * row_bytes, 0);
     } else if ((p.c_rs * os) % 16 == 0 && ((size_t)p.C & 15) == 0) {
         // narrow outputs: 16 rows of the wave tile are put together in a wave-private slab of the
@@ -299,7 +246,7 @@ __global__ void __launch_bounds__(Cfg::NT, 1) gemm_mfma16_kernel(GemmArgs p)
             for (int i = 0; i < TM; ++i) {
 #pragma unroll
                 for (int j = 0; j < TN; ++j) {
-                    auto w = pack(acc[i][j]);
+                    auto w = pack(fin4(acc[i][j]));
                     *(decltype(w)*)(mine + j * 16 * OS) = w;
                 }
 #pragma unroll
@@ -332,7 +279,7 @@ __global__ void __launch_bounds__(Cfg::NT, 1) gemm_mfma16_kernel(GemmArgs p)
 #pragma unroll
                 for (int j = 0; j < TN; ++j) {
                     const unsigned so = (unsigned)(i * 16) * row_bytes + (unsigned)(j * 16) * OS;
-                    auto w = pack(acc[i][j]);
+                    auto w = pack(fin4(acc[i][j]));
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
                         static_assert(OS == 2, "16-bit elements");
@@ -347,6 +294,70 @@ __global__ void __launch_bounds__(Cfg::NT, 1) gemm_mfma16_kernel(GemmArgs p)
             if (p.out_type == T_F16) by_element(std::integral_constant<int, 2>{}, pack_f16);
             else by_element(std::integral_constant<int, 2>{}, pack_bf16);
         }
+    }
+
+    };
+
+    if constexpr (!Cfg::GENERAL) {
+        // the host sends only SET 0 + ReLU / no epilogue here
+        if (p.epilogue == EPI_RELU) store_tile([](scalar_t v) { return v > scalar_t(0) ? v : scalar_t(0); });
+        else store_tile([](scalar_t v) { return v; });
+    } else {
+        // pass A, one copy for all output types: the aligned dword that holds the element is read and
+        // the element cut out of it; the loads of a block row sit behind one uniform branch, the
+        // arithmetic does not (c = 0 when C is not read).
+        const bool read_c = p.prologue != PRO_SET;
+        const scalar_t c_mul = p.prologue == PRO_SCALE ? (scalar_t)p.prologue_arg : scalar_t(read_c ? 1 : 0); // x1 is exact
+        const unsigned sh = (p.out_type == T_I32 || p.out_type == T_F32) ? 2 : (p.out_type == T_I8 ? 0 : 1);
+        const unsigned m_f32 = p.out_type == T_F32 ? ~0u : 0u, m_f16 = p.out_type == T_F16 ? ~0u : 0u, m_bf16 = p.out_type == T_BF16 ? ~0u : 0u;
+        char* tile_base = (char*)p.C + (((int64_t)m0 * p.c_rs + n0) << sh);
+        const unsigned base_mis = (unsigned)(size_t)tile_base & 3u; // the descriptor starts at the dword that holds the tile's first element
+        const CTile tile = c_tile(tile_base - base_mis);
+        const unsigned row_bytes = (unsigned)p.c_rs << sh;
+        const unsigned lane_off = base_mis + (unsigned)lrow * row_bytes + ((unsigned)lcol << sh);
+        // pass B operands: SET constant and the epilogue op as wave-uniform selects
+        const scalar_t set_value = p.prologue == PRO_SET ? (scalar_t)p.prologue_arg : scalar_t(0);
+        const scalar_t epi_arg = (scalar_t)p.epilogue_arg;
+        // (blended with masks: a select on a wave-uniform condition comes back as a branch per element)
+        const unsigned k_relu = p.epilogue == EPI_RELU ? ~0u : 0u, k_nocond = p.epilogue == EPI_RELU_NOCOND ? ~0u : 0u,
+                       k_scale = p.epilogue == EPI_SCALE ? ~0u : 0u, k_set = p.epilogue == EPI_SET ? ~0u : 0u,
+                       k_none = p.epilogue == EPI_NONE ? ~0u : 0u;
+        auto bits = [](scalar_t x) { return __builtin_bit_cast(unsigned, x); };
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                scalar_t c[4] = {scalar_t(0), scalar_t(0), scalar_t(0), scalar_t(0)};
+                if (read_c) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const unsigned off = lane_off + ((unsigned)(i * 16) * row_bytes + ((unsigned)(j * 16 + e) << sh));
+                        const unsigned mis = off & 3u; // byte of the element inside its dword
+                        const unsigned word = __builtin_amdgcn_raw_buffer_load_b32(tile.rsrc, off - mis, 0, 0);
+                        if constexpr (IN == IN_I8) { // int16 / int8 widen with their sign
+                            c[e] = sh == 2 ? (int)word : __builtin_amdgcn_sbfe((int)word, mis * 8, 8u << sh);
+                        } else {
+                            const unsigned half = word >> (mis * 8);
+                            const unsigned as_f16 = __float_as_uint((float)__builtin_bit_cast(_Float16, (unsigned short)half));
+                            c[e] = __uint_as_float((word & m_f32) | (as_f16 & m_f16) | ((half << 16) & m_bf16));
+                        }
+                    }
+                }
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    scalar_t v;
+                    if constexpr (IN == IN_I8) v = wrap_add(acc[i][j][e], wrap_mul(c[e], c_mul));
+                    else v = acc[i][j][e] + c[e] * c_mul;
+                    v = wrap_add(v, set_value);
+                    const scalar_t r = v > scalar_t(0) ? v : scalar_t(0);
+                    const scalar_t n = v * (v > scalar_t(0) ? scalar_t(1) : scalar_t(0));
+                    const scalar_t m = wrap_mul(v, epi_arg);
+                    acc[i][j][e] = __builtin_bit_cast(scalar_t, (bits(r) & k_relu) | (bits(n) & k_nocond) | (bits(m) & k_scale) |
+                                                                    (bits(epi_arg) & k_set) | (bits(v) & k_none));
+                }
+                __builtin_amdgcn_sched_barrier(0); // block by block: a handful of temporaries next to the 128 accumulators
+            }
+        store_tile([](scalar_t v) { return v; });
     }
 
     if constexpr (Cfg::TIMED) {

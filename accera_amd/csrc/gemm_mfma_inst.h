@@ -13,14 +13,15 @@ namespace acc950 {
 
 #define VA(AKC, BM, BN, WM, WN, BKC, DIRECT, EDGE, KB, STAGES)                                         \
     { BM, BN, WM, WN, AKC, BKC, DIRECT, EDGE, KB, STAGES, false, false,                                \
-      &launch_mfma<MfmaConfig<ACC950_IN, BM, BN, WM, WN, AKC, BKC, DIRECT, EDGE, KB, STAGES>> }
+      &launch_mfma<MfmaConfig<ACC950_IN, BM, BN, WM, WN, AKC, BKC, DIRECT, EDGE, KB, STAGES>>, nullptr }
 #define VPA(AKC, BM, BN, WM, WN, BKC, KB, STAGES)                                                       \
     { BM, BN, WM, WN, AKC, BKC, true, false, KB, STAGES, true, false,                                  \
-      &launch_mfma<MfmaConfig<ACC950_IN, BM, BN, WM, WN, AKC, BKC, true, false, KB, STAGES, true>> }
+      &launch_mfma<MfmaConfig<ACC950_IN, BM, BN, WM, WN, AKC, BKC, true, false, KB, STAGES, true>>, nullptr }
 // ping-pong on the 16x16 MFMA shapes
 #define V16(AKC, BM, BN, WM, WN, BKC, KB, STAGES)                                                       \
     { BM, BN, WM, WN, AKC, BKC, true, false, KB, STAGES, true, true,                                   \
-      &launch_mfma16<Mfma16Config<ACC950_IN, BM, BN, WM, WN, AKC, BKC, KB, STAGES>> }
+      &launch_mfma16<Mfma16Config<ACC950_IN, BM, BN, WM, WN, AKC, BKC, KB, STAGES, false>>,           \
+      &launch_mfma16<Mfma16Config<ACC950_IN, BM, BN, WM, WN, AKC, BKC, KB, STAGES, true>> }
 #define V(BM, BN, WM, WN, BKC, DIRECT, EDGE, KB, STAGES) VA(true, BM, BN, WM, WN, BKC, DIRECT, EDGE, KB, STAGES)
 #define VP(BM, BN, WM, WN, BKC, KB, STAGES) VPA(true, BM, BN, WM, WN, BKC, KB, STAGES)
 // column-major A (M contiguous; the "transA" shapes of the reference's sweep lists,
@@ -75,7 +76,7 @@ static const MfmaVariant kVariants[] = {
 // (256x256 ping-pong on the 16x16 MFMA shapes, row-major B): same code plus four clock stamps per workgroup.
 hipError_t ACC950_TIMED_FN(const GemmArgs& a, hipStream_t stream, LaunchGeom* geom, bool dry_run)
 {
-    return launch_mfma16<Mfma16Config<ACC950_IN, 256, 256, 2, 4, true, false, 64, 4, true>>(a, stream, geom, dry_run);
+    return launch_mfma16<Mfma16Config<ACC950_IN, 256, 256, 2, 4, true, false, 64, 4, false, true>>(a, stream, geom, dry_run);
 }
 
 const MfmaVariant* ACC950_TABLE_FN(int* count)

@@ -15,6 +15,7 @@ struct MfmaVariant {
     bool pingpong;       // sibling waves alternate memory and compute clusters
     bool mi16;           // 16x16 MFMA shapes (else 32x32)
     LaunchFn launch;
+    LaunchFn launch_general; // build that carries every prologue / epilogue op, when `launch` is a lean build (else null)
 };
 
 const MfmaVariant* mfma_variants_f16(int* count);
