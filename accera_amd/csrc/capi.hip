@@ -240,7 +240,10 @@ int auto_mfma_variant(const Problem& pb)
         // rank inside one tile shape: ping-pong kb64 x4 > ping-pong others > 8-wave > 4-wave (kb64 x4 first)
         int rank = v.pingpong ? (v.kb == 64 && v.stages == 4 ? 8 : 6) : (v.waves_m * v.waves_n == 8 ? 4 : 2);
         if (!v.pingpong && v.kb == 64 && v.stages == 4) rank += 1;
-        if (v.mi16) rank += 4; // measured 4-9 % faster than the 32x32 shapes on every large problem
+        // 16x16 shapes: measured 4-9 % faster than the 32x32 shapes on every large problem, in the lean build
+        // (C = A*B, C = relu(A*B)); their full build reads C element by element and lost 20 % to the 32x32 form
+        const bool lean = pb.g.prologue == PRO_SET && pb.g.prologue_arg == 0.f && (pb.g.epilogue == EPI_RELU || pb.g.epilogue == EPI_NONE);
+        if (v.mi16) rank += lean ? 4 : -8;
         const bool better = best < 0 || cost < best_cost * 0.999 ||
                             (cost <= best_cost * 1.001 && ((int64_t)v.bm * v.bn > (int64_t)tab[best].bm * tab[best].bn ||
                                                            ((int64_t)v.bm * v.bn == (int64_t)tab[best].bm * tab[best].bn && rank > best_rank)));

@@ -482,7 +482,8 @@ def _match(source):
 
 def _variant_for_tile(spec, bm, bn):
     """Best-ranked MFMA variant with block tile bm x bn that accepts the problem, else VARIANT_AUTO."""
-    best = _lib.VARIANT_AUTO
+    best, best_rank = _lib.VARIANT_AUTO, -9
+    lean = spec.prologue == _lib.PROLOGUE_SET and spec.prologue_arg == 0 and spec.epilogue in (_lib.EPILOGUE_RELU, _lib.EPILOGUE_NONE)
     for v in range(_lib.num_variants()):
         name = _lib.variant_name(v)
         if f"mfma {bm}x{bn} " not in name:
@@ -492,8 +493,10 @@ def _variant_for_tile(spec, bm, bn):
                                  spec.A.strides[-2:], spec.B.strides[-2:], spec.C.strides[-2:], v, 0)
         except _lib.Acc950Error:
             continue
-        if best == _lib.VARIANT_AUTO or ("pingpong" in name and "pingpong" not in _lib.variant_name(best)):
-            best = v
+        # ping-pong over software-pipelined; the 16x16 MFMA shapes where the library runs their lean build
+        rank = 2 * ("pingpong" in name) + (1 if "mi16" in name and lean else -1 if "mi16" in name else 0)
+        if best == _lib.VARIANT_AUTO or rank > best_rank:
+            best, best_rank = v, rank
     return best
 
 
