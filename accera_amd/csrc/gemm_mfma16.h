@@ -303,16 +303,21 @@ __global__ void __launch_bounds__(Cfg::NT, 1) gemm_mfma16_kernel(GemmArgs p)
         if (p.epilogue == EPI_RELU) store_tile([](scalar_t v) { return v > scalar_t(0) ? v : scalar_t(0); });
         else store_tile([](scalar_t v) { return v; });
     } else {
-        // pass A, one copy for all output types: the aligned dword that holds the element is read and
-        // the element cut out of it; the loads of a block row sit behind one uniform branch, the
-        // arithmetic does not (c = 0 when C is not read).
+        // pass A: the four elements of C a lane owns in a block arrive in one load -- 16 bytes (32-bit
+        // elements), or the 12 / 8 bytes from the dword boundary below them (16- / 8-bit elements, rows
+        // of C may start at any element), realigned with v_alignbyte.  The loads of a block sit behind
+        // one uniform branch per element width; the arithmetic does not (c = 0 when C is not read).
+        // The descriptor ends with the last row of C, so the few bytes a realigned load reads past its
+        // elements are never fetched from beyond the matrix.
         const bool read_c = p.prologue != PRO_SET;
         const scalar_t c_mul = p.prologue == PRO_SCALE ? (scalar_t)p.prologue_arg : scalar_t(read_c ? 1 : 0); // x1 is exact
         const unsigned sh = (p.out_type == T_I32 || p.out_type == T_F32) ? 2 : (p.out_type == T_I8 ? 0 : 1);
-        const unsigned m_f32 = p.out_type == T_F32 ? ~0u : 0u, m_f16 = p.out_type == T_F16 ? ~0u : 0u, m_bf16 = p.out_type == T_BF16 ? ~0u : 0u;
+        const unsigned m_f16 = p.out_type == T_F16 ? ~0u : 0u, m_bf16 = p.out_type == T_BF16 ? ~0u : 0u;
         char* tile_base = (char*)p.C + (((int64_t)m0 * p.c_rs + n0) << sh);
         const unsigned base_mis = (unsigned)(size_t)tile_base & 3u; // the descriptor starts at the dword that holds the tile's first element
-        const CTile tile = c_tile(tile_base - base_mis);
+        // (up to the end of the dword that holds the last element: the range check is per dword)
+        const int64_t c_bytes_left = (((((int64_t)(p.M - 1 - m0)) * p.c_rs + (p.N - n0)) << sh) + base_mis + 3) & ~(int64_t)3;
+        const CTile tile = CTile{__builtin_amdgcn_make_buffer_rsrc(tile_base - base_mis, 0, (int)(unsigned)(c_bytes_left < 0xffffffffll ? c_bytes_left : 0xffffffffll), 0x00020000)};
         const unsigned row_bytes = (unsigned)p.c_rs << sh;
         const unsigned lane_off = base_mis + (unsigned)lrow * row_bytes + ((unsigned)lcol << sh);
         // pass B operands: SET constant and the epilogue op as wave-uniform selects
@@ -329,17 +334,36 @@ __global__ void __launch_bounds__(Cfg::NT, 1) gemm_mfma16_kernel(GemmArgs p)
             for (int j = 0; j < TN; ++j) {
                 scalar_t c[4] = {scalar_t(0), scalar_t(0), scalar_t(0), scalar_t(0)};
                 if (read_c) {
+                    const unsigned off = lane_off + ((unsigned)(i * 16) * row_bytes + ((unsigned)(j * 16) << sh));
+                    const unsigned mis = off & 3u; // bytes between the dword boundary and the first element
+                    if (sh == 2) {
+                        // (the builtins return GCC-style vectors; assigning one to an ext_vector type compiles, to something else)
+                        const u32x4 w = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(tile.rsrc, off, 0, 0));
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        const unsigned off = lane_off + ((unsigned)(i * 16) * row_bytes + ((unsigned)(j * 16 + e) << sh));
-                        const unsigned mis = off & 3u; // byte of the element inside its dword
-                        const unsigned word = __builtin_amdgcn_raw_buffer_load_b32(tile.rsrc, off - mis, 0, 0);
-                        if constexpr (IN == IN_I8) { // int16 / int8 widen with their sign
-                            c[e] = sh == 2 ? (int)word : __builtin_amdgcn_sbfe((int)word, mis * 8, 8u << sh);
-                        } else {
-                            const unsigned half = word >> (mis * 8);
-                            const unsigned as_f16 = __float_as_uint((float)__builtin_bit_cast(_Float16, (unsigned short)half));
-                            c[e] = __uint_as_float((word & m_f32) | (as_f16 & m_f16) | ((half << 16) & m_bf16));
+                        for (int e = 0; e < 4; ++e) {
+                            const unsigned x = w[e]; // (a bit cast applied to the element expression itself reads element 0 with this compiler)
+                            c[e] = __builtin_bit_cast(scalar_t, x);
+                        }
+                    } else if (sh == 1) {
+                        typedef unsigned u32x3 __attribute__((ext_vector_type(3)));
+                        const u32x3 w = __builtin_bit_cast(u32x3, __builtin_amdgcn_raw_buffer_load_b96(tile.rsrc, off - mis, 0, 0));
+                        const unsigned lo = __builtin_amdgcn_alignbyte(w[1], w[0], mis), hi = __builtin_amdgcn_alignbyte(w[2], w[1], mis);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            const unsigned half = ((e & 2) ? hi : lo) >> ((e & 1) * 16);
+                            if constexpr (IN == IN_I8) c[e] = (int)(short)half; // int16 widens with its sign
+                            else {
+                                const unsigned as_f16 = __float_as_uint((float)__builtin_bit_cast(_Float16, (unsigned short)half));
+                                c[e] = __uint_as_float((as_f16 & m_f16) | ((half << 16) & m_bf16));
+                            }
+                        }
+                    } else {
+                        if constexpr (IN == IN_I8) {
+                            typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+                            const u32x2 w = __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(tile.rsrc, off - mis, 0, 0));
+                            const unsigned v4 = __builtin_amdgcn_alignbyte(w[1], w[0], mis);
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) c[e] = __builtin_amdgcn_sbfe((int)v4, e * 8, 8); // int8 widens with its sign
                         }
                     }
                 }

@@ -433,7 +433,9 @@ OPS = [(ora.PRO_SET, 0.0, ora.EPI_SCALE, 5.0), (ora.PRO_SCALE, 0.5, ora.EPI_NONE
 @pytest.mark.parametrize("case", [("f16", "f32", 256, 512, 256, -1), ("bf16", "bf16", 256, 384, 128, -1), ("i8", "i32", 256, 256, 512, -1),
                                   ("i8", "i16", 256, 256, 512, -1), ("i8", "i8", 256, 512, 256, -1), ("i8", "i8", 33, 47, 29, -1),
                                   ("f16", "f16", 200, 144, 176, -1), ("f32", "f32", 96, 80, 72, -1), ("f16", "f32", 33, 47, 29, 200),
-                                  ("f16", "f16", 8, 1088, 512, -1), ("bf16", "f32", 24, 1024, 256, -1), ("f16", "f16", 5, 1000, 998, -1)])
+                                  ("f16", "f16", 8, 1088, 512, -1), ("bf16", "f32", 24, 1024, 256, -1), ("f16", "f16", 5, 1000, 998, -1),
+                                  ("f16", "f32", 256, 512, 256, "mi16"), ("bf16", "bf16", 512, 256, 128, "mi16"), ("f16", "f16", 256, 256, 192, "mi16"),
+                                  ("i8", "i32", 256, 256, 512, "mi16"), ("i8", "i16", 256, 256, 256, "mi16"), ("i8", "i8", 256, 512, 256, "mi16")])
 def test_fragment_ops_alpha_beta(case):
     """C = epilogue(prologue(C) + A@B) for the SET / SCALE ops of the reference's tensorized plan
     (Tensor_MatMul_ElementWiseOps_GPU.md:85-99; helpers CppPrinterUtils.h:630-655), on the MFMA,
@@ -441,6 +443,10 @@ def test_fragment_ops_alpha_beta(case):
     import accera_amd as acc
     import torch
     in_type, out_type, M, N, K, variant = case
+    if variant == "mi16":  # the full build of the 16x16-shape kernel (the automatic choice keeps it for C = A*B and relu(A*B))
+        from accera_amd import _lib
+        variant = next(v for v in range(_lib.num_variants()) if "mi16" in _lib.variant_name(v) and "256x256 kb64" in _lib.variant_name(v)
+                       and "B=row-major" in _lib.variant_name(v) and "A=col" not in _lib.variant_name(v))
     for n, (pro, pa, epi, ea) in enumerate(OPS):
         rng = np.random.default_rng(300 + n)
         A, B = make_input(rng, (M, K), in_type), make_input(rng, (K, N), in_type)
