@@ -40,7 +40,10 @@ __global__ void __launch_bounds__(512) mfma_ceiling_kernel(const i32x4* src, flo
     const long long c1 = clock64(), w1 = wall_clock64();
     float s = 0;
     for (int j = 0; j < 16; ++j)
-        for (int r = 0; r < 4; ++r) s += IN == T_I8 ? (float)__builtin_bit_cast(int, acc[j][r]) : acc[j][r];
+        for (int r = 0; r < 4; ++r) {
+            const float x = acc[j][r];
+            s += IN == T_I8 ? (float)__float_as_int(x) : x;
+        }
     out[blockIdx.x * blockDim.x + threadIdx.x] = s;
     if (threadIdx.x == 0 && blockIdx.x == 0) { clk[0] = c1 - c0; clk[1] = w1 - w0; }
 }
