@@ -328,6 +328,7 @@ __global__ void __launch_bounds__(Cfg::NT, 1) gemm_mfma16_kernel(GemmArgs p)
                        k_scale = p.epilogue == EPI_SCALE ? ~0u : 0u, k_set = p.epilogue == EPI_SET ? ~0u : 0u,
                        k_none = p.epilogue == EPI_NONE ? ~0u : 0u;
         auto bits = [](scalar_t x) { return __builtin_bit_cast(unsigned, x); };
+        const bool simple = (p.epilogue == EPI_RELU || p.epilogue == EPI_NONE) && set_value == scalar_t(0);
 #pragma unroll
         for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -367,6 +368,17 @@ __global__ void __launch_bounds__(Cfg::NT, 1) gemm_mfma16_kernel(GemmArgs p)
                         }
                     }
                 }
+                if (simple) {
+                    // C = relu(C + A*B) or C + A*B, beta included: v, then max(v, 0) or max(v, v)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        scalar_t v;
+                        if constexpr (IN == IN_I8) v = wrap_add(acc[i][j][e], wrap_mul(c[e], c_mul));
+                        else v = acc[i][j][e] + c[e] * c_mul;
+                        const scalar_t lo = __builtin_bit_cast(scalar_t, bits(v) & k_none);
+                        acc[i][j][e] = v > lo ? v : lo;
+                    }
+                } else
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     scalar_t v;
