@@ -144,6 +144,40 @@ def cpu_baseline(c, threads, budget_rows=None):
                 sample=f"rows 0..{M - 1} of A against all of B ({M}x{N}x{K}), one pass, OpenMP over column tiles")
 
 
+def vendor_library(c, first_set, steps):
+    """The vendor GEMM library (torch.matmul -> hipBLASLt / rocBLAS, torch._int_mm for int8) on the same
+    operands: a yardstick beside the reference's own rocBLAS benchmarker
+    (/root/reference/tools/benchmarkers/rocblas/main.cpp).  It writes an output of the input type (int32 for
+    int8) and has no fused epilogue; nothing in the product path calls it."""
+    import torch
+    A, B, _ = first_set
+    try:
+        if c["in_type"] == "i8":
+            call = lambda: torch._int_mm(A, B)
+        else:
+            out = torch.empty((c["M"], c["N"]), dtype=A.dtype, device="cuda")
+            call = lambda: torch.matmul(A, B, out=out)
+        for _ in range(min(steps, 50)):
+            call()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        n = max(min(steps, 200), 10)
+        e0.record()
+        for _ in range(n):
+            call()
+        e1.record()
+        torch.cuda.synchronize()
+        dt = e0.elapsed_time(e1) * 1e-3 / n
+    except RuntimeError as e:
+        return {"error": str(e).splitlines()[0][:80]}
+    if c["bound"] == "hbm":
+        return {"value": round(algorithmic_bytes(c) / dt / 1e9, 1), "unit": "GB/s", "ms_per_step": round(dt * 1e3, 5),
+                "call": "torch.matmul, output of the input type, no epilogue"}
+    return {"value": round(algorithmic_flops(c) / dt / 1e12, 1), "unit": "TFLOP/s" if c["in_type"] != "i8" else "TOP/s",
+            "ms_per_step": round(dt * 1e3, 5),
+            "call": "torch._int_mm, int32 output, no epilogue" if c["in_type"] == "i8" else "torch.matmul, output of the input type, no epilogue"}
+
+
 def traffic_bytes(name):
     """HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE and scaled by the
     plain copy kernel of known size (written to profiles/traffic.json by accera_amd.profiling)."""
@@ -208,7 +242,8 @@ def measure(name, steps, warmup, variant=-1, k_splits=0):
     return dict(config=name, workload=c["workload"], value=round(value, 3), unit=vunit, ms_per_step=round(wall / steps * 1e3, 5),
                 roofline=dict(bound=c["bound"], achieved=round(achieved, 3), peak=peak, unit=unit,
                               frac=round(achieved / peak, 4), traffic=traffic_bytes(name)),
-                flops_per_launch=flops, bytes_per_launch=nbytes, in_kernel=in_kernel)
+                flops_per_launch=flops, bytes_per_launch=nbytes, in_kernel=in_kernel,
+                vendor_library=vendor_library(c, first_set, steps))
 
 
 def main():
@@ -256,6 +291,7 @@ def main():
         "roofline": m["roofline"],
         "machine_ceiling": machine_ceiling(c),
         "in_kernel": m["in_kernel"],
+        "vendor_library": m["vendor_library"],
     }
     if not args.no_cpu:
         threads = min(16, os.cpu_count() or 1)
