@@ -477,6 +477,14 @@ def _match(source):
         if i in first and j in first:
             spec.block_tile = (first[i], first[j])
             spec.variant = _variant_for_tile(spec, *spec.block_tile)
+    if spec.variant == _lib.VARIANT_AUTO and spec.batch is None:
+        # no tile named by the plan: a choice recorded for this very shape by `accera_amd.tune --save`, if any
+        from . import tuned
+        lean = spec.prologue == _lib.PROLOGUE_SET and spec.prologue_arg == 0 and spec.epilogue in (_lib.EPILOGUE_RELU, _lib.EPILOGUE_NONE)
+        hit = tuned.lookup(spec.A.element_type.lib_id, spec.C.element_type.lib_id, spec.M, spec.N, spec.K,
+                           spec.A.strides[-2:], spec.B.strides[-2:], spec.C.strides[-2:], lean)
+        if hit and hit[1] == 0:  # (package functions carry a variant, not a K split)
+            spec.variant = hit[0]
     return spec
 
 

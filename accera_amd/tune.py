@@ -11,6 +11,8 @@ tools/benchmarkers/gemm_*.csv; transX = 1 means the operand is stored column-maj
     NumPy product on sampled rows (rtol 1e-2 as the reference's driver),
   * times it with HIP events (min over batches of the mean time per launch),
   * writes one CSV row per (shape, variant) and prints the best variant per shape,
+  * with --save records the best variant per shape in the table the automatic choice consults
+    (accera_amd/tuned.py),
   * with --baseline also times the vendor GEMM library on the same operands (torch.matmul, i.e.
     hipBLASLt / rocBLAS; torch._int_mm for int8), the counterpart of the reference's rocBLAS
     benchmarker (/root/reference/tools/benchmarkers/rocblas/main.cpp).  The vendor call writes an
@@ -172,6 +174,9 @@ def main(argv=None):
     ap.add_argument("--output", default=None, help="csv of all (shape, variant) results")
     ap.add_argument("--min-time", type=float, default=0.05, help="seconds of timed launches per variant")
     ap.add_argument("--baseline", action="store_true", help="also time the vendor GEMM library (torch.matmul) on each shape")
+    ap.add_argument("--save", nargs="?", const="", default=None, metavar="JSON",
+                    help="record the best variant per shape in the table that automatic kernel choices consult "
+                         "(default: accera_amd/shapes/tuned_gfx950.json)")
     args = ap.parse_args(argv)
     with open(args.input) as f:
         rows = [r for r in csv.DictReader(f) if r.get("m")]
@@ -182,6 +187,10 @@ def main(argv=None):
             w = csv.DictWriter(f, fieldnames=list(results[0]))
             w.writeheader()
             w.writerows(results)
+    if args.save is not None and results:
+        from . import tuned
+        n = tuned.save(results, args.save or tuned.DEFAULT_PATH)
+        print(f"{n} shapes recorded in {args.save or tuned.DEFAULT_PATH}")
     bad = [r for r in results if r["correct"] is False]
     for r in bad:
         print(f"MISMATCH {r['m']}x{r['n']}x{r['k']} variant {r['variant']} ({r['kernel']})", file=sys.stderr)

@@ -111,6 +111,7 @@ def run_gpu(c, steps, warmup, variant=-1, k_splits=0):
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     launch_s = ev0.elapsed_time(ev1) * 1e-3 / steps
+    run_gpu.asked = (calls[0].variant, calls[0].k_splits)  # a recorded per-shape choice, or what the caller passed
     return wall, launch_s, sets[0]
 
 
@@ -278,7 +279,7 @@ def main():
     m = measure(args.config, args.steps, args.warmup, args.variant, args.k_splits)
     grid, block, lds, chosen = _lib.launch_geometry(
         getattr(_lib, c["in_type"].upper()), getattr(_lib, c["out_type"].upper()), c["M"], c["N"], c["K"],
-        (c["K"], 1), (c["N"], 1) if c["b"] == "row" else (1, c["K"]), (c["N"], 1), args.variant, args.k_splits)
+        (c["K"], 1), (c["N"], 1) if c["b"] == "row" else (1, c["K"]), (c["N"], 1), *run_gpu.asked)
     out = {
         "metric": "GEMM+ReLU TFLOP/s (TOPS int8) & % MFMA peak at 4096^3 fp16; skinny GEMM HBM GB/s",
         "value": m["value"], "unit": m["unit"], "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,

@@ -112,3 +112,32 @@ def test_bound_call_handles_without_launching():
     bad = list(args)
     bad[22] = 57 + 1000   # unknown variant
     assert L.acc950_bind(*bad, ctypes.byref(h)) == _lib.INVALID_ARGUMENT
+
+
+def test_tuned_table_is_consulted_by_name_and_validated(tmp_path, monkeypatch):
+    """accera_amd.tuned: entries name kernels by description; unknown kernels and kernels the library
+    refuses for the problem are ignored."""
+    from accera_amd import tuned
+    path = tmp_path / "tuned.json"
+    monkeypatch.setenv("ACCERA_AMD_TUNED", str(path))
+    rows = [dict(m=4096, n=4096, k=4096, transA=0, transB=0, alpha=1.0, beta=0.0, type="f16", out_type="f32", variant=1, k_splits=0,
+                 kernel=_lib.variant_name(1), time_ms=0.2, TFlops=1.0, correct=True),
+            dict(m=4096, n=4096, k=4096, transA=0, transB=0, alpha=1.0, beta=0.0, type="f16", out_type="f32", variant=0, k_splits=0,
+                 kernel=_lib.variant_name(0), time_ms=0.3, TFlops=1.0, correct=True),
+            dict(m=4096, n=4096, k=4096, transA=0, transB=0, alpha=1.0, beta=0.0, type="f16", out_type="f32", variant=5, k_splits=0,
+                 kernel=_lib.variant_name(5), time_ms=0.1, TFlops=1.0, correct=False),          # failed its check: never recorded
+            dict(m=1000, n=1000, k=1000, transA=0, transB=0, alpha=1.0, beta=0.0, type="f16", out_type="f32", variant=1, k_splits=0,
+                 kernel=_lib.variant_name(1), time_ms=0.1, TFlops=1.0, correct=True),           # kernel cannot take this shape
+            dict(m=512, n=512, k=512, transA=0, transB=0, alpha=1.0, beta=0.0, type="f16", out_type="f32", variant=1, k_splits=0,
+                 kernel="a kernel this library does not have", time_ms=0.1, TFlops=1.0, correct=True),
+            dict(m=4096, n=4096, k=4096, transA=0, transB=0, alpha=1.0, beta=0.0, type="f16", out_type="f32", variant=-2, k_splits=0,
+                 kernel="vendor library (torch.matmul)", time_ms=0.05, TFlops=1.0, correct="")]
+    assert tuned.save(rows, str(path)) == 3
+    tuned.reset()
+    args = (_lib.F16, _lib.F32, 4096, 4096, 4096, (4096, 1), (4096, 1), (4096, 1))
+    assert tuned.lookup(*args, True) == (1, 0)                 # fastest verified row
+    assert tuned.lookup(*args, False) is None                  # other op class: not recorded
+    assert tuned.lookup(_lib.F16, _lib.F32, 1000, 1000, 1000, (1000, 1), (1000, 1), (1000, 1), True) is None
+    assert tuned.lookup(_lib.F16, _lib.F32, 512, 512, 512, (512, 1), (512, 1), (512, 1), True) is None
+    assert tuned.lookup(_lib.F16, _lib.F32, 4096, 4096, 4096, (4096, 1), (4096, 1), (4100, 1), True) is None  # padded C: not a table shape
+    tuned.reset()
