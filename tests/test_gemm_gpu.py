@@ -586,3 +586,34 @@ def test_errors_are_reported_not_thrown():
         acc.gemm_relu(Ah, Ah.t(), Ch, variant=57)
     with pytest.raises(ValueError):
         acc.gemm_relu(Ah.cpu(), Ah.t(), Ch)  # no CPU path
+
+
+def test_random_problems_through_the_automatic_choice():
+    """Seeded random shapes, types, layouts and ops through the automatic kernel choice (MFMA tiles of
+    every size, edge and thread-bound kernels, skinny kernels), each checked against the oracle."""
+    import accera_amd as acc
+    import torch
+    rng = np.random.default_rng(2024)
+    pairs = [("f16", "f32"), ("f16", "f16"), ("bf16", "f32"), ("bf16", "bf16"), ("i8", "i32"), ("i8", "i16"), ("i8", "i8"), ("f32", "f32")]
+    ops = [(ora.PRO_SET0, 0.0, ora.EPI_RELU, 0.0), (ora.PRO_SET0, 0.0, ora.EPI_NONE, 0.0), (ora.PRO_NONE, 0.0, ora.EPI_RELU, 0.0),
+           (ora.PRO_SCALE, 0.5, ora.EPI_SCALE, 2.0), (ora.PRO_SET, 3.0, ora.EPI_RELU_NOCOND, 0.0), (ora.PRO_NONE, 0.0, ora.EPI_SET, 1.0)]
+    sizes_m = [1, 5, 8, 16, 31, 64, 100, 128, 200, 256, 384, 512, 768, 1024]
+    sizes_n = [8, 16, 40, 64, 72, 128, 192, 256, 384, 512, 768, 1000, 1024, 1088, 2048]
+    sizes_k = [16, 32, 64, 96, 128, 176, 256, 336, 512, 998, 1024, 2048]
+    for case in range(60):
+        in_type, out_type = pairs[rng.integers(len(pairs))]
+        M, N, K = (int(s[rng.integers(len(s))]) for s in (sizes_m, sizes_n, sizes_k))
+        pro, pa, epi, ea = ops[rng.integers(len(ops))]
+        a_col, b_col = bool(rng.integers(2)) and in_type != "f32", bool(rng.integers(2))
+        print("case", case, in_type, out_type, M, N, K, "A col" if a_col else "A row", "B col" if b_col else "B row", pro, pa, epi, ea, flush=True)
+        A, B = make_input(rng, (M, K), in_type), make_input(rng, (K, N), in_type)
+        if a_col:
+            A = np.asfortranarray(A)
+        if b_col:
+            B = np.asfortranarray(B)
+        C0 = make_c0(rng, (M, N), out_type, scale=100)
+        dC = to_device(C0, out_type)
+        acc.gemm_relu(to_device(A, in_type), to_device(B, in_type), dC, prologue=pro, prologue_arg=pa, epilogue=epi, epilogue_arg=ea)
+        torch.cuda.synchronize()
+        want = ora.gemm_relu_exact(A, B, C0, in_type, out_type, pro, epi, prologue_arg=pa, epilogue_arg=ea)
+        assert_matches(to_host(dC, out_type), want, out_type, K)
