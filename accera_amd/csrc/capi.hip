@@ -130,6 +130,12 @@ bool mfma_can_take(const MfmaVariant& v, const Problem& pb)
         if (g.c_rs % 16 || (g.batch > 1 && g.c_bs % 16)) return false;
         if (pb.have_pointers && !aligned16(g.C)) return false;
     }
+    if (v.w4) {
+        const bool lean = g.prologue == PRO_SET && g.prologue_arg == 0.f && (g.epilogue == EPI_RELU || g.epilogue == EPI_NONE);
+        const int os = elem_size(g.out_type);
+        if (!lean || g.K % (4 * bk) || (g.c_rs * os) % 16 || (g.batch > 1 && (g.c_bs * os) % 16)) return false;
+        if (pb.have_pointers && !aligned16(g.C)) return false;
+    }
     if (v.edge) {
         if (g.K % vec) return false;
         if (!v.b_kc && g.N % vec) return false;
@@ -236,7 +242,7 @@ int auto_mfma_variant(const Problem& pb)
         if (!v.direct) cost *= 1.2;
         // measured on sweeps: 4-wave tiles reach about 85 % of the ping-pong kernel's rate when two
         // workgroups share a CU and about 70 % when a workgroup has the CU to itself
-        if (v.waves_m * v.waves_n <= 4) cost /= wgs_per_cu == 2 ? 0.85 : 0.7;
+        if (v.waves_m * v.waves_n <= 4 && !v.w4) cost /= wgs_per_cu == 2 ? 0.85 : 0.7;
         // rank inside one tile shape: ping-pong kb64 x4 > ping-pong others > 8-wave > 4-wave (kb64 x4 first)
         int rank = v.pingpong ? (v.kb == 64 && v.stages == 4 ? 8 : 6) : (v.waves_m * v.waves_n == 8 ? 4 : 2);
         if (!v.pingpong && v.kb == 64 && v.stages == 4) rank += 1;
@@ -244,6 +250,9 @@ int auto_mfma_variant(const Problem& pb)
         // (C = A*B, C = relu(A*B)); their full build reads C element by element and lost 20 % to the 32x32 form
         const bool lean = pb.g.prologue == PRO_SET && pb.g.prologue_arg == 0.f && (pb.g.epilogue == EPI_RELU || pb.g.epilogue == EPI_NONE);
         if (v.mi16) rank += lean ? 4 : -8;
+        // four waves with 128x128 wave tiles: 4-9 % faster than the eight-wave form on large 16-bit problems
+        // (a third less LDS traffic, and the part is at its power limit there); int8 measured 1-2 % slower
+        if (v.w4) rank = elem_size(pb.g.in_type) == 2 ? 13 : 11;
         const bool better = best < 0 || cost < best_cost * 0.999 ||
                             (cost <= best_cost * 1.001 && ((int64_t)v.bm * v.bn > (int64_t)tab[best].bm * tab[best].bn ||
                                                            ((int64_t)v.bm * v.bn == (int64_t)tab[best].bm * tab[best].bn && rank > best_rank)));
@@ -495,7 +504,7 @@ int acc950_mfma_phase_probe(int in_type, int out_type, int M, int N, int K, cons
     Problem pb;
     int rc = make_problem(in_type, out_type, M, N, K, A, K, 1, B, N, 1, C, N, 1, PRO_SET0, EPI_RELU, true, &pb);
     if (rc) return rc;
-    const MfmaVariant probe = {256, 256, 2, 4, true, false, true, false, 64, 4, true, false, nullptr, nullptr};
+    const MfmaVariant probe = {256, 256, 2, 4, true, false, true, false, 64, 4, true, false, false, nullptr, nullptr};
     int n_unused = 0;
     if (M < 256 || N < 256 || K < 1 || !mfma_table(pb.g.in_type, &n_unused) || !mfma_can_take(probe, pb))
         return fail(ACC950_UNSUPPORTED, "the phase probe runs the 256x256 ping-pong kernel: 8/16-bit inputs, dense row-major A, B, C, M and N multiples of 256, K of 64 bytes");
@@ -643,7 +652,7 @@ int acc950_variant_name(int variant, char* buf, size_t buf_len)
     const MfmaVariant& v = tab[variant];
     std::snprintf(buf, buf_len, "mfma %dx%d kb%d waves %dx%d %sB=%s fill=%s stages=%d%s%s%s", v.bm, v.bn, v.kb, v.waves_m, v.waves_n,
                   v.a_kc ? "" : "A=col-major ", v.b_kc ? "col-major" : "row-major", v.direct ? "direct" : "registers", v.stages,
-                  v.edge ? " edge" : "", v.pingpong ? " pingpong" : "", v.mi16 ? " mi16" : "");
+                  v.edge ? " edge" : "", v.pingpong ? " pingpong" : "", v.w4 ? " mi16 hand-laid loop" : v.mi16 ? " mi16" : "");
     return ACC950_OK;
 }
 

@@ -1,0 +1,330 @@
+// Four-wave MFMA GEMM on the 16x16 instruction shapes: one wave per SIMD, each with a 128x128
+// piece of a 256x256 output tile.
+//
+// Counterpart of the same tensorized plan of the reference as gemm_mfma16.h
+// (/root/reference/accera/transforms/src/exec/ExecutionPlanToAffineLoweringPass.cpp:5986-6533),
+// with the largest wave tile the register file takes.  A 128x128 wave tile reads 16 fragments
+// from LDS per 64 MFMAs; the eight-wave kernel's 128x64 wave tile reads 12 per 32.  LDS traffic
+// per unit of arithmetic drops by a third, and on a part that runs large GEMMs at its power
+// limit that is clock rate for the matrix cores.
+//
+// The 256 accumulator registers live in a[0:255] and the K loop is hand-laid assembly
+// (gemm_mfma16w4_loop.inc, written by gen_w4_loop.py) -- left to the compiler the same loop
+// moves accumulators between the register files and spills.  Tile staging, the LDS layout and
+// the stores are those of gemm_mfma16.h.
+//
+// Takes: A row-major, whole tiles, K a multiple of four k-steps (256 bytes), C = A*B or
+// C = relu(A*B) (SET 0 prologue), rows of C 16 bytes aligned.
+#pragma once
+#include "gemm_mfma16.h"
+#include "gemm_mfma16w4_loop.inc"
+
+namespace acc950 {
+
+template <int IN_, bool B_KC_, bool TIMED_ = false>
+struct Mfma16W4Config {
+    static constexpr bool TIMED = TIMED_;
+    static constexpr int IN = IN_, BM = 256, BN = 256, WAVES_M = 2, WAVES_N = 2, KB = 64, STAGES = 4, NT = 256;
+    static constexpr bool A_KC = true, B_KC = B_KC_;
+    static constexpr int LDS_BYTES = STAGES * (BM + BN) * KB;
+};
+
+// the four registers of accumulator block N, out of the AGPR file
+template <int N>
+__device__ __forceinline__ i32x4 w4_acc_block()
+{
+    int x0, x1, x2, x3;
+    asm volatile("v_accvgpr_read_b32 %0, a[%4]\n\tv_accvgpr_read_b32 %1, a[%5]\n\tv_accvgpr_read_b32 %2, a[%6]\n\tv_accvgpr_read_b32 %3, a[%7]"
+                 : "=v"(x0), "=v"(x1), "=v"(x2), "=v"(x3)
+                 : "n"(N * 4), "n"(N * 4 + 1), "n"(N * 4 + 2), "n"(N * 4 + 3));
+    return i32x4{x0, x1, x2, x3};
+}
+
+template <int B, int E, typename F>
+__device__ __forceinline__ void w4_static_for(F&& f)
+{
+    if constexpr (B < E) {
+        f(std::integral_constant<int, B>{});
+        w4_static_for<B + 1, E>(f);
+    }
+}
+
+template <typename Cfg>
+__global__ void __launch_bounds__(256, 1) gemm_mfma16w4_kernel(GemmArgs p)
+{
+    constexpr int IN = Cfg::IN, BM = 256, BN = 256, NT = 256, KB = 64, WAVES_N = 2;
+    constexpr bool B_KC = Cfg::B_KC;
+    constexpr int ES = InTraits<IN>::ES;
+    constexpr int BK = KB / ES;
+    constexpr int WTM = 128, WTN = 128, TM = 8, TN = 8;
+    // (swizzle and address arithmetic only: these are the tiles of the eight-wave kernel)
+    using TA = OperandTile<IN, BM, true, 512, KB, true>;
+    using TB = OperandTile<IN, BN, B_KC, 512, KB, true>;
+    using acc_t = typename In16Traits<IN>::acc_t;
+    using scalar_t = typename In16Traits<IN>::scalar_t;
+    constexpr int STAGE_BYTES = TA::TILE_BYTES + TB::TILE_BYTES;
+    static_assert(STAGE_BYTES == 32768 && TA::TILE_BYTES == 16384, "the loop's offsets are written for these");
+
+    extern __shared__ __attribute__((aligned(1024))) char smem[];
+    select_batch(p);
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int wr0 = (wave / WAVES_N) * WTM;
+    const int wc0 = (wave % WAVES_N) * WTN;
+
+    unsigned long long stamp_clk[4], stamp_ref[4];
+    auto stamp = [&](int i) {
+        if constexpr (Cfg::TIMED) {
+            __builtin_amdgcn_sched_barrier(0);
+            stamp_clk[i] = __builtin_amdgcn_s_memtime();
+            stamp_ref[i] = __builtin_amdgcn_s_memrealtime();
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    stamp(0);
+
+    int tile_m, tile_n;
+    tile_coords(blockIdx.x, p.tiles_m, p.tiles_n, tile_m, tile_n);
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+
+    const char* Ab = (const char*)p.A;
+    const char* Bb = (const char*)p.B;
+    const int64_t lda = p.a_rs;
+    const int64_t ldb = B_KC ? p.b_cs : p.b_rs;
+    const int KT = p.K / BK;
+
+    // ---- tile fills: 4 + 4 instructions per thread and K tile.  A (and a K-contiguous B): one
+    // instruction of the workgroup covers 64 rows.  B with N contiguous: 8 (16-bit) or 16 (8-bit)
+    // k rows, half a period of the swizzle, so even and odd instructions have their own lane offset.
+    const unsigned smem_addr = (unsigned)(size_t)(ACC950_LDS char*)smem;
+    const unsigned ldsb = __builtin_amdgcn_readfirstlane(smem_addr + (unsigned)(wave * 1024));
+    constexpr int B_CPR = TB::CPR;
+    constexpr int B_RPP = NT / B_CPR; // rows of B's tile one fill instruction of the workgroup covers
+    // K-contiguous tiles (64-byte rows): chunk c of row r sits at position c ^ kc_swz(r).  With this map
+    // the 16-row ds_read_b128 of a fragment is free of bank conflicts (the row/4 map of the eight-wave
+    // kernel costs two passes; there the sibling wave's MFMAs hide it, here nothing does).
+    auto kc_swz = [](int row) { return ((row >> 1) & 1) | ((((row >> 1) ^ (row >> 2)) & 1) << 1); };
+    const unsigned a_off = (unsigned)TA::global_off(tid / 4, (tid % 4) ^ kc_swz(tid / 4), 0, 0, lda);
+    unsigned b_off0, b_off1;
+    if constexpr (B_KC) {
+        b_off0 = b_off1 = (unsigned)TB::global_off(tid / 4, (tid % 4) ^ kc_swz(tid / 4), 0, 0, ldb);
+    } else {
+        b_off0 = (unsigned)TB::global_off(tid / B_CPR, TB::swizzle(tid / B_CPR, tid % B_CPR), 0, 0, ldb);
+        b_off1 = (unsigned)TB::global_off(tid / B_CPR, TB::swizzle(tid / B_CPR + B_RPP, tid % B_CPR), 0, 0, ldb);
+    }
+    const unsigned da = __builtin_amdgcn_readfirstlane((unsigned)(64 * lda * ES));
+    const unsigned db = __builtin_amdgcn_readfirstlane((unsigned)((B_KC ? 64 : B_RPP) * ldb * ES));
+    const unsigned sa = KB;
+    const unsigned sb = __builtin_amdgcn_readfirstlane(B_KC ? (unsigned)KB : (unsigned)(BK * ldb * ES));
+    const char* a_tile = Ab + (int64_t)m0 * lda * ES;
+    const char* b_tile = Bb + (B_KC ? (int64_t)n0 * ldb * ES : (int64_t)n0 * ES);
+#pragma unroll
+    for (int s = 0; s < 3; ++s) {
+#pragma unroll
+        for (int f = 0; f < 4; ++f)
+            TA::direct_issue(ldsb + s * STAGE_BYTES + f * 4096, a_off, a_tile + (int64_t)s * sa + (int64_t)f * da);
+#pragma unroll
+        for (int f = 0; f < 4; ++f)
+            TB::direct_issue(ldsb + s * STAGE_BYTES + TA::TILE_BYTES + f * 4096, (f & 1) ? b_off1 : b_off0,
+                             b_tile + (int64_t)s * sb + (int64_t)f * db);
+    }
+    const char* pa = a_tile + 3 * (int64_t)sa;
+    const char* pb = b_tile + 3 * (int64_t)sb;
+    const unsigned groups = __builtin_amdgcn_readfirstlane((unsigned)(KT / 4 - 1));
+
+    // ---- LDS addresses of the fragment reads (stage 0; the loop adds stage and block offsets)
+    const int kg = lane >> 4, li = lane & 15;
+    const unsigned a_rd = smem_addr + (unsigned)((wr0 + li) * 64 + (kg ^ kc_swz(li)) * 16);
+    unsigned b_rd[8];
+    if constexpr (B_KC) {
+#pragma unroll
+        for (int x = 0; x < 8; ++x) b_rd[x] = smem_addr + (unsigned)((wc0 + li) * 64 + (kg ^ kc_swz(li)) * 16);
+    } else if constexpr (ES == 2) {
+#pragma unroll
+        for (int x = 0; x < 8; ++x) {
+            const int col_byte = (wc0 + x * 16 + (li & 3) * 4) * 2, k = kg * 8 + (li >> 2);
+            b_rd[x] = smem_addr + (unsigned)(k * TB::ROW_BYTES + TB::swizzle(k, col_byte >> 4) * 16 + (col_byte & 15));
+        }
+    } else {
+#pragma unroll
+        for (int x = 0; x < 8; ++x) {
+            const int col_byte = wc0 + x * 16 + (li & 1) * 8, k = kg * 16 + (li >> 1);
+            b_rd[x] = smem_addr + (unsigned)(k * TB::ROW_BYTES + TB::swizzle(k, col_byte >> 4) * 16 + (col_byte & 15));
+        }
+    }
+
+    wait_vmcnt<16>(); // tile 0 has landed (tiles 1 and 2 in flight)
+    __syncthreads();
+    stamp(1);
+
+#define ACC950_W4_OPERANDS                                                                                              \
+    : [a_rd] "v"(a_rd), [b_rd0] "v"(b_rd[0]), [b_rd1] "v"(b_rd[1]), [b_rd2] "v"(b_rd[2]), [b_rd3] "v"(b_rd[3]),          \
+      [b_rd4] "v"(b_rd[4]), [b_rd5] "v"(b_rd[5]), [b_rd6] "v"(b_rd[6]), [b_rd7] "v"(b_rd[7]), [a_off] "v"(a_off),        \
+      [b_off0] "v"(b_off0), [b_off1] "v"(b_off1), [pa] "s"(pa), [pb] "s"(pb), [da] "s"(da), [db] "s"(db), [sa] "s"(sa),   \
+      [sb] "s"(sb), [ldsb] "s"(ldsb), [groups] "s"(groups)                                                             \
+    : "memory", "scc", "s72", "s73", "s74", "s75", "s76", "s77", "s78", "s79", ACC950_W4_V(10), ACC950_W4_V(11),        \
+      ACC950_W4_V(12), ACC950_W4_V(13), ACC950_W4_V(14), ACC950_W4_V(15), ACC950_W4_V(16), ACC950_W4_V(17),             \
+      ACC950_W4_V(18), ACC950_W4_V(19), ACC950_W4_V(20), ACC950_W4_V(21), ACC950_W4_V(22), ACC950_W4_V(23),             \
+      ACC950_W4_V(24), "v250", "v251", "v252", "v253", "v254", "v255", "a0", "a1", "a2", "a3", "a4", "a5", "a6", "a7",   \
+      "a8", "a9", ACC950_W4_A(1), ACC950_W4_A(2), ACC950_W4_A(3), ACC950_W4_A(4), ACC950_W4_A(5), ACC950_W4_A(6), ACC950_W4_A(7), ACC950_W4_A(8), ACC950_W4_A(9),   \
+      ACC950_W4_A(10), ACC950_W4_A(11), ACC950_W4_A(12), ACC950_W4_A(13), ACC950_W4_A(14), ACC950_W4_A(15),             \
+      ACC950_W4_A(16), ACC950_W4_A(17), ACC950_W4_A(18), ACC950_W4_A(19), ACC950_W4_A(20), ACC950_W4_A(21),             \
+      ACC950_W4_A(22), ACC950_W4_A(23), ACC950_W4_A(24), "a250", "a251", "a252", "a253", "a254", "a255"
+// ten registers of a file, by decade
+#define ACC950_W4_R(f, d) f #d "0", f #d "1", f #d "2", f #d "3", f #d "4", f #d "5", f #d "6", f #d "7", f #d "8", f #d "9"
+#define ACC950_W4_V(d) ACC950_W4_R("v", d)
+#define ACC950_W4_A(d) ACC950_W4_R("a", d)
+    if constexpr (B_KC) {
+        if constexpr (IN == IN_F16) asm volatile(ACC950_W4_LOOP_KC("v_mfma_f32_16x16x32_f16") : ACC950_W4_OPERANDS);
+        else if constexpr (IN == IN_BF16) asm volatile(ACC950_W4_LOOP_KC("v_mfma_f32_16x16x32_bf16") : ACC950_W4_OPERANDS);
+        else asm volatile(ACC950_W4_LOOP_KC("v_mfma_i32_16x16x64_i8") : ACC950_W4_OPERANDS);
+    } else {
+        if constexpr (IN == IN_F16) asm volatile(ACC950_W4_LOOP_MC16("v_mfma_f32_16x16x32_f16") : ACC950_W4_OPERANDS);
+        else if constexpr (IN == IN_BF16) asm volatile(ACC950_W4_LOOP_MC16("v_mfma_f32_16x16x32_bf16") : ACC950_W4_OPERANDS);
+        else asm volatile(ACC950_W4_LOOP_MC8("v_mfma_i32_16x16x64_i8") : ACC950_W4_OPERANDS);
+    }
+    stamp(2);
+#undef ACC950_W4_OPERANDS
+#undef ACC950_W4_R
+#undef ACC950_W4_V
+#undef ACC950_W4_A
+
+    // ---- write-back: block (i, j) leaves the AGPR file just before its store.  Lane l holds row
+    // i*16 + l%16 and columns j*16 + (l/16)*4 .. +3 of the wave tile.
+    const int lrow = wr0 + (lane & 15), lcol = wc0 + (lane >> 4) * 4;
+    const unsigned os = p.out_type == T_I8 ? 1 : (p.out_type == T_F32 || p.out_type == T_I32) ? 4 : 2;
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+    // One copy of the stores per epilogue (a uniform branch): with a single wave per SIMD the
+    // write-back is bound by instruction issue, so every instruction per block counts.
+    auto write_back = [&](auto relu_tag) {
+        constexpr bool RELU = decltype(relu_tag)::value;
+        auto block = [&](auto n_tag) -> acc_t {
+            acc_t v = __builtin_bit_cast(acc_t, w4_acc_block<decltype(n_tag)::value>());
+            if constexpr (RELU) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    if constexpr (IN == IN_I8) v[e] = v[e] > 0 ? v[e] : 0;
+                    else v[e] = __builtin_fmaxf(v[e], 0.f);
+                }
+            }
+            return v;
+        };
+        if (os == 4) {
+            const CTile tile = c_tile((char*)p.C + ((int64_t)m0 * p.c_rs + n0) * 4);
+            const unsigned row_bytes = (unsigned)p.c_rs * 4;
+            const unsigned lane_off = (unsigned)lrow * row_bytes + (unsigned)lcol * 4;
+            w4_static_for<0, TM>([&](auto i) {
+                const unsigned soff = (unsigned)(i.value * 16) * row_bytes;
+                w4_static_for<0, TN>([&](auto j) {
+                    constexpr int n = i.value * 8 + j.value;
+                    if constexpr (RELU) {
+                        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, block(std::integral_constant<int, n>{})), tile.rsrc,
+                                                               lane_off + j.value * 64, soff, 0);
+                    } else {
+                        // no arithmetic on the way out: the store reads the accumulator registers themselves
+                        const unsigned vo = lane_off, so = soff; // (asm operands do not capture on their own)
+                        const auto rsrc = tile.rsrc;
+                        asm volatile("buffer_store_dwordx4 a[%3:%4], %0, %1, %2 offen offset:%5"
+                                     :
+                                     : "v"(vo), "s"(rsrc), "s"(so), "n"(n * 4), "n"(n * 4 + 3), "n"(j.value * 64)
+                                     : "memory");
+                    }
+                });
+            });
+        } else {
+            // narrow outputs: 16 rows of the wave tile are put together in a wave-private slab of the
+            // (now idle) tile buffers and leave as 16-byte pieces that cover whole rows
+            __syncthreads();
+            auto staged = [&](auto os_tag, auto&& pack) {
+                constexpr int OS = decltype(os_tag)::value;
+                constexpr int ROW = WTN * OS;
+                constexpr int PITCH = (ROW / 32) % 2 == 0 ? ROW + 32 : ROW;
+                char* slab = smem + wave_u * (16 * PITCH);
+                const CTile tile = c_tile((char*)p.C + ((int64_t)(m0 + (wave_u / WAVES_N) * WTM) * p.c_rs + n0 + (wave_u % WAVES_N) * WTN) * OS);
+                const unsigned row_bytes = (unsigned)p.c_rs * OS;
+                constexpr int CPRW = ROW / 16;
+                constexpr int PIECES = (16 * CPRW + 63) / 64;
+                char* mine = slab + (lane & 15) * PITCH + ((lane >> 4) * 4) * OS;
+                w4_static_for<0, TM>([&](auto i) {
+                    w4_static_for<0, TN>([&](auto j) {
+                        auto w = pack(block(std::integral_constant<int, i.value * 8 + j.value>{}));
+                        *(decltype(w)*)(mine + j.value * 16 * OS) = w;
+                    });
+#pragma unroll
+                    for (int it = 0; it < PIECES; ++it) {
+                        const int id = it * 64 + lane;
+                        const int row = id / CPRW, cc = id % CPRW;
+                        const i32x4 v = *(const i32x4*)(slab + row * PITCH + cc * 16);
+                        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), tile.rsrc, (unsigned)row * row_bytes + cc * 16,
+                                                               (unsigned)(i.value * 16) * row_bytes, 0);
+                    }
+                });
+            };
+            auto pack_f16 = [](const acc_t& v) -> i32x2 {
+                typedef _Float16 h4 __attribute__((ext_vector_type(4)));
+                return __builtin_bit_cast(i32x2, h4{(_Float16)v[0], (_Float16)v[1], (_Float16)v[2], (_Float16)v[3]});
+            };
+            auto pack_bf16 = [](const acc_t& v) -> i32x2 {
+                typedef __bf16 b4 __attribute__((ext_vector_type(4)));
+                return __builtin_bit_cast(i32x2, b4{(__bf16)v[0], (__bf16)v[1], (__bf16)v[2], (__bf16)v[3]});
+            };
+            auto pack_i16 = [](const acc_t& v) -> i32x2 {
+                return i32x2{(int)(((unsigned)v[0] & 0xffffu) | ((unsigned)v[1] << 16)), (int)(((unsigned)v[2] & 0xffffu) | ((unsigned)v[3] << 16))};
+            };
+            auto pack_i8 = [](const acc_t& v) -> int {
+                return (int)(((unsigned)v[0] & 0xffu) | (((unsigned)v[1] & 0xffu) << 8) | (((unsigned)v[2] & 0xffu) << 16) | ((unsigned)v[3] << 24));
+            };
+            if constexpr (IN == IN_I8) {
+                if (os == 2) staged(std::integral_constant<int, 2>{}, pack_i16);
+                else staged(std::integral_constant<int, 1>{}, pack_i8);
+            } else {
+                if (p.out_type == T_F16) staged(std::integral_constant<int, 2>{}, pack_f16);
+                else staged(std::integral_constant<int, 2>{}, pack_bf16);
+            }
+        }
+    };
+    if (p.epilogue == EPI_RELU) write_back(std::true_type{});
+    else write_back(std::false_type{});
+
+    if constexpr (Cfg::TIMED) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // stores acknowledged
+        stamp(3);
+        if (threadIdx.x == 0 && p.stamps) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                p.stamps[(blockIdx.x * 4 + i) * 2] = stamp_clk[i];
+                p.stamps[(blockIdx.x * 4 + i) * 2 + 1] = stamp_ref[i];
+            }
+        }
+    }
+}
+
+template <typename Cfg>
+hipError_t launch_mfma16w4(const GemmArgs& a, hipStream_t stream, LaunchGeom* geom, bool dry_run)
+{
+    auto kern = gemm_mfma16w4_kernel<Cfg>;
+    GemmArgs args = a;
+    args.tiles_m = a.M / Cfg::BM;
+    args.tiles_n = a.N / Cfg::BN;
+    if (geom) {
+        geom->grid[0] = (unsigned)(args.tiles_m * args.tiles_n);
+        geom->grid[1] = 1;
+        geom->grid[2] = a.batch > 1 ? a.batch : 1;
+        geom->block[0] = Cfg::NT;
+        geom->block[1] = geom->block[2] = 1;
+        geom->dyn_lds = Cfg::LDS_BYTES;
+    }
+    if (dry_run) return hipSuccess;
+    static bool attr_set = false;
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES);
+        if (e != hipSuccess) return e;
+        attr_set = true;
+    }
+    hipLaunchKernelGGL(kern, dim3(args.tiles_m * args.tiles_n, 1, a.batch > 1 ? a.batch : 1), dim3(Cfg::NT), Cfg::LDS_BYTES, stream, args);
+    return hipGetLastError();
+}
+
+} // namespace acc950

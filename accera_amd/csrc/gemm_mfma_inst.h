@@ -6,22 +6,26 @@
 //  /root/reference/tools/benchmarkers/accera_gemm.py:187-348): block tile BMxBN, K tile
 // of KB bytes, waves laid out WAVES_M x WAVES_N, the tile fill either direct-to-LDS
 // (STAGES buffers deep) or register-staged, and whether partial edge tiles are handled.
-#include "gemm_mfma16.h"
+#include <cstdlib>
+#include "gemm_mfma16w4.h"
 #include "variants.h"
 
 namespace acc950 {
 
 #define VA(AKC, BM, BN, WM, WN, BKC, DIRECT, EDGE, KB, STAGES)                                         \
-    { BM, BN, WM, WN, AKC, BKC, DIRECT, EDGE, KB, STAGES, false, false,                                \
+    { BM, BN, WM, WN, AKC, BKC, DIRECT, EDGE, KB, STAGES, false, false, false,                         \
       &launch_mfma<MfmaConfig<ACC950_IN, BM, BN, WM, WN, AKC, BKC, DIRECT, EDGE, KB, STAGES>>, nullptr }
 #define VPA(AKC, BM, BN, WM, WN, BKC, KB, STAGES)                                                       \
-    { BM, BN, WM, WN, AKC, BKC, true, false, KB, STAGES, true, false,                                  \
+    { BM, BN, WM, WN, AKC, BKC, true, false, KB, STAGES, true, false, false,                           \
       &launch_mfma<MfmaConfig<ACC950_IN, BM, BN, WM, WN, AKC, BKC, true, false, KB, STAGES, true>>, nullptr }
 // ping-pong on the 16x16 MFMA shapes
 #define V16(AKC, BM, BN, WM, WN, BKC, KB, STAGES)                                                       \
-    { BM, BN, WM, WN, AKC, BKC, true, false, KB, STAGES, true, true,                                   \
+    { BM, BN, WM, WN, AKC, BKC, true, false, KB, STAGES, true, true, false,                            \
       &launch_mfma16<Mfma16Config<ACC950_IN, BM, BN, WM, WN, AKC, BKC, KB, STAGES, false>>,           \
       &launch_mfma16<Mfma16Config<ACC950_IN, BM, BN, WM, WN, AKC, BKC, KB, STAGES, true>> }
+// four waves, 128x128 wave tiles, hand-laid K loop
+#define V16W4(BKC) \
+    { 256, 256, 2, 2, true, BKC, true, false, 64, 4, false, true, true, &launch_mfma16w4<Mfma16W4Config<ACC950_IN, BKC>>, nullptr }
 #define V(BM, BN, WM, WN, BKC, DIRECT, EDGE, KB, STAGES) VA(true, BM, BN, WM, WN, BKC, DIRECT, EDGE, KB, STAGES)
 #define VP(BM, BN, WM, WN, BKC, KB, STAGES) VPA(true, BM, BN, WM, WN, BKC, KB, STAGES)
 // column-major A (M contiguous; the "transA" shapes of the reference's sweep lists,
@@ -63,11 +67,14 @@ static const MfmaVariant kVariants[] = {
     V16(false, 256, 256, 2, 4, false, 64, 4),
     V16(false, 256, 256, 2, 4, true, 64, 4),
     V16(true, 256, 192, 4, 2, true, 64, 4),
+    V16W4(false),
+    V16W4(true),
 };
 #undef LAYOUT_AT
 #undef VA
 #undef VPA
 #undef V16
+#undef V16W4
 #undef LAYOUT
 #undef V
 #undef VP
@@ -76,6 +83,7 @@ static const MfmaVariant kVariants[] = {
 // (256x256 ping-pong on the 16x16 MFMA shapes, row-major B): same code plus four clock stamps per workgroup.
 hipError_t ACC950_TIMED_FN(const GemmArgs& a, hipStream_t stream, LaunchGeom* geom, bool dry_run)
 {
+    if (std::getenv("ACC950_PROBE_W4")) return launch_mfma16w4<Mfma16W4Config<ACC950_IN, false, true>>(a, stream, geom, dry_run);
     return launch_mfma16<Mfma16Config<ACC950_IN, 256, 256, 2, 4, true, false, 64, 4, false, true>>(a, stream, geom, dry_run);
 }
 

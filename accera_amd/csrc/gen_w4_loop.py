@@ -1,0 +1,169 @@
+#!/usr/bin/env python3
+"""Writes gemm_mfma16w4_loop.inc: the K loop of the four-wave 256x256 GEMM kernel as one block of
+gfx950 assembly per layout of matrix B.
+
+    python3 gen_w4_loop.py > gemm_mfma16w4_loop.inc
+
+One wave per SIMD owns a 128x128 piece of the output tile: 8 x 8 blocks of 16x16, 256 accumulator
+registers, which only fit when they live in a[0:255] for the whole loop while v[128:255] hold
+two sets of operand fragments.  The compiler's register allocator does not keep that split on
+its own (it moves accumulators between the two files and spills), so the loop is laid out by
+hand: registers are fixed, and each k-step of 64 bytes is
+
+    s_waitcnt lgkmcnt(4)            fragments of this step are in registers (all but A's last four)
+    32 MFMAs (rows 0..63 of the wave tile), the 8 fill instructions of the step three ahead
+    and their address arithmetic spread between them, at most two per MFMA
+    s_waitcnt vmcnt(16); s_barrier  the tile of the next step has landed for every wave
+    32 MFMAs (rows 64..127), the fragment reads of the next step between them, one per MFMA
+
+The four LDS stages rotate with the k-step, so the body is written out for four steps; the last
+four steps (no more fills, then no more reads) are a second copy.  K must be a multiple of four
+steps.
+
+Register use (besides the operands the C++ side passes in):
+    a[0:255]    accumulators, block (i, j) at a[(i*8+j)*4 .. +3]
+    v[128:191]  fragments of even steps: B blocks 0..7 (v128..), A blocks 0..7 (v160..)
+    v[192:255]  fragments of odd steps
+    v[104:121]  LDS read addresses of the upper two stages (the 16-bit offset field reaches 64 KB)
+    s[72:73], s[74:75]  fill pointers of A and B (tile three ahead); s[76:77] scratch pointer; s78 loop count
+"""
+STAGE = 32768      # (256 + 256) rows x 64 bytes
+B_TILE = 16384     # B's tile follows A's inside a stage
+FRAG = 1024        # 16 rows x 64 bytes (K-contiguous operand)
+
+
+def acc(i, j):
+    n = (i * 8 + j) * 4
+    return f"a[{n}:{n + 3}]"
+
+
+def bfrag(buf, j):
+    n = 128 + buf * 64 + j * 4
+    return n
+
+
+def afrag(buf, i):
+    n = 160 + buf * 64 + i * 4
+    return n
+
+
+def mfma(i, j, buf):
+    b, a = bfrag(buf, j), afrag(buf, i)
+    return f'MFMA " {acc(i, j)}, v[{b}:{b + 3}], v[{a}:{a + 3}], {acc(i, j)}\\n"'
+
+
+def line(s):
+    return f'"{s}\\n"'
+
+
+def read_a(x, stage, buf):
+    base = "%[a_rd]" if stage < 2 else "v104"
+    off = (stage & 1) * STAGE + x * FRAG
+    n = afrag(buf, x)
+    return [line(f"ds_read_b128 v[{n}:{n + 3}], {base} offset:{off}")]
+
+
+def read_b(x, stage, buf, b_layout):
+    n = bfrag(buf, x)
+    if b_layout == "kc":
+        base = "%[b_rd0]" if stage < 2 else "v105"
+        off = (stage & 1) * STAGE + B_TILE + x * FRAG
+        return [line(f"ds_read_b128 v[{n}:{n + 3}], {base} offset:{off}")]
+    # B as it lies in memory (N contiguous): two transposing reads per block, 4 (16-bit) or 8 (8-bit)
+    # k rows = 2048 bytes apart; every block has its own address (the swizzle is an XOR)
+    op = "ds_read_b64_tr_b16" if b_layout == "mc16" else "ds_read_b64_tr_b8"
+    base = f"%[b_rd{x}]" if stage < 2 else f"v{106 + x}"
+    out = []
+    for q in range(2):
+        off = (stage & 1) * STAGE + B_TILE + q * 2048
+        out.append(line(f"{op} v[{n + 2 * q}:{n + 2 * q + 1}], {base} offset:{off}"))
+    return out
+
+
+def fill(f, phase, stage, b_layout):
+    """Fill instruction f (0..3 A, 4..7 B) of a K tile, spread over four MFMA slots: pointer, M0,
+    the load (the MFMA between the M0 write and the load is the wait state M0 needs), pointer advance."""
+    if f < 4:
+        ptr, d, s, lane, tile, g = "s[72:73]", "%[da]", "%[sa]", "%[a_off]", 0, f
+    else:
+        g = f - 4
+        ptr, d, s, tile = "s[74:75]", "%[db]", "%[sb]", B_TILE
+        lane = "%[b_off0]" if (b_layout == "kc" or g % 2 == 0) else "%[b_off1]"
+    if phase == 0:
+        if g == 0:
+            return [line(f"s_mov_b64 s[76:77], {ptr}")]
+        return [line(f"s_add_u32 s76, s76, {d}"), line("s_addc_u32 s77, s77, 0")]
+    if phase == 1:
+        return [line(f"s_add_u32 m0, %[ldsb], {stage * STAGE + tile + g * 4096}")]
+    if phase == 2:
+        return [line(f"global_load_lds_dwordx4 {lane}, s[76:77]")]
+    if g == 3:  # advance to the next K tile
+        lo, hi = (72, 73) if f < 4 else (74, 75)
+        return [line(f"s_add_u32 s{lo}, s{lo}, {s}"), line(f"s_addc_u32 s{hi}, s{hi}, 0")]
+    return []
+
+
+def step(pos, do_fill, wait, last, b_layout):
+    buf, nxt, fst = pos % 2, (pos + 1) % 4, (pos + 3) % 4
+    # fragments of B and of A's first four blocks are in registers (the last four reads may still be in flight)
+    out = [line("s_waitcnt lgkmcnt(4)")]
+    order = [(i, j) for i in range(8) for j in range(8)]
+    for s, (i, j) in enumerate(order[:32]):
+        out.append(mfma(i, j, buf))
+        if do_fill:
+            out += fill(s // 4, s % 4, fst, b_layout)
+    out.append(line("s_waitcnt lgkmcnt(0)"))
+    if not last:
+        out.append(line(f"s_waitcnt vmcnt({wait})"))
+        out.append(line("s_barrier"))
+    reads = []
+    if not last:
+        for x in range(8):
+            reads += read_b(x, nxt, buf ^ 1, b_layout)
+        for x in range(8):
+            reads += read_a(x, nxt, buf ^ 1)
+    for s, (i, j) in enumerate(order[32:]):
+        out.append(mfma(i, j, buf))
+        if s < len(reads):
+            out.append(reads[s])
+    return out
+
+
+def loop(b_layout):
+    out = [line("s_mov_b64 s[72:73], %[pa]"), line("s_mov_b64 s[74:75], %[pb]"), line("s_mov_b32 s78, %[groups]"),
+           line("v_add_u32 v104, 0x10000, %[a_rd]")]
+    if b_layout == "kc":
+        out.append(line("v_add_u32 v105, 0x10000, %[b_rd0]"))
+    else:
+        for x in range(8):
+            out.append(line(f"v_add_u32 v{106 + x}, 0x10000, %[b_rd{x}]"))
+    for n in range(256):
+        out.append(line(f"v_accvgpr_write_b32 a{n}, 0"))
+    for x in range(8):
+        out += read_b(x, 0, 0, b_layout)
+    for x in range(8):
+        out += read_a(x, 0, 0)
+    out += [line("s_nop 7"), line("s_cmp_eq_u32 s78, 0"), line("s_cbranch_scc1 2f"), line("1:")]
+    for pos in range(4):
+        out += step(pos, True, 16, False, b_layout)
+    out += [line("s_sub_u32 s78, s78, 1"), line("s_cmp_lg_u32 s78, 0"), line("s_cbranch_scc1 1b"), line("2:")]
+    out += step(0, True, 16, False, b_layout)
+    out += step(1, False, 8, False, b_layout)
+    out += step(2, False, 0, False, b_layout)
+    out += step(3, False, 0, True, b_layout)
+    out += [line("s_nop 15"), line("s_nop 15")]
+    return out
+
+
+def main():
+    print("// Generated by gen_w4_loop.py; do not edit.  The K loop of gemm_mfma16w4_kernel, one macro per")
+    print("// layout of B (K contiguous / N contiguous 16-bit / N contiguous 8-bit); MFMA is the mnemonic.")
+    for name in ("kc", "mc16", "mc8"):
+        body = loop(name)
+        print(f"#define ACC950_W4_LOOP_{name.upper()}(MFMA) \\")
+        print(" \\\n".join("    " + s for s in body))
+        print()
+
+
+if __name__ == "__main__":
+    main()

@@ -490,7 +490,7 @@ def _match(source):
 
 def _variant_for_tile(spec, bm, bn):
     """Best-ranked MFMA variant with block tile bm x bn that accepts the problem, else VARIANT_AUTO."""
-    best, best_rank = _lib.VARIANT_AUTO, -9
+    best, best_rank = _lib.VARIANT_AUTO, -8
     lean = spec.prologue == _lib.PROLOGUE_SET and spec.prologue_arg == 0 and spec.epilogue in (_lib.EPILOGUE_RELU, _lib.EPILOGUE_NONE)
     for v in range(_lib.num_variants()):
         name = _lib.variant_name(v)
@@ -503,7 +503,9 @@ def _variant_for_tile(spec, bm, bn):
             continue
         # ping-pong over software-pipelined; the 16x16 MFMA shapes where the library runs their lean build
         rank = 2 * ("pingpong" in name) + (1 if "mi16" in name and lean else -1 if "mi16" in name else 0)
-        if best == _lib.VARIANT_AUTO or rank > best_rank:
+        if "hand-laid loop" in name:  # four waves, C = A*B / relu(A*B) only; ahead of ping-pong on 16-bit inputs
+            rank = (4 if spec.A.element_type.lib_id in (_lib.F16, _lib.BF16) else 2) if lean else -9
+        if rank > best_rank:
             best, best_rank = v, rank
     return best
 

@@ -68,7 +68,8 @@ def test_mfma_all_variants(in_type, out_type, b_layout):
         a_layout = "col" if "A=col-major" in name else "row"
         bm, bn = map(int, re.search(r"mfma (\d+)x(\d+)", name).groups())
         M, N = max(512, 2 * bm), (max(512, 2 * bn) if 512 % bn == 0 else 3 * bn)
-        for k_tiles in (1, 2, 3, 7):
+        # (the hand-laid loop takes K in steps of four tiles: the pipeline's depth, twice and five times it)
+        for k_tiles in ((4, 8, 20) if "hand-laid" in name else (1, 2, 3, 7)):
             run_case(in_type, out_type, M, N, k_tiles * kb, b_layout=b_layout, variant=v, seed=v + k_tiles, a_layout=a_layout)
         if "edge" in name:
             # ragged M, N (multiple of the 16-byte vector only) and a K tail
@@ -88,6 +89,10 @@ def test_mfma_all_variants_narrow_integer_outputs(out_type):
             a_layout = "col" if "A=col-major" in name else "row"
             bm, bn = map(int, re.search(r"mfma (\d+)x(\d+)", name).groups())
             M, N = max(512, 2 * bm), (max(512, 2 * bn) if 512 % bn == 0 else 3 * bn)
+            if "hand-laid" in name:  # C = A*B and relu(A*B) only, K in steps of four tiles
+                run_case("i8", out_type, M, N, 4 * kb, b_layout=b_layout, variant=v, seed=v)
+                run_case("i8", out_type, M, N, 12 * kb, b_layout=b_layout, variant=v, seed=v + 1, epilogue=ora.EPI_NONE)
+                continue
             run_case("i8", out_type, M, N, 2 * kb, b_layout=b_layout, variant=v, seed=v, a_layout=a_layout)
             run_case("i8", out_type, M, N, 3 * kb, b_layout=b_layout, variant=v, seed=v + 1, a_layout=a_layout, prologue=ora.PRO_NONE)
             if "edge" in name:
@@ -227,6 +232,47 @@ def test_large_tile_kernels_on_padded_output_rows(in_type, out_type, pad):
         want = ora.gemm_relu_exact(A, B, np.ascontiguousarray(Cbig[:, :N]), in_type, out_type, prologue, ora.EPI_RELU)
         assert_matches(got[:, :N], want, out_type, K)
         assert np.array_equal(got[:, N:], Cbig[:, N:]), "padding columns were written"
+
+
+def _hand_laid(b_layout):
+    from accera_amd import _lib
+    return next(v for v, n in _variants(b_layout) if "hand-laid" in n)
+
+
+@pytest.mark.parametrize("in_type,out_type", [("f16", "f32"), ("f16", "f16"), ("bf16", "bf16"), ("bf16", "f32"),
+                                              ("i8", "i32"), ("i8", "i16"), ("i8", "i8")])
+@pytest.mark.parametrize("b_layout", ["row", "col"])
+def test_four_wave_kernel_every_output_type(in_type, out_type, b_layout):
+    """The kernel with the hand-laid K loop (accumulators pinned in the AGPR file): both epilogues it
+    takes, every store path (32-bit straight from the accumulator registers, narrow types through
+    LDS), 6 output tiles so that the tile map and both wave rows / columns are exercised, K at one,
+    two and five rounds of the four LDS stages."""
+    v = _hand_laid(b_layout)
+    kb = 64 if in_type == "i8" else 32
+    for k_tiles, epi in ((4, ora.EPI_RELU), (8, ora.EPI_NONE), (20, ora.EPI_RELU)):
+        print("variant", v, in_type, out_type, b_layout, "k tiles", k_tiles, flush=True)
+        run_case(in_type, out_type, 512, 768, k_tiles * kb, b_layout=b_layout, variant=v, seed=700 + k_tiles, epilogue=epi)
+
+
+def test_four_wave_kernel_is_refused_for_what_it_does_not_take():
+    """Accumulating into C, the SCALE / SET ops and a K that is not a multiple of four tiles go to the
+    other kernels: naming the variant for them is an error, never a wrong result."""
+    import accera_amd as acc
+    import torch
+    from accera_amd import _lib
+    v = _hand_laid("row")
+    rng = np.random.default_rng(5)
+    A, B = make_input(rng, (256, 160), "f16"), make_input(rng, (160, 256), "f16")
+    dC = to_device(np.zeros((256, 256), np.float32), "f32")
+    with pytest.raises(_lib.Acc950Error):
+        acc.gemm_relu(to_device(A, "f16"), to_device(B, "f16"), dC, variant=v)  # K = 5 tiles
+    A, B = make_input(rng, (256, 128), "f16"), make_input(rng, (128, 256), "f16")
+    for kw in (dict(prologue=acc.PROLOGUE_NONE), dict(epilogue=acc.EPILOGUE_SCALE, epilogue_arg=2.0), dict(prologue=acc.PROLOGUE_SET, prologue_arg=1.0)):
+        with pytest.raises(_lib.Acc950Error):
+            acc.gemm_relu(to_device(A, "f16"), to_device(B, "f16"), dC, variant=v, **kw)
+    acc.gemm_relu(to_device(A, "f16"), to_device(B, "f16"), dC, variant=v)  # and what it does take still runs
+    torch.cuda.synchronize()
+    assert_matches(to_host(dC, "f32"), ora.gemm_relu_exact(A, B, np.zeros((256, 256), np.float32), "f16", "f32", ora.PRO_SET0, ora.EPI_RELU), "f32", 128)
 
 
 def test_int8_output_rows_at_odd_distances_take_the_thread_bound_kernel():
