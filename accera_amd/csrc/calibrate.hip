@@ -102,12 +102,12 @@ int acc950_mfma_ceiling(int in_type, int data_mode, int iters, double* tera_ops,
         };
         launch(200);
         if (hipDeviceSynchronize() != hipSuccess) break;
-        hipEventRecord(e0, 0);
+        if (hipEventRecord(e0, 0) != hipSuccess) break;
         launch(iters);
-        hipEventRecord(e1, 0);
+        if (hipEventRecord(e1, 0) != hipSuccess) break;
         if (hipDeviceSynchronize() != hipSuccess) break;
         float ms = 0;
-        hipEventElapsedTime(&ms, e0, e1);
+        if (hipEventElapsedTime(&ms, e0, e1) != hipSuccess) break;
         long long c[2];
         if (hipMemcpy(c, clk, 16, hipMemcpyDeviceToHost) != hipSuccess) break;
         const double ops = 256.0 * 8 * iters * 16 * (in_type == T_I8 ? 32768.0 : 16384.0);

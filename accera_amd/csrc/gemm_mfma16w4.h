@@ -29,15 +29,19 @@ struct Mfma16W4Config {
     static constexpr int LDS_BYTES = STAGES * (BM + BN) * KB;
 };
 
-// the four registers of accumulator block N, out of the AGPR file
+// accumulator blocks N and N+1 (eight registers) out of the AGPR file.  The moves go through the matrix
+// pipeline and take a while to land; eight in a row, and a whole row of blocks before the first use,
+// keep that latency out of the write-back's critical path.
+struct W4BlockPair { i32x4 a, b; };
 template <int N>
-__device__ __forceinline__ i32x4 w4_acc_block()
+__device__ __forceinline__ W4BlockPair w4_acc_pair()
 {
-    int x0, x1, x2, x3;
-    asm volatile("v_accvgpr_read_b32 %0, a[%4]\n\tv_accvgpr_read_b32 %1, a[%5]\n\tv_accvgpr_read_b32 %2, a[%6]\n\tv_accvgpr_read_b32 %3, a[%7]"
-                 : "=v"(x0), "=v"(x1), "=v"(x2), "=v"(x3)
-                 : "n"(N * 4), "n"(N * 4 + 1), "n"(N * 4 + 2), "n"(N * 4 + 3));
-    return i32x4{x0, x1, x2, x3};
+    int x0, x1, x2, x3, y0, y1, y2, y3;
+    asm volatile("v_accvgpr_read_b32 %0, a[%8]\n\tv_accvgpr_read_b32 %1, a[%9]\n\tv_accvgpr_read_b32 %2, a[%10]\n\tv_accvgpr_read_b32 %3, a[%11]\n\t"
+                 "v_accvgpr_read_b32 %4, a[%12]\n\tv_accvgpr_read_b32 %5, a[%13]\n\tv_accvgpr_read_b32 %6, a[%14]\n\tv_accvgpr_read_b32 %7, a[%15]"
+                 : "=v"(x0), "=v"(x1), "=v"(x2), "=v"(x3), "=v"(y0), "=v"(y1), "=v"(y2), "=v"(y3)
+                 : "n"(N * 4), "n"(N * 4 + 1), "n"(N * 4 + 2), "n"(N * 4 + 3), "n"(N * 4 + 4), "n"(N * 4 + 5), "n"(N * 4 + 6), "n"(N * 4 + 7));
+    return W4BlockPair{i32x4{x0, x1, x2, x3}, i32x4{y0, y1, y2, y3}};
 }
 
 template <int B, int E, typename F>
@@ -200,16 +204,23 @@ __global__ void __launch_bounds__(256, 1) gemm_mfma16w4_kernel(GemmArgs p)
     // write-back is bound by instruction issue, so every instruction per block counts.
     auto write_back = [&](auto relu_tag) {
         constexpr bool RELU = decltype(relu_tag)::value;
-        auto block = [&](auto n_tag) -> acc_t {
-            acc_t v = __builtin_bit_cast(acc_t, w4_acc_block<decltype(n_tag)::value>());
+        // row i of the wave tile's blocks, epilogue applied
+        auto load_row = [&](auto i_tag, acc_t (&row)[TN]) {
+            constexpr int i = decltype(i_tag)::value;
+            w4_static_for<0, TN / 2>([&](auto h) {
+                const W4BlockPair pr = w4_acc_pair<i * 8 + h.value * 2>();
+                row[h.value * 2] = __builtin_bit_cast(acc_t, pr.a);
+                row[h.value * 2 + 1] = __builtin_bit_cast(acc_t, pr.b);
+            });
             if constexpr (RELU) {
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    if constexpr (IN == IN_I8) v[e] = v[e] > 0 ? v[e] : 0;
-                    else v[e] = __builtin_fmaxf(v[e], 0.f);
-                }
+                for (int j = 0; j < TN; ++j)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        if constexpr (IN == IN_I8) row[j][e] = row[j][e] > 0 ? row[j][e] : 0;
+                        else row[j][e] = __builtin_fmaxf(row[j][e], 0.f);
+                    }
             }
-            return v;
         };
         if (os == 4) {
             const CTile tile = c_tile((char*)p.C + ((int64_t)m0 * p.c_rs + n0) * 4);
@@ -217,11 +228,12 @@ __global__ void __launch_bounds__(256, 1) gemm_mfma16w4_kernel(GemmArgs p)
             const unsigned lane_off = (unsigned)lrow * row_bytes + (unsigned)lcol * 4;
             w4_static_for<0, TM>([&](auto i) {
                 const unsigned soff = (unsigned)(i.value * 16) * row_bytes;
+                acc_t row[TN];
+                if constexpr (RELU) load_row(i, row);
                 w4_static_for<0, TN>([&](auto j) {
                     constexpr int n = i.value * 8 + j.value;
                     if constexpr (RELU) {
-                        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, block(std::integral_constant<int, n>{})), tile.rsrc,
-                                                               lane_off + j.value * 64, soff, 0);
+                        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, row[j.value]), tile.rsrc, lane_off + j.value * 64, soff, 0);
                     } else {
                         // no arithmetic on the way out: the store reads the accumulator registers themselves
                         const unsigned vo = lane_off, so = soff; // (asm operands do not capture on their own)
@@ -247,18 +259,27 @@ __global__ void __launch_bounds__(256, 1) gemm_mfma16w4_kernel(GemmArgs p)
                 constexpr int CPRW = ROW / 16;
                 constexpr int PIECES = (16 * CPRW + 63) / 64;
                 char* mine = slab + (lane & 15) * PITCH + ((lane >> 4) * 4) * OS;
+                // (the accumulator reads of the next row are issued between this row's LDS writes and reads)
+                acc_t row[TN], next_row[TN];
+                load_row(std::integral_constant<int, 0>{}, row);
                 w4_static_for<0, TM>([&](auto i) {
-                    w4_static_for<0, TN>([&](auto j) {
-                        auto w = pack(block(std::integral_constant<int, i.value * 8 + j.value>{}));
-                        *(decltype(w)*)(mine + j.value * 16 * OS) = w;
-                    });
+#pragma unroll
+                    for (int j = 0; j < TN; ++j) {
+                        auto w = pack(row[j]);
+                        *(decltype(w)*)(mine + j * 16 * OS) = w;
+                    }
+                    if constexpr (i.value + 1 < TM) load_row(std::integral_constant<int, i.value + 1>{}, next_row);
 #pragma unroll
                     for (int it = 0; it < PIECES; ++it) {
                         const int id = it * 64 + lane;
-                        const int row = id / CPRW, cc = id % CPRW;
-                        const i32x4 v = *(const i32x4*)(slab + row * PITCH + cc * 16);
-                        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), tile.rsrc, (unsigned)row * row_bytes + cc * 16,
+                        const int r = id / CPRW, cc = id % CPRW;
+                        const i32x4 v = *(const i32x4*)(slab + r * PITCH + cc * 16);
+                        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), tile.rsrc, (unsigned)r * row_bytes + cc * 16,
                                                                (unsigned)(i.value * 16) * row_bytes, 0);
+                    }
+                    if constexpr (i.value + 1 < TM) {
+#pragma unroll
+                        for (int j = 0; j < TN; ++j) row[j] = next_row[j];
                     }
                 });
             };

@@ -503,8 +503,8 @@ def _variant_for_tile(spec, bm, bn):
             continue
         # ping-pong over software-pipelined; the 16x16 MFMA shapes where the library runs their lean build
         rank = 2 * ("pingpong" in name) + (1 if "mi16" in name and lean else -1 if "mi16" in name else 0)
-        if "hand-laid loop" in name:  # four waves, C = A*B / relu(A*B) only; ahead of ping-pong on 16-bit inputs
-            rank = (4 if spec.A.element_type.lib_id in (_lib.F16, _lib.BF16) else 2) if lean else -9
+        if "hand-laid loop" in name:  # four waves, C = A*B / relu(A*B) only; measured ahead of the ping-pong form
+            rank = 4 if lean else -9
         if rank > best_rank:
             best, best_rank = v, rank
     return best

@@ -121,11 +121,11 @@ def sweep(rows, in_type, relu, check, out_type=None, min_time_s=0.05, log=print,
         best = None
         for v, sp in candidates(in_id, out_id, M, N, K, sa, sb, sc):
             C = C0.clone()
-            call = GemmCall(A, B, C, prologue=pro, epilogue=epi, variant=v, k_splits=sp, prologue_arg=parg, epilogue_arg=earg)
             try:
+                call = GemmCall(A, B, C, prologue=pro, epilogue=epi, variant=v, k_splits=sp, prologue_arg=parg, epilogue_arg=earg)
                 call()
             except _lib.Acc950Error:
-                continue  # refused with the actual pointers (alignment)
+                continue  # refused with the actual pointers (alignment) or fragment ops (kernels that only take C = A*B)
             ok = ""
             if check:
                 C.copy_(C0)
