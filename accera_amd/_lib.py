@@ -81,7 +81,7 @@ def check(rc):
 
 
 def mfma_phase_probe(in_type, out_type, M, N, K, a_ptr, b_ptr, c_ptr):
-    """In-kernel phase times of the 256x256 ping-pong kernel on device operands; returns a dict."""
+    """In-kernel phase times of the 256x256 kernel the automatic choice takes, on device operands; returns a dict."""
     out = (ctypes.c_double * 8)()
     check(lib().acc950_mfma_phase_probe(in_type, out_type, M, N, K, a_ptr, b_ptr, c_ptr, out))
     return {"prologue_us": out[0] / 1e3, "main_loop_us": out[1] / 1e3, "write_back_us": out[2] / 1e3,

@@ -507,7 +507,7 @@ int acc950_mfma_phase_probe(int in_type, int out_type, int M, int N, int K, cons
     const MfmaVariant probe = {256, 256, 2, 4, true, false, true, false, 64, 4, true, false, false, nullptr, nullptr};
     int n_unused = 0;
     if (M < 256 || N < 256 || K < 1 || !mfma_table(pb.g.in_type, &n_unused) || !mfma_can_take(probe, pb))
-        return fail(ACC950_UNSUPPORTED, "the phase probe runs the 256x256 ping-pong kernel: 8/16-bit inputs, dense row-major A, B, C, M and N multiples of 256, K of 64 bytes");
+        return fail(ACC950_UNSUPPORTED, "the phase probe runs the 256x256 kernels: 8/16-bit inputs, dense row-major A, B, C, M and N multiples of 256, K of 64 bytes");
     GemmArgs g = pb.g;
     const int tiles = (M / 256) * (N / 256);
     hipError_t e = hipMalloc((void**)&g.stamps, (size_t)tiles * 8 * sizeof(unsigned long long));
@@ -540,7 +540,8 @@ int acc950_mfma_phase_probe(int in_type, int out_type, int M, int N, int K, cons
         out[3 + q] = ns[q] > 0 ? cyc[q] / ns[q] : 0;  // shader clock in that phase [GHz]
     }
     out[6] = (double)(last - first) * 10.0;           // first workgroup start to last workgroup end [ns]
-    // MFMA pipe occupancy of the main loop: two waves per SIMD, 8 MFMAs of 32 cycles per k step each
+    // MFMA pipe occupancy of the main loop: per SIMD, 512 MFMA cycles per 32 bytes of K (two waves x 8 MFMAs of 32 cycles,
+    // or one wave x 32 MFMAs of 16 cycles)
     const int es = g.in_type == T_I8 ? 1 : 2;
     const double mfma_cycles = 2.0 * 8.0 * 32.0 * ((double)K * es / 32.0);
     out[7] = cyc[1] > 0 ? mfma_cycles / (cyc[1] / tiles) : 0;

@@ -15,6 +15,7 @@ prints per-kernel averages of every counter in the given files.
 import argparse
 import collections
 import csv
+import re
 import json
 import os
 import sys
@@ -38,7 +39,9 @@ def _dominant(acc, counter):
     for k, cs in acc.items():
         if "acc950_copy_kernel" in k or "acc950_stream_read_kernel" in k or "mfma_ceiling" in k or counter not in cs:
             continue
-        if not any(s in k for s in ("gemm_mfma_kernel", "gemm_mfma16_kernel", "gemm_skinny", "gemm_f32_kernel", "gemm_generic_kernel")):
+        if not any(s in k for s in ("gemm_mfma_kernel", "gemm_mfma16_kernel", "gemm_mfma16w4_kernel", "gemm_skinny", "gemm_f32_kernel", "gemm_generic_kernel")):
+            continue
+        if re.search(r"Config<[^>]*, true>\s*>", k):  # the build with clock stamps (last template argument), run by the phase probe
             continue
         tot = sum(cs[counter])
         if best is None or tot > best[1]:

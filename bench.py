@@ -226,7 +226,7 @@ def measure(name, steps, warmup, variant=-1, k_splits=0):
     in_kernel = None
     if c["bound"] == "mfma" and c["in_type"] in ("f16", "bf16", "i8") and c["b"] == "row" and c["M"] % 256 == 0 and c["N"] % 256 == 0 \
             and variant < 0:
-        # clock stamps inside the 256x256 ping-pong kernel on the same operands: phase times, the
+        # clock stamps inside the 256x256 kernel of the automatic choice on the same operands: phase times, the
         # engine clock in each phase, and how busy the MFMA pipe is at that clock
         from accera_amd import _lib
         A, B, C = first_set

@@ -204,14 +204,15 @@ int acc950_variant_name(int variant, char* buf, size_t buf_len);
  * The sustained clock under MFMA load depends on the operand data, so the random-data
  * figure is the practical compute roof for random GEMM inputs on the device at hand.
  *
- * acc950_mfma_phase_probe: runs a build of the 256x256 ping-pong MFMA kernel (the one the
- * automatic choice takes for large aligned problems) that reads the shader-clock counter
+ * acc950_mfma_phase_probe: runs a build of the 256x256 MFMA kernel the automatic choice takes
+ * for large aligned problems (four waves with the hand-laid K loop when K is a multiple of four
+ * K tiles of 64 bytes, else the eight-wave ping-pong form) that reads the shader-clock counter
  * and the constant 100 MHz counter at four points in every workgroup, on dense row-major
  * DEVICE operands (M, N multiples of 256, SET-0 prologue, ReLU epilogue), synchronously.
  * out[0..2] = average time of prologue / main loop / write-back in ns, out[3..5] = shader
  * clock in GHz during each phase, out[6] = first workgroup start to last workgroup end in
- * ns, out[7] = fraction of the main loop's cycles the MFMA pipe is busy (its 32-cycle
- * MFMAs / shader cycles).  Tells a loop that keeps the matrix cores busy at a throttled
+ * ns, out[7] = fraction of the main loop's cycles the MFMA pipe is busy (the cycles its
+ * MFMAs occupy / shader cycles).  Tells a loop that keeps the matrix cores busy at a throttled
  * clock from one that stalls.
  *
  * acc950_copy_probe / acc950_stream_read_probe: a plain copy (reads and writes `bytes`)
