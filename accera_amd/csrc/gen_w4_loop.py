@@ -111,7 +111,11 @@ def step(pos, do_fill, wait, last, b_layout):
     for s, (i, j) in enumerate(order[:32]):
         out.append(mfma(i, j, buf))
         if do_fill:
-            out += fill(s // 4, s % 4, fst, b_layout)
+            # A's fills come last in odd steps and first in even ones: the two 64-byte halves of a 128-byte
+            # line of a K-contiguous operand belong to k-steps 2m and 2m+1, filled in steps 2m-3 and 2m-2;
+            # requested back to back, the second half is still in the CU's vector cache
+            f = s // 4 if pos % 2 == 0 else (s // 4 + 4) % 8
+            out += fill(f, s % 4, fst, b_layout)
     out.append(line("s_waitcnt lgkmcnt(0)"))
     if not last:
         out.append(line(f"s_waitcnt vmcnt({wait})"))
