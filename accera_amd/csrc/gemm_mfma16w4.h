@@ -13,8 +13,9 @@
 // moves accumulators between the register files and spills.  Tile staging, the LDS layout and
 // the stores are those of gemm_mfma16.h.
 //
-// Takes: A row-major, whole tiles, K a multiple of four k-steps (256 bytes), C = A*B or
-// C = relu(A*B) (SET 0 prologue), rows of C 16 bytes aligned.
+// Takes: A row-major, whole tiles, K a multiple of four k-steps (256 bytes), rows of C 16 bytes aligned;
+// C = A*B or relu(A*B) (SET 0 prologue) for every output type, C += A*B (then ReLU or nothing) for
+// 32-bit outputs, where the tile of C is loaded straight into the accumulator registers.
 #pragma once
 #include "gemm_mfma16.h"
 #include "gemm_mfma16w4_loop.inc"
@@ -159,6 +160,14 @@ __global__ void __launch_bounds__(256, 1) gemm_mfma16w4_kernel(GemmArgs p)
         }
     }
 
+    // C += A*B with a 32-bit C: the loop starts from the tile of C instead of zeros (the host sends nothing else
+    // with a prologue other than SET 0 here).  Lane l owns row i*16 + l%16, columns j*16 + (l/16)*4 .. +3 of block (i, j).
+    const unsigned accum = __builtin_amdgcn_readfirstlane(p.prologue == PRO_NONE ? 1u : 0u);
+    const CTile c_in = c_tile((char*)p.C + ((int64_t)m0 * p.c_rs + n0) * 4);
+    const unsigned c_off = (unsigned)(wr0 + (lane & 15)) * ((unsigned)p.c_rs * 4) + (unsigned)(wc0 + (lane >> 4) * 4) * 4;
+    const unsigned c_row16 = __builtin_amdgcn_readfirstlane((unsigned)p.c_rs * 64);
+    const auto c_rsrc = c_in.rsrc;
+
     wait_vmcnt<16>(); // tile 0 has landed (tiles 1 and 2 in flight)
     __syncthreads();
     stamp(1);
@@ -167,7 +176,8 @@ __global__ void __launch_bounds__(256, 1) gemm_mfma16w4_kernel(GemmArgs p)
     : [a_rd] "v"(a_rd), [b_rd0] "v"(b_rd[0]), [b_rd1] "v"(b_rd[1]), [b_rd2] "v"(b_rd[2]), [b_rd3] "v"(b_rd[3]),          \
       [b_rd4] "v"(b_rd[4]), [b_rd5] "v"(b_rd[5]), [b_rd6] "v"(b_rd[6]), [b_rd7] "v"(b_rd[7]), [a_off] "v"(a_off),        \
       [b_off0] "v"(b_off0), [b_off1] "v"(b_off1), [pa] "s"(pa), [pb] "s"(pb), [da] "s"(da), [db] "s"(db), [sa] "s"(sa),   \
-      [sb] "s"(sb), [ldsb] "s"(ldsb), [groups] "s"(groups)                                                             \
+      [sb] "s"(sb), [ldsb] "s"(ldsb), [groups] "s"(groups), [accum] "s"(accum), [c_off] "v"(c_off),                     \
+      [c_rsrc] "s"(c_rsrc), [c_row16] "s"(c_row16)                                                                      \
     : "memory", "scc", "s72", "s73", "s74", "s75", "s76", "s77", "s78", "s79", ACC950_W4_V(10), ACC950_W4_V(11),        \
       ACC950_W4_V(12), ACC950_W4_V(13), ACC950_W4_V(14), ACC950_W4_V(15), ACC950_W4_V(16), ACC950_W4_V(17),             \
       ACC950_W4_V(18), ACC950_W4_V(19), ACC950_W4_V(20), ACC950_W4_V(21), ACC950_W4_V(22), ACC950_W4_V(23),             \

@@ -25,7 +25,8 @@ Register use (besides the operands the C++ side passes in):
     v[128:191]  fragments of even steps: B blocks 0..7 (v128..), A blocks 0..7 (v160..)
     v[192:255]  fragments of odd steps
     v[104:121]  LDS read addresses of the upper two stages (the 16-bit offset field reaches 64 KB)
-    s[72:73], s[74:75]  fill pointers of A and B (tile three ahead); s[76:77] scratch pointer; s78 loop count
+    s[72:73], s[74:75]  fill pointers of A and B (tile three ahead); s[76:77] scratch pointer; s78 loop count;
+    s79 row offset while C is loaded
 """
 STAGE = 32768      # (256 + 256) rows x 64 bytes
 B_TILE = 16384     # B's tile follows A's inside a stage
@@ -141,8 +142,17 @@ def loop(b_layout):
     else:
         for x in range(8):
             out.append(line(f"v_add_u32 v{106 + x}, 0x10000, %[b_rd{x}]"))
+    # accumulators: zero, or (C += A*B with 32-bit C) the tile of C, loaded straight into the AGPR file
+    out += [line("s_cmp_eq_u32 %[accum], 0"), line("s_cbranch_scc1 3f"), line("s_mov_b32 s79, 0")]
+    for i in range(8):
+        for j in range(8):
+            n = (i * 8 + j) * 4
+            out.append(line(f"buffer_load_dwordx4 a[{n}:{n + 3}], %[c_off], %[c_rsrc], s79 offen offset:{j * 64}"))
+        out.append(line("s_add_u32 s79, s79, %[c_row16]"))
+    out += [line("s_waitcnt vmcnt(0)"), line("s_branch 4f"), line("3:")]
     for n in range(256):
         out.append(line(f"v_accvgpr_write_b32 a{n}, 0"))
+    out.append(line("4:"))
     for x in range(8):
         out += read_b(x, 0, 0, b_layout)
     for x in range(8):

@@ -49,11 +49,12 @@ class GemmCall:
     def __init__(self, A, B, C, prologue=_lib.PROLOGUE_SET0, epilogue=_lib.EPILOGUE_RELU, variant=_lib.VARIANT_AUTO,
                  k_splits=0, stream=None, prologue_arg=0.0, epilogue_arg=0.0):
         problem = _problem(A, B, C)
+        hit = None
         if variant == _lib.VARIANT_AUTO and k_splits == 0 and problem[2] == 1:
             # a recorded choice for this very shape (accera_amd.tune --save) goes before the library's cost model
             from . import tuned
-            lean = prologue == _lib.PROLOGUE_SET0 and float(prologue_arg) == 0.0 and epilogue in (_lib.EPILOGUE_RELU, _lib.EPILOGUE_NONE)
-            hit = tuned.lookup(problem[0], problem[1], problem[3], problem[4], problem[5], problem[8:10], problem[12:14], problem[16:18], lean)
+            hit = tuned.lookup(problem[0], problem[1], problem[3], problem[4], problem[5], problem[8:10], problem[12:14], problem[16:18],
+                               tuned.ops_class(prologue, prologue_arg, epilogue))
             if hit:
                 variant, k_splits = hit
         if stream is None:
@@ -62,8 +63,14 @@ class GemmCall:
         self.tensors = (A, B, C)
         L = _lib.lib()
         handle = ctypes.c_int(-1)
-        _lib.check(L.acc950_bind(*problem, prologue, float(prologue_arg), epilogue, float(epilogue_arg), variant, k_splits, stream,
-                                 ctypes.byref(handle)))
+        rc = L.acc950_bind(*problem, prologue, float(prologue_arg), epilogue, float(epilogue_arg), variant, k_splits, stream,
+                           ctypes.byref(handle))
+        if rc and hit:
+            # the recorded kernel does not take this call after all (pointer alignment, ops): the library chooses
+            self.variant, self.k_splits = _lib.VARIANT_AUTO, 0
+            rc = L.acc950_bind(*problem, prologue, float(prologue_arg), epilogue, float(epilogue_arg), _lib.VARIANT_AUTO, 0, stream,
+                               ctypes.byref(handle))
+        _lib.check(rc)
         self._handle = handle.value
         self._launch, self._unbind = L.acc950_launch, L.acc950_unbind
 

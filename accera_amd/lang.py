@@ -480,9 +480,9 @@ def _match(source):
     if spec.variant == _lib.VARIANT_AUTO and spec.batch is None:
         # no tile named by the plan: a choice recorded for this very shape by `accera_amd.tune --save`, if any
         from . import tuned
-        lean = spec.prologue == _lib.PROLOGUE_SET and spec.prologue_arg == 0 and spec.epilogue in (_lib.EPILOGUE_RELU, _lib.EPILOGUE_NONE)
         hit = tuned.lookup(spec.A.element_type.lib_id, spec.C.element_type.lib_id, spec.M, spec.N, spec.K,
-                           spec.A.strides[-2:], spec.B.strides[-2:], spec.C.strides[-2:], lean)
+                           spec.A.strides[-2:], spec.B.strides[-2:], spec.C.strides[-2:],
+                           tuned.ops_class(spec.prologue, spec.prologue_arg, spec.epilogue))
         if hit and hit[1] == 0:  # (package functions carry a variant, not a K split)
             spec.variant = hit[0]
     return spec
@@ -503,8 +503,10 @@ def _variant_for_tile(spec, bm, bn):
             continue
         # ping-pong over software-pipelined; the 16x16 MFMA shapes where the library runs their lean build
         rank = 2 * ("pingpong" in name) + (1 if "mi16" in name and lean else -1 if "mi16" in name else 0)
-        if "hand-laid loop" in name:  # four waves, C = A*B / relu(A*B) only; measured ahead of the ping-pong form
-            rank = 4 if lean else -9
+        if "hand-laid loop" in name:  # four waves; C = A*B / relu(A*B), or C += A*B into a 32-bit C; ahead of the ping-pong form
+            adds = (spec.prologue == _lib.PROLOGUE_NONE and spec.epilogue in (_lib.EPILOGUE_RELU, _lib.EPILOGUE_NONE)
+                    and spec.C.element_type.lib_id in (_lib.F32, _lib.I32))
+            rank = 4 if (lean or adds) else -9
         if rank > best_rank:
             best, best_rank = v, rank
     return best

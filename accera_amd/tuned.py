@@ -18,9 +18,24 @@ _table = None
 _names = None
 
 
-def key(in_id, out_id, M, N, K, a_col_major, b_col_major, lean):
-    """lean: C = A*B or C = relu(A*B) (no C read, no SET / SCALE operand)."""
-    return f"{in_id}-{out_id}-{M}x{N}x{K}-{'c' if a_col_major else 'r'}{'c' if b_col_major else 'r'}-{'lean' if lean else 'full'}"
+def ops_class(prologue, prologue_arg, epilogue):
+    """Kernels differ in the prologue / epilogue ops they take, so a choice is recorded per class:
+    "lean"  C = A*B or relu(A*B)          (SET 0 prologue: C is not read)
+    "acc"   C += A*B, then ReLU or nothing (C read, no operand)
+    "full"  everything else               (SCALE / SET with an operand, the other epilogue ops)"""
+    plain = epilogue in (_lib.EPILOGUE_RELU, _lib.EPILOGUE_NONE)
+    if plain and prologue == _lib.PROLOGUE_SET and float(prologue_arg) == 0.0:
+        return "lean"
+    if plain and prologue == _lib.PROLOGUE_NONE:
+        return "acc"
+    return "full"
+
+
+def key(in_id, out_id, M, N, K, a_col_major, b_col_major, ops):
+    """ops: a class of ops_class() (True / False are read as "lean" / "full")."""
+    if isinstance(ops, bool):
+        ops = "lean" if ops else "full"
+    return f"{in_id}-{out_id}-{M}x{N}x{K}-{'c' if a_col_major else 'r'}{'c' if b_col_major else 'r'}-{ops}"
 
 
 def _load():
@@ -43,9 +58,10 @@ def _variant_by_name(name):
     return _names.get(name)
 
 
-def lookup(in_id, out_id, M, N, K, a_strides, b_strides, c_strides, lean):
-    """(variant, k_splits) recorded for this problem, or None.  Only plain row- / column-major
-    operands and a row-major C are looked up; the library still validates the choice."""
+def lookup(in_id, out_id, M, N, K, a_strides, b_strides, c_strides, ops):
+    """(variant, k_splits) recorded for this problem and class of ops (ops_class), or None.  Only plain
+    row- / column-major operands and a row-major C are looked up; the library still validates the choice
+    when the call is bound, and callers fall back to its own choice if it refuses."""
     if tuple(c_strides) != (N, 1):
         return None
     a_col = tuple(a_strides) == (1, M) and M != 1
@@ -54,7 +70,7 @@ def lookup(in_id, out_id, M, N, K, a_strides, b_strides, c_strides, lean):
         return None
     if not b_col and tuple(b_strides) != (N, 1):
         return None
-    rec = _load().get(key(in_id, out_id, M, N, K, a_col, b_col, lean))
+    rec = _load().get(key(in_id, out_id, M, N, K, a_col, b_col, ops))
     if not rec:
         return None
     v = _variant_by_name(rec.get("kernel", ""))
@@ -80,9 +96,10 @@ def save(results, path=DEFAULT_PATH, merge=True):
     for r in results:
         if r["variant"] < 0 or r["correct"] is False:
             continue
-        lean = float(r["beta"]) == 0.0 and float(r["alpha"]) == 1.0
+        alpha, beta = float(r["alpha"]), float(r["beta"])
+        ops = "lean" if (alpha == 1.0 and beta == 0.0) else "acc" if (alpha == 1.0 and beta == 1.0) else "full"
         k = key(getattr(_lib, r["type"].upper()), getattr(_lib, r["out_type"].upper()), r["m"], r["n"], r["k"],
-                bool(r["transA"]), bool(r["transB"]), lean)
+                bool(r["transA"]), bool(r["transB"]), ops)
         if k not in best or r["time_ms"] < best[k]["time_ms"]:
             best[k] = r
     for k, r in best.items():

@@ -137,6 +137,11 @@ def test_tuned_table_is_consulted_by_name_and_validated(tmp_path, monkeypatch):
     args = (_lib.F16, _lib.F32, 4096, 4096, 4096, (4096, 1), (4096, 1), (4096, 1))
     assert tuned.lookup(*args, True) == (1, 0)                 # fastest verified row
     assert tuned.lookup(*args, False) is None                  # other op class: not recorded
+    assert tuned.lookup(*args, "acc") is None and tuned.lookup(*args, "lean") == (1, 0)
+    assert tuned.ops_class(_lib.PROLOGUE_SET0, 0.0, _lib.EPILOGUE_RELU) == "lean"
+    assert tuned.ops_class(_lib.PROLOGUE_NONE, 0.0, _lib.EPILOGUE_NONE) == "acc"
+    assert tuned.ops_class(_lib.PROLOGUE_SET, 1.0, _lib.EPILOGUE_RELU) == "full"
+    assert tuned.ops_class(_lib.PROLOGUE_NONE, 0.0, _lib.EPILOGUE_SCALE) == "full"
     assert tuned.lookup(_lib.F16, _lib.F32, 1000, 1000, 1000, (1000, 1), (1000, 1), (1000, 1), True) is None
     assert tuned.lookup(_lib.F16, _lib.F32, 512, 512, 512, (512, 1), (512, 1), (512, 1), True) is None
     assert tuned.lookup(_lib.F16, _lib.F32, 4096, 4096, 4096, (4096, 1), (4096, 1), (4100, 1), True) is None  # padded C: not a table shape
