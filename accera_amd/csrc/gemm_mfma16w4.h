@@ -1,5 +1,5 @@
 // Four-wave MFMA GEMM on the 16x16 instruction shapes: one wave per SIMD, each with a 128x128
-// piece of a 256x256 output tile.
+// piece of a 256x256 output tile (or 128x96 of a 256x192 one).
 //
 // Counterpart of the same tensorized plan of the reference as gemm_mfma16.h
 // (/root/reference/accera/transforms/src/exec/ExecutionPlanToAffineLoweringPass.cpp:5986-6533),
@@ -22,12 +22,14 @@
 
 namespace acc950 {
 
-template <int IN_, bool B_KC_, bool TIMED_ = false>
+// BN: 256, or 192 (K-contiguous B only; N = 3072 = 16 x 192 gives one tile per CU) with 128x96 wave tiles
+template <int IN_, bool B_KC_, bool TIMED_ = false, int BN_ = 256>
 struct Mfma16W4Config {
     static constexpr bool TIMED = TIMED_;
-    static constexpr int IN = IN_, BM = 256, BN = 256, WAVES_M = 2, WAVES_N = 2, KB = 64, STAGES = 4, NT = 256;
+    static constexpr int IN = IN_, BM = 256, BN = BN_, WAVES_M = 2, WAVES_N = 2, KB = 64, STAGES = 4, NT = 256;
     static constexpr bool A_KC = true, B_KC = B_KC_;
     static constexpr int LDS_BYTES = STAGES * (BM + BN) * KB;
+    static_assert(BN == 256 || (BN == 192 && B_KC), "tile widths the loop is written for");
 };
 
 // accumulator blocks N and N+1 (eight registers) out of the AGPR file.  The moves go through the matrix
@@ -57,18 +59,19 @@ __device__ __forceinline__ void w4_static_for(F&& f)
 template <typename Cfg>
 __global__ void __launch_bounds__(256, 1) gemm_mfma16w4_kernel(GemmArgs p)
 {
-    constexpr int IN = Cfg::IN, BM = 256, BN = 256, NT = 256, KB = 64, WAVES_N = 2;
+    constexpr int IN = Cfg::IN, BM = 256, BN = Cfg::BN, NT = 256, KB = 64, WAVES_N = 2;
     constexpr bool B_KC = Cfg::B_KC;
     constexpr int ES = InTraits<IN>::ES;
     constexpr int BK = KB / ES;
-    constexpr int WTM = 128, WTN = 128, TM = 8, TN = 8;
+    constexpr int WTM = 128, WTN = BN / 2, TM = 8, TN = WTN / 16;
+    constexpr int FILLS_B = BN * KB / (NT * 16), FILLS = 4 + FILLS_B; // fill instructions per thread and K tile
     // (swizzle and address arithmetic only: these are the tiles of the eight-wave kernel)
     using TA = OperandTile<IN, BM, true, 512, KB, true>;
     using TB = OperandTile<IN, BN, B_KC, 512, KB, true>;
     using acc_t = typename In16Traits<IN>::acc_t;
     using scalar_t = typename In16Traits<IN>::scalar_t;
     constexpr int STAGE_BYTES = TA::TILE_BYTES + TB::TILE_BYTES;
-    static_assert(STAGE_BYTES == 32768 && TA::TILE_BYTES == 16384, "the loop's offsets are written for these");
+    static_assert(STAGE_BYTES == 16384 + TN * 2048 && TA::TILE_BYTES == 16384, "the loop's offsets are written for these");
 
     extern __shared__ __attribute__((aligned(1024))) char smem[];
     select_batch(p);
@@ -131,7 +134,7 @@ __global__ void __launch_bounds__(256, 1) gemm_mfma16w4_kernel(GemmArgs p)
         for (int f = 0; f < 4; ++f)
             TA::direct_issue(ldsb + s * STAGE_BYTES + f * 4096, a_off, a_tile + (int64_t)s * sa + (int64_t)f * da);
 #pragma unroll
-        for (int f = 0; f < 4; ++f)
+        for (int f = 0; f < FILLS_B; ++f)
             TB::direct_issue(ldsb + s * STAGE_BYTES + TA::TILE_BYTES + f * 4096, (f & 1) ? b_off1 : b_off0,
                              b_tile + (int64_t)s * sb + (int64_t)f * db);
     }
@@ -168,7 +171,7 @@ __global__ void __launch_bounds__(256, 1) gemm_mfma16w4_kernel(GemmArgs p)
     const unsigned c_row16 = __builtin_amdgcn_readfirstlane((unsigned)p.c_rs * 64);
     const auto c_rsrc = c_in.rsrc;
 
-    wait_vmcnt<16>(); // tile 0 has landed (tiles 1 and 2 in flight)
+    wait_vmcnt<2 * FILLS>(); // tile 0 has landed (tiles 1 and 2 in flight)
     __syncthreads();
     stamp(1);
 
@@ -190,7 +193,11 @@ __global__ void __launch_bounds__(256, 1) gemm_mfma16w4_kernel(GemmArgs p)
 #define ACC950_W4_R(f, d) f #d "0", f #d "1", f #d "2", f #d "3", f #d "4", f #d "5", f #d "6", f #d "7", f #d "8", f #d "9"
 #define ACC950_W4_V(d) ACC950_W4_R("v", d)
 #define ACC950_W4_A(d) ACC950_W4_R("a", d)
-    if constexpr (B_KC) {
+    if constexpr (B_KC && BN == 192) {
+        if constexpr (IN == IN_F16) asm volatile(ACC950_W4_LOOP_KC6("v_mfma_f32_16x16x32_f16") : ACC950_W4_OPERANDS);
+        else if constexpr (IN == IN_BF16) asm volatile(ACC950_W4_LOOP_KC6("v_mfma_f32_16x16x32_bf16") : ACC950_W4_OPERANDS);
+        else asm volatile(ACC950_W4_LOOP_KC6("v_mfma_i32_16x16x64_i8") : ACC950_W4_OPERANDS);
+    } else if constexpr (B_KC) {
         if constexpr (IN == IN_F16) asm volatile(ACC950_W4_LOOP_KC("v_mfma_f32_16x16x32_f16") : ACC950_W4_OPERANDS);
         else if constexpr (IN == IN_BF16) asm volatile(ACC950_W4_LOOP_KC("v_mfma_f32_16x16x32_bf16") : ACC950_W4_OPERANDS);
         else asm volatile(ACC950_W4_LOOP_KC("v_mfma_i32_16x16x64_i8") : ACC950_W4_OPERANDS);
@@ -218,7 +225,7 @@ __global__ void __launch_bounds__(256, 1) gemm_mfma16w4_kernel(GemmArgs p)
         auto load_row = [&](auto i_tag, acc_t (&row)[TN]) {
             constexpr int i = decltype(i_tag)::value;
             w4_static_for<0, TN / 2>([&](auto h) {
-                const W4BlockPair pr = w4_acc_pair<i * 8 + h.value * 2>();
+                const W4BlockPair pr = w4_acc_pair<i * TN + h.value * 2>();
                 row[h.value * 2] = __builtin_bit_cast(acc_t, pr.a);
                 row[h.value * 2 + 1] = __builtin_bit_cast(acc_t, pr.b);
             });
@@ -241,7 +248,7 @@ __global__ void __launch_bounds__(256, 1) gemm_mfma16w4_kernel(GemmArgs p)
                 acc_t row[TN];
                 if constexpr (RELU) load_row(i, row);
                 w4_static_for<0, TN>([&](auto j) {
-                    constexpr int n = i.value * 8 + j.value;
+                    constexpr int n = i.value * TN + j.value;
                     if constexpr (RELU) {
                         __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, row[j.value]), tile.rsrc, lane_off + j.value * 64, soff, 0);
                     } else {
@@ -282,6 +289,7 @@ __global__ void __launch_bounds__(256, 1) gemm_mfma16w4_kernel(GemmArgs p)
 #pragma unroll
                     for (int it = 0; it < PIECES; ++it) {
                         const int id = it * 64 + lane;
+                        if ((16 * CPRW) % 64 != 0 && id >= 16 * CPRW) break;
                         const int r = id / CPRW, cc = id % CPRW;
                         const i32x4 v = *(const i32x4*)(slab + r * PITCH + cc * 16);
                         __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), tile.rsrc, (unsigned)r * row_bytes + cc * 16,

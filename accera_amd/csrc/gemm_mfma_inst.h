@@ -25,6 +25,8 @@ namespace acc950 {
 // four waves, 128x128 wave tiles, hand-laid K loop
 #define V16W4(BKC) \
     { 256, 256, 2, 2, true, BKC, true, false, 64, 4, false, true, true, &launch_mfma16w4<Mfma16W4Config<ACC950_IN, BKC>>, nullptr }
+#define V16W4_192 \
+    { 256, 192, 2, 2, true, true, true, false, 64, 4, false, true, true, &launch_mfma16w4<Mfma16W4Config<ACC950_IN, true, false, 192>>, nullptr }
 #define V(BM, BN, WM, WN, BKC, DIRECT, EDGE, KB, STAGES) VA(true, BM, BN, WM, WN, BKC, DIRECT, EDGE, KB, STAGES)
 #define VP(BM, BN, WM, WN, BKC, KB, STAGES) VPA(true, BM, BN, WM, WN, BKC, KB, STAGES)
 // column-major A (M contiguous; the "transA" shapes of the reference's sweep lists,
@@ -68,12 +70,14 @@ static const MfmaVariant kVariants[] = {
     V16(true, 256, 192, 4, 2, true, 64, 4),
     V16W4(false),
     V16W4(true),
+    V16W4_192,
 };
 #undef LAYOUT_AT
 #undef VA
 #undef VPA
 #undef V16
 #undef V16W4
+#undef V16W4_192
 #undef LAYOUT
 #undef V
 #undef VP

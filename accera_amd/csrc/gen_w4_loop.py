@@ -13,7 +13,7 @@ hand: registers are fixed, and each k-step of 64 bytes is
     s_waitcnt lgkmcnt(4)            fragments of this step are in registers (all but A's last four)
     32 MFMAs (rows 0..63 of the wave tile), the 8 fill instructions of the step three ahead
     and their address arithmetic spread between them, at most two per MFMA
-    s_waitcnt vmcnt(16); s_barrier  the tile of the next step has landed for every wave
+    s_waitcnt vmcnt(2 tiles' fills); s_barrier  the tile of the next step has landed for every wave
     32 MFMAs (rows 64..127), the fragment reads of the next step between them, one per MFMA
 
 The four LDS stages rotate with the k-step, so the body is written out for four steps; the last
@@ -21,20 +21,27 @@ four steps (no more fills, then no more reads) are a second copy.  K must be a m
 steps.
 
 Register use (besides the operands the C++ side passes in):
-    a[0:255]    accumulators, block (i, j) at a[(i*8+j)*4 .. +3]
+    a[0:255]    accumulators, block (i, j) at a[(i*TN+j)*4 .. +3] (TN = 8 blocks of columns per wave, 6 for the 192-wide tile)
     v[128:191]  fragments of even steps: B blocks 0..7 (v128..), A blocks 0..7 (v160..)
     v[192:255]  fragments of odd steps
     v[104:121]  LDS read addresses of the upper two stages (the 16-bit offset field reaches 64 KB)
     s[72:73], s[74:75]  fill pointers of A and B (tile three ahead); s[76:77] scratch pointer; s78 loop count;
     s79 row offset while C is loaded
 """
-STAGE = 32768      # (256 + 256) rows x 64 bytes
-B_TILE = 16384     # B's tile follows A's inside a stage
+B_TILE = 16384     # B's tile follows A's (256 rows x 64 bytes) inside a stage
 FRAG = 1024        # 16 rows x 64 bytes (K-contiguous operand)
+TN = 8             # blocks of 16 columns per wave: 8 (256-wide tile) or 6 (192-wide, K-contiguous B only)
+STAGE = 32768      # A's tile + B's tile (2 * TN * 16 rows x 64 bytes)
+
+
+def set_width(tn):
+    global TN, STAGE
+    TN = tn
+    STAGE = B_TILE + 2 * tn * FRAG
 
 
 def acc(i, j):
-    n = (i * 8 + j) * 4
+    n = (i * TN + j) * 4
     return f"a[{n}:{n + 3}]"
 
 
@@ -81,53 +88,59 @@ def read_b(x, stage, buf, b_layout):
     return out
 
 
-def fill(f, phase, stage, b_layout):
-    """Fill instruction f (0..3 A, 4..7 B) of a K tile, spread over four MFMA slots: pointer, M0,
-    the load (the MFMA between the M0 write and the load is the wait state M0 needs), pointer advance."""
+def fill(f, stage, b_layout):
+    """Fill instruction f (0..3 A, 4.. B) of a K tile as a list of MFMA slots: pointer, M0, the load (the MFMA
+    between the M0 write and the load is the wait state M0 needs; the last pass also advances the pointer)."""
     if f < 4:
-        ptr, d, s, lane, tile, g = "s[72:73]", "%[da]", "%[sa]", "%[a_off]", 0, f
+        ptr, d, s, lane, tile, g, last = "s[72:73]", "%[da]", "%[sa]", "%[a_off]", 0, f, 3
     else:
         g = f - 4
-        ptr, d, s, tile = "s[74:75]", "%[db]", "%[sb]", B_TILE
+        ptr, d, s, tile, last = "s[74:75]", "%[db]", "%[sb]", B_TILE, (2 * TN * FRAG) // 4096 - 1
         lane = "%[b_off0]" if (b_layout == "kc" or g % 2 == 0) else "%[b_off1]"
-    if phase == 0:
-        if g == 0:
-            return [line(f"s_mov_b64 s[76:77], {ptr}")]
-        return [line(f"s_add_u32 s76, s76, {d}"), line("s_addc_u32 s77, s77, 0")]
-    if phase == 1:
-        return [line(f"s_add_u32 m0, %[ldsb], {stage * STAGE + tile + g * 4096}")]
-    if phase == 2:
-        return [line(f"global_load_lds_dwordx4 {lane}, s[76:77]")]
-    if g == 3:  # advance to the next K tile
+    slots = []
+    if g == 0:
+        slots.append([line(f"s_mov_b64 s[76:77], {ptr}")])
+    else:
+        slots.append([line(f"s_add_u32 s76, s76, {d}"), line("s_addc_u32 s77, s77, 0")])
+    slots.append([line(f"s_add_u32 m0, %[ldsb], {stage * STAGE + tile + g * 4096}")])
+    slots.append([line(f"global_load_lds_dwordx4 {lane}, s[76:77]")])
+    if g == last:  # advance to the next K tile
         lo, hi = (72, 73) if f < 4 else (74, 75)
-        return [line(f"s_add_u32 s{lo}, s{lo}, {s}"), line(f"s_addc_u32 s{hi}, s{hi}, 0")]
-    return []
+        slots[-1] += [line(f"s_add_u32 s{lo}, s{lo}, {s}"), line(f"s_addc_u32 s{hi}, s{hi}, 0")]
+    return slots
 
 
 def step(pos, do_fill, wait, last, b_layout):
     buf, nxt, fst = pos % 2, (pos + 1) % 4, (pos + 3) % 4
     # fragments of B and of A's first four blocks are in registers (the last four reads may still be in flight)
     out = [line("s_waitcnt lgkmcnt(4)")]
-    order = [(i, j) for i in range(8) for j in range(8)]
-    for s, (i, j) in enumerate(order[:32]):
+    order = [(i, j) for i in range(8) for j in range(TN)]
+    half = 4 * TN
+    extra = [[] for _ in range(half)]
+    if do_fill:
+        # A's fills come last in odd steps and first in even ones: the two 64-byte halves of a 128-byte
+        # line of a K-contiguous operand belong to k-steps 2m and 2m+1, filled in steps 2m-3 and 2m-2;
+        # requested back to back, the second half is still in the CU's vector cache
+        nb = (2 * TN * FRAG) // 4096
+        fills = list(range(4 + nb)) if pos % 2 == 0 else list(range(4, 4 + nb)) + list(range(4))
+        per = half // len(fills)  # MFMA slots per fill: 4 (256-wide) or 3 (192-wide)
+        for n, f in enumerate(fills):
+            for k, ins in enumerate(fill(f, fst, b_layout)):
+                extra[n * per + k] += ins
+    for s, (i, j) in enumerate(order[:half]):
         out.append(mfma(i, j, buf))
-        if do_fill:
-            # A's fills come last in odd steps and first in even ones: the two 64-byte halves of a 128-byte
-            # line of a K-contiguous operand belong to k-steps 2m and 2m+1, filled in steps 2m-3 and 2m-2;
-            # requested back to back, the second half is still in the CU's vector cache
-            f = s // 4 if pos % 2 == 0 else (s // 4 + 4) % 8
-            out += fill(f, s % 4, fst, b_layout)
+        out += extra[s]
     out.append(line("s_waitcnt lgkmcnt(0)"))
     if not last:
         out.append(line(f"s_waitcnt vmcnt({wait})"))
         out.append(line("s_barrier"))
     reads = []
     if not last:
-        for x in range(8):
+        for x in range(TN):
             reads += read_b(x, nxt, buf ^ 1, b_layout)
         for x in range(8):
             reads += read_a(x, nxt, buf ^ 1)
-    for s, (i, j) in enumerate(order[32:]):
+    for s, (i, j) in enumerate(order[half:]):
         out.append(mfma(i, j, buf))
         if s < len(reads):
             out.append(reads[s])
@@ -136,33 +149,34 @@ def step(pos, do_fill, wait, last, b_layout):
 
 def loop(b_layout):
     out = [line("s_mov_b64 s[72:73], %[pa]"), line("s_mov_b64 s[74:75], %[pb]"), line("s_mov_b32 s78, %[groups]"),
-           line("v_add_u32 v104, 0x10000, %[a_rd]")]
+           line(f"v_add_u32 v104, {2 * STAGE}, %[a_rd]")]
     if b_layout == "kc":
-        out.append(line("v_add_u32 v105, 0x10000, %[b_rd0]"))
+        out.append(line(f"v_add_u32 v105, {2 * STAGE}, %[b_rd0]"))
     else:
         for x in range(8):
-            out.append(line(f"v_add_u32 v{106 + x}, 0x10000, %[b_rd{x}]"))
+            out.append(line(f"v_add_u32 v{106 + x}, {2 * STAGE}, %[b_rd{x}]"))
     # accumulators: zero, or (C += A*B with 32-bit C) the tile of C, loaded straight into the AGPR file
     out += [line("s_cmp_eq_u32 %[accum], 0"), line("s_cbranch_scc1 3f"), line("s_mov_b32 s79, 0")]
     for i in range(8):
-        for j in range(8):
-            n = (i * 8 + j) * 4
+        for j in range(TN):
+            n = (i * TN + j) * 4
             out.append(line(f"buffer_load_dwordx4 a[{n}:{n + 3}], %[c_off], %[c_rsrc], s79 offen offset:{j * 64}"))
         out.append(line("s_add_u32 s79, s79, %[c_row16]"))
     out += [line("s_waitcnt vmcnt(0)"), line("s_branch 4f"), line("3:")]
-    for n in range(256):
+    for n in range(32 * TN):
         out.append(line(f"v_accvgpr_write_b32 a{n}, 0"))
     out.append(line("4:"))
-    for x in range(8):
+    for x in range(TN):
         out += read_b(x, 0, 0, b_layout)
     for x in range(8):
         out += read_a(x, 0, 0)
     out += [line("s_nop 7"), line("s_cmp_eq_u32 s78, 0"), line("s_cbranch_scc1 2f"), line("1:")]
+    per_tile = 4 + (2 * TN * FRAG) // 4096  # fill instructions per K tile and thread
     for pos in range(4):
-        out += step(pos, True, 16, False, b_layout)
+        out += step(pos, True, 2 * per_tile, False, b_layout)
     out += [line("s_sub_u32 s78, s78, 1"), line("s_cmp_lg_u32 s78, 0"), line("s_cbranch_scc1 1b"), line("2:")]
-    out += step(0, True, 16, False, b_layout)
-    out += step(1, False, 8, False, b_layout)
+    out += step(0, True, 2 * per_tile, False, b_layout)
+    out += step(1, False, per_tile, False, b_layout)
     out += step(2, False, 0, False, b_layout)
     out += step(3, False, 0, True, b_layout)
     out += [line("s_nop 15"), line("s_nop 15")]
@@ -172,9 +186,10 @@ def loop(b_layout):
 def main():
     print("// Generated by gen_w4_loop.py; do not edit.  The K loop of gemm_mfma16w4_kernel, one macro per")
     print("// layout of B (K contiguous / N contiguous 16-bit / N contiguous 8-bit); MFMA is the mnemonic.")
-    for name in ("kc", "mc16", "mc8"):
+    for name, tn in (("kc", 8), ("mc16", 8), ("mc8", 8), ("kc", 6)):
+        set_width(tn)
         body = loop(name)
-        print(f"#define ACC950_W4_LOOP_{name.upper()}(MFMA) \\")
+        print(f"#define ACC950_W4_LOOP_{name.upper()}{'' if tn == 8 else tn}(MFMA) \\")
         print(" \\\n".join("    " + s for s in body))
         print()
 

@@ -247,17 +247,17 @@ def test_four_wave_kernel_every_output_type(in_type, out_type, b_layout):
     takes, every store path (32-bit straight from the accumulator registers, narrow types through
     LDS), 6 output tiles so that the tile map and both wave rows / columns are exercised, K at one,
     two and five rounds of the four LDS stages."""
-    v = _hand_laid(b_layout)
     kb = 64 if in_type == "i8" else 32
-    for k_tiles, epi in ((4, ora.EPI_RELU), (8, ora.EPI_NONE), (20, ora.EPI_RELU)):
-        print("variant", v, in_type, out_type, b_layout, "k tiles", k_tiles, flush=True)
-        run_case(in_type, out_type, 512, 768, k_tiles * kb, b_layout=b_layout, variant=v, seed=700 + k_tiles, epilogue=epi)
-    if out_type in ("f32", "i32"):
-        # C += A*B: the tile of C is loaded into the accumulator registers before the loop
-        for k_tiles, epi in ((4, ora.EPI_NONE), (12, ora.EPI_RELU)):
-            print("variant", v, in_type, out_type, b_layout, "accumulating, k tiles", k_tiles, flush=True)
-            run_case(in_type, out_type, 512, 768, k_tiles * kb, b_layout=b_layout, variant=v, seed=720 + k_tiles, epilogue=epi,
-                     prologue=ora.PRO_NONE)
+    for v in [v for v, n in _variants(b_layout) if "hand-laid" in n]:  # 256x256, and 256x192 for column-major B
+        for k_tiles, epi in ((4, ora.EPI_RELU), (8, ora.EPI_NONE), (20, ora.EPI_RELU)):
+            print("variant", v, in_type, out_type, b_layout, "k tiles", k_tiles, flush=True)
+            run_case(in_type, out_type, 512, 768, k_tiles * kb, b_layout=b_layout, variant=v, seed=700 + k_tiles, epilogue=epi)
+        if out_type in ("f32", "i32"):
+            # C += A*B: the tile of C is loaded into the accumulator registers before the loop
+            for k_tiles, epi in ((4, ora.EPI_NONE), (12, ora.EPI_RELU)):
+                print("variant", v, in_type, out_type, b_layout, "accumulating, k tiles", k_tiles, flush=True)
+                run_case(in_type, out_type, 512, 768, k_tiles * kb, b_layout=b_layout, variant=v, seed=720 + k_tiles, epilogue=epi,
+                         prologue=ora.PRO_NONE)
 
 
 def test_four_wave_kernel_is_refused_for_what_it_does_not_take():
