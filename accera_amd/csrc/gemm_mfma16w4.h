@@ -269,7 +269,10 @@ __global__ void __launch_bounds__(256, 1) gemm_mfma16w4_kernel(GemmArgs p)
             auto staged = [&](auto os_tag, auto&& pack) {
                 constexpr int OS = decltype(os_tag)::value;
                 constexpr int ROW = WTN * OS;
-                constexpr int PITCH = (ROW / 32) % 2 == 0 ? ROW + 32 : ROW;
+                // 16 bytes past a row: the 16 row starts are an odd number of 4-bank steps apart, so a lane group's
+                // 8- or 4-byte pieces of 16 rows land on 64 different banks
+                constexpr int PITCH = ROW + 16;
+                static_assert(ROW % 32 == 0, "(ROW / 16 + 1) must be odd for the 16 row starts to differ mod 64 banks");
                 char* slab = smem + wave_u * (16 * PITCH);
                 const CTile tile = c_tile((char*)p.C + ((int64_t)(m0 + (wave_u / WAVES_N) * WTM) * p.c_rs + n0 + (wave_u % WAVES_N) * WTN) * OS);
                 const unsigned row_bytes = (unsigned)p.c_rs * OS;
