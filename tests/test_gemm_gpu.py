@@ -577,7 +577,8 @@ def test_benchmark_configurations_at_full_size(cfg):
 @pytest.mark.parametrize("case", [("f16", "f32", 3, 1280, 768, 1024, -1), ("bf16", "bf16", 8, 256, 384, 128, -1), ("i8", "i32", 4, 256, 256, 512, -1),
                                   ("i8", "i16", 3, 256, 256, 512, -1), ("i8", "i8", 5, 128, 384, 256, -1),
                                   ("f32", "f32", 32, 128, 128, 128, -1), ("f16", "f16", 5, 100, 72, 40, -1), ("f16", "f16", 6, 8, 1088, 512, -1),
-                                  ("f16", "f16", 3, 8, 1088, 512, 100), ("bf16", "f32", 2, 5, 1000, 998, -1), ("f16", "f32", 1, 64, 64, 64, -1)])
+                                  ("f16", "f16", 3, 8, 1088, 512, 100), ("bf16", "f32", 2, 5, 1000, 998, -1), ("f16", "f32", 1, 64, 64, 64, -1),
+                                  ("f16", "f32", 3, 512, 768, 512, "hand-laid"), ("i8", "i32", 2, 256, 512, 1024, "hand-laid")])
 def test_batched_gemm(case):
     """C[b] = relu(A[b] @ B[b]) in one launch: the reference's batch matmul nest
     (mfma_tests.py:435-549; shapes 3 x 1280x768x1024, 8 x ..., 32 x 128^3, 1 x 64^3 from :2519-2549) on
@@ -585,6 +586,8 @@ def test_batched_gemm(case):
     import accera_amd as acc
     import torch
     in_type, out_type, batch, M, N, K, variant = case
+    if variant == "hand-laid":  # the four-wave kernel, named (it also accumulates into a 32-bit C)
+        variant = _hand_laid("row")
     rng = np.random.default_rng(batch * 1000 + M)
     A = np.stack([make_input(rng, (M, K), in_type, "normal") for _ in range(batch)])
     B = np.stack([make_input(rng, (K, N), in_type, "normal") for _ in range(batch)])
