@@ -123,6 +123,8 @@ def step(pos, do_fill, wait, last, b_layout):
         # requested back to back, the second half is still in the CU's vector cache
         nb = (2 * TN * FRAG) // 4096
         fills = list(range(4 + nb)) if pos % 2 == 0 else list(range(4, 4 + nb)) + list(range(4))
+        # fill() chains the scratch pointer from one pass of an operand to its next: passes must come in order
+        assert [f for f in fills if f < 4] == [0, 1, 2, 3] and [f for f in fills if f >= 4] == list(range(4, 4 + nb))
         per = half // len(fills)  # MFMA slots per fill: 4 (256-wide) or 3 (192-wide)
         for n, f in enumerate(fills):
             for k, ins in enumerate(fill(f, fst, b_layout)):
