@@ -1,0 +1,155 @@
+"""The K loop of the four-wave GEMM kernel is generated assembly text (accera_amd/csrc/gen_w4_loop.py ->
+gemm_mfma16w4_loop.inc).  These checks read that text on the CPU: the include in the tree is what the
+generator writes, and every k-step keeps the invariants the kernel's correctness (and the safety of its
+global addresses) rests on -- one MFMA per accumulator block, fragment reads that land in the other
+register set and stay inside the LDS stage they are meant for, fill passes of an operand in order (the
+scratch pointer is chained from pass to pass), one pointer advance per operand and step, and wait
+counts that match the number of fills in flight."""
+import importlib.util
+import os
+import re
+
+import pytest
+
+CSRC = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "accera_amd", "csrc")
+
+
+def _gen():
+    spec = importlib.util.spec_from_file_location("gen_w4_loop", os.path.join(CSRC, "gen_w4_loop.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    return mod
+
+
+def _text(lines):
+    """Generator lines -> plain instructions ('MFMA a[..], ..' for the MFMA macro lines)."""
+    out = []
+    for l in lines:
+        m = re.match(r'^MFMA " (.*)\\n"$', l)
+        out.append("MFMA " + m.group(1) if m else re.match(r'^"(.*)\\n"$', l).group(1))
+    return out
+
+
+def test_include_in_the_tree_is_what_the_generator_writes(capsys):
+    g = _gen()
+    g.main()
+    assert capsys.readouterr().out == open(os.path.join(CSRC, "gemm_mfma16w4_loop.inc")).read()
+
+
+@pytest.mark.parametrize("layout,tn", [("kc", 8), ("mc16", 8), ("mc8", 8), ("kc", 6)])
+def test_every_k_step_keeps_its_invariants(layout, tn):
+    g = _gen()
+    g.set_width(tn)
+    stage_bytes, b_tile = g.STAGE, g.B_TILE
+    assert stage_bytes == 16384 + tn * 2048 and 4 * stage_bytes <= 160 * 1024
+    nb = tn * 2048 // 4096                      # fill passes of B per K tile
+    per_tile = 4 + nb
+    for pos in range(4):
+        for do_fill, wait, last in ((True, 2 * per_tile, False), (False, per_tile, False), (False, 0, False), (False, 0, True)):
+            ins = _text(g.step(pos, do_fill, wait, last, layout))
+            buf, nxt, fst = pos % 2, (pos + 1) % 4, (pos + 3) % 4
+            # ---- MFMAs: every accumulator block once, operands from this step's register set
+            blocks = []
+            for i in ins:
+                m = re.match(r"MFMA a\[(\d+):(\d+)\], v\[(\d+):(\d+)\], v\[(\d+):(\d+)\], a\[(\d+):(\d+)\]$", i)
+                if not m:
+                    continue
+                d0, d1, b0, b1, a0, a1, c0, c1 = map(int, m.groups())
+                assert (d0, d1) == (c0, c1) and d1 == d0 + 3 and d0 % 4 == 0 and d1 < 32 * tn
+                blk = d0 // 4
+                bi, bj = divmod(blk, tn)
+                assert b0 == 128 + buf * 64 + bj * 4 and b1 == b0 + 3      # B's fragment: first operand
+                assert a0 == 160 + buf * 64 + bi * 4 and a1 == a0 + 3      # A's fragment: second operand
+                blocks.append(blk)
+            assert sorted(blocks) == list(range(8 * tn))
+            # ---- fragment reads of the next step: other register set, inside the next step's LDS stage
+            reads = [i for i in ins if i.startswith("ds_read")]
+            assert len(reads) == (0 if last else 8 + (tn if layout == "kc" else 2 * tn))
+            written = set()
+            for r in reads:
+                m = re.match(r"(ds_read_b128|ds_read_b64_tr_b16|ds_read_b64_tr_b8) v\[(\d+):(\d+)\], (\S+) offset:(\d+)$", r)
+                op, v0, v1, base, off = m.group(1), int(m.group(2)), int(m.group(3)), m.group(4), int(m.group(5))
+                assert 128 + (buf ^ 1) * 64 <= v0 and v1 < 128 + (buf ^ 1) * 64 + 64, "reads must not touch the registers in use"
+                assert not written & set(range(v0, v1 + 1))
+                written |= set(range(v0, v1 + 1))
+                upper = not base.startswith("%")                  # v104.. hold the addresses of stages 2 and 3
+                assert upper == (nxt >= 2)
+                assert off < 65536                                # the instruction's offset field
+                in_stage = off - (nxt & 1) * stage_bytes
+                assert 0 <= in_stage < stage_bytes
+                is_b = 128 + (buf ^ 1) * 64 <= v0 < 160 + (buf ^ 1) * 64
+                assert (in_stage >= b_tile) == is_b
+                assert (op == "ds_read_b128") == (layout == "kc" or not is_b)
+            assert len(written) == (0 if last else (8 + tn) * 4)
+            # ---- fills of the tile three steps ahead
+            loads = [n for n, i in enumerate(ins) if i.startswith("global_load_lds")]
+            assert len(loads) == (per_tile if do_fill else 0)
+            if do_fill:
+                first_mfma_after_barrier = ins.index("s_barrier")
+                assert max(loads) < first_mfma_after_barrier      # all issued before this step's wait
+                seen = {"a": [], "b": []}
+                chain = None                                       # operand the scratch pointer currently belongs to
+                m0 = None
+                advanced = []
+                for n, i in enumerate(ins[:first_mfma_after_barrier]):
+                    if i.startswith("s_mov_b64 s[76:77], "):
+                        chain = {"s[72:73]": "a", "s[74:75]": "b"}[i.split(", ")[1]]
+                        assert not seen[chain], "an operand's first pass starts from its tile pointer"
+                    elif i.startswith("s_add_u32 s76, s76, "):
+                        assert chain == {"%[da]": "a", "%[db]": "b"}[i.split(", ")[2]] and seen[chain]
+                        assert ins[n + 1] == "s_addc_u32 s77, s77, 0"
+                    elif i.startswith("s_add_u32 m0, %[ldsb], "):
+                        m0 = int(i.split(", ")[2])
+                    elif i.startswith("global_load_lds"):
+                        assert ins[n - 1].startswith("MFMA"), "one instruction between the M0 write and its use"
+                        lane = i.split()[1].rstrip(",")
+                        g_pass = len(seen[chain])
+                        tile = 0 if chain == "a" else b_tile
+                        assert m0 == fst * stage_bytes + tile + g_pass * 4096
+                        assert m0 + 4096 <= 4 * stage_bytes
+                        if chain == "a":
+                            assert lane == "%[a_off]"
+                        else:
+                            assert lane == ("%[b_off0]" if layout == "kc" or g_pass % 2 == 0 else "%[b_off1]")
+                        seen[chain].append(g_pass)
+                        m0 = None
+                    elif re.match(r"s_add_u32 s7[24], s7[24], %\[s[ab]\]$", i):
+                        op = "a" if "s72" in i else "b"
+                        assert i.endswith("%[sa]") == (op == "a")
+                        assert len(seen[op]) == (4 if op == "a" else nb), "the tile pointer moves on after the operand's last pass"
+                        advanced.append(op)
+                assert seen == {"a": [0, 1, 2, 3], "b": list(range(nb))} and sorted(advanced) == ["a", "b"]
+            # ---- waits
+            assert ins[0] == "s_waitcnt lgkmcnt(4)"
+            assert ("s_barrier" in ins) == (not last)
+            if not last:
+                b = ins.index("s_barrier")
+                assert ins[b - 1] == f"s_waitcnt vmcnt({wait})" and ins[b - 2] == "s_waitcnt lgkmcnt(0)"
+
+
+@pytest.mark.parametrize("layout,tn", [("kc", 8), ("mc16", 8), ("kc", 6)])
+def test_whole_loop_shape(layout, tn):
+    """Preamble, four-step body with its back branch, and the four closing steps (one with fills, three without)."""
+    g = _gen()
+    g.set_width(tn)
+    ins = _text(g.loop(layout))
+    per_tile = 4 + tn * 2048 // 4096
+    assert ins.count("1:") == 1 and ins.count("2:") == 1 and ins.index("1:") < ins.index("s_cbranch_scc1 1b") < ins.index("2:")
+    body = ins[ins.index("1:"):ins.index("2:")]
+    tail = ins[ins.index("2:"):]
+    assert sum(i.startswith("MFMA") for i in body) == 4 * 8 * tn == sum(i.startswith("MFMA") for i in tail)
+    assert body.count("s_barrier") == 4 and tail.count("s_barrier") == 3
+    assert sum(i.startswith("global_load_lds") for i in body) == 4 * per_tile
+    assert sum(i.startswith("global_load_lds") for i in tail) == per_tile
+    assert [i for i in tail if i.startswith("s_waitcnt vmcnt")] == [f"s_waitcnt vmcnt({2 * per_tile})", f"s_waitcnt vmcnt({per_tile})", "s_waitcnt vmcnt(0)"]
+    # accumulators: zeroed, or loaded from C block by block (64 bytes per block and row group, 16 rows further per row of blocks)
+    pre = ins[:ins.index("1:")]
+    assert sum(i.startswith("v_accvgpr_write_b32") for i in pre) == 32 * tn
+    c_loads = [i for i in pre if i.startswith("buffer_load_dwordx4")]
+    assert len(c_loads) == 8 * tn
+    for n, i in enumerate(c_loads):
+        m = re.match(r"buffer_load_dwordx4 a\[(\d+):(\d+)\], %\[c_off\], %\[c_rsrc\], s79 offen offset:(\d+)$", i)
+        assert int(m.group(1)) == n * 4 and int(m.group(2)) == n * 4 + 3 and int(m.group(3)) == (n % tn) * 64
+    assert pre.count("s_add_u32 s79, s79, %[c_row16]") == 8
+    # the loop ends with enough idle cycles for the last MFMA results to be readable
+    assert ins[-2:] == ["s_nop 15", "s_nop 15"]
