@@ -11,7 +11,8 @@ its own (it moves accumulators between the two files and spills), so the loop is
 hand: registers are fixed, and each k-step of 64 bytes is
 
     s_waitcnt lgkmcnt(4)            fragments of this step are in registers (all but A's last four)
-    32 MFMAs (rows 0..63 of the wave tile), the 8 fill instructions of the step three ahead
+    32 MFMAs (rows 0..63 of the wave tile, column by column with the rows back and forth, so that
+    consecutive MFMAs share one operand: 0.6-1 % faster than row by row), the 8 fill instructions of the step three ahead
     and their address arithmetic spread between them, at most two per MFMA
     s_waitcnt vmcnt(2 tiles' fills); s_barrier  the tile of the next step has landed for every wave
     32 MFMAs (rows 64..127), the fragment reads of the next step between them, one per MFMA
@@ -114,7 +115,12 @@ def step(pos, do_fill, wait, last, b_layout):
     buf, nxt, fst = pos % 2, (pos + 1) % 4, (pos + 3) % 4
     # fragments of B and of A's first four blocks are in registers (the last four reads may still be in flight)
     out = [line("s_waitcnt lgkmcnt(4)")]
-    order = [(i, j) for i in range(8) for j in range(TN)]
+    # (columns back and forth: consecutive MFMAs always share one operand)
+    order = []
+    for h in range(2):  # rows 0..3 of blocks before the barrier, 4..7 after; inside a half column by column, rows back and forth
+        for j in range(TN):
+            rows = range(4 * h, 4 * h + 4)
+            order += [(i, j) for i in (rows if j % 2 == 0 else reversed(rows))]
     half = 4 * TN
     extra = [[] for _ in range(half)]
     if do_fill:
