@@ -14,8 +14,9 @@
 // the stores are those of gemm_mfma16.h.
 //
 // Takes: A row-major, whole tiles, K a multiple of four k-steps (256 bytes), rows of C 16 bytes aligned;
-// C = A*B or relu(A*B) (SET 0 prologue) for every output type, C += A*B (then ReLU or nothing) for
-// 32-bit outputs, where the tile of C is loaded straight into the accumulator registers.
+// C = A*B or relu(A*B) (SET 0 prologue) for every output type; C += A*B (then ReLU or nothing) for 32-bit
+// outputs, where the tile of C is loaded straight into the accumulator registers, and for 16-bit outputs,
+// where it is widened on the way in.
 #pragma once
 #include "gemm_mfma16.h"
 #include "gemm_mfma16w4_loop.inc"
@@ -163,13 +164,57 @@ __global__ void __launch_bounds__(256, 1) gemm_mfma16w4_kernel(GemmArgs p)
         }
     }
 
-    // C += A*B with a 32-bit C: the loop starts from the tile of C instead of zeros (the host sends nothing else
-    // with a prologue other than SET 0 here).  Lane l owns row i*16 + l%16, columns j*16 + (l/16)*4 .. +3 of block (i, j).
-    const unsigned accum = __builtin_amdgcn_readfirstlane(p.prologue == PRO_NONE ? 1u : 0u);
+    // C += A*B: the loop starts from the tile of C instead of zeros (the host sends nothing else with a prologue
+    // other than SET 0 here).  A 32-bit C is loaded by the loop's preamble:  Lane l owns row i*16 + l%16, columns j*16 + (l/16)*4 .. +3 of block (i, j).
+    const bool c_is_32bit = p.out_type == T_F32 || p.out_type == T_I32;
+    const unsigned accum = __builtin_amdgcn_readfirstlane(p.prologue != PRO_NONE ? 0u : c_is_32bit ? 1u : 2u); // 2: set up below
     const CTile c_in = c_tile((char*)p.C + ((int64_t)m0 * p.c_rs + n0) * 4);
     const unsigned c_off = (unsigned)(wr0 + (lane & 15)) * ((unsigned)p.c_rs * 4) + (unsigned)(wc0 + (lane >> 4) * 4) * 4;
     const unsigned c_row16 = __builtin_amdgcn_readfirstlane((unsigned)p.c_rs * 64);
     const auto c_rsrc = c_in.rsrc;
+
+    if (accum == 2) {
+        // C += A*B with a 16-bit C (fp16 / bf16 / int16): the lane's four elements of every block are loaded,
+        // widened and written into the accumulator registers here; the loop then leaves them as they are.
+        // (All fills are waited for first: the compiler counts only its own loads when it places the waits.)
+        wait_vmcnt<0>();
+        const CTile c16 = c_tile((char*)p.C + ((int64_t)m0 * p.c_rs + n0) * 2);
+        const unsigned rb = (unsigned)p.c_rs * 2;
+        const unsigned off16 = (unsigned)(wr0 + (lane & 15)) * rb + (unsigned)(wc0 + (lane >> 4) * 4) * 2;
+        const unsigned m_f16 = p.out_type == T_F16 ? ~0u : 0u, m_bf16 = p.out_type == T_BF16 ? ~0u : 0u;
+        typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+        // four rows of blocks at a time: their loads are all in flight before the first is used
+        w4_static_for<0, TM / 4>([&](auto q) {
+            u32x2 w[4][TN];
+#pragma unroll
+            for (int ii = 0; ii < 4; ++ii)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+                    w[ii][j] = __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(c16.rsrc, off16 + j * 32,
+                                                                                             (unsigned)((q.value * 4 + ii) * 16) * rb, 0));
+            w4_static_for<0, 4>([&](auto ii) {
+                w4_static_for<0, TN>([&](auto j) {
+                    const unsigned w0 = w[ii.value][j.value][0], w1 = w[ii.value][j.value][1];
+                    int x[4];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const unsigned half = (((e & 2) ? w1 : w0) >> ((e & 1) * 16)) & 0xffffu;
+                        if constexpr (IN == IN_I8) x[e] = (int)(short)half; // int16 widens with its sign
+                        else {
+                            const unsigned short h = (unsigned short)half;
+                            const unsigned as_f16 = __float_as_uint((float)__builtin_bit_cast(_Float16, h));
+                            x[e] = (int)((as_f16 & m_f16) | ((half << 16) & m_bf16));
+                        }
+                    }
+                    constexpr int n = ((q.value * 4 + ii.value) * TN + j.value) * 4;
+                    const int x0 = x[0], x1 = x[1], x2 = x[2], x3 = x[3]; // (asm operands do not capture on their own)
+                    asm volatile("v_accvgpr_write_b32 a[%4], %0\n\tv_accvgpr_write_b32 a[%5], %1\n\tv_accvgpr_write_b32 a[%6], %2\n\tv_accvgpr_write_b32 a[%7], %3"
+                                 :
+                                 : "v"(x0), "v"(x1), "v"(x2), "v"(x3), "n"(n), "n"(n + 1), "n"(n + 2), "n"(n + 3));
+                });
+            });
+        });
+    }
 
     wait_vmcnt<2 * FILLS>(); // tile 0 has landed (tiles 1 and 2 in flight)
     __syncthreads();

@@ -164,7 +164,9 @@ def loop(b_layout):
         for x in range(8):
             out.append(line(f"v_add_u32 v{106 + x}, {2 * STAGE}, %[b_rd{x}]"))
     # accumulators: zero, or (C += A*B with 32-bit C) the tile of C, loaded straight into the AGPR file
-    out += [line("s_cmp_eq_u32 %[accum], 0"), line("s_cbranch_scc1 3f"), line("s_mov_b32 s79, 0")]
+    # (or nothing: a 16-bit C has been widened into them by the code before the loop)
+    out += [line("s_cmp_eq_u32 %[accum], 0"), line("s_cbranch_scc1 3f"), line("s_cmp_eq_u32 %[accum], 2"), line("s_cbranch_scc1 4f"),
+            line("s_mov_b32 s79, 0")]
     for i in range(8):
         for j in range(TN):
             n = (i * TN + j) * 4
