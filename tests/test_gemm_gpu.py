@@ -260,6 +260,34 @@ def test_four_wave_kernel_every_output_type(in_type, out_type, b_layout):
                          prologue=ora.PRO_NONE)
 
 
+@pytest.mark.parametrize("in_type,out_type,b_layout", [("f16", "f32", "row"), ("bf16", "bf16", "col"), ("i8", "i32", "row"), ("i8", "i8", "col")])
+def test_four_wave_kernel_on_views_of_larger_matrices(in_type, out_type, b_layout):
+    """Leading dimensions larger than the logical widths (every fill stride and the row stride of C differ from
+    the tile's extent), overwriting and accumulating; what lies beside the views stays as it was."""
+    import accera_amd as acc
+    import torch
+    rng = np.random.default_rng(41)
+    M, N, K = 512, 768, 256 if in_type == "i8" else 384
+    esz = 1 if in_type == "i8" else 2
+    for v in [v for v, n in _variants(b_layout) if "hand-laid" in n]:
+        Abig = make_input(rng, (M, K + 128 // esz), in_type)
+        Bbig = make_input(rng, (N, K + 64 // esz) if b_layout == "col" else (K, N + 256 // esz), in_type)
+        Bview = Bbig[:, :K].T if b_layout == "col" else Bbig[:, :N]
+        pad_c = 16 if out_type == "i8" else 8
+        for prologue in ((ora.PRO_SET0, ora.PRO_NONE) if out_type != "i8" else (ora.PRO_SET0,)):
+            Cbig = make_c0(rng, (M, N + pad_c), out_type)
+            dA, dB, dC = to_device(Abig, in_type), to_device(Bbig, in_type), to_device(Cbig, out_type)
+            dBv = dB[:, :K].t() if b_layout == "col" else dB[:, :N]
+            print("variant", v, in_type, out_type, b_layout, "prologue", prologue, flush=True)
+            acc.gemm_relu(dA[:, :K], dBv, dC[:, :N], prologue=prologue, variant=v)
+            torch.cuda.synchronize()
+            got = to_host(dC, out_type)
+            want = ora.gemm_relu_exact(np.ascontiguousarray(Abig[:, :K]), np.ascontiguousarray(Bview), np.ascontiguousarray(Cbig[:, :N]),
+                                       in_type, out_type, prologue, ora.EPI_RELU)
+            assert_matches(got[:, :N], want, out_type, K)
+            assert np.array_equal(got[:, N:], Cbig[:, N:]), "columns beside the view were written"
+
+
 def test_four_wave_kernel_is_refused_for_what_it_does_not_take():
     """Accumulating into an int8 C, the SCALE / SET ops and a K that is not a multiple of four tiles go to
     the other kernels: naming the variant for them is an error, never a wrong result."""
