@@ -137,13 +137,16 @@ bool mfma_can_take(const MfmaVariant& v, const Problem& pb)
         const bool lean = epi_ok && ((g.prologue == PRO_SET && g.prologue_arg == 0.f) || (g.prologue == PRO_NONE && os >= 2));
         if (!lean || g.K % (4 * bk) || (g.c_rs * os) % 16 || (g.batch > 1 && (g.c_bs * os) % 16)) return false;
         if (pb.have_pointers && !aligned16(g.C)) return false;
+        // any M >= one tile when C is only written: the last row of tiles is moved up to end at row M
+        if (g.M % v.bm && (g.M < v.bm || g.prologue != PRO_SET)) return false;
+        if (g.N % v.bn || g.K % bk) return false;
     }
     if (v.edge) {
         if (g.K % vec) return false;
         if (!v.b_kc && g.N % vec) return false;
         if (!v.a_kc && g.M % vec) return false;
     } else {
-        if (g.M % v.bm || g.N % v.bn || g.K % bk) return false;
+        if (!v.w4 && (g.M % v.bm || g.N % v.bn || g.K % bk)) return false;
     }
     // offsets inside one output tile are 32-bit in the write-back
     if ((int64_t)v.bm * g.c_rs * 4 >= (1ll << 32)) return false;

@@ -288,6 +288,23 @@ def test_four_wave_kernel_on_views_of_larger_matrices(in_type, out_type, b_layou
             assert np.array_equal(got[:, N:], Cbig[:, N:]), "columns beside the view were written"
 
 
+@pytest.mark.parametrize("in_type,out_type,M", [("f16", "f32", 600), ("bf16", "bf16", 1000), ("i8", "i32", 257), ("f16", "f16", 511)])
+def test_four_wave_kernel_any_number_of_rows(in_type, out_type, M):
+    """M that is not a multiple of the tile height: the last row of tiles ends at row M and overlaps the one
+    before it (allowed when C is only written).  Accumulating into C with such an M is refused."""
+    import accera_amd as acc
+    from accera_amd import _lib
+    kb = 64 if in_type == "i8" else 32
+    for b_layout in ("row", "col"):
+        for v in [v for v, n in _variants(b_layout) if "hand-laid" in n]:
+            print("variant", v, in_type, out_type, b_layout, "M", M, flush=True)
+            run_case(in_type, out_type, M, 768, 8 * kb, b_layout=b_layout, variant=v, seed=M)
+            with pytest.raises(_lib.Acc950Error):
+                run_case(in_type, out_type, M, 768, 8 * kb, b_layout=b_layout, variant=v, seed=M, prologue=ora.PRO_NONE)
+    with pytest.raises(_lib.Acc950Error):  # fewer rows than one tile
+        run_case(in_type, out_type, 200, 768, 8 * kb, variant=_hand_laid("row"))
+
+
 def test_four_wave_kernel_is_refused_for_what_it_does_not_take():
     """Accumulating into an int8 C, the SCALE / SET ops and a K that is not a multiple of four tiles go to
     the other kernels: naming the variant for them is an error, never a wrong result."""
