@@ -137,9 +137,11 @@ bool mfma_can_take(const MfmaVariant& v, const Problem& pb)
         const bool lean = epi_ok && ((g.prologue == PRO_SET && g.prologue_arg == 0.f) || (g.prologue == PRO_NONE && os >= 2));
         if (!lean || g.K % (4 * bk) || (g.c_rs * os) % 16 || (g.batch > 1 && (g.c_bs * os) % 16)) return false;
         if (pb.have_pointers && !aligned16(g.C)) return false;
-        // any M >= one tile when C is only written: the last row of tiles is moved up to end at row M
+        // any M, N >= one tile when C is only written: the last row / column of tiles is moved to end at M / N
+        // (its first column must still be 16 bytes aligned in B's and C's rows)
         if (g.M % v.bm && (g.M < v.bm || g.prologue != PRO_SET)) return false;
-        if (g.N % v.bn || g.K % bk) return false;
+        if (g.N % v.bn && (g.N < v.bn || g.prologue != PRO_SET || g.N % vec || (g.N * os) % 16)) return false;
+        if (g.K % bk) return false;
     }
     if (v.edge) {
         if (g.K % vec) return false;

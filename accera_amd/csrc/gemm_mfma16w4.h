@@ -13,8 +13,8 @@
 // moves accumulators between the register files and spills.  Tile staging, the LDS layout and
 // the stores are those of gemm_mfma16.h.
 //
-// Takes: A row-major, N a multiple of the tile width, M a multiple of 256 (any M >= 256 when C is not read: the
-// last row of tiles then overlaps the one before), K a multiple of four k-steps (256 bytes), rows of C 16 bytes aligned;
+// Takes: A row-major, M and N multiples of the tile (any M >= 256 and any 16-byte-aligned N >= the tile width
+// when C is not read: the last row / column of tiles then overlaps the one before), K a multiple of four k-steps (256 bytes), rows of C 16 bytes aligned;
 // C = A*B or relu(A*B) (SET 0 prologue) for every output type; C += A*B (then ReLU or nothing) for 32-bit
 // outputs, where the tile of C is loaded straight into the accumulator registers, and for 16-bit outputs,
 // where it is widened on the way in.
@@ -97,9 +97,11 @@ __global__ void __launch_bounds__(256, 1) gemm_mfma16w4_kernel(GemmArgs p)
 
     int tile_m, tile_n;
     tile_coords(blockIdx.x, p.tiles_m, p.tiles_n, tile_m, tile_n);
-    // M need not be a multiple of the tile: the last row of tiles starts at M - 256 and overlaps its neighbour.
-    // The rows both compute get the same bits from both (the host allows this only when C is not read).
-    const int m0 = tile_m * BM + BM <= p.M ? tile_m * BM : p.M - BM, n0 = tile_n * BN;
+    // M and N need not be multiples of the tile: the last row / column of tiles ends at M / N and overlaps its
+    // neighbour.  What both compute gets the same bits from both (the host allows this only when C is not read,
+    // and only for N whose last tile still starts on a 16-byte boundary of B's and C's rows).
+    const int m0 = tile_m * BM + BM <= p.M ? tile_m * BM : p.M - BM;
+    const int n0 = tile_n * BN + BN <= p.N ? tile_n * BN : p.N - BN;
 
     const char* Ab = (const char*)p.A;
     const char* Bb = (const char*)p.B;
@@ -397,7 +399,7 @@ hipError_t launch_mfma16w4(const GemmArgs& a, hipStream_t stream, LaunchGeom* ge
     auto kern = gemm_mfma16w4_kernel<Cfg>;
     GemmArgs args = a;
     args.tiles_m = (a.M + Cfg::BM - 1) / Cfg::BM;
-    args.tiles_n = a.N / Cfg::BN;
+    args.tiles_n = (a.N + Cfg::BN - 1) / Cfg::BN;
     if (geom) {
         geom->grid[0] = (unsigned)(args.tiles_m * args.tiles_n);
         geom->grid[1] = 1;

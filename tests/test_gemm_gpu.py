@@ -290,8 +290,8 @@ def test_four_wave_kernel_on_views_of_larger_matrices(in_type, out_type, b_layou
 
 @pytest.mark.parametrize("in_type,out_type,M", [("f16", "f32", 600), ("bf16", "bf16", 1000), ("i8", "i32", 257), ("f16", "f16", 511)])
 def test_four_wave_kernel_any_number_of_rows(in_type, out_type, M):
-    """M that is not a multiple of the tile height: the last row of tiles ends at row M and overlaps the one
-    before it (allowed when C is only written).  Accumulating into C with such an M is refused."""
+    """M and N that are not multiples of the tile: the last row / column of tiles ends at M / N and overlaps the
+    one before it (allowed when C is only written).  Accumulating into C with such sizes is refused."""
     import accera_amd as acc
     from accera_amd import _lib
     kb = 64 if in_type == "i8" else 32
@@ -299,6 +299,7 @@ def test_four_wave_kernel_any_number_of_rows(in_type, out_type, M):
         for v in [v for v, n in _variants(b_layout) if "hand-laid" in n]:
             print("variant", v, in_type, out_type, b_layout, "M", M, flush=True)
             run_case(in_type, out_type, M, 768, 8 * kb, b_layout=b_layout, variant=v, seed=M)
+            run_case(in_type, out_type, M, 768 + 16 + 64 * (M % 3), 4 * kb, b_layout=b_layout, variant=v, seed=M + 1)  # N ragged too
             with pytest.raises(_lib.Acc950Error):
                 run_case(in_type, out_type, M, 768, 8 * kb, b_layout=b_layout, variant=v, seed=M, prologue=ora.PRO_NONE)
     with pytest.raises(_lib.Acc950Error):  # fewer rows than one tile
