@@ -135,7 +135,7 @@ bool mfma_can_take(const MfmaVariant& v, const Problem& pb)
         const int os = elem_size(g.out_type);
         const bool epi_ok = g.epilogue == EPI_RELU || g.epilogue == EPI_NONE;
         const bool lean = epi_ok && ((g.prologue == PRO_SET && g.prologue_arg == 0.f) || (g.prologue == PRO_NONE && os >= 2));
-        if (!lean || g.K % (4 * bk) || (g.c_rs * os) % 16 || (g.batch > 1 && (g.c_bs * os) % 16)) return false;
+        if (!lean || g.K % bk || g.K < 4 * bk || (g.c_rs * os) % 16 || (g.batch > 1 && (g.c_bs * os) % 16)) return false;
         if (pb.have_pointers && !aligned16(g.C)) return false;
         // any M, N >= one tile when C is only written: the last row / column of tiles is moved to end at M / N
         // (its first column must still be 16 bytes aligned in B's and C's rows)

@@ -14,7 +14,8 @@
 // the stores are those of gemm_mfma16.h.
 //
 // Takes: A row-major, M and N multiples of the tile (any M >= 256 and any 16-byte-aligned N >= the tile width
-// when C is not read: the last row / column of tiles then overlaps the one before), K a multiple of four k-steps (256 bytes), rows of C 16 bytes aligned;
+// when C is not read: the last row / column of tiles then overlaps the one before), K a multiple of one k-step (64 bytes)
+// and at least four of them, rows of C 16 bytes aligned;
 // C = A*B or relu(A*B) (SET 0 prologue) for every output type; C += A*B (then ReLU or nothing) for 32-bit
 // outputs, where the tile of C is loaded straight into the accumulator registers, and for 16-bit outputs,
 // where it is widened on the way in.
@@ -134,19 +135,23 @@ __global__ void __launch_bounds__(256, 1) gemm_mfma16w4_kernel(GemmArgs p)
     const unsigned sb = __builtin_amdgcn_readfirstlane(B_KC ? (unsigned)KB : (unsigned)(BK * ldb * ES));
     const char* a_tile = Ab + (int64_t)m0 * lda * ES;
     const char* b_tile = Bb + (B_KC ? (int64_t)n0 * ldb * ES : (int64_t)n0 * ES);
+    // The loop's last k-step runs at position 3 of its four-step pattern, so the first one starts at position
+    // p0 = (4 - KT % 4) % 4: tile s goes to LDS stage (s + p0) % 4, and a partial first trip through the body
+    // counts as one more trip.
+    const unsigned p0 = __builtin_amdgcn_readfirstlane((unsigned)((4 - KT % 4) % 4));
 #pragma unroll
     for (int s = 0; s < 3; ++s) {
+        const unsigned stage = ldsb + ((s + p0) & 3) * STAGE_BYTES;
 #pragma unroll
         for (int f = 0; f < 4; ++f)
-            TA::direct_issue(ldsb + s * STAGE_BYTES + f * 4096, a_off, a_tile + (int64_t)s * sa + (int64_t)f * da);
+            TA::direct_issue(stage + f * 4096, a_off, a_tile + (int64_t)s * sa + (int64_t)f * da);
 #pragma unroll
         for (int f = 0; f < FILLS_B; ++f)
-            TB::direct_issue(ldsb + s * STAGE_BYTES + TA::TILE_BYTES + f * 4096, (f & 1) ? b_off1 : b_off0,
-                             b_tile + (int64_t)s * sb + (int64_t)f * db);
+            TB::direct_issue(stage + TA::TILE_BYTES + f * 4096, (f & 1) ? b_off1 : b_off0, b_tile + (int64_t)s * sb + (int64_t)f * db);
     }
     const char* pa = a_tile + 3 * (int64_t)sa;
     const char* pb = b_tile + 3 * (int64_t)sb;
-    const unsigned groups = __builtin_amdgcn_readfirstlane((unsigned)(KT / 4 - 1));
+    const unsigned groups = __builtin_amdgcn_readfirstlane((unsigned)(KT / 4 - 1 + (KT % 4 ? 1 : 0)));
 
     // ---- LDS addresses of the fragment reads (stage 0; the loop adds stage and block offsets)
     const int kg = lane >> 4, li = lane & 15;
@@ -229,7 +234,7 @@ __global__ void __launch_bounds__(256, 1) gemm_mfma16w4_kernel(GemmArgs p)
     : [a_rd] "v"(a_rd), [b_rd0] "v"(b_rd[0]), [b_rd1] "v"(b_rd[1]), [b_rd2] "v"(b_rd[2]), [b_rd3] "v"(b_rd[3]),          \
       [b_rd4] "v"(b_rd[4]), [b_rd5] "v"(b_rd[5]), [b_rd6] "v"(b_rd[6]), [b_rd7] "v"(b_rd[7]), [a_off] "v"(a_off),        \
       [b_off0] "v"(b_off0), [b_off1] "v"(b_off1), [pa] "s"(pa), [pb] "s"(pb), [da] "s"(da), [db] "s"(db), [sa] "s"(sa),   \
-      [sb] "s"(sb), [ldsb] "s"(ldsb), [groups] "s"(groups), [accum] "s"(accum), [c_off] "v"(c_off),                     \
+      [sb] "s"(sb), [ldsb] "s"(ldsb), [groups] "s"(groups), [accum] "s"(accum), [c_off] "v"(c_off), [p0] "s"(p0),       \
       [c_rsrc] "s"(c_rsrc), [c_row16] "s"(c_row16)                                                                      \
     : "memory", "scc", "s72", "s73", "s74", "s75", "s76", "s77", "s78", "s79", ACC950_W4_V(10), ACC950_W4_V(11),        \
       ACC950_W4_V(12), ACC950_W4_V(13), ACC950_W4_V(14), ACC950_W4_V(15), ACC950_W4_V(16), ACC950_W4_V(17),             \

@@ -18,8 +18,8 @@ hand: registers are fixed, and each k-step of 64 bytes is
     32 MFMAs (rows 64..127), the fragment reads of the next step between them, one per MFMA
 
 The four LDS stages rotate with the k-step, so the body is written out for four steps; the last
-four steps (no more fills, then no more reads) are a second copy.  K must be a multiple of four
-steps.
+four steps (no more fills, then no more reads) are a second copy.  A number of k-steps that is not
+a multiple of four enters the body in the middle (see loop()); at least four steps.
 
 Register use (besides the operands the C++ side passes in):
     a[0:255]    accumulators, block (i, j) at a[(i*TN+j)*4 .. +3] (TN = 8 blocks of columns per wave, 6 for the 192-wide tile)
@@ -176,13 +176,26 @@ def loop(b_layout):
     for n in range(32 * TN):
         out.append(line(f"v_accvgpr_write_b32 a{n}, 0"))
     out.append(line("4:"))
-    for x in range(TN):
-        out += read_b(x, 0, 0, b_layout)
-    for x in range(8):
-        out += read_a(x, 0, 0)
-    out += [line("s_nop 7"), line("s_cmp_eq_u32 s78, 0"), line("s_cbranch_scc1 2f"), line("1:")]
+    # Entry.  The last k-step always runs at position 3 of the closing copy, so the first one starts at position
+    # p0 = (4 - steps % 4) % 4: its tile lies in LDS stage p0 (the code before the loop put it there), its fragments
+    # go to register set p0 % 2, and the body is entered at that position (labels 5, 6, 7 = positions 1, 2, 3).
+    def first_reads(pos):
+        r = []
+        for x in range(TN):
+            r += read_b(x, pos, pos % 2, b_layout)
+        for x in range(8):
+            r += read_a(x, pos, pos % 2)
+        return r + [line("s_nop 7")]
+    out += [line("s_cmp_eq_u32 %[p0], 0"), line("s_cbranch_scc1 10f"), line("s_cmp_eq_u32 %[p0], 1"), line("s_cbranch_scc1 11f"),
+            line("s_cmp_eq_u32 %[p0], 2"), line("s_cbranch_scc1 12f")]
+    out += first_reads(3) + [line("s_branch 7f"), line("11:")]
+    out += first_reads(1) + [line("s_branch 5f"), line("12:")]
+    out += first_reads(2) + [line("s_branch 6f"), line("10:")]
+    out += first_reads(0) + [line("s_cmp_eq_u32 s78, 0"), line("s_cbranch_scc1 2f"), line("1:")]
     per_tile = 4 + (2 * TN * FRAG) // 4096  # fill instructions per K tile and thread
     for pos in range(4):
+        if pos:
+            out.append(line(f"{4 + pos}:"))
         out += step(pos, True, 2 * per_tile, False, b_layout)
     out += [line("s_sub_u32 s78, s78, 1"), line("s_cmp_lg_u32 s78, 0"), line("s_cbranch_scc1 1b"), line("2:")]
     out += step(0, True, 2 * per_tile, False, b_layout)

@@ -207,7 +207,7 @@ int acc950_variant_name(int variant, char* buf, size_t buf_len);
  * figure is the practical compute roof for random GEMM inputs on the device at hand.
  *
  * acc950_mfma_phase_probe: runs a build of the 256x256 MFMA kernel the automatic choice takes
- * for large aligned problems (four waves with the hand-laid K loop when K is a multiple of four
+ * for large aligned problems (four waves with the hand-laid K loop when K has at least four
  * K tiles of 64 bytes, else the eight-wave ping-pong form) that reads the shader-clock counter
  * and the constant 100 MHz counter at four points in every workgroup, on dense row-major
  * DEVICE operands (M, N multiples of 256, SET-0 prologue, ReLU epilogue), synchronously.

@@ -68,8 +68,9 @@ def test_mfma_all_variants(in_type, out_type, b_layout):
         a_layout = "col" if "A=col-major" in name else "row"
         bm, bn = map(int, re.search(r"mfma (\d+)x(\d+)", name).groups())
         M, N = max(512, 2 * bm), (max(512, 2 * bn) if 512 % bn == 0 else 3 * bn)
-        # (the hand-laid loop takes K in steps of four tiles: the pipeline's depth, twice and five times it)
-        for k_tiles in ((4, 8, 20) if "hand-laid" in name else (1, 2, 3, 7)):
+        # (the hand-laid loop takes at least four K tiles, the depth of its pipeline; every remainder modulo four enters
+        # its four-step body at another position)
+        for k_tiles in ((4, 5, 6, 7, 8, 9, 20) if "hand-laid" in name else (1, 2, 3, 7)):
             run_case(in_type, out_type, M, N, k_tiles * kb, b_layout=b_layout, variant=v, seed=v + k_tiles, a_layout=a_layout)
         if "edge" in name:
             # ragged M, N (multiple of the 16-byte vector only) and a K tail
@@ -307,17 +308,17 @@ def test_four_wave_kernel_any_number_of_rows(in_type, out_type, M):
 
 
 def test_four_wave_kernel_is_refused_for_what_it_does_not_take():
-    """Accumulating into an int8 C, the SCALE / SET ops and a K that is not a multiple of four tiles go to
-    the other kernels: naming the variant for them is an error, never a wrong result."""
+    """Accumulating into an int8 C, the SCALE / SET ops and a K of fewer than four tiles go to the other
+    kernels: naming the variant for them is an error, never a wrong result."""
     import accera_amd as acc
     import torch
     from accera_amd import _lib
     v = _hand_laid("row")
     rng = np.random.default_rng(5)
-    A, B = make_input(rng, (256, 160), "f16"), make_input(rng, (160, 256), "f16")
+    A, B = make_input(rng, (256, 96), "f16"), make_input(rng, (96, 256), "f16")
     dC = to_device(np.zeros((256, 256), np.float32), "f32")
     with pytest.raises(_lib.Acc950Error):
-        acc.gemm_relu(to_device(A, "f16"), to_device(B, "f16"), dC, variant=v)  # K = 5 tiles
+        acc.gemm_relu(to_device(A, "f16"), to_device(B, "f16"), dC, variant=v)  # K = 3 tiles: fewer than the pipeline is deep
     A, B = make_input(rng, (256, 128), "f16"), make_input(rng, (128, 256), "f16")
     for kw in (dict(prologue=acc.PROLOGUE_SCALE, prologue_arg=0.5), dict(epilogue=acc.EPILOGUE_SCALE, epilogue_arg=2.0),
                dict(prologue=acc.PROLOGUE_SET, prologue_arg=1.0)):

@@ -135,7 +135,23 @@ def test_whole_loop_shape(layout, tn):
     ins = _text(g.loop(layout))
     per_tile = 4 + tn * 2048 // 4096
     assert ins.count("1:") == 1 and ins.count("2:") == 1 and ins.index("1:") < ins.index("s_cbranch_scc1 1b") < ins.index("2:")
-    body = ins[ins.index("1:"):ins.index("2:")]
+    # the body can be entered at each of its four positions (a step count that is not a multiple of four); every entry
+    # first reads the fragments of the first tile from the stage of that position into that position's register set
+    assert ins.index("1:") < ins.index("5:") < ins.index("6:") < ins.index("7:") < ins.index("s_cbranch_scc1 1b")
+    entry = ins[ins.index("4:"):ins.index("1:")]
+    for label, jump, pos in ((None, "s_branch 7f", 3), ("11:", "s_branch 5f", 1), ("12:", "s_branch 6f", 2), ("10:", "s_cbranch_scc1 2f", 0)):
+        start = entry.index(label) + 1 if label else entry.index("s_cbranch_scc1 12f") + 1
+        block = entry[start:entry.index(jump, start)]
+        reads = [i for i in block if i.startswith("ds_read")]
+        assert len(reads) == 8 + (tn if layout == "kc" else 2 * tn)
+        for r in reads:
+            m = re.match(r"\S+ v\[(\d+):(\d+)\], (\S+) offset:(\d+)$", r)
+            v0, base, off = int(m.group(1)), m.group(3), int(m.group(4))
+            assert 128 + (pos % 2) * 64 <= v0 < 192 + (pos % 2) * 64
+            assert (not base.startswith("%")) == (pos >= 2) and 0 <= off - (pos & 1) * g.STAGE < g.STAGE
+    step_starts = [ins.index("1:"), ins.index("5:"), ins.index("6:"), ins.index("7:")]
+    assert all(ins[n + 1] == "s_waitcnt lgkmcnt(4)" for n in step_starts)
+    body = [i for i in ins[ins.index("1:"):ins.index("2:")] if i not in ("5:", "6:", "7:")]
     tail = ins[ins.index("2:"):]
     assert sum(i.startswith("MFMA") for i in body) == 4 * 8 * tn == sum(i.startswith("MFMA") for i in tail)
     assert body.count("s_barrier") == 4 and tail.count("s_barrier") == 3
