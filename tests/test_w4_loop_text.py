@@ -169,3 +169,94 @@ def test_whole_loop_shape(layout, tn):
     assert pre.count("s_add_u32 s79, s79, %[c_row16]") == 8
     # the loop ends with enough idle cycles for the last MFMA results to be readable
     assert ins[-2:] == ["s_nop 15", "s_nop 15"]
+
+
+def _run_fills(g, layout, tn, KT, b_tiles_before_loop):
+    """Executes the scalar side of the loop text for KT k-steps: follows the branches, keeps the fill pointers as
+    numbers and records every global_load_lds as (operand, K tile, pass, LDS stage).  The code before the loop
+    has issued A's tiles 0..2 and B's tiles 0..b_tiles_before_loop-1; pa / pb point at the next tiles."""
+    g.set_width(tn)
+    ins = _text(g.loop(layout))
+    DA, DB, SA, SB = 1 << 20, 1 << 21, 1 << 30, 1 << 34      # distinct powers of two: an address decodes uniquely
+    p0 = (4 - KT % 4) % 4
+    groups = KT // 4 - 1 + (1 if KT % 4 else 0)
+    env = {"%[pa]": 3 * SA, "%[pb]": (1 << 50) + b_tiles_before_loop * SB, "%[groups]": groups, "%[p0]": p0, "%[accum]": 0,
+           "%[da]": DA, "%[db]": DB, "%[sa]": SA, "%[sb]": SB, "%[ldsb]": 0, "%[c_row16]": 0}
+    labels = {}
+    for n, i in enumerate(ins):
+        if re.match(r"^\d+:$", i):
+            labels.setdefault(i[:-1], []).append(n)
+    reg, scc, m0, pc, fills, steps = {}, 0, None, 0, [], 0
+
+    def val(tok):
+        tok = tok.strip()
+        if tok in env:
+            return env[tok]
+        if re.match(r"^s\d+$", tok):
+            return reg.get(tok, 0)
+        return int(tok, 0)
+
+    def pair(tok):  # s[a:b] or an operand
+        m = re.match(r"s\[(\d+):(\d+)\]", tok.strip())
+        return (reg.get("s" + m.group(1), 0) | (reg.get("s" + m.group(2), 0) << 32)) if m else env[tok.strip()]
+
+    while pc < len(ins):
+        i = ins[pc]
+        pc += 1
+        op, _, rest = i.partition(" ")
+        a = [x.strip() for x in rest.split(",")] if rest else []
+        if op == "s_mov_b64":
+            m = re.match(r"s\[(\d+):(\d+)\]", a[0])
+            v = pair(rest.split(",", 1)[1])
+            reg["s" + m.group(1)], reg["s" + m.group(2)] = v & 0xffffffff, v >> 32
+        elif op == "s_mov_b32":
+            reg[a[0]] = val(a[1])
+        elif op == "s_add_u32":
+            t = val(a[1]) + val(a[2])
+            scc = t >> 32
+            if a[0] == "m0":
+                m0 = t & 0xffffffff
+            else:
+                reg[a[0]] = t & 0xffffffff
+        elif op == "s_addc_u32":
+            t = val(a[1]) + val(a[2]) + scc
+            scc, reg[a[0]] = t >> 32, t & 0xffffffff
+        elif op == "s_sub_u32":
+            reg[a[0]] = val(a[1]) - val(a[2])
+        elif op == "s_cmp_eq_u32":
+            scc = int(val(a[0]) == val(a[1]))
+        elif op == "s_cmp_lg_u32":
+            scc = int(val(a[0]) != val(a[1]))
+        elif op in ("s_cbranch_scc1", "s_branch"):
+            if op == "s_branch" or scc:
+                lab, way = a[0][:-1], a[0][-1]
+                cands = labels[lab]
+                pc = min(c for c in cands if c >= pc) if way == "f" else max(c for c in cands if c < pc)
+        elif op == "global_load_lds_dwordx4":
+            addr = pair(rest.split(",", 1)[1])
+            operand = "b" if addr >> 50 else "a"       # (bit 50 marks B's address space in this model)
+            addr &= (1 << 50) - 1
+            stride, delta = (SB, DB) if operand == "b" else (SA, DA)
+            tile, within = divmod(addr, stride)
+            assert within % delta == 0
+            stage, in_stage = divmod(m0, g.STAGE)
+            assert in_stage == (g.B_TILE if operand == "b" else 0) + (within // delta) * 4096
+            fills.append((operand, tile, within // delta, stage))
+            m0 = None
+        elif op == "s_waitcnt" and a and a[0].startswith("lgkmcnt(4)"):
+            steps += 1
+    return fills, steps, p0
+
+
+@pytest.mark.parametrize("layout,tn", [("kc", 8), ("mc16", 8), ("kc", 6)])
+@pytest.mark.parametrize("KT", [4, 5, 6, 7, 8, 9, 10, 11, 12, 23, 128])
+def test_fill_addresses_over_a_whole_k_loop(layout, tn, KT):
+    """Every pass of every K tile from 3 on is filled exactly once, from the address of that tile and pass, into
+    the LDS stage its k-step will read ((tile + entry position) mod 4), and nothing beyond the last tile is touched."""
+    g = _gen()
+    fills, steps, p0 = _run_fills(g, layout, tn, KT, 3)
+    nb = tn * 2048 // 4096
+    assert steps == KT
+    want = sorted([("a", t, p, (t + p0) % 4) for t in range(3, KT) for p in range(4)] +
+                  [("b", t, p, (t + p0) % 4) for t in range(3, KT) for p in range(nb)])
+    assert sorted(fills) == want
