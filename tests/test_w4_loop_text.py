@@ -187,6 +187,15 @@ def _run_fills(g, layout, tn, KT, b_tiles_before_loop):
         if re.match(r"^\d+:$", i):
             labels.setdefault(i[:-1], []).append(n)
     reg, scc, m0, pc, fills, steps = {}, 0, None, 0, [], 0
+    nb_ = tn * 2048 // 4096
+    # fills in flight, oldest first: what the code before the loop issued (tile by tile, A's passes then B's), then the loop's
+    issued = []
+    for t in range(3):
+        issued += [("a", t, p) for p in range(4)]
+        if t < b_tiles_before_loop:
+            issued += [("b", t, p) for p in range(nb_)]
+    if b_tiles_before_loop > 3:
+        issued += [("b", t, p) for t in range(3, b_tiles_before_loop) for p in range(nb_)]
 
     def val(tok):
         tok = tok.strip()
@@ -242,7 +251,16 @@ def _run_fills(g, layout, tn, KT, b_tiles_before_loop):
             stage, in_stage = divmod(m0, g.STAGE)
             assert in_stage == (g.B_TILE if operand == "b" else 0) + (within // delta) * 4096
             fills.append((operand, tile, within // delta, stage))
+            issued.append((operand, tile, within // delta))
             m0 = None
+        elif op == "s_waitcnt" and a and a[0].startswith("vmcnt(") and steps:
+            # loads complete in order: all but the youngest N are done.  The tile of the next k-step must be among them.
+            n_out = int(a[0][6:-1])
+            done = set(issued[:len(issued) - n_out]) if n_out else set(issued)
+            nxt_tile = steps                                   # this is k-step steps-1; the barrier that follows publishes the next tile
+            if nxt_tile < KT:
+                need = {("a", nxt_tile, p) for p in range(4)} | {("b", nxt_tile, p) for p in range(nb_)}
+                assert need <= done, (steps - 1, sorted(need - done))
         elif op == "s_waitcnt" and a and a[0].startswith("lgkmcnt(4)"):
             steps += 1
     return fills, steps, p0
