@@ -139,18 +139,25 @@ __global__ void __launch_bounds__(256, 1) gemm_mfma16w4_kernel(GemmArgs p)
     // p0 = (4 - KT % 4) % 4: tile s goes to LDS stage (s + p0) % 4, and a partial first trip through the body
     // counts as one more trip.
     const unsigned p0 = __builtin_amdgcn_readfirstlane((unsigned)((4 - KT % 4) % 4));
+    // With paired fills a K-contiguous B is fetched two K tiles at a time on the even positions of the loop's pattern
+    // (both 64-byte halves of a cache line in neighbouring requests), so its third tile is issued here only when the
+    // first k-step sits at an odd position; otherwise the loop's first step fetches tiles 2 and 3.
+    constexpr bool B_PAIRED = B_KC && (BN == 192 || IN == IN_I8); // measured: behind the plain scheme for 16-bit inputs on 256-wide tiles
+    const unsigned b_tiles_here = B_PAIRED ? 2u + (p0 & 1u) : 3u;
 #pragma unroll
     for (int s = 0; s < 3; ++s) {
         const unsigned stage = ldsb + ((s + p0) & 3) * STAGE_BYTES;
 #pragma unroll
         for (int f = 0; f < 4; ++f)
             TA::direct_issue(stage + f * 4096, a_off, a_tile + (int64_t)s * sa + (int64_t)f * da);
+        if ((unsigned)s < b_tiles_here) {
 #pragma unroll
-        for (int f = 0; f < FILLS_B; ++f)
-            TB::direct_issue(stage + TA::TILE_BYTES + f * 4096, (f & 1) ? b_off1 : b_off0, b_tile + (int64_t)s * sb + (int64_t)f * db);
+            for (int f = 0; f < FILLS_B; ++f)
+                TB::direct_issue(stage + TA::TILE_BYTES + f * 4096, (f & 1) ? b_off1 : b_off0, b_tile + (int64_t)s * sb + (int64_t)f * db);
+        }
     }
     const char* pa = a_tile + 3 * (int64_t)sa;
-    const char* pb = b_tile + 3 * (int64_t)sb;
+    const char* pb = b_tile + (int64_t)b_tiles_here * sb;
     const unsigned groups = __builtin_amdgcn_readfirstlane((unsigned)(KT / 4 - 1 + (KT % 4 ? 1 : 0)));
 
     // ---- LDS addresses of the fragment reads (stage 0; the loop adds stage and block offsets)
@@ -226,7 +233,7 @@ __global__ void __launch_bounds__(256, 1) gemm_mfma16w4_kernel(GemmArgs p)
         });
     }
 
-    wait_vmcnt<2 * FILLS>(); // tile 0 has landed (tiles 1 and 2 in flight)
+    wait_vmcnt<B_PAIRED ? 4 + FILLS : 2 * FILLS>(); // tile 0 has landed (tile 1 and tile 2 -- A's part of it at least -- in flight)
     __syncthreads();
     stamp(1);
 
@@ -236,7 +243,7 @@ __global__ void __launch_bounds__(256, 1) gemm_mfma16w4_kernel(GemmArgs p)
       [b_off0] "v"(b_off0), [b_off1] "v"(b_off1), [pa] "s"(pa), [pb] "s"(pb), [da] "s"(da), [db] "s"(db), [sa] "s"(sa),   \
       [sb] "s"(sb), [ldsb] "s"(ldsb), [groups] "s"(groups), [accum] "s"(accum), [c_off] "v"(c_off), [p0] "s"(p0),       \
       [c_rsrc] "s"(c_rsrc), [c_row16] "s"(c_row16)                                                                      \
-    : "memory", "scc", "s72", "s73", "s74", "s75", "s76", "s77", "s78", "s79", ACC950_W4_V(10), ACC950_W4_V(11),        \
+    : "memory", "scc", "s72", "s73", "s74", "s75", "s76", "s77", "s78", "s79", "s80", "s81", ACC950_W4_V(10), ACC950_W4_V(11), \
       ACC950_W4_V(12), ACC950_W4_V(13), ACC950_W4_V(14), ACC950_W4_V(15), ACC950_W4_V(16), ACC950_W4_V(17),             \
       ACC950_W4_V(18), ACC950_W4_V(19), ACC950_W4_V(20), ACC950_W4_V(21), ACC950_W4_V(22), ACC950_W4_V(23),             \
       ACC950_W4_V(24), "v250", "v251", "v252", "v253", "v254", "v255", "a0", "a1", "a2", "a3", "a4", "a5", "a6", "a7",   \
@@ -249,13 +256,13 @@ __global__ void __launch_bounds__(256, 1) gemm_mfma16w4_kernel(GemmArgs p)
 #define ACC950_W4_V(d) ACC950_W4_R("v", d)
 #define ACC950_W4_A(d) ACC950_W4_R("a", d)
     if constexpr (B_KC && BN == 192) {
-        if constexpr (IN == IN_F16) asm volatile(ACC950_W4_LOOP_KC6("v_mfma_f32_16x16x32_f16") : ACC950_W4_OPERANDS);
-        else if constexpr (IN == IN_BF16) asm volatile(ACC950_W4_LOOP_KC6("v_mfma_f32_16x16x32_bf16") : ACC950_W4_OPERANDS);
-        else asm volatile(ACC950_W4_LOOP_KC6("v_mfma_i32_16x16x64_i8") : ACC950_W4_OPERANDS);
+        if constexpr (IN == IN_F16) asm volatile(ACC950_W4_LOOP_KCP6("v_mfma_f32_16x16x32_f16") : ACC950_W4_OPERANDS);
+        else if constexpr (IN == IN_BF16) asm volatile(ACC950_W4_LOOP_KCP6("v_mfma_f32_16x16x32_bf16") : ACC950_W4_OPERANDS);
+        else asm volatile(ACC950_W4_LOOP_KCP6("v_mfma_i32_16x16x64_i8") : ACC950_W4_OPERANDS);
     } else if constexpr (B_KC) {
         if constexpr (IN == IN_F16) asm volatile(ACC950_W4_LOOP_KC("v_mfma_f32_16x16x32_f16") : ACC950_W4_OPERANDS);
         else if constexpr (IN == IN_BF16) asm volatile(ACC950_W4_LOOP_KC("v_mfma_f32_16x16x32_bf16") : ACC950_W4_OPERANDS);
-        else asm volatile(ACC950_W4_LOOP_KC("v_mfma_i32_16x16x64_i8") : ACC950_W4_OPERANDS);
+        else asm volatile(ACC950_W4_LOOP_KCP("v_mfma_i32_16x16x64_i8") : ACC950_W4_OPERANDS);
     } else {
         if constexpr (IN == IN_F16) asm volatile(ACC950_W4_LOOP_MC16("v_mfma_f32_16x16x32_f16") : ACC950_W4_OPERANDS);
         else if constexpr (IN == IN_BF16) asm volatile(ACC950_W4_LOOP_MC16("v_mfma_f32_16x16x32_bf16") : ACC950_W4_OPERANDS);

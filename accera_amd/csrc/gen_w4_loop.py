@@ -26,7 +26,7 @@ Register use (besides the operands the C++ side passes in):
     v[128:191]  fragments of even steps: B blocks 0..7 (v128..), A blocks 0..7 (v160..)
     v[192:255]  fragments of odd steps
     v[104:121]  LDS read addresses of the upper two stages (the 16-bit offset field reaches 64 KB)
-    s[72:73], s[74:75]  fill pointers of A and B (tile three ahead); s[76:77] scratch pointer; s78 loop count;
+    s[72:73], s[74:75]  fill pointers of A and B (the next tile to fetch); s[76:77], s[80:81] scratch pointers; s78 loop count;
     s79 row offset while C is loaded
 """
 B_TILE = 16384     # B's tile follows A's (256 rows x 64 bytes) inside a stage
@@ -74,7 +74,7 @@ def read_a(x, stage, buf):
 
 def read_b(x, stage, buf, b_layout):
     n = bfrag(buf, x)
-    if b_layout == "kc":
+    if b_layout in ("kc", "kcp"):
         base = "%[b_rd0]" if stage < 2 else "v105"
         off = (stage & 1) * STAGE + B_TILE + x * FRAG
         return [line(f"ds_read_b128 v[{n}:{n + 3}], {base} offset:{off}")]
@@ -97,7 +97,7 @@ def fill(f, stage, b_layout):
     else:
         g = f - 4
         ptr, d, s, tile, last = "s[74:75]", "%[db]", "%[sb]", B_TILE, (2 * TN * FRAG) // 4096 - 1
-        lane = "%[b_off0]" if (b_layout == "kc" or g % 2 == 0) else "%[b_off1]"
+        lane = "%[b_off0]" if (b_layout in ("kc", "kcp") or g % 2 == 0) else "%[b_off1]"
     slots = []
     if g == 0:
         slots.append([line(f"s_mov_b64 s[76:77], {ptr}")])
@@ -109,6 +109,43 @@ def fill(f, stage, b_layout):
         lo, hi = (72, 73) if f < 4 else (74, 75)
         slots[-1] += [line(f"s_add_u32 s{lo}, s{lo}, {s}"), line(f"s_addc_u32 s{hi}, s{hi}, 0")]
     return slots
+
+
+def kc_fills(pos, half):
+    """Fill instructions of one k-step of the "kcp" scheme (B K-contiguous, fills paired), as lists per MFMA slot.  Both operands' K tiles are
+    half cache lines, so both are fetched as pairs of neighbouring requests: A's tile t+3 last in odd steps and first
+    in even ones (as for the other layouts), and B two tiles at a time, t+2 and t+3 pass by pass, on even steps only."""
+    nb = (2 * TN * FRAG) // 4096
+    slots = []
+    for g in range(4):  # A, tile t+3 -> stage (pos+3) % 4
+        first = [line("s_mov_b64 s[76:77], s[72:73]")] if g == 0 else [line("s_add_u32 s76, s76, %[da]"), line("s_addc_u32 s77, s77, 0")]
+        slots.append(first + [line(f"s_add_u32 m0, %[ldsb], {((pos + 3) % 4) * STAGE + g * 4096}")])
+        slots.append([line("global_load_lds_dwordx4 %[a_off], s[76:77]")])
+    slots[-1] += [line("s_add_u32 s72, s72, %[sa]"), line("s_addc_u32 s73, s73, 0")]
+    if pos % 2:
+        return [[] for _ in range(half - len(slots))] + slots
+    for g in range(nb):  # B, tiles t+2 and t+3 -> stages (pos+2) % 4 and (pos+3) % 4
+        if g == 0:
+            ptrs = [line("s_mov_b64 s[76:77], s[74:75]"), line("s_add_u32 s80, s74, %[sb]"), line("s_addc_u32 s81, s75, 0")]
+        else:
+            ptrs = [line("s_add_u32 s76, s76, %[db]"), line("s_addc_u32 s77, s77, 0"), line("s_add_u32 s80, s80, %[db]"), line("s_addc_u32 s81, s81, 0")]
+        slots.append(ptrs + [line(f"s_add_u32 m0, %[ldsb], {((pos + 2) % 4) * STAGE + B_TILE + g * 4096}")])
+        slots.append([line("global_load_lds_dwordx4 %[b_off0], s[76:77]"),
+                      line(f"s_add_u32 m0, %[ldsb], {((pos + 3) % 4) * STAGE + B_TILE + g * 4096}")])
+        slots.append([line("global_load_lds_dwordx4 %[b_off0], s[80:81]")])
+    slots[-1] += [line("s_add_u32 s74, s74, %[sb]"), line("s_addc_u32 s75, s75, 0"), line("s_add_u32 s74, s74, %[sb]"), line("s_addc_u32 s75, s75, 0")]
+    assert len(slots) <= half
+    return slots + [[] for _ in range(half - len(slots))]
+
+
+def kc_wait(pos, tiles_left):
+    """vmcnt before the barrier of a k-step with K-contiguous B: how many fills issued after the next tile's last one
+    may still be in flight.  tiles_left: K tiles after this step's (>= 3 inside the body)."""
+    nb = (2 * TN * FRAG) // 4096
+    if tiles_left >= 3:
+        return 8 + 2 * nb if pos % 2 == 0 else 5   # even: A(t+2), A(t+3), B(t+2), B(t+3); odd: B(t+2)'s last pass, A(t+3)
+    assert pos == 4 - 1 - tiles_left                 # the closing steps sit at positions 1 and 2
+    return 1 if tiles_left == 2 else 0              # position 1: B's last tile's last pass; position 2: nothing
 
 
 def step(pos, do_fill, wait, last, b_layout):
@@ -123,7 +160,9 @@ def step(pos, do_fill, wait, last, b_layout):
             order += [(i, j) for i in (rows if j % 2 == 0 else reversed(rows))]
     half = 4 * TN
     extra = [[] for _ in range(half)]
-    if do_fill:
+    if do_fill and b_layout == "kcp":
+        extra = kc_fills(pos, half)
+    elif do_fill:
         # A's fills come last in odd steps and first in even ones: the two 64-byte halves of a 128-byte
         # line of a K-contiguous operand belong to k-steps 2m and 2m+1, filled in steps 2m-3 and 2m-2;
         # requested back to back, the second half is still in the CU's vector cache
@@ -158,7 +197,7 @@ def step(pos, do_fill, wait, last, b_layout):
 def loop(b_layout):
     out = [line("s_mov_b64 s[72:73], %[pa]"), line("s_mov_b64 s[74:75], %[pb]"), line("s_mov_b32 s78, %[groups]"),
            line(f"v_add_u32 v104, {2 * STAGE}, %[a_rd]")]
-    if b_layout == "kc":
+    if b_layout in ("kc", "kcp"):
         out.append(line(f"v_add_u32 v105, {2 * STAGE}, %[b_rd0]"))
     else:
         for x in range(8):
@@ -193,13 +232,14 @@ def loop(b_layout):
     out += first_reads(2) + [line("s_branch 6f"), line("10:")]
     out += first_reads(0) + [line("s_cmp_eq_u32 s78, 0"), line("s_cbranch_scc1 2f"), line("1:")]
     per_tile = 4 + (2 * TN * FRAG) // 4096  # fill instructions per K tile and thread
+    kc = b_layout == "kcp"
     for pos in range(4):
         if pos:
             out.append(line(f"{4 + pos}:"))
-        out += step(pos, True, 2 * per_tile, False, b_layout)
+        out += step(pos, True, kc_wait(pos, 3) if kc else 2 * per_tile, False, b_layout)
     out += [line("s_sub_u32 s78, s78, 1"), line("s_cmp_lg_u32 s78, 0"), line("s_cbranch_scc1 1b"), line("2:")]
-    out += step(0, True, 2 * per_tile, False, b_layout)
-    out += step(1, False, per_tile, False, b_layout)
+    out += step(0, True, kc_wait(0, 3) if kc else 2 * per_tile, False, b_layout)
+    out += step(1, False, kc_wait(1, 2) if kc else per_tile, False, b_layout)
     out += step(2, False, 0, False, b_layout)
     out += step(3, False, 0, True, b_layout)
     out += [line("s_nop 15"), line("s_nop 15")]
@@ -208,8 +248,10 @@ def loop(b_layout):
 
 def main():
     print("// Generated by gen_w4_loop.py; do not edit.  The K loop of gemm_mfma16w4_kernel, one macro per")
-    print("// layout of B (K contiguous / N contiguous 16-bit / N contiguous 8-bit); MFMA is the mnemonic.")
-    for name, tn in (("kc", 8), ("mc16", 8), ("mc8", 8), ("kc", 6)):
+    print("// layout of B (K contiguous, plain or with paired fills / N contiguous 16-bit / N contiguous 8-bit); MFMA is the mnemonic.")
+    # kcp: K-contiguous B with its half-line fills paired (two K tiles per even step); measured ahead of the plain
+    # scheme for the 192-wide tile and for int8, behind it for 16-bit inputs on the 256-wide tile
+    for name, tn in (("kc", 8), ("kcp", 8), ("mc16", 8), ("mc8", 8), ("kcp", 6)):
         set_width(tn)
         body = loop(name)
         print(f"#define ACC950_W4_LOOP_{name.upper()}{'' if tn == 8 else tn}(MFMA) \\")

@@ -36,7 +36,7 @@ def test_include_in_the_tree_is_what_the_generator_writes(capsys):
     assert capsys.readouterr().out == open(os.path.join(CSRC, "gemm_mfma16w4_loop.inc")).read()
 
 
-@pytest.mark.parametrize("layout,tn", [("kc", 8), ("mc16", 8), ("mc8", 8), ("kc", 6)])
+@pytest.mark.parametrize("layout,tn", [("kc", 8), ("kcp", 8), ("mc16", 8), ("mc8", 8), ("kcp", 6)])
 def test_every_k_step_keeps_its_invariants(layout, tn):
     g = _gen()
     g.set_width(tn)
@@ -45,7 +45,8 @@ def test_every_k_step_keeps_its_invariants(layout, tn):
     nb = tn * 2048 // 4096                      # fill passes of B per K tile
     per_tile = 4 + nb
     for pos in range(4):
-        for do_fill, wait, last in ((True, 2 * per_tile, False), (False, per_tile, False), (False, 0, False), (False, 0, True)):
+        for do_fill, wait, last in ((True, g.kc_wait(pos, 3) if layout == "kcp" else 2 * per_tile, False), (False, per_tile, False),
+                                    (False, 0, False), (False, 0, True)):
             ins = _text(g.step(pos, do_fill, wait, last, layout))
             buf, nxt, fst = pos % 2, (pos + 1) % 4, (pos + 3) % 4
             # ---- MFMAs: every accumulator block once, operands from this step's register set
@@ -64,7 +65,7 @@ def test_every_k_step_keeps_its_invariants(layout, tn):
             assert sorted(blocks) == list(range(8 * tn))
             # ---- fragment reads of the next step: other register set, inside the next step's LDS stage
             reads = [i for i in ins if i.startswith("ds_read")]
-            assert len(reads) == (0 if last else 8 + (tn if layout == "kc" else 2 * tn))
+            assert len(reads) == (0 if last else 8 + (tn if layout in ("kc", "kcp") else 2 * tn))
             written = set()
             for r in reads:
                 m = re.match(r"(ds_read_b128|ds_read_b64_tr_b16|ds_read_b64_tr_b8) v\[(\d+):(\d+)\], (\S+) offset:(\d+)$", r)
@@ -79,12 +80,22 @@ def test_every_k_step_keeps_its_invariants(layout, tn):
                 assert 0 <= in_stage < stage_bytes
                 is_b = 128 + (buf ^ 1) * 64 <= v0 < 160 + (buf ^ 1) * 64
                 assert (in_stage >= b_tile) == is_b
-                assert (op == "ds_read_b128") == (layout == "kc" or not is_b)
+                assert (op == "ds_read_b128") == (layout in ("kc", "kcp") or not is_b)
             assert len(written) == (0 if last else (8 + tn) * 4)
             # ---- fills of the tile three steps ahead
             loads = [n for n, i in enumerate(ins) if i.startswith("global_load_lds")]
-            assert len(loads) == (per_tile if do_fill else 0)
-            if do_fill:
+            for n in loads:
+                assert ins[n - 1].startswith("MFMA"), "one instruction between the M0 write and its use"
+                assert any(i.startswith("s_add_u32 m0,") for i in ins[max(0, n - 8):n - 1])
+            if layout == "kcp":
+                # (K-contiguous B with paired fills: A's tile t+3 every step, B's tiles t+2 and t+3 on even positions; addresses, stages and
+                # waits of this scheme are checked over whole loops by the model below)
+                assert len(loads) == ((4 + (2 * nb if pos % 2 == 0 else 0)) if do_fill else 0)
+                if do_fill:
+                    assert max(loads) < ins.index("s_barrier")
+            else:
+                assert len(loads) == (per_tile if do_fill else 0)
+            if do_fill and layout != "kcp":
                 first_mfma_after_barrier = ins.index("s_barrier")
                 assert max(loads) < first_mfma_after_barrier      # all issued before this step's wait
                 seen = {"a": [], "b": []}
@@ -127,7 +138,7 @@ def test_every_k_step_keeps_its_invariants(layout, tn):
                 assert ins[b - 1] == f"s_waitcnt vmcnt({wait})" and ins[b - 2] == "s_waitcnt lgkmcnt(0)"
 
 
-@pytest.mark.parametrize("layout,tn", [("kc", 8), ("mc16", 8), ("kc", 6)])
+@pytest.mark.parametrize("layout,tn", [("kc", 8), ("kcp", 8), ("mc16", 8), ("kcp", 6)])
 def test_whole_loop_shape(layout, tn):
     """Preamble, four-step body with its back branch, and the four closing steps (one with fills, three without)."""
     g = _gen()
@@ -143,7 +154,7 @@ def test_whole_loop_shape(layout, tn):
         start = entry.index(label) + 1 if label else entry.index("s_cbranch_scc1 12f") + 1
         block = entry[start:entry.index(jump, start)]
         reads = [i for i in block if i.startswith("ds_read")]
-        assert len(reads) == 8 + (tn if layout == "kc" else 2 * tn)
+        assert len(reads) == 8 + (tn if layout in ("kc", "kcp") else 2 * tn)
         for r in reads:
             m = re.match(r"\S+ v\[(\d+):(\d+)\], (\S+) offset:(\d+)$", r)
             v0, base, off = int(m.group(1)), m.group(3), int(m.group(4))
@@ -156,8 +167,13 @@ def test_whole_loop_shape(layout, tn):
     assert sum(i.startswith("MFMA") for i in body) == 4 * 8 * tn == sum(i.startswith("MFMA") for i in tail)
     assert body.count("s_barrier") == 4 and tail.count("s_barrier") == 3
     assert sum(i.startswith("global_load_lds") for i in body) == 4 * per_tile
-    assert sum(i.startswith("global_load_lds") for i in tail) == per_tile
-    assert [i for i in tail if i.startswith("s_waitcnt vmcnt")] == [f"s_waitcnt vmcnt({2 * per_tile})", f"s_waitcnt vmcnt({per_tile})", "s_waitcnt vmcnt(0)"]
+    nb = tn * 2048 // 4096
+    if layout == "kcp":  # the closing copy's first step fetches A's last tile and B's last two
+        assert sum(i.startswith("global_load_lds") for i in tail) == 4 + 2 * nb
+        assert [i for i in tail if i.startswith("s_waitcnt vmcnt")] == [f"s_waitcnt vmcnt({8 + 2 * nb})", "s_waitcnt vmcnt(1)", "s_waitcnt vmcnt(0)"]
+    else:
+        assert sum(i.startswith("global_load_lds") for i in tail) == per_tile
+        assert [i for i in tail if i.startswith("s_waitcnt vmcnt")] == [f"s_waitcnt vmcnt({2 * per_tile})", f"s_waitcnt vmcnt({per_tile})", "s_waitcnt vmcnt(0)"]
     # accumulators: zeroed, or loaded from C block by block (64 bytes per block and row group, 16 rows further per row of blocks)
     pre = ins[:ins.index("1:")]
     assert sum(i.startswith("v_accvgpr_write_b32") for i in pre) == 32 * tn
@@ -266,15 +282,19 @@ def _run_fills(g, layout, tn, KT, b_tiles_before_loop):
     return fills, steps, p0
 
 
-@pytest.mark.parametrize("layout,tn", [("kc", 8), ("mc16", 8), ("kc", 6)])
+@pytest.mark.parametrize("layout,tn", [("kc", 8), ("kcp", 8), ("mc16", 8), ("kcp", 6)])
 @pytest.mark.parametrize("KT", [4, 5, 6, 7, 8, 9, 10, 11, 12, 23, 128])
 def test_fill_addresses_over_a_whole_k_loop(layout, tn, KT):
     """Every pass of every K tile from 3 on is filled exactly once, from the address of that tile and pass, into
     the LDS stage its k-step will read ((tile + entry position) mod 4), and nothing beyond the last tile is touched."""
     g = _gen()
-    fills, steps, p0 = _run_fills(g, layout, tn, KT, 3)
+    p0 = (4 - KT % 4) % 4
+    # with paired fills a K-contiguous B is fetched two tiles at a time on the even positions of the body: the code before the loop issues
+    # B's tiles 0 and 1, and tile 2 as well when the first k-step sits at an odd position
+    b_before = 3 if layout != "kcp" else 2 + (p0 & 1)
+    fills, steps, p0 = _run_fills(g, layout, tn, KT, b_before)
     nb = tn * 2048 // 4096
     assert steps == KT
     want = sorted([("a", t, p, (t + p0) % 4) for t in range(3, KT) for p in range(4)] +
-                  [("b", t, p, (t + p0) % 4) for t in range(3, KT) for p in range(nb)])
+                  [("b", t, p, (t + p0) % 4) for t in range(b_before, KT) for p in range(nb)])
     assert sorted(fills) == want
