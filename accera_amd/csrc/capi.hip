@@ -131,10 +131,9 @@ bool mfma_can_take(const MfmaVariant& v, const Problem& pb)
         if (pb.have_pointers && !aligned16(g.C)) return false;
     }
     if (v.w4) {
-        // C = A*B / relu(A*B); with a 32- or 16-bit C also C += A*B (the accumulators start from C)
+        // every op, except that an int8 C is only written (SET prologue), never read
         const int os = elem_size(g.out_type);
-        const bool epi_ok = g.epilogue == EPI_RELU || g.epilogue == EPI_NONE;
-        const bool lean = epi_ok && ((g.prologue == PRO_SET && g.prologue_arg == 0.f) || (g.prologue == PRO_NONE && os >= 2));
+        const bool lean = g.prologue == PRO_SET || os >= 2;
         if (!lean || g.K % bk || g.K < 4 * bk || (g.c_rs * os) % 16 || (g.batch > 1 && (g.c_bs * os) % 16)) return false;
         if (pb.have_pointers && !aligned16(g.C)) return false;
         // any M, N >= one tile when C is only written: the last row / column of tiles is moved to end at M / N

@@ -16,9 +16,9 @@
 // Takes: A row-major, M and N multiples of the tile (any M >= 256 and any 16-byte-aligned N >= the tile width
 // when C is not read: the last row / column of tiles then overlaps the one before), K a multiple of one k-step (64 bytes)
 // and at least four of them, rows of C 16 bytes aligned;
-// C = A*B or relu(A*B) (SET 0 prologue) for every output type; C += A*B (then ReLU or nothing) for 32-bit
-// outputs, where the tile of C is loaded straight into the accumulator registers, and for 16-bit outputs,
-// where it is widened on the way in.
+// every prologue / epilogue op (an int8 C is only written, never read): C = A*B starts from zeros, C += A*B with a
+// 32-bit C loads the tile of C straight into the accumulator registers, everything else (a 16-bit C, beta * C,
+// a SET constant) is written into them by ordinary code before the loop.
 #pragma once
 #include "gemm_mfma16.h"
 #include "gemm_mfma16w4_loop.inc"
@@ -183,54 +183,94 @@ __global__ void __launch_bounds__(256, 1) gemm_mfma16w4_kernel(GemmArgs p)
 
     // C += A*B: the loop starts from the tile of C instead of zeros (the host sends nothing else with a prologue
     // other than SET 0 here).  A 32-bit C is loaded by the loop's preamble:  Lane l owns row i*16 + l%16, columns j*16 + (l/16)*4 .. +3 of block (i, j).
+    // How the accumulators start: 0 zeros (SET 0: C = A*B), 1 the loop's preamble loads a 32-bit C into them (C += A*B),
+    // 2 the code below sets them up (a 16-bit C, beta * C, or a SET constant) and the loop leaves them as they are.
     const bool c_is_32bit = p.out_type == T_F32 || p.out_type == T_I32;
-    const unsigned accum = __builtin_amdgcn_readfirstlane(p.prologue != PRO_NONE ? 0u : c_is_32bit ? 1u : 2u); // 2: set up below
+    const unsigned accum = __builtin_amdgcn_readfirstlane(
+        p.prologue == PRO_SET ? (p.prologue_arg == 0.f ? 0u : 2u) : (p.prologue == PRO_NONE && c_is_32bit) ? 1u : 2u);
     const CTile c_in = c_tile((char*)p.C + ((int64_t)m0 * p.c_rs + n0) * 4);
     const unsigned c_off = (unsigned)(wr0 + (lane & 15)) * ((unsigned)p.c_rs * 4) + (unsigned)(wc0 + (lane >> 4) * 4) * 4;
     const unsigned c_row16 = __builtin_amdgcn_readfirstlane((unsigned)p.c_rs * 64);
     const auto c_rsrc = c_in.rsrc;
 
     if (accum == 2) {
-        // C += A*B with a 16-bit C (fp16 / bf16 / int16): the lane's four elements of every block are loaded,
-        // widened and written into the accumulator registers here; the loop then leaves them as they are.
+        // The lane's four elements of every block are written into the accumulator registers here: the SET constant,
+        // or C widened (16-bit types) and scaled (SCALE prologue; x 1 is exact otherwise).
         // (All fills are waited for first: the compiler counts only its own loads when it places the waits.)
-        wait_vmcnt<0>();
-        const CTile c16 = c_tile((char*)p.C + ((int64_t)m0 * p.c_rs + n0) * 2);
-        const unsigned rb = (unsigned)p.c_rs * 2;
-        const unsigned off16 = (unsigned)(wr0 + (lane & 15)) * rb + (unsigned)(wc0 + (lane >> 4) * 4) * 2;
-        const unsigned m_f16 = p.out_type == T_F16 ? ~0u : 0u, m_bf16 = p.out_type == T_BF16 ? ~0u : 0u;
-        typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
-        // four rows of blocks at a time: their loads are all in flight before the first is used
-        w4_static_for<0, TM / 4>([&](auto q) {
-            u32x2 w[4][TN];
+        auto put = [](auto n_tag, int x0, int x1, int x2, int x3) {
+            constexpr int n = decltype(n_tag)::value;
+            asm volatile("v_accvgpr_write_b32 a[%4], %0\n\tv_accvgpr_write_b32 a[%5], %1\n\tv_accvgpr_write_b32 a[%6], %2\n\tv_accvgpr_write_b32 a[%7], %3"
+                         :
+                         : "v"(x0), "v"(x1), "v"(x2), "v"(x3), "n"(n), "n"(n + 1), "n"(n + 2), "n"(n + 3));
+        };
+        const scalar_t c_mul = p.prologue == PRO_SCALE ? (scalar_t)p.prologue_arg : scalar_t(1);
+        auto scaled = [&](scalar_t c) -> int {
+            if constexpr (IN == IN_I8) return wrap_mul(c, c_mul);
+            else return (int)__float_as_uint(c * c_mul);
+        };
+        if (p.prologue == PRO_SET) {
+            const scalar_t set_v = (scalar_t)p.prologue_arg;
+            int x;
+            if constexpr (IN == IN_I8) x = set_v;
+            else x = (int)__float_as_uint(set_v);
+            w4_static_for<0, TM * TN>([&](auto b) { put(std::integral_constant<int, b.value * 4>{}, x, x, x, x); });
+        } else if (c_is_32bit) {
+            wait_vmcnt<0>();
+            // four rows of blocks at a time: their loads are all in flight before the first is used
+            w4_static_for<0, TM / 4>([&](auto q) {
+                u32x4 w[4][TN];
 #pragma unroll
-            for (int ii = 0; ii < 4; ++ii)
+                for (int ii = 0; ii < 4; ++ii)
 #pragma unroll
-                for (int j = 0; j < TN; ++j)
-                    w[ii][j] = __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(c16.rsrc, off16 + j * 32,
-                                                                                             (unsigned)((q.value * 4 + ii) * 16) * rb, 0));
-            w4_static_for<0, 4>([&](auto ii) {
-                w4_static_for<0, TN>([&](auto j) {
-                    const unsigned w0 = w[ii.value][j.value][0], w1 = w[ii.value][j.value][1];
-                    int x[4];
+                    for (int j = 0; j < TN; ++j)
+                        w[ii][j] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(c_rsrc, c_off + j * 64,
+                                                                                                 (unsigned)((q.value * 4 + ii) * 16) * ((unsigned)p.c_rs * 4), 0));
+                w4_static_for<0, 4>([&](auto ii) {
+                    w4_static_for<0, TN>([&](auto j) {
+                        int x[4];
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        const unsigned half = (((e & 2) ? w1 : w0) >> ((e & 1) * 16)) & 0xffffu;
-                        if constexpr (IN == IN_I8) x[e] = (int)(short)half; // int16 widens with its sign
-                        else {
-                            const unsigned short h = (unsigned short)half;
-                            const unsigned as_f16 = __float_as_uint((float)__builtin_bit_cast(_Float16, h));
-                            x[e] = (int)((as_f16 & m_f16) | ((half << 16) & m_bf16));
+                        for (int e = 0; e < 4; ++e) {
+                            const unsigned bits = w[ii.value][j.value][e]; // (a bit cast applied to the element expression itself reads element 0)
+                            x[e] = scaled(__builtin_bit_cast(scalar_t, bits));
                         }
-                    }
-                    constexpr int n = ((q.value * 4 + ii.value) * TN + j.value) * 4;
-                    const int x0 = x[0], x1 = x[1], x2 = x[2], x3 = x[3]; // (asm operands do not capture on their own)
-                    asm volatile("v_accvgpr_write_b32 a[%4], %0\n\tv_accvgpr_write_b32 a[%5], %1\n\tv_accvgpr_write_b32 a[%6], %2\n\tv_accvgpr_write_b32 a[%7], %3"
-                                 :
-                                 : "v"(x0), "v"(x1), "v"(x2), "v"(x3), "n"(n), "n"(n + 1), "n"(n + 2), "n"(n + 3));
+                        put(std::integral_constant<int, ((q.value * 4 + ii.value) * TN + j.value) * 4>{}, x[0], x[1], x[2], x[3]);
+                    });
                 });
             });
-        });
+        } else {
+            wait_vmcnt<0>();
+            const CTile c16 = c_tile((char*)p.C + ((int64_t)m0 * p.c_rs + n0) * 2);
+            const unsigned rb = (unsigned)p.c_rs * 2;
+            const unsigned off16 = (unsigned)(wr0 + (lane & 15)) * rb + (unsigned)(wc0 + (lane >> 4) * 4) * 2;
+            const unsigned m_f16 = p.out_type == T_F16 ? ~0u : 0u, m_bf16 = p.out_type == T_BF16 ? ~0u : 0u;
+            typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+            w4_static_for<0, TM / 4>([&](auto q) {
+                u32x2 w[4][TN];
+#pragma unroll
+                for (int ii = 0; ii < 4; ++ii)
+#pragma unroll
+                    for (int j = 0; j < TN; ++j)
+                        w[ii][j] = __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(c16.rsrc, off16 + j * 32,
+                                                                                                 (unsigned)((q.value * 4 + ii) * 16) * rb, 0));
+                w4_static_for<0, 4>([&](auto ii) {
+                    w4_static_for<0, TN>([&](auto j) {
+                        const unsigned w0 = w[ii.value][j.value][0], w1 = w[ii.value][j.value][1];
+                        int x[4];
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            const unsigned half = (((e & 2) ? w1 : w0) >> ((e & 1) * 16)) & 0xffffu;
+                            if constexpr (IN == IN_I8) x[e] = scaled((int)(short)half); // int16 widens with its sign
+                            else {
+                                const unsigned short h = (unsigned short)half;
+                                const unsigned as_f16 = __float_as_uint((float)__builtin_bit_cast(_Float16, h));
+                                x[e] = scaled(__uint_as_float((as_f16 & m_f16) | ((half << 16) & m_bf16)));
+                            }
+                        }
+                        put(std::integral_constant<int, ((q.value * 4 + ii.value) * TN + j.value) * 4>{}, x[0], x[1], x[2], x[3]);
+                    });
+                });
+            });
+        }
     }
 
     wait_vmcnt<B_PAIRED ? 4 + FILLS : 2 * FILLS>(); // tile 0 has landed (tile 1 and tile 2 -- A's part of it at least -- in flight)
@@ -281,8 +321,10 @@ __global__ void __launch_bounds__(256, 1) gemm_mfma16w4_kernel(GemmArgs p)
     const int wave_u = __builtin_amdgcn_readfirstlane(wave);
     // One copy of the stores per epilogue (a uniform branch): with a single wave per SIMD the
     // write-back is bound by instruction issue, so every instruction per block counts.
-    auto write_back = [&](auto relu_tag) {
-        constexpr bool RELU = decltype(relu_tag)::value;
+    // (epi_tag: 0 nothing, 1 ReLU, 2 the other epilogue ops, applied element by element from the call's arguments)
+    auto write_back = [&](auto epi_tag) {
+        constexpr int EPI = decltype(epi_tag)::value;
+        constexpr bool RELU = EPI == 1;
         // row i of the wave tile's blocks, epilogue applied
         auto load_row = [&](auto i_tag, acc_t (&row)[TN]) {
             constexpr int i = decltype(i_tag)::value;
@@ -299,6 +341,11 @@ __global__ void __launch_bounds__(256, 1) gemm_mfma16w4_kernel(GemmArgs p)
                         if constexpr (IN == IN_I8) row[j][e] = row[j][e] > 0 ? row[j][e] : 0;
                         else row[j][e] = __builtin_fmaxf(row[j][e], 0.f);
                     }
+            } else if constexpr (EPI == 2) {
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) row[j][e] = apply_epilogue<scalar_t>(row[j][e], p.epilogue, p.epilogue_arg);
             }
         };
         if (os == 4) {
@@ -308,10 +355,10 @@ __global__ void __launch_bounds__(256, 1) gemm_mfma16w4_kernel(GemmArgs p)
             w4_static_for<0, TM>([&](auto i) {
                 const unsigned soff = (unsigned)(i.value * 16) * row_bytes;
                 acc_t row[TN];
-                if constexpr (RELU) load_row(i, row);
+                if constexpr (EPI != 0) load_row(i, row);
                 w4_static_for<0, TN>([&](auto j) {
                     constexpr int n = i.value * TN + j.value;
-                    if constexpr (RELU) {
+                    if constexpr (EPI != 0) {
                         __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, row[j.value]), tile.rsrc, lane_off + j.value * 64, soff, 0);
                     } else {
                         // no arithmetic on the way out: the store reads the accumulator registers themselves
@@ -389,8 +436,9 @@ __global__ void __launch_bounds__(256, 1) gemm_mfma16w4_kernel(GemmArgs p)
             }
         }
     };
-    if (p.epilogue == EPI_RELU) write_back(std::true_type{});
-    else write_back(std::false_type{});
+    if (p.epilogue == EPI_RELU) write_back(std::integral_constant<int, 1>{});
+    else if (p.epilogue == EPI_NONE) write_back(std::integral_constant<int, 0>{});
+    else write_back(std::integral_constant<int, 2>{});
 
     if constexpr (Cfg::TIMED) {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // stores acknowledged

@@ -503,10 +503,9 @@ def _variant_for_tile(spec, bm, bn):
             continue
         # ping-pong over software-pipelined; the 16x16 MFMA shapes where the library runs their lean build
         rank = 2 * ("pingpong" in name) + (1 if "mi16" in name and lean else -1 if "mi16" in name else 0)
-        if "hand-laid loop" in name:  # four waves; C = A*B / relu(A*B), or C += A*B (not into an int8 C); ahead of the ping-pong form
-            adds = (spec.prologue == _lib.PROLOGUE_NONE and spec.epilogue in (_lib.EPILOGUE_RELU, _lib.EPILOGUE_NONE)
-                    and spec.C.element_type.lib_id != _lib.I8)
-            rank = 4 if (lean or adds) else -9
+        if "hand-laid loop" in name:  # four waves: every op, but an int8 C is only written; ahead of the ping-pong form
+            reads_int8_c = spec.prologue != _lib.PROLOGUE_SET and spec.C.element_type.lib_id == _lib.I8
+            rank = -9 if reads_int8_c else 4
         if rank > best_rank:
             best, best_rank = v, rank
     return best
