@@ -91,7 +91,7 @@ int acc950_gemm_relu(int in_type, int out_type, int M, int N, int K,
  * ACC950_VARIANT_SKINNY_BASE + i, ACC950_VARIANT_F32_MFMA or ACC950_VARIANT_GENERIC.  `k_splits` (skinny
  * kernels only; 0 = automatic) splits K over workgroups.  A named variant that does not take the
  * problem -- its sizes, layouts, alignment, or its prologue / epilogue ops (the four-wave kernels
- * take C = A*B, relu(A*B) and, unless C is int8, C += A*B only) -- returns ACC950_UNSUPPORTED; nothing runs.
+ * do not read an int8 C) -- returns ACC950_UNSUPPORTED; nothing runs.
  */
 int acc950_gemm_relu_ex(int in_type, int out_type, int M, int N, int K,
                         const void* A, int64_t a_row_stride, int64_t a_col_stride,
