@@ -727,3 +727,45 @@ def test_random_problems_through_the_automatic_choice():
         torch.cuda.synchronize()
         want = ora.gemm_relu_exact(A, B, C0, in_type, out_type, pro, epi, prologue_arg=pa, epilogue_arg=ea)
         assert_matches(to_host(dC, out_type), want, out_type, K)
+
+
+def test_random_problems_on_the_four_wave_kernel():
+    """Seeded random sizes (M and N ragged or whole tiles, every K remainder modulo four k-steps), types, B layouts
+    and ops on the kernels with the hand-laid loop, named explicitly; what a kernel refuses is skipped, never wrong."""
+    import accera_amd as acc
+    import torch
+    from accera_amd import _lib
+    rng = np.random.default_rng(950)
+    pairs = [("f16", "f32"), ("f16", "f16"), ("bf16", "f32"), ("bf16", "bf16"), ("i8", "i32"), ("i8", "i16"), ("i8", "i8")]
+    ops = [(ora.PRO_SET0, 0.0, ora.EPI_RELU, 0.0), (ora.PRO_SET0, 0.0, ora.EPI_NONE, 0.0), (ora.PRO_NONE, 0.0, ora.EPI_RELU, 0.0),
+           (ora.PRO_SCALE, 0.5, ora.EPI_SCALE, 2.0), (ora.PRO_SET, 3.0, ora.EPI_RELU_NOCOND, 0.0), (ora.PRO_NONE, 0.0, ora.EPI_SET, 1.0),
+           (ora.PRO_SCALE, -1.5, ora.EPI_RELU, 0.0)]
+    ran = 0
+    for case in range(48):
+        in_type, out_type = pairs[rng.integers(len(pairs))]
+        b_layout = ("row", "col")[rng.integers(2)]
+        variants = [v for v, n in _variants(b_layout) if "hand-laid" in n]
+        v = variants[rng.integers(len(variants))]
+        kb = 64 if in_type == "i8" else 32
+        pro, pa, epi, ea = ops[rng.integers(len(ops))]
+        whole = pro != ora.PRO_SET or rng.integers(2) == 0          # ragged sizes only when C is not read
+        tile_n = 192 if "256x192" in _lib.variant_name(v) else 256
+        M = int(rng.integers(1, 5)) * 256 if whole else int(rng.integers(256, 1100))
+        N = int(rng.integers(1, 5)) * tile_n if whole else int(rng.integers(tile_n // 16, 70)) * 16
+        K = int(rng.integers(4, 14)) * kb
+        print("case", case, "variant", v, in_type, out_type, M, N, K, b_layout, pro, pa, epi, ea, flush=True)
+        A, B = make_input(rng, (M, K), in_type), make_input(rng, (K, N), in_type)
+        if b_layout == "col":
+            B = np.asfortranarray(B)
+        C0 = make_c0(rng, (M, N), out_type, scale=100)
+        dC = to_device(C0, out_type)
+        try:
+            acc.gemm_relu(to_device(A, in_type), to_device(B, in_type), dC, prologue=pro, prologue_arg=pa, epilogue=epi, epilogue_arg=ea,
+                          variant=v)
+        except _lib.Acc950Error:
+            continue  # (an int8 C that would be read)
+        torch.cuda.synchronize()
+        want = ora.gemm_relu_exact(A, B, C0, in_type, out_type, pro, epi, prologue_arg=pa, epilogue_arg=ea)
+        assert_matches(to_host(dC, out_type), want, out_type, K)
+        ran += 1
+    assert ran >= 30, ran
