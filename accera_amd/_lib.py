@@ -1,4 +1,4 @@
-"""ctypes binding of libaccera_mi355x.so (the C ABI declared in include/accera_mi355x_gemm.h).
+"""ctypes binding of libaccera_mi355x.so (the C ABI declared in include/accera_mi355x_gemm.h, the measurement aids in include/accera_mi355x_probes.h).
 
 There is no CPU fallback: if the shared library is missing, loading raises with the
 build command; if a call fails, the library's own error text is raised.
@@ -22,8 +22,10 @@ EXPORTS = [
     "acc950_init", "acc950_gemm_relu", "acc950_gemm_relu_ex", "acc950_gemm_relu_host", "acc950_gemm_ops", "acc950_gemm_ops_host",
     "acc950_gemm_batched", "acc950_gemm_batched_host", "acc950_bind", "acc950_launch", "acc950_unbind",
     "acc950_launch_geometry", "acc950_num_variants", "acc950_num_skinny_variants",
-    "acc950_variant_name", "acc950_last_error", "acc950_mfma_ceiling", "acc950_mfma_phase_probe", "acc950_copy_probe", "acc950_stream_read_probe",
+    "acc950_variant_name", "acc950_last_error",
 ]
+# measurement aids (include/accera_mi355x_probes.h): not part of the product ABI
+PROBE_EXPORTS = ["acc950_mfma_ceiling", "acc950_mfma_phase_probe", "acc950_copy_probe", "acc950_stream_read_probe", "acc950_workspace_probe"]
 
 
 class Acc950Error(RuntimeError):
@@ -67,8 +69,9 @@ def lib():
     L.acc950_mfma_phase_probe.argtypes = [ci, ci, ci, ci, ci, vp, vp, vp, ctypes.POINTER(ctypes.c_double)]
     L.acc950_copy_probe.argtypes = [vp, vp, ctypes.c_size_t, vp]
     L.acc950_stream_read_probe.argtypes = [vp, ctypes.c_size_t, vp, vp]
+    L.acc950_workspace_probe.argtypes = [vp, ctypes.POINTER(vp), ctypes.POINTER(vp)]
     L.acc950_last_error.restype = ctypes.c_char_p
-    for name in EXPORTS:
+    for name in EXPORTS + PROBE_EXPORTS:
         if name != "acc950_last_error":
             getattr(L, name).restype = ci
     _lib = L
@@ -95,6 +98,13 @@ def mfma_ceiling(in_type, data_mode=2, iters=20000):
     t, g = ctypes.c_double(), ctypes.c_double()
     check(lib().acc950_mfma_ceiling(in_type, data_mode, iters, ctypes.byref(t), ctypes.byref(g)))
     return t.value, g.value
+
+
+def workspace_probe(stream):
+    """(partial sums, counters) device addresses of the K-split workspace of `stream` (a raw hipStream_t or None)."""
+    a, b = ctypes.c_void_p(), ctypes.c_void_p()
+    check(lib().acc950_workspace_probe(stream, ctypes.byref(a), ctypes.byref(b)))
+    return a.value, b.value
 
 
 def variant_name(variant):

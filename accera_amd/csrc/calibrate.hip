@@ -9,6 +9,7 @@
 //   * Copy kernel of known size: reference point for scaling the rocprof FETCH_SIZE /
 //     WRITE_SIZE counters, and a streaming read kernel for the achievable HBM rate.
 #include "../../include/accera_mi355x_gemm.h"
+#include "../../include/accera_mi355x_probes.h"
 #include "common.h"
 
 #include <cstdlib>

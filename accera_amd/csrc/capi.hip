@@ -1,6 +1,7 @@
 // C ABI of the library (include/accera_mi355x_gemm.h): argument checking, kernel
 // selection, the host-pointer path and the launch-geometry query.
 #include "../../include/accera_mi355x_gemm.h"
+#include "../../include/accera_mi355x_probes.h"
 #include "common.h"
 #include "skinny.h"
 #include <vector>
@@ -8,8 +9,10 @@
 
 #include <cstdio>
 #include <cstring>
+#include <map>
 #include <mutex>
 #include <string>
+#include <utility>
 
 using namespace acc950;
 
@@ -181,32 +184,47 @@ int auto_skinny_variant(const Problem& pb)
     return -1;
 }
 
-// ---- scratch for the skinny kernels' K split -----------------------------------------
+// ---- workspace of the skinny kernels' K split ------------------------------------------
+// Partial sums (fp32) and one arrival counter per column block.  One workspace per (device, stream): launches on one
+// stream run one after the other and may share it, launches on different streams may overlap and must not.  A
+// workspace only grows, and an outgrown block stays allocated until the process ends, because launches queued
+// earlier may still be using it.  The pointers are copied out while the lock is held.
+struct Workspace {
+    float* scratch = nullptr;
+    size_t floats = 0;
+    unsigned* counters = nullptr; // zero between launches: the kernels leave them so
+    size_t n_counters = 0;
+};
 std::mutex g_ws_mutex;
-float* g_scratch = nullptr;
-size_t g_scratch_floats = 0;
-unsigned* g_counters = nullptr;
-size_t g_counters_n = 0;
+std::map<std::pair<int, hipStream_t>, Workspace> g_ws;
 
-hipError_t ensure_workspace(size_t floats, size_t counters)
+hipError_t workspace_for(hipStream_t stream, size_t floats, size_t counters, float** scratch, unsigned** cnt)
 {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
     std::lock_guard<std::mutex> lock(g_ws_mutex);
-    if (floats > g_scratch_floats) {
-        if (g_scratch) { hipError_t e = hipFree(g_scratch); if (e != hipSuccess) return e; g_scratch = nullptr; g_scratch_floats = 0; }
-        size_t want = floats < (1u << 20) ? (1u << 20) : floats;
-        hipError_t e = hipMalloc((void**)&g_scratch, want * sizeof(float));
+    Workspace& w = g_ws[std::make_pair(dev, stream)];
+    if (floats > w.floats) {
+        const size_t want = floats < (1u << 20) ? (1u << 20) : floats + floats / 2;
+        float* p = nullptr;
+        e = hipMalloc((void**)&p, want * sizeof(float));
         if (e != hipSuccess) return e;
-        g_scratch_floats = want;
+        w.scratch = p; // (the block it replaces is left to earlier launches)
+        w.floats = want;
     }
-    if (counters > g_counters_n) {
-        if (g_counters) { hipError_t e = hipFree(g_counters); if (e != hipSuccess) return e; g_counters = nullptr; g_counters_n = 0; }
-        size_t want = counters < 4096 ? 4096 : counters;
-        hipError_t e = hipMalloc((void**)&g_counters, want * sizeof(unsigned));
+    if (counters > w.n_counters) {
+        const size_t want = counters < 4096 ? 4096 : counters + counters / 2;
+        unsigned* p = nullptr;
+        e = hipMalloc((void**)&p, want * sizeof(unsigned));
         if (e != hipSuccess) return e;
-        e = hipMemset(g_counters, 0, want * sizeof(unsigned));
-        if (e != hipSuccess) return e;
-        g_counters_n = want;
+        e = hipMemset(p, 0, want * sizeof(unsigned));
+        if (e != hipSuccess) { (void)hipFree(p); return e; }
+        w.counters = p;
+        w.n_counters = want;
     }
+    *scratch = w.scratch;
+    *cnt = w.counters;
     return hipSuccess;
 }
 
@@ -347,10 +365,9 @@ int run(const Problem& pb, const Choice& c, hipStream_t stream, LaunchGeom* geom
             const size_t nb = g.batch > 1 ? (size_t)g.batch : 1;
             s.scratch_bs = (int64_t)skinny_scratch_floats(sv, g.N, ws_splits);
             s.counter_bs = skinny_column_blocks(sv, g.N);
-            e = ensure_workspace(nb * (size_t)s.scratch_bs, nb * (size_t)s.counter_bs);
+            const size_t floats = nb * (size_t)s.scratch_bs, counters = nb * (size_t)s.counter_bs;
+            e = workspace_for(stream, floats, counters, &s.scratch, &s.counters);
             if (e != hipSuccess) return fail_hip(e, "workspace allocation");
-            s.scratch = g_scratch;
-            s.counters = g_counters;
         }
         e = launch_skinny(sv, s, stream, geom, dry_run);
     } else {
@@ -502,6 +519,18 @@ int acc950_gemm_relu(int in_type, int out_type, int M, int N, int K,
 {
     return acc950_gemm_relu_ex(in_type, out_type, M, N, K, A, a_rs, a_cs, B, b_rs, b_cs, C, c_rs, c_cs, prologue, epilogue,
                                ACC950_VARIANT_AUTO, 0, stream);
+}
+
+int acc950_workspace_probe(void* stream, void** partial_sums, void** counters)
+{
+    if (!partial_sums || !counters) return fail(ACC950_INVALID_ARGUMENT, "null output");
+    float* f = nullptr;
+    unsigned* c = nullptr;
+    hipError_t e = workspace_for((hipStream_t)stream, 1, 1, &f, &c);
+    if (e != hipSuccess) return fail_hip(e, "workspace allocation");
+    *partial_sums = f;
+    *counters = c;
+    return ACC950_OK;
 }
 
 int acc950_mfma_phase_probe(int in_type, int out_type, int M, int N, int K, const void* A, const void* B, void* C, double* out)

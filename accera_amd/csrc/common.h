@@ -2,6 +2,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <mutex>
 
 namespace acc950 {
 
@@ -144,5 +145,27 @@ struct LaunchGeom {
 };
 
 typedef hipError_t (*LaunchFn)(const GemmArgs&, hipStream_t, LaunchGeom*, bool dry_run);
+
+// Raises a kernel's dynamic LDS limit once per device, whichever host thread launches it first
+// (one object per kernel instantiation, as a function-local static of its launcher).
+class LdsLimitOnce {
+public:
+    hipError_t ensure(const void* kernel, int bytes)
+    {
+        int dev = 0;
+        hipError_t e = hipGetDevice(&dev);
+        if (e != hipSuccess) return e;
+        const uint64_t bit = 1ull << (dev & 63);
+        std::lock_guard<std::mutex> lock(mutex_);
+        if (done_ & bit) return hipSuccess;
+        e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+        if (e == hipSuccess) done_ |= bit;
+        return e;
+    }
+
+private:
+    std::mutex mutex_;
+    uint64_t done_ = 0;
+};
 
 } // namespace acc950

@@ -311,10 +311,15 @@ typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 struct CTile {
     __amdgpu_buffer_rsrc_t rsrc;
 };
-__device__ __forceinline__ CTile c_tile(void* base)
+// Descriptor that starts `back` bytes before element (row, col) of C (elements of `os` bytes) and ends with the
+// last row of C: the kernels test the edges themselves, and an access that slips past the end of the matrix all
+// the same is dropped by the hardware's range check instead of reaching memory.
+__device__ __forceinline__ CTile c_tile(const GemmArgs& p, int row, int col, unsigned os, unsigned back = 0)
 {
-    // no range check by the hardware: the kernels test the edges themselves
-    return CTile{__builtin_amdgcn_make_buffer_rsrc(base, 0, -1, 0x00020000)};
+    char* base = (char*)p.C + ((int64_t)row * p.c_rs + col) * os - back;
+    const int64_t bytes = ((int64_t)(p.M - 1 - row) * p.c_rs + (p.N - col)) * os + back;
+    const unsigned records = bytes <= 0 ? 0u : bytes > 0xffffffffll ? 0xffffffffu : (unsigned)bytes;
+    return CTile{__builtin_amdgcn_make_buffer_rsrc(base, 0, records, 0x00020000)};
 }
 template <typename T>
 __device__ __forceinline__ T c_load(CTile t, unsigned voff, unsigned soff)
@@ -618,7 +623,7 @@ __global__ void __launch_bounds__(Cfg::NT, Cfg::WGS_PER_CU) gemm_mfma_kernel(Gem
     auto for_each_element = [&](auto out_tag, auto&& fn) {
         using out_t = decltype(out_tag);
         constexpr unsigned OS = sizeof(out_t);
-        const CTile tile = c_tile((char*)p.C + ((int64_t)m0 * p.c_rs + n0) * OS); // uniform
+        const CTile tile = c_tile(p, m0, n0, OS); // uniform
         const unsigned row_bytes = (unsigned)p.c_rs * OS;
         const unsigned lane_off = (unsigned)row_in_tile * row_bytes + (unsigned)col_in_tile * OS;
 #pragma unroll
@@ -659,7 +664,7 @@ __global__ void __launch_bounds__(Cfg::NT, Cfg::WGS_PER_CU) gemm_mfma_kernel(Gem
         const unsigned m_f32 = p.out_type == T_F32 ? ~0u : 0u, m_f16 = p.out_type == T_F16 ? ~0u : 0u, m_bf16 = p.out_type == T_BF16 ? ~0u : 0u;
         char* tile_base = (char*)p.C + (((int64_t)m0 * p.c_rs + n0) << sh);
         const unsigned base_mis = (unsigned)(size_t)tile_base & 3u;  // the descriptor starts at the dword that holds the tile's first element
-        const CTile tile = c_tile(tile_base - base_mis);
+        const CTile tile = c_tile(p, m0, n0, 1u << sh, base_mis);
         const unsigned row_bytes = (unsigned)p.c_rs << sh;
         const unsigned lane_off = base_mis + (unsigned)row_in_tile * row_bytes + ((unsigned)col_in_tile << sh);
 #pragma unroll
@@ -721,7 +726,7 @@ __global__ void __launch_bounds__(Cfg::NT, Cfg::WGS_PER_CU) gemm_mfma_kernel(Gem
     auto stream_slab = [&](auto out_tag, const char* slab, int i) {
         constexpr int OS = sizeof(decltype(out_tag));
         const int wave_u = __builtin_amdgcn_readfirstlane(wave);
-        const CTile tile = c_tile((char*)p.C + ((int64_t)(m0 + (wave_u / WAVES_N) * WTM) * p.c_rs + n0 + (wave_u % WAVES_N) * WTN) * OS);
+        const CTile tile = c_tile(p, m0 + (wave_u / WAVES_N) * WTM, n0 + (wave_u % WAVES_N) * WTN, OS);
         const unsigned row_bytes = (unsigned)p.c_rs * OS;
         constexpr int CPRW = WTN * OS / 16;       // 16-byte pieces per row of the wave tile
         constexpr int PIECES = 32 * CPRW / 64;    // per lane and 32-row slab
@@ -836,6 +841,8 @@ template <typename Cfg>
 hipError_t launch_mfma(const GemmArgs& a, hipStream_t stream, LaunchGeom* geom, bool dry_run)
 {
     auto kern = gemm_mfma_kernel<Cfg>;
+    // an int8 C is written in 16-byte pieces of 16-byte aligned rows; no kernel here has a path for anything else
+    if (a.out_type == T_I8 && (a.c_rs % 16 || ((size_t)a.C & 15) || (a.batch > 1 && a.c_bs % 16))) return hipErrorInvalidValue;
     GemmArgs args = a;
     args.tiles_m = (a.M + Cfg::BM - 1) / Cfg::BM;
     args.tiles_n = (a.N + Cfg::BN - 1) / Cfg::BN;
@@ -848,12 +855,8 @@ hipError_t launch_mfma(const GemmArgs& a, hipStream_t stream, LaunchGeom* geom, 
         geom->dyn_lds = Cfg::LDS_BYTES;
     }
     if (dry_run) return hipSuccess;
-    static bool attr_set = false; // per instantiation; benign if set twice
-    if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES);
-        if (e != hipSuccess) return e;
-        attr_set = true;
-    }
+    static LdsLimitOnce lds_limit; // per instantiation
+    if (hipError_t e = lds_limit.ensure((const void*)kern, Cfg::LDS_BYTES); e != hipSuccess) return e;
     hipLaunchKernelGGL(kern, dim3(args.tiles_m * args.tiles_n, 1, a.batch > 1 ? a.batch : 1), dim3(Cfg::NT), Cfg::LDS_BYTES, stream, args);
     return hipGetLastError();
 }

@@ -237,7 +237,7 @@ __global__ void __launch_bounds__(Cfg::NT, 1) gemm_mfma16_kernel(GemmArgs p)
         auto fin4 = [&](const acc_t& v) { return acc_t{fin(v[0]), fin(v[1]), fin(v[2]), fin(v[3])}; };
     if (os == 4) {
         // one 16-byte store per block and lane
-        const CTile tile = c_tile((char*)p.C + ((int64_t)m0 * p.c_rs + n0) * 4);
+        const CTile tile = c_tile(p, m0, n0, 4);
         const unsigned row_bytes = (unsigned)p.c_rs * 4;
         const unsigned lane_off = (unsigned)lrow * row_bytes + (unsigned)lcol * 4;
 #pragma unroll
@@ -256,7 +256,7 @@ __global__ void __launch_bounds__(Cfg::NT, 1) gemm_mfma16_kernel(GemmArgs p)
             constexpr int PITCH = (ROW / 32) % 2 == 0 ? ROW + 32 : ROW; // an odd number of 32-byte units: rows spread over the banks
             static_assert(NT / 64 * 16 * PITCH <= Cfg::LDS_BYTES, "slabs fit the tile buffers");
             char* slab = smem + wave_u * (16 * PITCH);
-            const CTile tile = c_tile((char*)p.C + ((int64_t)(m0 + (wave_u / WAVES_N) * WTM) * p.c_rs + n0 + (wave_u % WAVES_N) * WTN) * OS);
+            const CTile tile = c_tile(p, m0 + (wave_u / WAVES_N) * WTM, n0 + (wave_u % WAVES_N) * WTN, OS);
             const unsigned row_bytes = (unsigned)p.c_rs * OS;
             constexpr int CPRW = ROW / 16;                    // 16-byte pieces per row of the wave tile
             constexpr int PIECES = (16 * CPRW + 63) / 64;     // per lane and 16-row slab
@@ -288,7 +288,7 @@ __global__ void __launch_bounds__(Cfg::NT, 1) gemm_mfma16_kernel(GemmArgs p)
         }
     } else {
         // rows of C that are not 16-byte aligned: single elements
-        const CTile tile = c_tile((char*)p.C + ((int64_t)m0 * p.c_rs + n0) * os);
+        const CTile tile = c_tile(p, m0, n0, os);
         const unsigned row_bytes = (unsigned)p.c_rs * os;
         const unsigned lane_off = (unsigned)lrow * row_bytes + (unsigned)lcol * os;
         auto by_element = [&](auto os_tag, auto&& pack) {
@@ -433,6 +433,8 @@ template <typename Cfg>
 hipError_t launch_mfma16(const GemmArgs& a, hipStream_t stream, LaunchGeom* geom, bool dry_run)
 {
     auto kern = gemm_mfma16_kernel<Cfg>;
+    // an int8 C is written in 16-byte pieces of 16-byte aligned rows; no kernel here has a path for anything else
+    if (a.out_type == T_I8 && (a.c_rs % 16 || ((size_t)a.C & 15) || (a.batch > 1 && a.c_bs % 16))) return hipErrorInvalidValue;
     GemmArgs args = a;
     args.tiles_m = (a.M + Cfg::BM - 1) / Cfg::BM;
     args.tiles_n = (a.N + Cfg::BN - 1) / Cfg::BN;
@@ -445,12 +447,8 @@ hipError_t launch_mfma16(const GemmArgs& a, hipStream_t stream, LaunchGeom* geom
         geom->dyn_lds = Cfg::LDS_BYTES;
     }
     if (dry_run) return hipSuccess;
-    static bool attr_set = false; // per instantiation; benign if set twice
-    if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES);
-        if (e != hipSuccess) return e;
-        attr_set = true;
-    }
+    static LdsLimitOnce lds_limit; // per instantiation
+    if (hipError_t e = lds_limit.ensure((const void*)kern, Cfg::LDS_BYTES); e != hipSuccess) return e;
     hipLaunchKernelGGL(kern, dim3(args.tiles_m * args.tiles_n, 1, a.batch > 1 ? a.batch : 1), dim3(Cfg::NT), Cfg::LDS_BYTES, stream, args);
     return hipGetLastError();
 }

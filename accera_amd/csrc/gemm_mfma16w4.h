@@ -188,7 +188,7 @@ __global__ void __launch_bounds__(256, 1) gemm_mfma16w4_kernel(GemmArgs p)
     const bool c_is_32bit = p.out_type == T_F32 || p.out_type == T_I32;
     const unsigned accum = __builtin_amdgcn_readfirstlane(
         p.prologue == PRO_SET ? (p.prologue_arg == 0.f ? 0u : 2u) : (p.prologue == PRO_NONE && c_is_32bit) ? 1u : 2u);
-    const CTile c_in = c_tile((char*)p.C + ((int64_t)m0 * p.c_rs + n0) * 4);
+    const CTile c_in = c_tile(p, m0, n0, 4);
     const unsigned c_off = (unsigned)(wr0 + (lane & 15)) * ((unsigned)p.c_rs * 4) + (unsigned)(wc0 + (lane >> 4) * 4) * 4;
     const unsigned c_row16 = __builtin_amdgcn_readfirstlane((unsigned)p.c_rs * 64);
     const auto c_rsrc = c_in.rsrc;
@@ -239,7 +239,7 @@ __global__ void __launch_bounds__(256, 1) gemm_mfma16w4_kernel(GemmArgs p)
             });
         } else {
             wait_vmcnt<0>();
-            const CTile c16 = c_tile((char*)p.C + ((int64_t)m0 * p.c_rs + n0) * 2);
+            const CTile c16 = c_tile(p, m0, n0, 2);
             const unsigned rb = (unsigned)p.c_rs * 2;
             const unsigned off16 = (unsigned)(wr0 + (lane & 15)) * rb + (unsigned)(wc0 + (lane >> 4) * 4) * 2;
             const unsigned m_f16 = p.out_type == T_F16 ? ~0u : 0u, m_bf16 = p.out_type == T_BF16 ? ~0u : 0u;
@@ -349,7 +349,7 @@ __global__ void __launch_bounds__(256, 1) gemm_mfma16w4_kernel(GemmArgs p)
             }
         };
         if (os == 4) {
-            const CTile tile = c_tile((char*)p.C + ((int64_t)m0 * p.c_rs + n0) * 4);
+            const CTile tile = c_tile(p, m0, n0, 4);
             const unsigned row_bytes = (unsigned)p.c_rs * 4;
             const unsigned lane_off = (unsigned)lrow * row_bytes + (unsigned)lcol * 4;
             w4_static_for<0, TM>([&](auto i) {
@@ -383,7 +383,7 @@ __global__ void __launch_bounds__(256, 1) gemm_mfma16w4_kernel(GemmArgs p)
                 constexpr int PITCH = ROW + 16;
                 static_assert(ROW % 32 == 0, "(ROW / 16 + 1) must be odd for the 16 row starts to differ mod 64 banks");
                 char* slab = smem + wave_u * (16 * PITCH);
-                const CTile tile = c_tile((char*)p.C + ((int64_t)(m0 + (wave_u / WAVES_N) * WTM) * p.c_rs + n0 + (wave_u % WAVES_N) * WTN) * OS);
+                const CTile tile = c_tile(p, m0 + (wave_u / WAVES_N) * WTM, n0 + (wave_u % WAVES_N) * WTN, OS);
                 const unsigned row_bytes = (unsigned)p.c_rs * OS;
                 constexpr int CPRW = ROW / 16;
                 constexpr int PIECES = (16 * CPRW + 63) / 64;
@@ -457,6 +457,8 @@ template <typename Cfg>
 hipError_t launch_mfma16w4(const GemmArgs& a, hipStream_t stream, LaunchGeom* geom, bool dry_run)
 {
     auto kern = gemm_mfma16w4_kernel<Cfg>;
+    // an int8 C is written in 16-byte pieces of 16-byte aligned rows; no kernel here has a path for anything else
+    if (a.out_type == T_I8 && (a.c_rs % 16 || ((size_t)a.C & 15) || (a.batch > 1 && a.c_bs % 16))) return hipErrorInvalidValue;
     GemmArgs args = a;
     args.tiles_m = (a.M + Cfg::BM - 1) / Cfg::BM;
     args.tiles_n = (a.N + Cfg::BN - 1) / Cfg::BN;
@@ -469,12 +471,8 @@ hipError_t launch_mfma16w4(const GemmArgs& a, hipStream_t stream, LaunchGeom* ge
         geom->dyn_lds = Cfg::LDS_BYTES;
     }
     if (dry_run) return hipSuccess;
-    static bool attr_set = false;
-    if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES);
-        if (e != hipSuccess) return e;
-        attr_set = true;
-    }
+    static LdsLimitOnce lds_limit; // per instantiation
+    if (hipError_t e = lds_limit.ensure((const void*)kern, Cfg::LDS_BYTES); e != hipSuccess) return e;
     hipLaunchKernelGGL(kern, dim3(args.tiles_m * args.tiles_n, 1, a.batch > 1 ? a.batch : 1), dim3(Cfg::NT), Cfg::LDS_BYTES, stream, args);
     return hipGetLastError();
 }

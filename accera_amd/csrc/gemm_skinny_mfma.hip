@@ -309,12 +309,10 @@ hipError_t launch_one(const SkinnyArgs& a, hipStream_t stream, LaunchGeom* geom,
     }
     if (dry_run) return hipSuccess;
     if (lds > 160 * 1024) return hipErrorInvalidValue;
-    static bool attr_set = false;
-    if (lds > 64 * 1024 && !attr_set) {
-        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return e;
-        attr_set = true;
-    }
+    // (the LDS need grows with M and the ring depth, never past the instantiation's largest: ask for that once)
+    static LdsLimitOnce lds_limit;
+    if (lds > 64 * 1024)
+        if (hipError_t e = lds_limit.ensure((const void*)kern, 160 * 1024); e != hipSuccess) return e;
     hipLaunchKernelGGL(kern, grid, block, lds, stream, a);
     return hipGetLastError();
 }

@@ -1,11 +1,16 @@
 #!/usr/bin/env python3
 """Benchmark of the matmul + fused-ReLU hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c2] [--no-cpu] [--all]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c2] [--no-cpu] [--only] [--all]
 
 A "step" is one GEMM+ReLU launch on device-resident synthetic inputs.  The default
 workload is the configuration the headline metric is quoted on: fp16 inputs, fp32
-accumulate / output, M=N=K=4096, C = max(A.B, 0).  One JSON line is printed with
+accumulate / output, M=N=K=4096, C = max(A.B, 0).  The metric also names the int8 GEMM and
+the skinny decode GEMM, so the default run measures those two as well, the same way, and
+reports them under "other_configs", each with its own roofline block (`--only` leaves them
+out).  Before the W untimed warm-up steps of a configuration its kernel is launched for
+SETTLE_MS of wall time (reported as settle_ms): after idling the engine clock takes some tens
+of milliseconds of load to settle, whatever W is.  One JSON line is printed with
   value         whole-job TFLOP/s (2*M*N*K per step, the formula of the reference's
                 harness: /root/reference/tools/benchmarkers/accera_gemm.py:648-654)
   roofline      algorithmic FLOP (or bytes) per launch / average launch duration from
@@ -13,7 +18,7 @@ accumulate / output, M=N=K=4096, C = max(A.B, 0).  One JSON line is printed with
   cpu_baseline  the CPU oracle (a restatement of the reference's HOST schedule, not an
                 Accera-generated package) timed on this box's host cores
 
-`--all` adds the other four BASELINE configurations under "other_configs".
+`--all` measures all five BASELINE configurations.
 """
 import argparse
 import json
@@ -28,6 +33,7 @@ sys.path.insert(0, ROOT)
 
 PEAK = {"f16": 2500.0, "bf16": 2500.0, "i8": 5000.0, "f32": 157.3}  # dense MFMA TFLOP/s (TOP/s)
 HBM_PEAK_GBS = 8000.0
+SETTLE_MS = 150.0  # launches of the kernel under test before the counted warm-up, by wall time
 
 CONFIGS = {
     # name: in, out, M, N, K, B layout, bound
@@ -98,6 +104,15 @@ def run_gpu(c, steps, warmup, variant=-1, k_splits=0):
     def step(i):
         calls[i % n_sets]()
 
+    # clock settle by wall time, then the counted warm-up
+    t_settle = time.perf_counter()
+    n = 0
+    while (time.perf_counter() - t_settle) * 1e3 < SETTLE_MS:
+        for _ in range(32):
+            step(n)
+            n += 1
+        torch.cuda.synchronize()
+    run_gpu.settle_ms = round((time.perf_counter() - t_settle) * 1e3, 1)
     for i in range(warmup):
         step(i)
     torch.cuda.synchronize()
@@ -241,23 +256,36 @@ def measure(name, steps, warmup, variant=-1, k_splits=0):
         achieved, peak, unit = flops / launch_s / 1e12, PEAK[c["in_type"]], "TFLOP/s" if c["in_type"] != "i8" else "TOP/s"
         value, vunit = flops * steps / wall / 1e12, unit
     return dict(config=name, workload=c["workload"], value=round(value, 3), unit=vunit, ms_per_step=round(wall / steps * 1e3, 5),
+                steps=steps, warmup=warmup, settle_ms=run_gpu.settle_ms, rotating_input_sets=run_gpu.rotating_sets,
+                dtype={"f16": "f16", "bf16": "bf16", "i8": "int8", "f32": "f32"}[c["in_type"]],
+                kernel=_kernel_record(c),
                 roofline=dict(bound=c["bound"], achieved=round(achieved, 3), peak=peak, unit=unit,
                               frac=round(achieved / peak, 4), traffic=traffic_bytes(name)),
                 flops_per_launch=flops, bytes_per_launch=nbytes, in_kernel=in_kernel,
+                machine_ceiling=machine_ceiling(c),
                 vendor_library=vendor_library(c, first_set, steps))
+
+
+def _kernel_record(c):
+    """Name and launch geometry of the kernel the timed calls ran."""
+    from accera_amd import _lib
+    grid, block, lds, chosen = _lib.launch_geometry(
+        getattr(_lib, c["in_type"].upper()), getattr(_lib, c["out_type"].upper()), c["M"], c["N"], c["K"],
+        (c["K"], 1), (c["N"], 1) if c["b"] == "row" else (1, c["K"]), (c["N"], 1), *run_gpu.asked)
+    return {"name": _lib.variant_name(chosen), "grid": grid, "block": block, "dynamic_lds_bytes": lds}
 
 
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=500)
-    ap.add_argument("--warmup", type=int, default=500,
-                    help="untimed steps; the engine clock takes some tens of ms of load to settle after idle")
+    ap.add_argument("--warmup", type=int, default=50, help="untimed steps (after the time-based clock settle)")
     ap.add_argument("--config", default="c2", choices=sorted(CONFIGS))
     ap.add_argument("--variant", type=int, default=-1)
     ap.add_argument("--k-splits", type=int, default=0)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--all", action="store_true", help="also measure the other BASELINE configurations")
+    ap.add_argument("--only", action="store_true", help="measure --config alone (default: c4 and c5 ride along with c2)")
+    ap.add_argument("--all", action="store_true", help="measure all five BASELINE configurations")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs on ONE GPU only (no collectives, no sharding); run with --gpus 1", file=sys.stderr)
@@ -277,20 +305,18 @@ def main():
     torch.cuda.synchronize()
     del probe
     m = measure(args.config, args.steps, args.warmup, args.variant, args.k_splits)
-    grid, block, lds, chosen = _lib.launch_geometry(
-        getattr(_lib, c["in_type"].upper()), getattr(_lib, c["out_type"].upper()), c["M"], c["N"], c["K"],
-        (c["K"], 1), (c["N"], 1) if c["b"] == "row" else (1, c["K"]), (c["N"], 1), *run_gpu.asked)
     out = {
         "metric": "GEMM+ReLU TFLOP/s (TOPS int8) & % MFMA peak at 4096^3 fp16; skinny GEMM HBM GB/s",
-        "value": m["value"], "unit": m["unit"], "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "value": m["value"], "unit": m["unit"], "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "settle_ms": m["settle_ms"],
         "ms_per_step": m["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": {"f16": "f16", "bf16": "bf16", "i8": "int8", "f32": "f32"}[c["in_type"]], "data": "synthetic",
-        "config": {"workload": c["workload"], "M": c["M"], "N": c["N"], "K": c["K"], "kernel": _lib.variant_name(chosen),
-                   "grid": grid, "block": block, "dynamic_lds_bytes": lds, "device": torch.cuda.get_device_name(0),
+        "dtype": m["dtype"], "data": "synthetic",
+        "config": {"workload": c["workload"], "M": c["M"], "N": c["N"], "K": c["K"], "kernel": m["kernel"]["name"],
+                   "grid": m["kernel"]["grid"], "block": m["kernel"]["block"], "dynamic_lds_bytes": m["kernel"]["dynamic_lds_bytes"],
+                   "device": torch.cuda.get_device_name(0),
                    "arch": torch.cuda.get_device_properties(0).gcnArchName,
                    "compute_units": torch.cuda.get_device_properties(0).multi_processor_count},
         "roofline": m["roofline"],
-        "machine_ceiling": machine_ceiling(c),
+        "machine_ceiling": m["machine_ceiling"],
         "in_kernel": m["in_kernel"],
         "vendor_library": m["vendor_library"],
     }
@@ -299,9 +325,11 @@ def main():
         # bounded sample: about 10-30 s of single-core work spread over the host cores
         rows = {"c2": None, "c4": 2048, "c3": None, "c1": None, "c5": None}[args.config]
         out["cpu_baseline"] = cpu_baseline(c, threads, rows)
-    if args.all:
-        out["other_configs"] = [measure(n, max(20, args.steps // 4) if n == "c4" else args.steps, args.warmup)
-                                for n in sorted(CONFIGS) if n != args.config]
+    # the rest of the metric: int8 GEMM (TOP/s against the int8 MFMA peak) and the skinny decode GEMM (HBM GB/s)
+    others = [n for n in sorted(CONFIGS) if n != args.config] if args.all else \
+        ([] if args.only or args.variant >= 0 or args.k_splits else [n for n in ("c4", "c5") if n != args.config])
+    if others:
+        out["other_configs"] = [measure(n, args.steps, args.warmup) for n in others]
     print(json.dumps(out), flush=True)
 
 

@@ -11,8 +11,8 @@ from accera_amd import _lib
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
-def _declared():
-    text = open(os.path.join(ROOT, "include", "accera_mi355x_gemm.h")).read()
+def _declared(header="accera_mi355x_gemm.h"):
+    text = open(os.path.join(ROOT, "include", header)).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(acc950_\w+)\s*\(", text)))
 
@@ -21,7 +21,9 @@ def test_every_declared_symbol_is_exported():
     names = _declared()
     assert len(names) >= 9 and set(_lib.EXPORTS) == set(names)
     L = ctypes.CDLL(_lib.LIB_PATH)
-    for n in names:
+    probes = _declared("accera_mi355x_probes.h")
+    assert set(_lib.PROBE_EXPORTS) == set(probes) and not set(probes) & set(names)
+    for n in names + probes:
         assert getattr(L, n) is not None, n
 
 
