@@ -19,13 +19,13 @@ OK, INVALID_ARGUMENT, UNSUPPORTED, HIP_ERROR = 0, 1, 2, 3
 VARIANT_AUTO, VARIANT_SKINNY_BASE, VARIANT_GENERIC, VARIANT_F32_MFMA = -1, 100, 200, 201
 
 EXPORTS = [
-    "acc950_init", "acc950_gemm_relu", "acc950_gemm_relu_ex", "acc950_gemm_relu_host", "acc950_gemm_ops", "acc950_gemm_ops_host",
+    "acc950_init", "acc950_gemm_relu", "acc950_gemm_relu_ex", "acc950_gemm_relu_host", "acc950_gemm_ops", "acc950_gemm_ops_host", "acc950_gemm_ops_static",
     "acc950_gemm_batched", "acc950_gemm_batched_host", "acc950_bind", "acc950_launch", "acc950_unbind",
     "acc950_launch_geometry", "acc950_num_variants", "acc950_num_skinny_variants",
     "acc950_variant_name", "acc950_last_error",
 ]
 # measurement aids (include/accera_mi355x_probes.h): not part of the product ABI
-PROBE_EXPORTS = ["acc950_mfma_ceiling", "acc950_mfma_phase_probe", "acc950_copy_probe", "acc950_stream_read_probe", "acc950_workspace_probe"]
+PROBE_EXPORTS = ["acc950_mfma_ceiling", "acc950_mfma_phase_probe", "acc950_copy_probe", "acc950_stream_read_probe", "acc950_workspace_probe", "acc950_allocation_probe"]
 
 
 class Acc950Error(RuntimeError):
@@ -55,6 +55,7 @@ def lib():
     L.acc950_gemm_relu_host.argtypes = [ci, ci, ci, ci, ci] + mat * 3 + [ci, ci]
     cd = ctypes.c_double
     L.acc950_gemm_ops.argtypes = [ci, ci, ci, ci, ci] + mat * 3 + [ci, cd, ci, cd, ci, ci, vp]
+    L.acc950_gemm_ops_static.argtypes = L.acc950_gemm_ops.argtypes
     L.acc950_gemm_ops_host.argtypes = [ci, ci, ci, ci, ci] + mat * 3 + [ci, cd, ci, cd]
     bmat = [vp, i64, i64, i64]
     L.acc950_gemm_batched.argtypes = [ci, ci, ci, ci, ci, ci] + bmat * 3 + [ci, cd, ci, cd, ci, ci, vp]
@@ -69,6 +70,7 @@ def lib():
     L.acc950_mfma_phase_probe.argtypes = [ci, ci, ci, ci, ci, vp, vp, vp, ctypes.POINTER(ctypes.c_double)]
     L.acc950_copy_probe.argtypes = [vp, vp, ctypes.c_size_t, vp]
     L.acc950_stream_read_probe.argtypes = [vp, ctypes.c_size_t, vp, vp]
+    L.acc950_allocation_probe.argtypes = [ctypes.POINTER(ctypes.c_ulonglong)]
     L.acc950_workspace_probe.argtypes = [vp, ctypes.POINTER(vp), ctypes.POINTER(vp)]
     L.acc950_last_error.restype = ctypes.c_char_p
     for name in EXPORTS + PROBE_EXPORTS:
@@ -98,6 +100,13 @@ def mfma_ceiling(in_type, data_mode=2, iters=20000):
     t, g = ctypes.c_double(), ctypes.c_double()
     check(lib().acc950_mfma_ceiling(in_type, data_mode, iters, ctypes.byref(t), ctypes.byref(g)))
     return t.value, g.value
+
+
+def allocation_probe():
+    """Device allocations made by the GEMM entry points of this process so far."""
+    n = ctypes.c_ulonglong()
+    check(lib().acc950_allocation_probe(ctypes.byref(n)))
+    return n.value
 
 
 def workspace_probe(stream):

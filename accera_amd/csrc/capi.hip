@@ -7,6 +7,7 @@
 #include <vector>
 #include "variants.h"
 
+#include <atomic>
 #include <cstdio>
 #include <cstring>
 #include <map>
@@ -197,6 +198,7 @@ struct Workspace {
 };
 std::mutex g_ws_mutex;
 std::map<std::pair<int, hipStream_t>, Workspace> g_ws;
+std::atomic<unsigned long long> g_device_allocations{0}; // hipMalloc calls made by the GEMM entry points (acc950_allocation_probe)
 
 hipError_t workspace_for(hipStream_t stream, size_t floats, size_t counters, float** scratch, unsigned** cnt)
 {
@@ -210,6 +212,7 @@ hipError_t workspace_for(hipStream_t stream, size_t floats, size_t counters, flo
         float* p = nullptr;
         e = hipMalloc((void**)&p, want * sizeof(float));
         if (e != hipSuccess) return e;
+        ++g_device_allocations;
         w.scratch = p; // (the block it replaces is left to earlier launches)
         w.floats = want;
     }
@@ -218,6 +221,7 @@ hipError_t workspace_for(hipStream_t stream, size_t floats, size_t counters, flo
         unsigned* p = nullptr;
         e = hipMalloc((void**)&p, want * sizeof(unsigned));
         if (e != hipSuccess) return e;
+        ++g_device_allocations;
         e = hipMemset(p, 0, want * sizeof(unsigned));
         if (e != hipSuccess) { (void)hipFree(p); return e; }
         w.counters = p;
@@ -225,6 +229,35 @@ hipError_t workspace_for(hipStream_t stream, size_t floats, size_t counters, flo
     }
     *scratch = w.scratch;
     *cnt = w.counters;
+    return hipSuccess;
+}
+
+// ---- the workspace that is never allocated (acc950_gemm_ops_static) ------------------------
+// Lives in the library's own device image: kStaticFloats partial sums followed by kStaticCounters arrival counters.
+// Zero when the image is loaded; the kernels leave the counters zero.  Every GPU holds its own copy at its own
+// address, looked up once per device.
+constexpr size_t kStaticFloats = ACC950_STATIC_WORKSPACE_BYTES / sizeof(float) - 4096;
+constexpr size_t kStaticCounters = 4096;
+static __device__ __align__(256) float scratch[kStaticFloats + kStaticCounters];
+constexpr int kMaxDevices = 64;
+std::mutex g_static_mutex;
+float* g_static_ptr[kMaxDevices] = {};
+
+// Device address of `scratch` on the current device (the array's name is only a host-side handle).
+hipError_t static_workspace(float** ptr)
+{
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
+    std::lock_guard<std::mutex> lock(g_static_mutex);
+    if (!g_static_ptr[dev]) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return e;
+        g_static_ptr[dev] = (float*)p;
+    }
+    *ptr = g_static_ptr[dev];
     return hipSuccess;
 }
 
@@ -330,7 +363,8 @@ int choose(const Problem& pb, int variant, int k_splits, Choice* c)
     return ACC950_OK;
 }
 
-int run(const Problem& pb, const Choice& c, hipStream_t stream, LaunchGeom* geom, bool dry_run)
+// static_ws: the K-split workspace is the one in the library's own device image; nothing is allocated
+int run(const Problem& pb, const Choice& c, hipStream_t stream, LaunchGeom* geom, bool dry_run, bool static_ws = false)
 {
     const GemmArgs& g = pb.g;
     if (g.M == 0 || g.N == 0) {
@@ -366,8 +400,20 @@ int run(const Problem& pb, const Choice& c, hipStream_t stream, LaunchGeom* geom
             s.scratch_bs = (int64_t)skinny_scratch_floats(sv, g.N, ws_splits);
             s.counter_bs = skinny_column_blocks(sv, g.N);
             const size_t floats = nb * (size_t)s.scratch_bs, counters = nb * (size_t)s.counter_bs;
-            e = workspace_for(stream, floats, counters, &s.scratch, &s.counters);
-            if (e != hipSuccess) return fail_hip(e, "workspace allocation");
+            if (static_ws) {
+                if (floats > kStaticFloats || counters > kStaticCounters)
+                    return fail(ACC950_UNSUPPORTED, "this problem's K split needs " + std::to_string(floats * sizeof(float)) + " bytes of partial sums and " +
+                                std::to_string(counters) + " counters; the built-in workspace holds " + std::to_string(kStaticFloats * sizeof(float)) +
+                                " bytes and " + std::to_string(kStaticCounters) + " counters");
+                float* base = nullptr;
+                e = static_workspace(&base);
+                if (e != hipSuccess) return fail_hip(e, "address of the built-in workspace");
+                s.scratch = base;
+                s.counters = (unsigned*)(base + kStaticFloats);
+            } else {
+                e = workspace_for(stream, floats, counters, &s.scratch, &s.counters);
+                if (e != hipSuccess) return fail_hip(e, "workspace allocation");
+            }
         }
         e = launch_skinny(sv, s, stream, geom, dry_run);
     } else {
@@ -391,7 +437,7 @@ hipError_t reserve(DevBuf& b, size_t bytes)
     if (bytes <= b.bytes) return hipSuccess;
     if (b.p) { hipError_t e = hipFree(b.p); if (e != hipSuccess) return e; b.p = nullptr; b.bytes = 0; }
     hipError_t e = hipMalloc(&b.p, bytes);
-    if (e == hipSuccess) b.bytes = bytes;
+    if (e == hipSuccess) { b.bytes = bytes; ++g_device_allocations; }
     return e;
 }
 
@@ -416,6 +462,9 @@ int acc950_init(int device_id)
     if (e != hipSuccess) return fail_hip(e, "hipGetDeviceProperties");
     if (std::strncmp(prop.gcnArchName, "gfx950", 6) != 0)
         return fail(ACC950_UNSUPPORTED, std::string("this library is built for gfx950 only, device is ") + prop.gcnArchName);
+    float* ws = nullptr; // this device's copy of the built-in workspace, so that acc950_gemm_ops_static need not look it up
+    e = static_workspace(&ws);
+    if (e != hipSuccess) return fail_hip(e, "address of the built-in workspace");
     return ACC950_OK;
 }
 
@@ -432,6 +481,21 @@ int acc950_gemm_ops(int in_type, int out_type, int M, int N, int K,
     rc = choose(pb, variant, k_splits, &c);
     if (rc) return rc;
     return run(pb, c, (hipStream_t)stream, nullptr, false);
+}
+
+int acc950_gemm_ops_static(int in_type, int out_type, int M, int N, int K,
+                           const void* A, int64_t a_rs, int64_t a_cs, const void* B, int64_t b_rs, int64_t b_cs,
+                           void* C, int64_t c_rs, int64_t c_cs, int prologue, double prologue_arg, int epilogue, double epilogue_arg,
+                           int variant, int k_splits, void* stream)
+{
+    Problem pb;
+    int rc = make_problem(in_type, out_type, M, N, K, A, a_rs, a_cs, B, b_rs, b_cs, C, c_rs, c_cs, prologue, epilogue, true, &pb,
+                          prologue_arg, epilogue_arg);
+    if (rc) return rc;
+    Choice c;
+    rc = choose(pb, variant, k_splits, &c);
+    if (rc) return rc;
+    return run(pb, c, (hipStream_t)stream, nullptr, false, true);
 }
 
 int acc950_gemm_batched(int in_type, int out_type, int batch, int M, int N, int K,
@@ -519,6 +583,13 @@ int acc950_gemm_relu(int in_type, int out_type, int M, int N, int K,
 {
     return acc950_gemm_relu_ex(in_type, out_type, M, N, K, A, a_rs, a_cs, B, b_rs, b_cs, C, c_rs, c_cs, prologue, epilogue,
                                ACC950_VARIANT_AUTO, 0, stream);
+}
+
+int acc950_allocation_probe(unsigned long long* count)
+{
+    if (!count) return fail(ACC950_INVALID_ARGUMENT, "null output");
+    *count = g_device_allocations.load();
+    return ACC950_OK;
 }
 
 int acc950_workspace_probe(void* stream, void** partial_sums, void** counters)

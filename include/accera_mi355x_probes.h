@@ -53,6 +53,11 @@ int acc950_stream_read_probe(const void* src, size_t bytes, void* scratch4, void
  */
 int acc950_workspace_probe(void* stream, void** partial_sums, void** counters);
 
+/* Number of device allocations (hipMalloc) the GEMM entry points of this process have made so far: K-split
+ * workspaces and the device buffers of the host-pointer path.  A test of an entry point that must not allocate
+ * reads it before and after. */
+int acc950_allocation_probe(unsigned long long* count);
+
 #if defined(__cplusplus)
 }
 #endif

@@ -1,0 +1,58 @@
+"""The entry point that allocates nothing (acc950_gemm_ops_static) against acc950_gemm_ops: same kernels, the K-split
+workspace in the library's own device image instead of a per-stream allocation.  Two calls in a row, the second on
+a smaller problem, both bit-identical to the allocating entry point and within tolerance of the CPU oracle."""
+import numpy as np
+import pytest
+
+import oracle as ora
+from tests.util import assert_matches, make_input, out_zeros, to_device, to_host
+
+pytestmark = pytest.mark.gpu
+
+
+def _call(entry, dA, dB, dC, M, N, K, k_splits, stream):
+    from accera_amd import _lib
+    return entry(_lib.F16, _lib.F16, M, N, K, dA.data_ptr(), K, 1, dB.data_ptr(), N, 1, dC.data_ptr(), N, 1,
+                 _lib.PROLOGUE_SET0, 0.0, _lib.EPILOGUE_RELU, 0.0, _lib.VARIANT_AUTO, k_splits, stream)
+
+
+def test_static_workspace_entry_point_matches_the_allocating_one():
+    import torch
+    from accera_amd import _lib
+    L = _lib.lib()
+    _lib.check(L.acc950_init(0))
+    stream = torch.cuda.current_stream().cuda_stream
+    rng = np.random.default_rng(2024)
+    # decode shape first (its slow-phase column blocks are shared by two workgroups each: 2.7 MiB of partial sums),
+    # then a smaller problem with an explicit K split over four workgroups per column block
+    cases = [(8, 11008, 4096, 0), (4, 2048, 1024, 4)]
+    data = []
+    for M, N, K, ks in cases:
+        A = make_input(rng, (M, K), "f16", "normal")
+        B = (make_input(rng, (K, N), "f16", "normal").astype(np.float32) * 0.05).astype(np.float16)
+        dA, dB = to_device(A, "f16"), to_device(B, "f16")
+        d_ref, d_new = to_device(np.full((M, N), 7, np.float16), "f16"), to_device(np.full((M, N), 9, np.float16), "f16")
+        _lib.check(_call(L.acc950_gemm_ops, dA, dB, d_ref, M, N, K, ks, stream))
+        data.append((A, B, dA, dB, d_ref, d_new))
+    torch.cuda.synchronize()
+    allocations_before = _lib.allocation_probe()
+    assert allocations_before >= 2  # the allocating entry point made this stream's workspace
+    for rep in range(2):  # the pair of calls twice: the second round finds the array as the first left it
+        for (M, N, K, ks), (A, B, dA, dB, d_ref, d_new) in zip(cases, data):
+            d_new.fill_(9)
+            _lib.check(_call(L.acc950_gemm_ops_static, dA, dB, d_new, M, N, K, ks, stream))
+    torch.cuda.synchronize()
+    assert _lib.allocation_probe() == allocations_before, "the static entry point must not allocate device memory"
+    for (M, N, K, ks), (A, B, dA, dB, d_ref, d_new) in zip(cases, data):
+        got, ref = to_host(d_new, "f16"), to_host(d_ref, "f16")
+        assert np.array_equal(got.view(np.uint16), ref.view(np.uint16)), (M, N, K)
+        want = ora.gemm_relu_exact(A, B, out_zeros(M, N, "f16"), "f16", "f16", ora.PRO_SET0, ora.EPI_RELU)
+        assert_matches(got, want, "f16", K)
+        assert (got == 0).any() and (got > 0).any()
+    # a K split whose partial sums do not fit the array is refused, nothing runs
+    (M, N, K, _), (A, B, dA, dB, d_ref, d_new) = cases[0], data[0]
+    d_new.fill_(9)
+    rc = _call(L.acc950_gemm_ops_static, dA, dB, d_new, M, N, K, 8, stream)
+    assert rc == _lib.UNSUPPORTED and b"built-in workspace" in L.acc950_last_error()
+    torch.cuda.synchronize()
+    assert (to_host(d_new, "f16") == 9).all()
