@@ -309,7 +309,8 @@ int auto_mfma_variant(const Problem& pb)
         if (v.mi16) rank += lean ? 4 : -8;
         // four waves with 128x128 wave tiles: measured 3-9 % faster than the eight-wave form on large problems
         // (a third less LDS traffic, and the part is at its power limit there)
-        if (v.w4) rank = 13;
+        // (walking several tiles per workgroup pays when there is more than one round of tiles over the CUs)
+        if (v.w4) rank = v.persist ? (tiles > kComputeUnits ? 14 : 12) : 13;
         const bool better = best < 0 || cost < best_cost * 0.999 ||
                             (cost <= best_cost * 1.001 && ((int64_t)v.bm * v.bn > (int64_t)tab[best].bm * tab[best].bn ||
                                                            ((int64_t)v.bm * v.bn == (int64_t)tab[best].bm * tab[best].bn && rank > best_rank)));
@@ -610,7 +611,7 @@ int acc950_mfma_phase_probe(int in_type, int out_type, int M, int N, int K, cons
     Problem pb;
     int rc = make_problem(in_type, out_type, M, N, K, A, K, 1, B, N, 1, C, N, 1, PRO_SET0, EPI_RELU, true, &pb);
     if (rc) return rc;
-    const MfmaVariant probe = {256, 256, 2, 4, true, false, true, false, 64, 4, true, false, false, nullptr, nullptr};
+    const MfmaVariant probe = {256, 256, 2, 4, true, false, true, false, 64, 4, true, false, false, false, nullptr, nullptr};
     int n_unused = 0;
     if (M < 256 || N < 256 || K < 1 || !mfma_table(pb.g.in_type, &n_unused) || !mfma_can_take(probe, pb))
         return fail(ACC950_UNSUPPORTED, "the phase probe runs the 256x256 kernels: 8/16-bit inputs, dense row-major A, B, C, M and N multiples of 256, K of 64 bytes");
@@ -759,7 +760,7 @@ int acc950_variant_name(int variant, char* buf, size_t buf_len)
     const MfmaVariant& v = tab[variant];
     std::snprintf(buf, buf_len, "mfma %dx%d kb%d waves %dx%d %sB=%s fill=%s stages=%d%s%s%s", v.bm, v.bn, v.kb, v.waves_m, v.waves_n,
                   v.a_kc ? "" : "A=col-major ", v.b_kc ? "col-major" : "row-major", v.direct ? "direct" : "registers", v.stages,
-                  v.edge ? " edge" : "", v.pingpong ? " pingpong" : "", v.w4 ? " mi16 hand-laid loop" : v.mi16 ? " mi16" : "");
+                  v.edge ? " edge" : "", v.pingpong ? " pingpong" : "", v.w4 ? (v.persist ? " mi16 hand-laid loop multi-tile" : " mi16 hand-laid loop") : v.mi16 ? " mi16" : "");
     return ACC950_OK;
 }
 

@@ -26,12 +26,17 @@
 namespace acc950 {
 
 // BN: 256, or 192 (K-contiguous B only; N = 3072 = 16 x 192 gives one tile per CU) with 128x96 wave tiles
-template <int IN_, bool B_KC_, bool TIMED_ = false, int BN_ = 256>
+// PERSIST: one workgroup per CU walks several output tiles (grid = min(tiles, CUs)); the closing k-steps of a tile
+// fetch the first K tiles of the next one, and that tile's loop starts while this tile's stores are still on their way.
+template <int IN_, bool B_KC_, bool TIMED_ = false, int BN_ = 256, bool PERSIST_ = false>
 struct Mfma16W4Config {
-    static constexpr bool TIMED = TIMED_;
+    static constexpr bool TIMED = TIMED_, PERSIST = PERSIST_;
+    static_assert(!PERSIST_ || BN_ == 256, "the 192-wide tile is for problems of one tile per CU");
     static constexpr int IN = IN_, BM = 256, BN = BN_, WAVES_M = 2, WAVES_N = 2, KB = 64, STAGES = 4, NT = 256;
     static constexpr bool A_KC = true, B_KC = B_KC_;
-    static constexpr int LDS_BYTES = STAGES * (BM + BN) * KB;
+    // (a workgroup that walks several tiles stages its write-back behind the last LDS stage while the others already receive
+    // the next tile: it asks for the whole LDS of the CU)
+    static constexpr int LDS_BYTES = PERSIST_ ? 160 * 1024 : STAGES * (BM + BN) * KB;
     static_assert(BN == 256 || (BN == 192 && B_KC), "tile widths the loop is written for");
 };
 
@@ -96,13 +101,33 @@ __global__ void __launch_bounds__(256, 1) gemm_mfma16w4_kernel(GemmArgs p)
     };
     stamp(0);
 
-    int tile_m, tile_n;
-    tile_coords(blockIdx.x, p.tiles_m, p.tiles_n, tile_m, tile_n);
     // M and N need not be multiples of the tile: the last row / column of tiles ends at M / N and overlaps its
     // neighbour.  What both compute gets the same bits from both (the host allows this only when C is not read,
     // and only for N whose last tile still starts on a 16-byte boundary of B's and C's rows).
-    const int m0 = tile_m * BM + BM <= p.M ? tile_m * BM : p.M - BM;
-    const int n0 = tile_n * BN + BN <= p.N ? tile_n * BN : p.N - BN;
+    auto tile_origin = [&](int id, int& r0, int& c0) {
+        int tile_m, tile_n;
+        tile_coords(id, p.tiles_m, p.tiles_n, tile_m, tile_n);
+        r0 = tile_m * BM + BM <= p.M ? tile_m * BM : p.M - BM;
+        c0 = tile_n * BN + BN <= p.N ? tile_n * BN : p.N - BN;
+    };
+    // (a workgroup that walks several tiles takes ids blockIdx.x, blockIdx.x + gridDim.x, ...: in every round the
+    // workgroups of one XCD -- ids equal modulo 8 -- work on one compact rectangle of tiles, as when every tile has its own workgroup)
+    const int total_tiles = p.tiles_m * p.tiles_n;
+    if constexpr (Cfg::PERSIST) {
+        // Tiles take equal time, so workgroups that start together reach every write-back together, and all of C's
+        // bytes of a round then queue at the memory at once while the matrix cores wait.  Groups of workgroups (taken
+        // across the XCDs: ids / 8) start a little apart instead; the offsets last for the whole launch, and one
+        // group's stores drain while the others compute.  (A bounded wait on the constant 100 MHz counter.)
+        const unsigned grp = p.stagger_groups > 1 ? (blockIdx.x >> 3) % (unsigned)p.stagger_groups : 0u;
+        if (grp) {
+            const unsigned long long t0 = __builtin_amdgcn_s_memrealtime();
+            const unsigned long long wait = (unsigned long long)grp * (unsigned)p.stagger_ticks;
+            while (__builtin_amdgcn_s_memrealtime() - t0 < wait) __builtin_amdgcn_s_sleep(16);
+        }
+    }
+    int tile_id = blockIdx.x;
+    int m0, n0;
+    tile_origin(tile_id, m0, n0);
 
     const char* Ab = (const char*)p.A;
     const char* Bb = (const char*)p.B;
@@ -133,8 +158,10 @@ __global__ void __launch_bounds__(256, 1) gemm_mfma16w4_kernel(GemmArgs p)
     const unsigned db = __builtin_amdgcn_readfirstlane((unsigned)((B_KC ? 64 : B_RPP) * ldb * ES));
     const unsigned sa = KB;
     const unsigned sb = __builtin_amdgcn_readfirstlane(B_KC ? (unsigned)KB : (unsigned)(BK * ldb * ES));
-    const char* a_tile = Ab + (int64_t)m0 * lda * ES;
-    const char* b_tile = Bb + (B_KC ? (int64_t)n0 * ldb * ES : (int64_t)n0 * ES);
+    auto a_panel = [&](int r0) { return Ab + (int64_t)r0 * lda * ES; };
+    auto b_panel = [&](int c0) { return Bb + (B_KC ? (int64_t)c0 * ldb * ES : (int64_t)c0 * ES); };
+    const char* a_tile = a_panel(m0);
+    const char* b_tile = b_panel(n0);
     // The loop's last k-step runs at position 3 of its four-step pattern, so the first one starts at position
     // p0 = (4 - KT % 4) % 4: tile s goes to LDS stage (s + p0) % 4, and a partial first trip through the body
     // counts as one more trip.
@@ -144,20 +171,22 @@ __global__ void __launch_bounds__(256, 1) gemm_mfma16w4_kernel(GemmArgs p)
     // first k-step sits at an odd position; otherwise the loop's first step fetches tiles 2 and 3.
     constexpr bool B_PAIRED = B_KC && (BN == 192 || IN == IN_I8); // measured: behind the plain scheme for 16-bit inputs on 256-wide tiles
     const unsigned b_tiles_here = B_PAIRED ? 2u + (p0 & 1u) : 3u;
+    // the first three K tiles of an output tile, issued ahead of its loop
+    auto first_fills = [&](const char* a_src, const char* b_src) {
 #pragma unroll
-    for (int s = 0; s < 3; ++s) {
-        const unsigned stage = ldsb + ((s + p0) & 3) * STAGE_BYTES;
+        for (int s = 0; s < 3; ++s) {
+            const unsigned stage = ldsb + ((s + p0) & 3) * STAGE_BYTES;
 #pragma unroll
-        for (int f = 0; f < 4; ++f)
-            TA::direct_issue(stage + f * 4096, a_off, a_tile + (int64_t)s * sa + (int64_t)f * da);
-        if ((unsigned)s < b_tiles_here) {
+            for (int f = 0; f < 4; ++f)
+                TA::direct_issue(stage + f * 4096, a_off, a_src + (int64_t)s * sa + (int64_t)f * da);
+            if ((unsigned)s < b_tiles_here) {
 #pragma unroll
-            for (int f = 0; f < FILLS_B; ++f)
-                TB::direct_issue(stage + TA::TILE_BYTES + f * 4096, (f & 1) ? b_off1 : b_off0, b_tile + (int64_t)s * sb + (int64_t)f * db);
+                for (int f = 0; f < FILLS_B; ++f)
+                    TB::direct_issue(stage + TA::TILE_BYTES + f * 4096, (f & 1) ? b_off1 : b_off0, b_src + (int64_t)s * sb + (int64_t)f * db);
+            }
         }
-    }
-    const char* pa = a_tile + 3 * (int64_t)sa;
-    const char* pb = b_tile + (int64_t)b_tiles_here * sb;
+    };
+    first_fills(a_tile, b_tile);
     const unsigned groups = __builtin_amdgcn_readfirstlane((unsigned)(KT / 4 - 1 + (KT % 4 ? 1 : 0)));
 
     // ---- LDS addresses of the fragment reads (stage 0; the loop adds stage and block offsets)
@@ -188,9 +217,29 @@ __global__ void __launch_bounds__(256, 1) gemm_mfma16w4_kernel(GemmArgs p)
     const bool c_is_32bit = p.out_type == T_F32 || p.out_type == T_I32;
     const unsigned accum = __builtin_amdgcn_readfirstlane(
         p.prologue == PRO_SET ? (p.prologue_arg == 0.f ? 0u : 2u) : (p.prologue == PRO_NONE && c_is_32bit) ? 1u : 2u);
-    const CTile c_in = c_tile(p, m0, n0, 4);
     const unsigned c_off = (unsigned)(wr0 + (lane & 15)) * ((unsigned)p.c_rs * 4) + (unsigned)(wc0 + (lane >> 4) * 4) * 4;
     const unsigned c_row16 = __builtin_amdgcn_readfirstlane((unsigned)p.c_rs * 64);
+    const unsigned os = p.out_type == T_I8 ? 1 : (p.out_type == T_F32 || p.out_type == T_I32) ? 4 : 2;
+    // The closing k-steps of a tile can fetch for the next one when its K tile s belongs in LDS stage s (entry at
+    // position 0) and the loop has such closing steps (not the paired-fill loops).
+    constexpr bool TAIL_PREFETCH = Cfg::PERSIST && !B_PAIRED;
+    bool came_prefetched = false; // this tile's first three K tiles were issued by the previous tile's closing steps (before its stores)
+
+    // ---- one output tile per trip (a single trip unless the workgroup walks several tiles)
+    for (;;) {
+    const int next_id = tile_id + (int)gridDim.x;
+    const bool has_next = Cfg::PERSIST && next_id < total_tiles;
+    int m0_next = m0, n0_next = n0;
+    if (has_next) tile_origin(next_id, m0_next, n0_next);
+    const char* pa_n = a_panel(m0_next);
+    const char* pb_n = b_panel(n0_next);
+    const bool prefetch_next = TAIL_PREFETCH && has_next && p0 == 0;
+    // bit 0: the closing steps fetch the next tile's K tiles 0..2; bit 1: the first k-steps allow for the previous tile's
+    // stores (64 per thread with a 32-bit C) between this tile's fills
+    const unsigned flags = __builtin_amdgcn_readfirstlane((prefetch_next ? 1u : 0u) | (came_prefetched && os == 4 && groups >= 1 ? 2u : 0u));
+    const char* pa = a_tile + 3 * (int64_t)sa;
+    const char* pb = b_tile + (int64_t)b_tiles_here * sb;
+    const CTile c_in = c_tile(p, m0, n0, 4);
     const auto c_rsrc = c_in.rsrc;
 
     if (accum == 2) {
@@ -273,8 +322,17 @@ __global__ void __launch_bounds__(256, 1) gemm_mfma16w4_kernel(GemmArgs p)
         }
     }
 
-    wait_vmcnt<B_PAIRED ? 4 + FILLS : 2 * FILLS>(); // tile 0 has landed (tile 1 and tile 2 -- A's part of it at least -- in flight)
-    __syncthreads();
+    // K tile 0 has landed (tile 1 and tile 2 -- A's part of it at least -- may be in flight).  Memory operations complete in
+    // the order issued, so after closing steps that fetched ahead the previous tile's stores (issued after these fills:
+    // 64, 32 or 16 per thread for 4-, 2-, 1-byte elements of C) may be in flight as well.
+    if (!came_prefetched) wait_vmcnt<B_PAIRED ? 4 + FILLS : 2 * FILLS>();
+    else if (os == 4) wait_vmcnt<63>();
+    else if (os == 2) wait_vmcnt<2 * FILLS + 32>();
+    else wait_vmcnt<2 * FILLS + 16>();
+    // (the bare instruction: a fence would make the compiler wait for the previous tile's stores here)
+    __builtin_amdgcn_sched_barrier(0);
+    asm volatile("s_barrier" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
     stamp(1);
 
 #define ACC950_W4_OPERANDS                                                                                              \
@@ -282,7 +340,7 @@ __global__ void __launch_bounds__(256, 1) gemm_mfma16w4_kernel(GemmArgs p)
       [b_rd4] "v"(b_rd[4]), [b_rd5] "v"(b_rd[5]), [b_rd6] "v"(b_rd[6]), [b_rd7] "v"(b_rd[7]), [a_off] "v"(a_off),        \
       [b_off0] "v"(b_off0), [b_off1] "v"(b_off1), [pa] "s"(pa), [pb] "s"(pb), [da] "s"(da), [db] "s"(db), [sa] "s"(sa),   \
       [sb] "s"(sb), [ldsb] "s"(ldsb), [groups] "s"(groups), [accum] "s"(accum), [c_off] "v"(c_off), [p0] "s"(p0),       \
-      [c_rsrc] "s"(c_rsrc), [c_row16] "s"(c_row16)                                                                      \
+      [c_rsrc] "s"(c_rsrc), [c_row16] "s"(c_row16), [pa_n] "s"(pa_n), [pb_n] "s"(pb_n), [flags] "s"(flags)               \
     : "memory", "scc", "s72", "s73", "s74", "s75", "s76", "s77", "s78", "s79", "s80", "s81", ACC950_W4_V(10), ACC950_W4_V(11), \
       ACC950_W4_V(12), ACC950_W4_V(13), ACC950_W4_V(14), ACC950_W4_V(15), ACC950_W4_V(16), ACC950_W4_V(17),             \
       ACC950_W4_V(18), ACC950_W4_V(19), ACC950_W4_V(20), ACC950_W4_V(21), ACC950_W4_V(22), ACC950_W4_V(23),             \
@@ -299,6 +357,13 @@ __global__ void __launch_bounds__(256, 1) gemm_mfma16w4_kernel(GemmArgs p)
         if constexpr (IN == IN_F16) asm volatile(ACC950_W4_LOOP_KCP6("v_mfma_f32_16x16x32_f16") : ACC950_W4_OPERANDS);
         else if constexpr (IN == IN_BF16) asm volatile(ACC950_W4_LOOP_KCP6("v_mfma_f32_16x16x32_bf16") : ACC950_W4_OPERANDS);
         else asm volatile(ACC950_W4_LOOP_KCP6("v_mfma_i32_16x16x64_i8") : ACC950_W4_OPERANDS);
+    } else if constexpr (TAIL_PREFETCH && B_KC) {
+        if constexpr (IN == IN_F16) asm volatile(ACC950_W4_LOOP_KC_P("v_mfma_f32_16x16x32_f16") : ACC950_W4_OPERANDS);
+        else asm volatile(ACC950_W4_LOOP_KC_P("v_mfma_f32_16x16x32_bf16") : ACC950_W4_OPERANDS);
+    } else if constexpr (TAIL_PREFETCH) {
+        if constexpr (IN == IN_F16) asm volatile(ACC950_W4_LOOP_MC16_P("v_mfma_f32_16x16x32_f16") : ACC950_W4_OPERANDS);
+        else if constexpr (IN == IN_BF16) asm volatile(ACC950_W4_LOOP_MC16_P("v_mfma_f32_16x16x32_bf16") : ACC950_W4_OPERANDS);
+        else asm volatile(ACC950_W4_LOOP_MC8_P("v_mfma_i32_16x16x64_i8") : ACC950_W4_OPERANDS);
     } else if constexpr (B_KC) {
         if constexpr (IN == IN_F16) asm volatile(ACC950_W4_LOOP_KC("v_mfma_f32_16x16x32_f16") : ACC950_W4_OPERANDS);
         else if constexpr (IN == IN_BF16) asm volatile(ACC950_W4_LOOP_KC("v_mfma_f32_16x16x32_bf16") : ACC950_W4_OPERANDS);
@@ -316,11 +381,8 @@ __global__ void __launch_bounds__(256, 1) gemm_mfma16w4_kernel(GemmArgs p)
 
     // ---- write-back: block (i, j) leaves the AGPR file just before its store.  Lane l holds row
     // i*16 + l%16 and columns j*16 + (l/16)*4 .. +3 of the wave tile.
-    const int lrow = wr0 + (lane & 15), lcol = wc0 + (lane >> 4) * 4;
-    const unsigned os = p.out_type == T_I8 ? 1 : (p.out_type == T_F32 || p.out_type == T_I32) ? 4 : 2;
     const int wave_u = __builtin_amdgcn_readfirstlane(wave);
-    // One copy of the stores per epilogue (a uniform branch): with a single wave per SIMD the
-    // write-back is bound by instruction issue, so every instruction per block counts.
+    // One copy of the stores per epilogue (a uniform branch).
     // (epi_tag: 0 nothing, 1 ReLU, 2 the other epilogue ops, applied element by element from the call's arguments)
     auto write_back = [&](auto epi_tag) {
         constexpr int EPI = decltype(epi_tag)::value;
@@ -348,32 +410,11 @@ __global__ void __launch_bounds__(256, 1) gemm_mfma16w4_kernel(GemmArgs p)
                     for (int e = 0; e < 4; ++e) row[j][e] = apply_epilogue<scalar_t>(row[j][e], p.epilogue, p.epilogue_arg);
             }
         };
-        if (os == 4) {
-            const CTile tile = c_tile(p, m0, n0, 4);
-            const unsigned row_bytes = (unsigned)p.c_rs * 4;
-            const unsigned lane_off = (unsigned)lrow * row_bytes + (unsigned)lcol * 4;
-            w4_static_for<0, TM>([&](auto i) {
-                const unsigned soff = (unsigned)(i.value * 16) * row_bytes;
-                acc_t row[TN];
-                if constexpr (EPI != 0) load_row(i, row);
-                w4_static_for<0, TN>([&](auto j) {
-                    constexpr int n = i.value * TN + j.value;
-                    if constexpr (EPI != 0) {
-                        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, row[j.value]), tile.rsrc, lane_off + j.value * 64, soff, 0);
-                    } else {
-                        // no arithmetic on the way out: the store reads the accumulator registers themselves
-                        const unsigned vo = lane_off, so = soff; // (asm operands do not capture on their own)
-                        const auto rsrc = tile.rsrc;
-                        asm volatile("buffer_store_dwordx4 a[%3:%4], %0, %1, %2 offen offset:%5"
-                                     :
-                                     : "v"(vo), "s"(rsrc), "s"(so), "n"(n * 4), "n"(n * 4 + 3), "n"(j.value * 64)
-                                     : "memory");
-                    }
-                });
-            });
-        } else {
-            // narrow outputs: 16 rows of the wave tile are put together in a wave-private slab of the
-            // (now idle) tile buffers and leave as 16-byte pieces that cover whole rows
+        {
+            // 16 rows of the wave tile are put together in a wave-private slab of the (now idle) tile buffers and leave as
+            // 16-byte pieces that cover whole rows of the wave tile: a store instruction that writes 2 rows x 512 bytes (or
+            // whole rows of a narrow type) passes through a CU's memory pipeline more than twice as fast as one that writes
+            // the accumulator layout's 16 rows x 64 bytes (measured: 256 KB per CU in 2.4-2.9 us against 6.2-7.0 us)
             __syncthreads();
             auto staged = [&](auto os_tag, auto&& pack) {
                 constexpr int OS = decltype(os_tag)::value;
@@ -382,7 +423,10 @@ __global__ void __launch_bounds__(256, 1) gemm_mfma16w4_kernel(GemmArgs p)
                 // 8- or 4-byte pieces of 16 rows land on 64 different banks
                 constexpr int PITCH = ROW + 16;
                 static_assert(ROW % 32 == 0, "(ROW / 16 + 1) must be odd for the 16 row starts to differ mod 64 banks");
-                char* slab = smem + wave_u * (16 * PITCH);
+                // (a workgroup that walks several tiles keeps the slabs in stage 3, the stage of the last k-step: the others
+                // may already be receiving the next tile)
+                static_assert((Cfg::PERSIST ? 3 * STAGE_BYTES : 0) + 4 * 16 * PITCH <= Cfg::LDS_BYTES, "four slabs fit (behind the first three stages)");
+                char* slab = smem + (Cfg::PERSIST ? 3 * STAGE_BYTES : 0) + wave_u * (16 * PITCH);
                 const CTile tile = c_tile(p, m0 + (wave_u / WAVES_N) * WTM, n0 + (wave_u % WAVES_N) * WTN, OS);
                 const unsigned row_bytes = (unsigned)p.c_rs * OS;
                 constexpr int CPRW = ROW / 16;
@@ -427,7 +471,9 @@ __global__ void __launch_bounds__(256, 1) gemm_mfma16w4_kernel(GemmArgs p)
             auto pack_i8 = [](const acc_t& v) -> int {
                 return (int)(((unsigned)v[0] & 0xffu) | (((unsigned)v[1] & 0xffu) << 8) | (((unsigned)v[2] & 0xffu) << 16) | ((unsigned)v[3] << 24));
             };
-            if constexpr (IN == IN_I8) {
+            auto pack_32 = [](const acc_t& v) -> i32x4 { return __builtin_bit_cast(i32x4, v); };
+            if (os == 4) staged(std::integral_constant<int, 4>{}, pack_32);
+            else if constexpr (IN == IN_I8) {
                 if (os == 2) staged(std::integral_constant<int, 2>{}, pack_i16);
                 else staged(std::integral_constant<int, 1>{}, pack_i8);
             } else {
@@ -441,16 +487,33 @@ __global__ void __launch_bounds__(256, 1) gemm_mfma16w4_kernel(GemmArgs p)
     else write_back(std::integral_constant<int, 2>{});
 
     if constexpr (Cfg::TIMED) {
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // stores acknowledged
+        // four stamps per output tile: start (the first tile's includes its fills), loop entered, loop left, stores
+        // issued -- acknowledged too when the workgroup has one tile; one that walks on does not wait for them
+        if constexpr (!Cfg::PERSIST) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         stamp(3);
         if (threadIdx.x == 0 && p.stamps) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                p.stamps[(blockIdx.x * 4 + i) * 2] = stamp_clk[i];
-                p.stamps[(blockIdx.x * 4 + i) * 2 + 1] = stamp_ref[i];
+                p.stamps[(tile_id * 4 + i) * 2] = stamp_clk[i];
+                p.stamps[(tile_id * 4 + i) * 2 + 1] = stamp_ref[i];
             }
         }
+        stamp(0);
     }
+    if constexpr (!Cfg::PERSIST) break;
+    if (!has_next) break;
+    if (!prefetch_next) {
+        __syncthreads(); // every wave has read its last fragments (stage 3) and is done with its slab
+        first_fills(pa_n, pb_n);
+    }
+    came_prefetched = prefetch_next;
+    tile_id = next_id;
+    m0 = m0_next;
+    n0 = n0_next;
+    a_tile = pa_n;
+    b_tile = pb_n;
+    } // tiles
+
 }
 
 template <typename Cfg>
@@ -462,8 +525,18 @@ hipError_t launch_mfma16w4(const GemmArgs& a, hipStream_t stream, LaunchGeom* ge
     GemmArgs args = a;
     args.tiles_m = (a.M + Cfg::BM - 1) / Cfg::BM;
     args.tiles_n = (a.N + Cfg::BN - 1) / Cfg::BN;
+    // one workgroup per tile, or one per CU that walks the tiles id, id + grid, ... (the LDS of a CU holds one workgroup)
+    unsigned grid_x = (unsigned)(args.tiles_m * args.tiles_n);
+    if (Cfg::PERSIST && grid_x > (unsigned)kComputeUnits) grid_x = kComputeUnits;
+    args.stagger_groups = args.stagger_ticks = 0;
+    if (Cfg::PERSIST && args.tiles_m * args.tiles_n > kComputeUnits) {
+        // measured on int8 8192^3 (four rounds): four groups 3 us apart gain 0.5 %; eight groups, or more than about
+        // 10 us in all, lose several per cent (workgroups of an XCD then no longer share their panels in its L2)
+        args.stagger_groups = 4;
+        args.stagger_ticks = 300;
+    }
     if (geom) {
-        geom->grid[0] = (unsigned)(args.tiles_m * args.tiles_n);
+        geom->grid[0] = grid_x;
         geom->grid[1] = 1;
         geom->grid[2] = a.batch > 1 ? a.batch : 1;
         geom->block[0] = Cfg::NT;
@@ -473,7 +546,7 @@ hipError_t launch_mfma16w4(const GemmArgs& a, hipStream_t stream, LaunchGeom* ge
     if (dry_run) return hipSuccess;
     static LdsLimitOnce lds_limit; // per instantiation
     if (hipError_t e = lds_limit.ensure((const void*)kern, Cfg::LDS_BYTES); e != hipSuccess) return e;
-    hipLaunchKernelGGL(kern, dim3(args.tiles_m * args.tiles_n, 1, a.batch > 1 ? a.batch : 1), dim3(Cfg::NT), Cfg::LDS_BYTES, stream, args);
+    hipLaunchKernelGGL(kern, dim3(grid_x, 1, a.batch > 1 ? a.batch : 1), dim3(Cfg::NT), Cfg::LDS_BYTES, stream, args);
     return hipGetLastError();
 }
 

@@ -12,21 +12,24 @@
 namespace acc950 {
 
 #define VA(AKC, BM, BN, WM, WN, BKC, DIRECT, EDGE, KB, STAGES)                                         \
-    { BM, BN, WM, WN, AKC, BKC, DIRECT, EDGE, KB, STAGES, false, false, false,                         \
+    { BM, BN, WM, WN, AKC, BKC, DIRECT, EDGE, KB, STAGES, false, false, false, false,                  \
       &launch_mfma<MfmaConfig<ACC950_IN, BM, BN, WM, WN, AKC, BKC, DIRECT, EDGE, KB, STAGES>>, nullptr }
 #define VPA(AKC, BM, BN, WM, WN, BKC, KB, STAGES)                                                       \
-    { BM, BN, WM, WN, AKC, BKC, true, false, KB, STAGES, true, false, false,                           \
+    { BM, BN, WM, WN, AKC, BKC, true, false, KB, STAGES, true, false, false, false,                    \
       &launch_mfma<MfmaConfig<ACC950_IN, BM, BN, WM, WN, AKC, BKC, true, false, KB, STAGES, true>>, nullptr }
 // ping-pong on the 16x16 MFMA shapes
 #define V16(AKC, BM, BN, WM, WN, BKC, KB, STAGES)                                                       \
-    { BM, BN, WM, WN, AKC, BKC, true, false, KB, STAGES, true, true, false,                            \
+    { BM, BN, WM, WN, AKC, BKC, true, false, KB, STAGES, true, true, false, false,                     \
       &launch_mfma16<Mfma16Config<ACC950_IN, BM, BN, WM, WN, AKC, BKC, KB, STAGES, false>>,           \
       &launch_mfma16<Mfma16Config<ACC950_IN, BM, BN, WM, WN, AKC, BKC, KB, STAGES, true>> }
 // four waves, 128x128 wave tiles, hand-laid K loop
 #define V16W4(BKC) \
-    { 256, 256, 2, 2, true, BKC, true, false, 64, 4, false, true, true, &launch_mfma16w4<Mfma16W4Config<ACC950_IN, BKC>>, nullptr }
+    { 256, 256, 2, 2, true, BKC, true, false, 64, 4, false, true, true, false, &launch_mfma16w4<Mfma16W4Config<ACC950_IN, BKC>>, nullptr }
 #define V16W4_192 \
-    { 256, 192, 2, 2, true, true, true, false, 64, 4, false, true, true, &launch_mfma16w4<Mfma16W4Config<ACC950_IN, true, false, 192>>, nullptr }
+    { 256, 192, 2, 2, true, true, true, false, 64, 4, false, true, true, false, &launch_mfma16w4<Mfma16W4Config<ACC950_IN, true, false, 192>>, nullptr }
+// the same, one workgroup per CU walking several output tiles
+#define V16W4P(BKC) \
+    { 256, 256, 2, 2, true, BKC, true, false, 64, 4, false, true, true, true, &launch_mfma16w4<Mfma16W4Config<ACC950_IN, BKC, false, 256, true>>, nullptr }
 #define V(BM, BN, WM, WN, BKC, DIRECT, EDGE, KB, STAGES) VA(true, BM, BN, WM, WN, BKC, DIRECT, EDGE, KB, STAGES)
 #define VP(BM, BN, WM, WN, BKC, KB, STAGES) VPA(true, BM, BN, WM, WN, BKC, KB, STAGES)
 // column-major A (M contiguous; the "transA" shapes of the reference's sweep lists,
@@ -71,6 +74,8 @@ static const MfmaVariant kVariants[] = {
     V16W4(false),
     V16W4(true),
     V16W4_192,
+    V16W4P(false),
+    V16W4P(true),
 };
 #undef LAYOUT_AT
 #undef VA
@@ -78,6 +83,7 @@ static const MfmaVariant kVariants[] = {
 #undef V16
 #undef V16W4
 #undef V16W4_192
+#undef V16W4P
 #undef LAYOUT
 #undef V
 #undef VP
@@ -88,6 +94,8 @@ static const MfmaVariant kVariants[] = {
 hipError_t ACC950_TIMED_FN(const GemmArgs& a, hipStream_t stream, LaunchGeom* geom, bool dry_run)
 {
     constexpr int K4 = 4 * 64 / InTraits<ACC950_IN>::ES;
+    if (a.K >= K4 && (a.M / 256) * (a.N / 256) > kComputeUnits) // more than one round of tiles: the multi-tile form
+        return launch_mfma16w4<Mfma16W4Config<ACC950_IN, false, true, 256, true>>(a, stream, geom, dry_run);
     if (a.K >= K4) return launch_mfma16w4<Mfma16W4Config<ACC950_IN, false, true>>(a, stream, geom, dry_run);
     return launch_mfma16<Mfma16Config<ACC950_IN, 256, 256, 2, 4, true, false, 64, 4, false, true>>(a, stream, geom, dry_run);
 }

@@ -33,6 +33,7 @@ B_TILE = 16384     # B's tile follows A's (256 rows x 64 bytes) inside a stage
 FRAG = 1024        # 16 rows x 64 bytes (K-contiguous operand)
 TN = 8             # blocks of 16 columns per wave: 8 (256-wide tile) or 6 (192-wide, K-contiguous B only)
 STAGE = 32768      # A's tile + B's tile (2 * TN * 16 rows x 64 bytes)
+RELAX_STORES = 47  # stores per thread the relaxed first k-steps of a later tile count on (see loop(): 2 tiles' fills + 47 = 63)
 
 
 def set_width(tn):
@@ -194,7 +195,18 @@ def step(pos, do_fill, wait, last, b_layout):
     return out
 
 
-def loop(b_layout):
+def loop(b_layout, persist=False):
+    """persist: the loop of a workgroup that walks several output tiles.  Two bits of %[flags]:
+    bit 0  the closing steps go on fetching: the first three K tiles of the workgroup's NEXT output tile (from
+           %[pa_n] / %[pb_n]) go into the stages the closing steps leave behind, so that the workgroup finds them in LDS
+           (or on the way) after its write-back.  Only for an entry at position 0 (a number of k-steps that is a
+           multiple of four: tile s of the next output tile then belongs in stage s), not for the paired-fill scheme.
+    bit 1  the stores of the previous tile's write-back (at least RELAX_STORES per thread) were issued after the fills
+           of this tile's K tiles 1 and 2 and may still be in flight: the first four k-steps are a copy of the body
+           whose first two waits allow for them (memory operations complete in the order issued, so a wait count
+           that does not know of the stores would wait for nearly all of them).  Entry at position 0 and at least one
+           trip through the body (the copy counts as one)."""
+    assert not (persist and b_layout == "kcp")
     out = [line("s_mov_b64 s[72:73], %[pa]"), line("s_mov_b64 s[74:75], %[pb]"), line("s_mov_b32 s78, %[groups]"),
            line(f"v_add_u32 v104, {2 * STAGE}, %[a_rd]")]
     if b_layout in ("kc", "kcp"):
@@ -230,18 +242,37 @@ def loop(b_layout):
     out += first_reads(3) + [line("s_branch 7f"), line("11:")]
     out += first_reads(1) + [line("s_branch 5f"), line("12:")]
     out += first_reads(2) + [line("s_branch 6f"), line("10:")]
-    out += first_reads(0) + [line("s_cmp_eq_u32 s78, 0"), line("s_cbranch_scc1 2f"), line("1:")]
+    out += first_reads(0)
     per_tile = 4 + (2 * TN * FRAG) // 4096  # fill instructions per K tile and thread
     kc = b_layout == "kcp"
+    if persist:
+        # in flight, oldest first, at the wait of step 0: tile 1, tile 2, the stores, tile 3; at that of step 1: tile 2, the
+        # stores, tiles 3 and 4; from step 2 on the tile waited for is younger than the stores
+        relaxed = min(63, 2 * per_tile + RELAX_STORES)
+        out += [line("s_bitcmp1_b32 %[flags], 1"), line("s_cbranch_scc0 13f")]
+        out += step(0, True, relaxed, False, b_layout) + step(1, True, relaxed, False, b_layout)
+        out += step(2, True, 2 * per_tile, False, b_layout) + step(3, True, 2 * per_tile, False, b_layout)
+        out += [line("s_sub_u32 s78, s78, 1"), line("13:")]
+    out += [line("s_cmp_eq_u32 s78, 0"), line("s_cbranch_scc1 2f"), line("1:")]
     for pos in range(4):
         if pos:
             out.append(line(f"{4 + pos}:"))
         out += step(pos, True, kc_wait(pos, 3) if kc else 2 * per_tile, False, b_layout)
     out += [line("s_sub_u32 s78, s78, 1"), line("s_cmp_lg_u32 s78, 0"), line("s_cbranch_scc1 1b"), line("2:")]
     out += step(0, True, kc_wait(0, 3) if kc else 2 * per_tile, False, b_layout)
+    if persist:
+        # closing steps that go on fetching: the fill pointers move to the next output tile; waits as in the body
+        out += [line("s_bitcmp1_b32 %[flags], 0"), line("s_cbranch_scc0 8f"),
+                line("s_mov_b64 s[72:73], %[pa_n]"), line("s_mov_b64 s[74:75], %[pb_n]")]
+        out += step(1, True, 2 * per_tile, False, b_layout)
+        out += step(2, True, 2 * per_tile, False, b_layout)
+        out += step(3, True, 0, True, b_layout)
+        out += [line("s_branch 9f"), line("8:")]
     out += step(1, False, kc_wait(1, 2) if kc else per_tile, False, b_layout)
     out += step(2, False, 0, False, b_layout)
     out += step(3, False, 0, True, b_layout)
+    if persist:
+        out.append(line("9:"))
     out += [line("s_nop 15"), line("s_nop 15")]
     return out
 
@@ -255,6 +286,13 @@ def main():
         set_width(tn)
         body = loop(name)
         print(f"#define ACC950_W4_LOOP_{name.upper()}{'' if tn == 8 else tn}(MFMA) \\")
+        print(" \\\n".join("    " + s for s in body))
+        print()
+    # the same loops for a workgroup that walks several output tiles (closing steps that prefetch the next tile)
+    for name in ("kc", "mc16", "mc8"):
+        set_width(8)
+        body = loop(name, persist=True)
+        print(f"#define ACC950_W4_LOOP_{name.upper()}_P(MFMA) \\")
         print(" \\\n".join("    " + s for s in body))
         print()
 

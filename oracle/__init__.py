@@ -152,7 +152,12 @@ def gemm_relu_exact(A, B, C0, in_type, out_type, prologue=PRO_SET0, epilogue=EPI
     pre-narrowing values when ``narrow_out`` is False).
     """
     Aw, Bw = widen(A, in_type), widen(B, in_type)
-    S = Aw @ Bw
+    if in_type == "i8" and Aw.shape[1] * 2 ** 14 < 2 ** 52:
+        # int8 products are at most 2^14 in size, so every partial sum is an integer below 2^52 and the float64 product
+        # (a BLAS call, much faster than NumPy's int64 loop) is exact in whatever order it adds
+        S = (Aw.astype(np.float64) @ Bw.astype(np.float64)).astype(np.int64)
+    else:
+        S = Aw @ Bw
     if prologue == PRO_SET:
         S = S + _op_arg(prologue_arg, in_type)
     elif prologue == PRO_SCALE:

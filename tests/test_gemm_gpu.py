@@ -773,6 +773,57 @@ def test_random_problems_on_the_four_wave_kernel():
     assert ran >= 30, ran
 
 
+@pytest.mark.parametrize("in_type,out_type,b_layout,M,N,K,pro,epi", [
+    # 17 x 16 = 272 tiles of 256 x 256 over 256 workgroups: sixteen of them walk two tiles; K a multiple of four k-steps, so
+    # the closing steps of a tile fetch for the next one and (32-bit C) its first k-steps run with the stores in flight
+    ("i8", "i32", "row", 4352, 4096, 512, "set0", "relu"),
+    ("f16", "f32", "row", 4352, 4096, 256, "set0", "relu"),
+    ("bf16", "f32", "col", 4352, 4096, 384, "set0", "none"),
+    # narrow outputs: the slabs of the write-back live in the stage the next tile's fills leave alone
+    ("f16", "f16", "row", 4352, 4096, 256, "set0", "relu"),
+    ("i8", "i8", "row", 4352, 4096, 512, "set0", "relu"),
+    # a number of k-steps that is not a multiple of four: the next tile is fetched after the write-back
+    ("i8", "i32", "row", 4352, 4096, 448, "set0", "relu"),
+    ("bf16", "bf16", "row", 4352, 4096, 288, "set0", "relu"),
+    # ragged M and N, 18 x 17 = 306 tiles (not a multiple of the eight XCDs either)
+    ("f16", "f32", "row", 4400, 4112, 256, "set0", "relu"),
+    ("i8", "i32", "col", 4400, 4112, 512, "set0", "relu"),
+    # C is read: C += A*B straight into the accumulators (32-bit C), and widened / scaled by ordinary code
+    ("i8", "i32", "row", 4352, 4096, 512, "none", "relu"),
+    ("f16", "f16", "row", 4352, 4096, 256, "scale", "scale"),
+    # three rounds over the workgroups
+    ("i8", "i32", "row", 8192, 6144, 256, "set0", "relu"),
+])
+def test_four_wave_kernel_walking_several_tiles(in_type, out_type, b_layout, M, N, K, pro, epi):
+    """More tiles than compute units on the multi-tile form of the hand-laid kernel, named explicitly, and the automatic
+    choice takes it when the tiles make whole rounds over the compute units."""
+    import accera_amd as acc
+    import torch
+    from accera_amd import _lib
+    v = [v for v, n in _variants(b_layout) if "multi-tile" in n]
+    assert len(v) == 1
+    pro_op, pa = {"set0": (ora.PRO_SET0, 0.0), "none": (ora.PRO_NONE, 0.0), "scale": (ora.PRO_SCALE, 0.5)}[pro]
+    epi_op, ea = {"relu": (ora.EPI_RELU, 0.0), "none": (ora.EPI_NONE, 0.0), "scale": (ora.EPI_SCALE, 2.0)}[epi]
+    rng = np.random.default_rng(M + N + K)
+    A, B = make_input(rng, (M, K), in_type), make_input(rng, (K, N), in_type)
+    if b_layout == "col":
+        B = np.asfortranarray(B)
+    C0 = make_c0(rng, (M, N), out_type, scale=100)
+    dA, dB = to_device(A, in_type), to_device(B, in_type)
+    want = ora.gemm_relu_exact(A, B, C0, in_type, out_type, pro_op, epi_op, prologue_arg=pa, epilogue_arg=ea)
+    for variant in (v[0], -1):
+        dC = to_device(C0, out_type)
+        call = acc.GemmCall(dA, dB, dC, prologue=pro_op, prologue_arg=pa, epilogue=epi_op, epilogue_arg=ea, variant=variant)
+        call()
+        torch.cuda.synchronize()
+        assert_matches(to_host(dC, out_type), want, out_type, K)
+    grid, block, lds, chosen = _lib.launch_geometry(getattr(_lib, in_type.upper()), getattr(_lib, out_type.upper()), M, N, K, (K, 1),
+                                                    (N, 1) if b_layout == "row" else (1, K), (N, 1))
+    if (M // 256) * (N // 256) % 256 == 0 and M % 256 == 0 and N % 256 == 0:
+        # whole rounds of tiles over the compute units (with a nearly empty last round the cost model prefers smaller tiles)
+        assert "multi-tile" in _lib.variant_name(chosen) and grid == [256, 1, 1]
+
+
 def test_skinny_workspaces_are_per_stream():
     """Launches on different streams may overlap, so each stream has its own K-split partial sums and arrival
     counters; the decode shape (whose slow-phase column blocks are shared by two workgroups each) runs on two streams

@@ -187,17 +187,19 @@ def test_whole_loop_shape(layout, tn):
     assert ins[-2:] == ["s_nop 15", "s_nop 15"]
 
 
-def _run_fills(g, layout, tn, KT, b_tiles_before_loop):
+def _run_fills(g, layout, tn, KT, b_tiles_before_loop, persist=False, flags=0, stores_in_flight=0):
     """Executes the scalar side of the loop text for KT k-steps: follows the branches, keeps the fill pointers as
     numbers and records every global_load_lds as (operand, K tile, pass, LDS stage).  The code before the loop
     has issued A's tiles 0..2 and B's tiles 0..b_tiles_before_loop-1; pa / pb point at the next tiles."""
     g.set_width(tn)
-    ins = _text(g.loop(layout))
+    ins = _text(g.loop(layout, persist) if persist else g.loop(layout))
     DA, DB, SA, SB = 1 << 20, 1 << 21, 1 << 30, 1 << 34      # distinct powers of two: an address decodes uniquely
+    NEXT = 1 << 49                                            # marks the panels of the workgroup's next output tile
     p0 = (4 - KT % 4) % 4
     groups = KT // 4 - 1 + (1 if KT % 4 else 0)
     env = {"%[pa]": 3 * SA, "%[pb]": (1 << 50) + b_tiles_before_loop * SB, "%[groups]": groups, "%[p0]": p0, "%[accum]": 0,
-           "%[da]": DA, "%[db]": DB, "%[sa]": SA, "%[sb]": SB, "%[ldsb]": 0, "%[c_row16]": 0}
+           "%[da]": DA, "%[db]": DB, "%[sa]": SA, "%[sb]": SB, "%[ldsb]": 0, "%[c_row16]": 0,
+           "%[pa_n]": NEXT, "%[pb_n]": (1 << 50) + NEXT, "%[flags]": flags}
     labels = {}
     for n, i in enumerate(ins):
         if re.match(r"^\d+:$", i):
@@ -212,6 +214,8 @@ def _run_fills(g, layout, tn, KT, b_tiles_before_loop):
             issued += [("b", t, p) for p in range(nb_)]
     if b_tiles_before_loop > 3:
         issued += [("b", t, p) for t in range(3, b_tiles_before_loop) for p in range(nb_)]
+    # stores of the previous output tile's write-back, issued after these fills (a workgroup that walks several tiles)
+    issued += [("store", n, 0) for n in range(stores_in_flight)]
 
     def val(tok):
         tok = tok.strip()
@@ -252,8 +256,10 @@ def _run_fills(g, layout, tn, KT, b_tiles_before_loop):
             scc = int(val(a[0]) == val(a[1]))
         elif op == "s_cmp_lg_u32":
             scc = int(val(a[0]) != val(a[1]))
-        elif op in ("s_cbranch_scc1", "s_branch"):
-            if op == "s_branch" or scc:
+        elif op == "s_bitcmp1_b32":
+            scc = (val(a[0]) >> val(a[1])) & 1
+        elif op in ("s_cbranch_scc1", "s_cbranch_scc0", "s_branch"):
+            if op == "s_branch" or scc == (op == "s_cbranch_scc1"):
                 lab, way = a[0][:-1], a[0][-1]
                 cands = labels[lab]
                 pc = min(c for c in cands if c >= pc) if way == "f" else max(c for c in cands if c < pc)
@@ -261,8 +267,12 @@ def _run_fills(g, layout, tn, KT, b_tiles_before_loop):
             addr = pair(rest.split(",", 1)[1])
             operand = "b" if addr >> 50 else "a"       # (bit 50 marks B's address space in this model)
             addr &= (1 << 50) - 1
+            ahead = bool(addr & NEXT)                  # a fetch for the next output tile
+            addr &= NEXT - 1
             stride, delta = (SB, DB) if operand == "b" else (SA, DA)
             tile, within = divmod(addr, stride)
+            if ahead:
+                tile += KT                             # K tile s of the next output tile is numbered KT + s
             assert within % delta == 0
             stage, in_stage = divmod(m0, g.STAGE)
             assert in_stage == (g.B_TILE if operand == "b" else 0) + (within // delta) * 4096
@@ -298,3 +308,37 @@ def test_fill_addresses_over_a_whole_k_loop(layout, tn, KT):
     want = sorted([("a", t, p, (t + p0) % 4) for t in range(3, KT) for p in range(4)] +
                   [("b", t, p, (t + p0) % 4) for t in range(b_before, KT) for p in range(nb)])
     assert sorted(fills) == want
+
+
+@pytest.mark.parametrize("layout", ["kc", "mc16", "mc8"])
+@pytest.mark.parametrize("KT", [4, 8, 12, 128])
+@pytest.mark.parametrize("flags,stores", [(0, 0), (1, 0), (2, 64), (3, 64), (3, 47), (2, 500)])
+def test_loop_of_a_workgroup_that_walks_several_tiles(layout, KT, flags, stores):
+    """The loops with closing steps that fetch ahead (entry at position 0 only).  Bit 0 of the flags: the three
+    closing steps fill K tiles 0..2 of the next output tile into stages 0..2, nothing else changes.  Bit 1: the first four
+    k-steps are the copy whose waits allow for the previous tile's stores; the model keeps those stores in flight
+    between the fills of K tile 2 and those of K tile 3 and still finds every k-step's tile landed at its barrier
+    (memory operations complete in the order issued)."""
+    g = _gen()
+    if flags & 2 and KT < 8:
+        pytest.skip("the relaxed copy of the first four k-steps counts as one trip through the body: at least eight k-steps")
+    fills, steps, p0 = _run_fills(g, layout, 8, KT, 3, persist=True, flags=flags, stores_in_flight=stores)
+    assert steps == KT and p0 == 0
+    last = KT + 3 if flags & 1 else KT
+    want = sorted([(o, t, p, t % 4) for o in "ab" for t in range(3, last) for p in range(4)])
+    assert sorted(fills) == want
+    # the closing steps that fetch ahead are the body's steps: same text up to the waits and the missing last barrier
+    ins = _text(g.loop(layout, persist=True))
+    assert ins.count("s_bitcmp1_b32 %[flags], 0") == 1 and ins.count("s_bitcmp1_b32 %[flags], 1") == 1
+    assert sum(i.startswith("MFMA") for i in ins) == 64 * (4 + 4 + 1 + 3 + 3)   # relaxed copy, body, closing step 0, the two sets of closing steps
+    relaxed = [i for i in ins[ins.index("s_bitcmp1_b32 %[flags], 1"):ins.index("13:")] if i.startswith("s_waitcnt vmcnt")]
+    assert relaxed == ["s_waitcnt vmcnt(63)", "s_waitcnt vmcnt(63)", "s_waitcnt vmcnt(16)", "s_waitcnt vmcnt(16)"]
+    assert g.RELAX_STORES + 16 == 63
+
+
+def test_relaxed_first_steps_need_the_stores_they_count_on():
+    """The model notices a wait that is too loose: with fewer stores in flight than the relaxed copy counts on, the
+    tile of the second k-step is not known to have landed."""
+    g = _gen()
+    with pytest.raises(AssertionError):
+        _run_fills(g, "mc8", 8, 8, 3, persist=True, flags=2, stores_in_flight=40)
