@@ -26,6 +26,7 @@ pattern raises NotImplementedError.  `Package.build` emits `<name>.hat` + `<name
 """
 import enum
 import hashlib
+import re
 import os
 import subprocess
 
@@ -67,11 +68,13 @@ class MMAFragmentOp(enum.Enum):  # /root/reference/docs/Reference/enumerations/M
 
 
 class MMAShape(enum.Enum):
-    """Accepted for source compatibility (/root/reference/accera/ir/include/value/ValueMMAOp.h:27-49);
-    the gfx950 kernels always issue the 32x32 MFMA with 32 bytes of K per step."""
+    """The reference's shape names (/root/reference/accera/ir/include/value/ValueMMAOp.h:27-49) plus the gfx950 ones.
+    M x N x K is the product one matrix instruction forms, in elements.  Only the shapes in
+    Target.MI355X_TENSORCORE_INFO exist on this target; `plan.tensorize` refuses the others, and the shape it is given
+    selects the kernel family (16x16 or 32x32 instruction shapes)."""
     M64xN64xK1_B4 = 0
     M64xN64xK1_B2 = 1
-    M32xN32xK2_B1 = 2
+    M32xN32xK2_B1 = 2     # gfx950: v_mfma_f32_32x32x2_f32
     M16xN16xK4_B1 = 3
     M64xN64xK4_B4 = 4
     M64xN64xK4_B2 = 5
@@ -81,8 +84,18 @@ class MMAShape(enum.Enum):
     M64xN64xK2_B2 = 9
     M32xN32xK4_B1 = 10
     M16xN16xK8_B1 = 11
-    M32xN32xK16_B1 = 12   # gfx950 native: v_mfma_f32_32x32x16_{f16,bf16}
-    M32xN32xK32_B1 = 13   # gfx950 native: v_mfma_i32_32x32x32_i8
+    M32xN32xK16_B1 = 12   # gfx950: v_mfma_f32_32x32x16_{f16,bf16}
+    M32xN32xK32_B1 = 13   # gfx950: v_mfma_i32_32x32x32_i8
+    M16xN16xK32_B1 = 14   # gfx950: v_mfma_f32_16x16x32_{f16,bf16}
+    M16xN16xK64_B1 = 15   # gfx950: v_mfma_i32_16x16x64_i8
+    M32xN8xK16_B1 = 16
+    M8xN32xK16_B1 = 17
+
+    @property
+    def dims(self):
+        """(M, N, K) of the shape."""
+        m, n, k = self.name.split("_")[0].split("x")
+        return int(m[1:]), int(n[1:]), int(k[1:])
 
 
 class MMASchedulingPolicy(enum.Enum):
@@ -101,6 +114,40 @@ class _MemorySpace(enum.Enum):
     SHARED = 2
     PRIVATE = 3
     MMA_FRAGMENT = 4
+
+
+class TensorCoreInformationEntry:
+    """One matrix-instruction shape for one (input, output) type pair
+    (/root/reference/accera/python/accera/Targets.py:748-753)."""
+
+    def __init__(self, shape, inType, outType):
+        self.shape, self.inType, self.outType = shape, inType, outType
+
+    def __repr__(self):
+        return f"TensorCoreInformationEntry({self.shape.name}, {self.inType.name} -> {self.outType.name})"
+
+
+class TensorCoreInformation:
+    """The matrix-core table of a target with the reference's queries (Targets.py:756-793)."""
+
+    def __init__(self, entries=()):
+        self.entries = list(entries)
+
+    def supports(self, input_type, output_type, shape, num_total_passes=1, num_fused_passes=-1):
+        if not (num_total_passes >= 1 and (num_fused_passes == -1 or num_total_passes % num_fused_passes == 0)):
+            return False
+        return any(e.inType == input_type and e.outType == output_type and e.shape == shape for e in self.entries)
+
+    def supports_shape(self, shape, num_total_passes=1, num_fused_passes=-1):
+        """Some type pair runs this shape (what plan.tensorize can check before it knows the arrays)."""
+        return any(self.supports(e.inType, e.outType, shape, num_total_passes, num_fused_passes) for e in self.entries)
+
+    def mma_shape_to_tuple(self, mma_shape):
+        return mma_shape.dims
+
+    def compute_tensor_splits(self, mma_shape, num_total_passes=1):
+        m, n, k = mma_shape.dims
+        return (m, n, k * num_total_passes)
 
 
 class Target:
@@ -134,15 +181,16 @@ class Target:
         def __getattr__(self, name):
             return Target._GridUnit[name]
 
-    # (input type, output type) -> MMA shapes the hardware runs natively
-    MI355X_TENSORCORE_INFO = {
-        (ScalarType.float16, ScalarType.float32): [MMAShape.M32xN32xK16_B1],
-        (ScalarType.bfloat16, ScalarType.float32): [MMAShape.M32xN32xK16_B1],
-        (ScalarType.int8, ScalarType.int32): [MMAShape.M32xN32xK32_B1],
-        (ScalarType.int8, ScalarType.int16): [MMAShape.M32xN32xK32_B1],
-        (ScalarType.int8, ScalarType.int8): [MMAShape.M32xN32xK32_B1],
-        (ScalarType.float32, ScalarType.float32): [MMAShape.M32xN32xK2_B1],
-    }
+    # the matrix instructions of gfx950 this library's kernels are built on, per (input, output) type pair: the 16x16
+    # shapes sum 64 bytes of K per instruction (the large-tile kernels), the 32x32 shapes 32 bytes
+    MI355X_TENSORCORE_INFO = TensorCoreInformation(
+        [TensorCoreInformationEntry(shape, tin, tout)
+         for tin, outs, shapes in (
+             (ScalarType.float16, (ScalarType.float32, ScalarType.float16), (MMAShape.M16xN16xK32_B1, MMAShape.M32xN32xK16_B1)),
+             (ScalarType.bfloat16, (ScalarType.float32, ScalarType.bfloat16), (MMAShape.M16xN16xK32_B1, MMAShape.M32xN32xK16_B1)),
+             (ScalarType.int8, (ScalarType.int32, ScalarType.int16, ScalarType.int8), (MMAShape.M16xN16xK64_B1, MMAShape.M32xN32xK32_B1)),
+             (ScalarType.float32, (ScalarType.float32,), (MMAShape.M32xN32xK2_B1,)))
+         for tout in outs for shape in shapes])
 
     def __init__(self, model=None, category=None, runtime=None):
         if isinstance(model, str):
@@ -348,8 +396,10 @@ def fuse(*schedules, partial=None):
 
 
 class Plan:
-    """Execution-plan calls of the reference (Plan.py:134-703, 793-956).  `tensorize` carries
-    semantics (prologue / epilogue op); the rest selects nothing here and is recorded."""
+    """Execution-plan calls of the reference (Plan.py:134-703, 793-956).  `tensorize` carries semantics (prologue /
+    epilogue op) and its `mma_shape` selects the kernel family; the block tile comes from the schedule's splits; the
+    rest (cache, bind, unroll, ...) selects nothing here -- the kernels always stage A and B through LDS several K
+    tiles deep and keep C in accumulator registers -- and is recorded."""
 
     def __init__(self, schedule, target):
         self.schedule = schedule
@@ -357,10 +407,24 @@ class Plan:
         self.commands = []
         self.prologue_op, self.prologue_arg = MMAFragmentOp.NONE, 0
         self.epilogue_op, self.epilogue_arg = MMAFragmentOp.NONE, 0
+        self.mma_shape, self.num_total_passes = None, 1
 
     def tensorize(self, indices, mma_shape=None, use_static_offsets=False, num_total_passes=1, num_fused_passes=None,
                   scheduling_policy=MMASchedulingPolicy.PASS_ORDER, prologue_op=MMAFragmentOp.NONE, prologue_arg=0,
                   epilogue_op=MMAFragmentOp.NONE, epilogue_arg=0, **_):
+        # (the checks of the reference's Plan.tensorize / _tensorize, lang/Plan.py:242-361)
+        if self.target.category != Target.Category.GPU:
+            raise ValueError("tensorization currently only supported on GPU targets")
+        indices = [indices] if isinstance(indices, Index) else list(indices)
+        if len(indices) < 3:
+            raise ValueError("tensorization requires at least three input indices")
+        if num_fused_passes is not None and num_fused_passes <= 0:
+            raise ValueError("Number of passes used for fusing must be a positive number greater than 0.")
+        if mma_shape is None:
+            raise ValueError("tensorize needs an mma_shape; this target's shapes are listed in target.tensor_core_info")
+        if not self.target.tensor_core_info.supports_shape(mma_shape, num_total_passes, -1 if num_fused_passes is None else num_fused_passes):
+            raise ValueError("The target does not support the given tensorization dimensions with shape=", mma_shape)
+        self.mma_shape, self.num_total_passes = mma_shape, num_total_passes
         if prologue_op not in (MMAFragmentOp.NONE, MMAFragmentOp.SET, MMAFragmentOp.SCALE):
             raise NotImplementedError("prologue must be NONE, SET or SCALE")
         if epilogue_op not in (MMAFragmentOp.NONE, MMAFragmentOp.ReLU, MMAFragmentOp.ReLU_NoConditional, MMAFragmentOp.SET,
@@ -394,6 +458,8 @@ class _GemmSpec:
         self.prologue, self.epilogue = prologue, epilogue
         self.prologue_arg, self.epilogue_arg = float(prologue_arg), float(epilogue_arg)
         self.block_tile = None               # (bm, bn) when a GPU plan's outermost splits of i and j name one
+        self.mma_shape = None                # the tensorized plan's instruction shape
+        self.gpu_target = False              # the function was added from a plan for a GPU target
         self.variant = _lib.VARIANT_AUTO     # kernel instantiation picked from the block tile, else automatic
 
 
@@ -466,6 +532,7 @@ def _match(source):
             epilogue, epilogue_arg = _lib.EPILOGUE_SET, plan.epilogue_arg
     spec = _GemmSpec(A, B, C, M, N, K, prologue, epilogue, prologue_arg, epilogue_arg, batch=mm.shape[0] if batched else None)
     if plan and plan.target.category == Target.Category.GPU:
+        spec.gpu_target = True
         # The outermost split of i and of j is the block tile of a GPU plan (the reference binds the
         # resulting outer indices to BLOCK_Y / BLOCK_X: lang/Plan.py:793-825, mfma_tests.py:89-97).  If
         # the library has an MFMA instantiation with that tile which takes this problem, the package
@@ -474,9 +541,19 @@ def _match(source):
         for cmd in sched.commands:
             if cmd[0] == "split" and cmd[1] in (i, j) and cmd[1] not in first:
                 first[cmd[1]] = int(cmd[2])
+        family = None
+        if plan.mma_shape is not None:
+            # the shape must exist for the nest's own types (tensorize could only check that some type pair has it)
+            if not plan.target.tensor_core_info.supports(A.element_type, C.element_type, plan.mma_shape, plan.num_total_passes):
+                raise ValueError("The target does not support the given tensorization dimensions with shape=", plan.mma_shape,
+                                 f"for {A.element_type.name} inputs and a {C.element_type.name} result")
+            spec.mma_shape = plan.mma_shape
+            if A.element_type != ScalarType.float32:
+                family = "mi16" if plan.mma_shape.dims[0] == 16 else "mi32"
         if i in first and j in first:
             spec.block_tile = (first[i], first[j])
-            spec.variant = _variant_for_tile(spec, *spec.block_tile)
+        if family or spec.block_tile:
+            spec.variant = _variant_for(spec, spec.block_tile, family)
     if spec.variant == _lib.VARIANT_AUTO and spec.batch is None:
         # no tile named by the plan: a choice recorded for this very shape by `accera_amd.tune --save`, if any
         from . import tuned
@@ -488,27 +565,53 @@ def _match(source):
     return spec
 
 
-def _variant_for_tile(spec, bm, bn):
-    """Best-ranked MFMA variant with block tile bm x bn that accepts the problem, else VARIANT_AUTO."""
-    best, best_rank = _lib.VARIANT_AUTO, -8
+def _variant_for(spec, tile=None, family=None):
+    """MFMA variant for a plan that names a block tile (bm, bn) and / or an instruction-shape family ("mi16": the
+    16x16 shapes, "mi32": the 32x32 ones).  Among the variants that accept the problem: those of the named tile if
+    there are any (else any tile), of the named family if there are any; the library's own choice when it is one of
+    them, else the best-ranked.  VARIANT_AUTO when nothing matches."""
     lean = spec.prologue == _lib.PROLOGUE_SET and spec.prologue_arg == 0 and spec.epilogue in (_lib.EPILOGUE_RELU, _lib.EPILOGUE_NONE)
+    geometry = (spec.A.element_type.lib_id, spec.C.element_type.lib_id, spec.M, spec.N, spec.K,
+                spec.A.strides[-2:], spec.B.strides[-2:], spec.C.strides[-2:])
+    cands = []
     for v in range(_lib.num_variants()):
         name = _lib.variant_name(v)
-        if f"mfma {bm}x{bn} " not in name:
-            continue
         try:
-            _lib.launch_geometry(spec.A.element_type.lib_id, spec.C.element_type.lib_id, spec.M, spec.N, spec.K,
-                                 spec.A.strides[-2:], spec.B.strides[-2:], spec.C.strides[-2:], v, 0)
+            _lib.launch_geometry(*geometry, v, 0)
         except _lib.Acc950Error:
             continue
-        # ping-pong over software-pipelined; the 16x16 MFMA shapes where the library runs their lean build
-        rank = 2 * ("pingpong" in name) + (1 if "mi16" in name and lean else -1 if "mi16" in name else 0)
-        if "hand-laid loop" in name:  # four waves: every op, but an int8 C is only written; ahead of the ping-pong form
-            reads_int8_c = spec.prologue != _lib.PROLOGUE_SET and spec.C.element_type.lib_id == _lib.I8
-            rank = -9 if reads_int8_c else 4
-        if rank > best_rank:
-            best, best_rank = v, rank
-    return best
+        if "hand-laid loop" in name and spec.prologue != _lib.PROLOGUE_SET and spec.C.element_type.lib_id == _lib.I8:
+            continue  # (the four-wave kernels do not read an int8 C)
+        cands.append((v, name))
+    named = []
+    if tile:
+        named = [(v, n) for v, n in cands if f"mfma {tile[0]}x{tile[1]} " in n]
+        if not named and not family:
+            return _lib.VARIANT_AUTO
+        cands = named or cands
+    if family:
+        cands = [(v, n) for v, n in cands if ("mi16" in n) == (family == "mi16")] or cands
+    if not cands:
+        return _lib.VARIANT_AUTO
+    try:
+        auto = _lib.launch_geometry(*geometry, _lib.VARIANT_AUTO, 0)[3]
+    except _lib.Acc950Error:
+        auto = None
+    if auto in [v for v, _ in cands]:
+        return auto
+    if auto is not None and auto >= _lib.num_variants() and not (tile and named):
+        return _lib.VARIANT_AUTO  # the library runs this problem on a streaming / fp32 / thread-bound kernel: no MFMA tile to name
+
+    def rank(name):
+        bm, bn = map(int, re.search(r"mfma (\d+)x(\d+)", name).groups())
+        tiles = -(-spec.M // bm) * -(-spec.N // bn)
+        # ping-pong over software-pipelined; the 16x16 shapes where the library runs their lean build; four waves with
+        # the hand-laid loop ahead of both (the multi-tile form when there is more than one round of tiles); then larger tiles
+        r = 2 * ("pingpong" in name) + (1 if "mi16" in name and lean else -1 if "mi16" in name else 0)
+        if "hand-laid loop" in name:
+            r = 4 + (("multi-tile" in name) == (tiles > 256))
+        return (r, bm * bn if tiles >= 256 else -bm * bn, "edge" not in name)
+    return sorted(cands, key=lambda c: rank(c[1]))[-1][0]  # (`max` is the DSL's elementwise maximum in this module)
 
 
 # ---- package -------------------------------------------------------------------------------------
@@ -565,18 +668,32 @@ class Package:
             call_args = (f"{s.A.element_type.lib_id}, {s.C.element_type.lib_id}, {nb}, {s.M}, {s.N}, {s.K}, "
                          f"{pa}, {abs_}, {ars}, {acs}, {pb}, {bbs}, {brs}, {bcs}, {pc}, {cbs}, {crs}, {ccs}, "
                          f"{s.prologue}, {s.prologue_arg!r}, {s.epilogue}, {s.epilogue_arg!r}")
+            # (a variant recorded at build time that the library refuses at call time -- pointer alignment, a table that
+            # changed under a rebuilt library -- gives way to the library's own choice)
+            retry = f" if (rc == ACC950_UNSUPPORTED) rc = acc950_gemm_batched_host({call_args}, ACC950_VARIANT_AUTO, 0);" \
+                if s.variant != _lib.VARIANT_AUTO else ""
+            retry_dev = f" if (rc == ACC950_UNSUPPORTED) rc = acc950_gemm_batched({call_args}, ACC950_VARIANT_AUTO, 0, stream);" \
+                if s.variant != _lib.VARIANT_AUTO else ""
             lines += [
                 f"void {f['name']}(void* a0, void* a1, void* a2)", "{",
-                f"    if (acc950_gemm_batched_host({call_args}, {s.variant}, 0) != ACC950_OK)",
-                f"        fprintf(stderr, \"{f['name']}: %s\\n\", acc950_last_error());", "}",
-                "/* same function on device pointers, asynchronous on `stream` (hipStream_t or NULL) */",
+                f"    int rc = acc950_gemm_batched_host({call_args}, {s.variant}, 0);{retry}",
+                f"    if (rc != ACC950_OK) fprintf(stderr, \"{f['name']}: %s\\n\", acc950_last_error());", "}",
+                "/* same function on device pointers, asynchronous on `stream` (hipStream_t or NULL): what the record",
+                f"   [device_functions.{f['name']}__gpu__] of the .hat stands for */",
                 f"int {f['name']}__device(void* a0, void* a1, void* a2, void* stream)", "{",
-                f"    return acc950_gemm_batched({call_args}, {s.variant}, 0, stream);", "}", ""]
+                f"    int rc = acc950_gemm_batched({call_args}, {s.variant}, 0, stream);{retry_dev}",
+                "    return rc;", "}", ""]
         return "\n".join(lines)
 
-    def build(self, name, format=None, mode=None, platform=None, tolerance=1e-5, output_dir=None, **_):
+    def build(self, name, format=None, mode=None, platform=None, tolerance=1e-5, output_dir=None, gpu_records=True, **_):
         """Emit `<output_dir>/<name>.hat` and `<name>.so` (HAT_DYNAMIC).  Returns the list of
-        files written (Package.py:551-788 returns the same kind of list)."""
+        files written (Package.py:551-788 returns the same kind of list).
+
+        gpu_records: functions added from a plan for a GPU target get the records the reference writes for such targets
+        (Package.py:714-743): `runtime = "ROCM"` and `launches = "<fn>__gpu__"` on the function and a
+        `[device_functions.<fn>__gpu__]` table with its `launch_parameters`, `dynamic_shared_mem_bytes` and `provider`.
+        Functions of HOST-target plans (the quick-start form) never do.  The host symbol `<fn>` takes host pointers
+        either way; False leaves the GPU records out altogether (a plain host-convention package)."""
         fmt = format or Package.Format.DEFAULT
         if not (fmt & Package.Format.HAT_DYNAMIC):
             raise NotImplementedError("only Package.Format.HAT_DYNAMIC is produced by this build")
@@ -594,7 +711,7 @@ class Package:
                "-laccera_mi355x", f"-Wl,-rpath,$ORIGIN/{rel}", f"-Wl,-rpath,{_lib.LIB_DIR}"]
         subprocess.check_call(cmd)
 
-        functions = []
+        functions, device_functions = [], []
         for f in self._functions:
             s = f["spec"]
             arguments = []
@@ -614,8 +731,18 @@ class Package:
                                      "prologue": s.prologue, "prologue_arg": s.prologue_arg, "epilogue": s.epilogue,
                                      "epilogue_arg": s.epilogue_arg}}
             aux.update(f["auxiliary"])
-            functions.append(_hat.Function(name=f["name"], base_name=f["base_name"], arguments=arguments, auxiliary=aux))
-        _hat.write_hat(hat_path, name, functions, link_target=f"{name}.so",
+            fn = _hat.Function(name=f["name"], base_name=f["base_name"], arguments=arguments, auxiliary=aux)
+            if gpu_records and s.gpu_target:
+                # the kernel is prebuilt: the "provider" is the kernel library, and the device function is reached through
+                # the package's `<fn>__device` entry (there is no source for hatlib's run-time compiler)
+                fn.runtime, fn.launches = "ROCM", f"{f['name']}__gpu__"
+                device_functions.append(_hat.Function(
+                    name=fn.launches, base_name=f["base_name"], arguments=arguments, calling_convention="device",
+                    description=f"Device function launched by {f['name']}", launch_parameters=grid + block,
+                    dynamic_shared_mem_bytes=lds, provider=os.path.basename(_lib.LIB_PATH), runtime="ROCM",
+                    auxiliary={"accera_mi355x": {"kernel": _lib.variant_name(variant), "entry": f"{f['name']}__device"}}))
+            functions.append(fn)
+        _hat.write_hat(hat_path, name, functions, link_target=f"{name}.so", device_functions=device_functions,
                        author=self._description.get("author", ""), version=self._description.get("version", ""),
                        license_url=self._description.get("license", ""),
                        required_gpu={"runtime": "ROCM", "model": "AMD MI355X", "instruction_set_version": "gfx950"},

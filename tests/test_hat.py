@@ -44,7 +44,17 @@ def _quickstart_package(tmp, M=512, N=512, K=512):
     return files
 
 
-def _gpu_plan_package(tmp, in_t, out_t, M, N, K, b_layout=None, epilogue=None, base_name="matmul_relu"):
+def _native_shape(in_t, wide=False):
+    """An instruction shape of the target for this input type: the 16x16 family (the 32x32 one with `wide`)."""
+    S = acc.MMAShape
+    if in_t == acc.ScalarType.float32:
+        return S.M32xN32xK2_B1
+    if in_t == acc.ScalarType.int8:
+        return S.M32xN32xK32_B1 if wide else S.M16xN16xK64_B1
+    return S.M32xN32xK16_B1 if wide else S.M16xN16xK32_B1
+
+
+def _gpu_plan_package(tmp, in_t, out_t, M, N, K, b_layout=None, epilogue=None, base_name="matmul_relu", mma_shape=None, **build_args):
     """mfma_tests.py:359-432 (`_matmul_relu`): tensorized plan with SET prologue and ReLU epilogue."""
     target = acc.Target(acc.Target.Model.AMD_MI355X)
     A = acc.Array(role=acc.Role.INPUT, element_type=in_t, shape=(M, K))
@@ -62,13 +72,13 @@ def _gpu_plan_package(tmp, in_t, out_t, M, N, K, b_layout=None, epilogue=None, b
     schedule.reorder(i, j, k, ii, jj, kk)
     plan = schedule.create_plan(target)
     plan.bind({i: target.GridUnit.BLOCK_Y, j: target.GridUnit.BLOCK_X, ii: target.GridUnit.WARP_Y, jj: target.GridUnit.WARP_X})
-    plan.tensorize(indices=(ii, jj, kk), mma_shape=acc.MMAShape.M32xN32xK16_B1, prologue_op=acc.MMAFragmentOp.SET,
+    plan.tensorize(indices=(ii, jj, kk), mma_shape=mma_shape or _native_shape(in_t), prologue_op=acc.MMAFragmentOp.SET,
                    prologue_arg=0, epilogue_op=epilogue or acc.MMAFragmentOp.ReLU)
     plan.cache(A, index=ii, double_buffer=True, location=target.MemorySpace.SHARED)
     plan.cache(C, index=ii, location=target.MemorySpace.MMA_FRAGMENT)
     package = acc.Package()
     name = package.add(plan, args=(A, B, C), base_name=base_name)
-    files = package.build(name="gpu_pkg", output_dir=str(tmp))
+    files = package.build(name="gpu_pkg", output_dir=str(tmp), **build_args)
     return files, name
 
 
@@ -91,6 +101,8 @@ def test_quickstart_builds_a_valid_hat(tmp_path):
         assert rec["return"]["declared_type"] == "void"
         aux = rec["auxiliary"]["accera_mi355x"]
         assert len(aux["launch_parameters"]) == 6 and aux["epilogue"] == acc.EPILOGUE_RELU and aux["prologue"] == acc.PROLOGUE_NONE
+        assert "launches" not in rec and "runtime" not in rec      # HOST-target plans: a host-convention function
+    assert "device_functions" not in doc
     assert doc["dependencies"]["link_target"] == "hello_accera.so"
     assert doc["target"]["required"]["GPU"]["instruction_set_version"] == "gfx950"
     assert "void (*matmul_relu_fusion_naive)(float*, float*, float*)" in doc["declaration"]["code"]
@@ -146,8 +158,8 @@ def test_block_tile_of_a_gpu_plan_selects_the_kernel(tmp_path):
         schedule.reorder(i, j, k, ii, jj, kk)
         plan = schedule.create_plan(target)
         plan.bind({i: target.GridUnit.BLOCK_Y, j: target.GridUnit.BLOCK_X})
-        plan.tensorize(indices=(ii, jj, kk), mma_shape=acc.MMAShape.M32xN32xK16_B1, prologue_op=acc.MMAFragmentOp.SET, prologue_arg=0,
-                       epilogue_op=acc.MMAFragmentOp.ReLU)
+        plan.tensorize(indices=(ii, jj, kk), mma_shape=acc.MMAShape.M16xN16xK32_B1 if tile[0] == 256 else acc.MMAShape.M32xN32xK16_B1,
+                       prologue_op=acc.MMAFragmentOp.SET, prologue_arg=0, epilogue_op=acc.MMAFragmentOp.ReLU)
         return plan
 
     package = acc.Package()
@@ -160,6 +172,91 @@ def test_block_tile_of_a_gpu_plan_selects_the_kernel(tmp_path):
     assert "mfma 256x256" in rec(n256)["kernel"] and rec(n256)["launch_parameters"][:3] == [16, 1, 1]
     assert "mfma 128x128" in rec(n128)["kernel"] and rec(n128)["launch_parameters"][:3] == [64, 1, 1]
     assert "mfma" in rec(n48)["kernel"]
+
+
+def test_gpu_target_functions_carry_the_reference_device_records(tmp_path):
+    """Package.py:714-743: `runtime` / `launches` on the function, and a [device_functions.<fn>__gpu__] record with the
+    launch geometry, the dynamic LDS size and the provider."""
+    from accera_amd import _lib
+    (hat_path, so_path), name = _gpu_plan_package(tmp_path, acc.ScalarType.float16, acc.ScalarType.float32, 4096, 4096, 4096)
+    doc = hat.parse(hat_path)
+    fn = doc["functions"][name]
+    assert fn["runtime"] == "ROCM" and fn["launches"] == name + "__gpu__" and fn["calling_convention"] == "cdecl"
+    dev = doc["device_functions"][name + "__gpu__"]
+    assert dev["name"] == name + "__gpu__" and dev["calling_convention"] == "device" and dev["runtime"] == "ROCM"
+    assert dev["description"] == f"Device function launched by {name}"
+    assert dev["arguments"] == fn["arguments"] and dev["return"] == fn["return"]
+    grid, block, lds, variant = _lib.launch_geometry(_lib.F16, _lib.F32, 4096, 4096, 4096, (4096, 1), (4096, 1), (4096, 1))
+    assert dev["launch_parameters"] == grid + block == fn["auxiliary"]["accera_mi355x"]["launch_parameters"]
+    assert dev["dynamic_shared_mem_bytes"] == lds > 0 and dev["provider"] == "libaccera_mi355x.so"
+    assert dev["auxiliary"]["accera_mi355x"]["entry"] == name + "__device"
+    assert doc["target"]["required"]["GPU"]["runtime"] == "ROCM" and doc["target"]["required"]["GPU"]["model"] == "AMD MI355X"
+    # both symbols are in the package library
+    import ctypes
+    L = ctypes.CDLL(so_path)
+    assert getattr(L, name) is not None and getattr(L, name + "__device") is not None
+    # the loader pairs them
+    _, functions = hat.load(hat_path)
+    assert functions[name].launches == name + "__gpu__" and functions[name].device_record == dev
+    # gpu_records=False: the same function as a plain host-convention record
+    (hat2, _), name2 = _gpu_plan_package(tmp_path / "plain", acc.ScalarType.float16, acc.ScalarType.float32, 4096, 4096, 4096,
+                                         gpu_records=False)
+    doc2 = hat.parse(hat2)
+    assert name2 == name and "device_functions" not in doc2 and "launches" not in doc2["functions"][name]
+
+
+def test_tensor_core_table_and_mma_shape_validation(tmp_path):
+    """Targets.py:756-793 (the table and its queries) and the checks of Plan.tensorize (lang/Plan.py:242-361)."""
+    T, S = acc.ScalarType, acc.MMAShape
+    target = acc.Target(acc.Target.Model.AMD_MI355X)
+    info = target.tensor_core_info
+    assert info.supports(T.float16, T.float32, S.M16xN16xK32_B1, 1, -1) and info.supports(T.bfloat16, T.bfloat16, S.M32xN32xK16_B1, 2, 1)
+    assert info.supports(T.int8, T.int32, S.M16xN16xK64_B1) and info.supports(T.int8, T.int8, S.M32xN32xK32_B1)
+    assert info.supports(T.float32, T.float32, S.M32xN32xK2_B1)
+    assert not info.supports(T.float16, T.float32, S.M16xN16xK16_B1)          # an MI100 shape gfx950 kernels do not use
+    assert not info.supports(T.int8, T.int32, S.M16xN16xK32_B1)               # a 16-bit shape with 8-bit inputs
+    assert not info.supports(T.float16, T.float32, S.M16xN16xK32_B1, 4, 3)    # passes must divide
+    assert info.mma_shape_to_tuple(S.M16xN16xK64_B1) == (16, 16, 64) and info.compute_tensor_splits(S.M32xN32xK16_B1, 4) == (32, 32, 64)
+
+    def plan_for(in_t, out_t, tgt=target):
+        A = acc.Array(role=acc.Role.INPUT, element_type=in_t, shape=(512, 512))
+        B = acc.Array(role=acc.Role.INPUT, element_type=in_t, shape=(512, 512))
+        C = acc.Array(role=acc.Role.INPUT_OUTPUT, element_type=out_t, shape=(512, 512))
+        nest = acc.Nest(shape=(512, 512, 512))
+        i, j, k = nest.get_indices()
+
+        @nest.iteration_logic
+        def _():
+            C[i, j] += A[i, k] * B[k, j]
+
+        return nest.create_schedule().create_plan(tgt), (i, j, k), (A, B, C)
+
+    plan, idx, arrays = plan_for(T.float16, T.float32)
+    with pytest.raises(ValueError, match="does not support the given tensorization dimensions"):
+        plan.tensorize(indices=idx, mma_shape=S.M16xN16xK16_B1)
+    with pytest.raises(ValueError, match="at least three"):
+        plan.tensorize(indices=idx[:2], mma_shape=S.M16xN16xK32_B1)
+    with pytest.raises(ValueError, match="fusing must be a positive"):
+        plan.tensorize(indices=idx, mma_shape=S.M16xN16xK32_B1, num_fused_passes=0)
+    host_plan, idx_h, _ = plan_for(T.float16, T.float32, acc.Target.HOST)
+    with pytest.raises(ValueError, match="only supported on GPU"):
+        host_plan.tensorize(indices=idx_h, mma_shape=S.M16xN16xK32_B1)
+    # a shape of the target, but not for these types: caught when the function is added
+    plan8, idx8, arrays8 = plan_for(T.int8, T.int32)
+    plan8.tensorize(indices=idx8, mma_shape=S.M16xN16xK32_B1)
+    with pytest.raises(ValueError, match="does not support"):
+        acc.Package().add(plan8, args=arrays8, base_name="bad_shape")
+    # the shape selects the kernel family
+    package = acc.Package()
+    names = {}
+    for tag, shape in (("small", S.M16xN16xK32_B1), ("wide", S.M32xN32xK16_B1)):
+        p, ix, arr = plan_for(T.float16, T.float32)
+        p.tensorize(indices=ix, mma_shape=shape, prologue_op=acc.MMAFragmentOp.SET, epilogue_op=acc.MMAFragmentOp.ReLU)
+        names[tag] = package.add(p, args=arr, base_name=tag)
+    files = package.build(name="shapes", output_dir=str(tmp_path))
+    fns = hat.parse(files[0])["functions"]
+    assert " mi16" in fns[names["small"]]["auxiliary"]["accera_mi355x"]["kernel"]
+    assert " mi16" not in fns[names["wide"]]["auxiliary"]["accera_mi355x"]["kernel"] and "mfma" in fns[names["wide"]]["auxiliary"]["accera_mi355x"]["kernel"]
 
 
 def test_only_the_matmul_pattern_is_accepted():
@@ -327,3 +424,61 @@ def test_run_benchmark_reports_hatlib_style_rows(tmp_path):
         assert r.function_name.startswith("matmul_relu_fusion_")
         assert 0 < r.min_of_means <= r.median_of_means and r.min_of_means <= r.mean
         assert r.mean_of_small_means <= r.mean and r.robust_mean > 0
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("in_t,out_t,shape,wide", [
+    (acc.ScalarType.float16, acc.ScalarType.float32, (512, 512, 256), False),
+    (acc.ScalarType.int8, acc.ScalarType.int32, (256, 512, 512), True),
+    (acc.ScalarType.float16, acc.ScalarType.float16, (8, 2048, 1024), False),
+])
+def test_device_function_of_a_package_on_device_pointers(tmp_path, in_t, out_t, shape, wide):
+    """What the [device_functions.<fn>__gpu__] record stands for: `<fn>__device(A, B, C, stream)` of the package library
+    on DEVICE pointers, asynchronous on a stream, checked against the oracle; and the loader's `device_id=` form of the
+    call (copies on this side of the boundary), hatlib's calling form for GPU packages (accera_gemm.py:612-615)."""
+    import ctypes
+    import torch
+    from tests.util import assert_matches, make_input, to_device, to_host
+    M, N, K = shape
+    (hat_path, so_path), name = _gpu_plan_package(tmp_path, in_t, out_t, M, N, K, mma_shape=_native_shape(in_t, wide))
+    tn = {acc.ScalarType.float16: "f16", acc.ScalarType.int8: "i8", acc.ScalarType.float32: "f32", acc.ScalarType.int32: "i32"}
+    it, ot = tn[in_t], tn[out_t]
+    rng = np.random.default_rng(11)
+    A, B = make_input(rng, (M, K), it), make_input(rng, (K, N), it)
+    want = ora.gemm_relu_exact(A, B, None, it, ot)
+    dA, dB = to_device(A, it), to_device(B, it)
+    dC = to_device(np.full((M, N), 5, ora.NP_STORAGE[ot]), ot)
+    L = ctypes.CDLL(so_path)
+    entry = getattr(L, name + "__device")
+    entry.restype, entry.argtypes = ctypes.c_int, [ctypes.c_void_p] * 4
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        assert entry(dA.data_ptr(), dB.data_ptr(), dC.data_ptr(), stream.cuda_stream) == 0
+    stream.synchronize()
+    assert_matches(to_host(dC, ot), want, ot, K)
+    # through the loader
+    _, functions = hat.load(hat_path)
+    f = functions[name]
+    assert f.device_record["launch_parameters"][3] % 64 == 0
+    C = np.full((M, N), 3, ora.NP_STORAGE[ot])
+    f(A, B, C, device_id=0)
+    assert_matches(C, want, ot, K)
+    dC.fill_(1)
+    f.launch_on_device([dA.data_ptr(), dB.data_ptr(), dC.data_ptr()])
+    torch.cuda.synchronize()
+    assert_matches(to_host(dC, ot), want, ot, K)
+
+
+@pytest.mark.gpu
+def test_run_benchmark_times_gpu_functions_device_resident(tmp_path):
+    """accera_gemm.py:621-626, 648: `run_benchmark(..., device_id=)` of a GPU package gives kernel time (inputs resident
+    in device memory, HIP events around each batch), far below the time of the host-pointer entry with its copies."""
+    (hat_path, _), name = _gpu_plan_package(tmp_path, acc.ScalarType.float16, acc.ScalarType.float32, 2048, 2048, 2048)
+    dev = hat.run_benchmark(hat_path, batch_size=10, min_time_in_sec=0.3, input_sets_minimum_size_MB=40, device_id=0)
+    host = hat.run_benchmark(hat_path, batch_size=3, min_time_in_sec=0.3, input_sets_minimum_size_MB=40, device_id=0, host_pointers=True)
+    assert len(dev) == len(host) == 1 and dev[0].function_name == name
+    r = dev[0]
+    assert 0 < r.min_of_means <= r.median_of_means and r.min_of_means <= r.mean
+    tflops = 2 * 2048 ** 3 / r.min_of_means / 1e12
+    assert 100 < tflops < 2500, tflops          # a kernel time, not a copy time (PCIe alone takes milliseconds here)
+    assert host[0].min_of_means > 5 * r.min_of_means
