@@ -178,6 +178,15 @@ struct OperandTile {
                      : "memory");
     }
 
+    // Same for an address the register allocator may have put into vector registers although it is the same in every
+    // lane (scalar registers run short around the hand-laid loop): lane 0's copy is taken explicitly.
+    __device__ static __forceinline__ void direct_issue_uniform(unsigned lds_addr, unsigned lane_off, const char* sbase)
+    {
+        const unsigned long long a = (unsigned long long)sbase;
+        const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)a), hi = __builtin_amdgcn_readfirstlane((unsigned)(a >> 32));
+        direct_issue(__builtin_amdgcn_readfirstlane(lds_addr), lane_off, (const char*)(((unsigned long long)hi << 32) | lo));
+    }
+
     // ---- fragment read: 32 rows starting at row0, k-step ks (32 bytes of K) ----
     __device__ static __forceinline__ i32x4 read_frag(const char* lds, int row0, int ks, int lane)
     {

@@ -104,7 +104,7 @@ __global__ void __launch_bounds__(256, 1) gemm_mfma16w4_kernel(GemmArgs p)
     // M and N need not be multiples of the tile: the last row / column of tiles ends at M / N and overlaps its
     // neighbour.  What both compute gets the same bits from both (the host allows this only when C is not read,
     // and only for N whose last tile still starts on a 16-byte boundary of B's and C's rows).
-    auto tile_origin = [&](int id, int& r0, int& c0) {
+    auto tile_origin = [&](int id, int& r0, int& c0) __attribute__((always_inline)) {
         int tile_m, tile_n;
         tile_coords(id, p.tiles_m, p.tiles_n, tile_m, tile_n);
         r0 = tile_m * BM + BM <= p.M ? tile_m * BM : p.M - BM;
@@ -158,8 +158,8 @@ __global__ void __launch_bounds__(256, 1) gemm_mfma16w4_kernel(GemmArgs p)
     const unsigned db = __builtin_amdgcn_readfirstlane((unsigned)((B_KC ? 64 : B_RPP) * ldb * ES));
     const unsigned sa = KB;
     const unsigned sb = __builtin_amdgcn_readfirstlane(B_KC ? (unsigned)KB : (unsigned)(BK * ldb * ES));
-    auto a_panel = [&](int r0) { return Ab + (int64_t)r0 * lda * ES; };
-    auto b_panel = [&](int c0) { return Bb + (B_KC ? (int64_t)c0 * ldb * ES : (int64_t)c0 * ES); };
+    auto a_panel = [&](int r0) __attribute__((always_inline)) { return Ab + (int64_t)r0 * lda * ES; };
+    auto b_panel = [&](int c0) __attribute__((always_inline)) { return Bb + (B_KC ? (int64_t)c0 * ldb * ES : (int64_t)c0 * ES); };
     const char* a_tile = a_panel(m0);
     const char* b_tile = b_panel(n0);
     // The loop's last k-step runs at position 3 of its four-step pattern, so the first one starts at position
@@ -172,17 +172,18 @@ __global__ void __launch_bounds__(256, 1) gemm_mfma16w4_kernel(GemmArgs p)
     constexpr bool B_PAIRED = B_KC && (BN == 192 || IN == IN_I8); // measured: behind the plain scheme for 16-bit inputs on 256-wide tiles
     const unsigned b_tiles_here = B_PAIRED ? 2u + (p0 & 1u) : 3u;
     // the first three K tiles of an output tile, issued ahead of its loop
-    auto first_fills = [&](const char* a_src, const char* b_src) {
+    // (always inline: the panel addresses are scalar-register operands of the fill instructions)
+    auto first_fills = [&](const char* a_src, const char* b_src) __attribute__((always_inline)) {
 #pragma unroll
         for (int s = 0; s < 3; ++s) {
             const unsigned stage = ldsb + ((s + p0) & 3) * STAGE_BYTES;
 #pragma unroll
             for (int f = 0; f < 4; ++f)
-                TA::direct_issue(stage + f * 4096, a_off, a_src + (int64_t)s * sa + (int64_t)f * da);
+                TA::direct_issue_uniform(stage + f * 4096, a_off, a_src + (int64_t)s * sa + (int64_t)f * da);
             if ((unsigned)s < b_tiles_here) {
 #pragma unroll
                 for (int f = 0; f < FILLS_B; ++f)
-                    TB::direct_issue(stage + TA::TILE_BYTES + f * 4096, (f & 1) ? b_off1 : b_off0, b_src + (int64_t)s * sb + (int64_t)f * db);
+                    TB::direct_issue_uniform(stage + TA::TILE_BYTES + f * 4096, (f & 1) ? b_off1 : b_off0, b_src + (int64_t)s * sb + (int64_t)f * db);
             }
         }
     };
@@ -233,12 +234,23 @@ __global__ void __launch_bounds__(256, 1) gemm_mfma16w4_kernel(GemmArgs p)
     if (has_next) tile_origin(next_id, m0_next, n0_next);
     const char* pa_n = a_panel(m0_next);
     const char* pb_n = b_panel(n0_next);
+    const char* pa_n_u = nullptr;
+    const char* pb_n_u = nullptr;
     const bool prefetch_next = TAIL_PREFETCH && has_next && p0 == 0;
     // bit 0: the closing steps fetch the next tile's K tiles 0..2; bit 1: the first k-steps allow for the previous tile's
     // stores (64 per thread with a 32-bit C) between this tile's fills
     const unsigned flags = __builtin_amdgcn_readfirstlane((prefetch_next ? 1u : 0u) | (came_prefetched && os == 4 && groups >= 1 ? 2u : 0u));
-    const char* pa = a_tile + 3 * (int64_t)sa;
-    const char* pb = b_tile + (int64_t)b_tiles_here * sb;
+    // (lane 0's copy of each address, explicitly: they are scalar-register operands of the loop, and with scalar registers
+    // short around it the compiler may keep a value that is the same in every lane in vector registers)
+    auto uniform_ptr = [](const char* q) __attribute__((always_inline)) {
+        const unsigned long long a = (unsigned long long)q;
+        const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)a), hi = __builtin_amdgcn_readfirstlane((unsigned)(a >> 32));
+        return (const char*)(((unsigned long long)hi << 32) | lo);
+    };
+    const char* pa = uniform_ptr(a_tile + 3 * (int64_t)sa);
+    const char* pb = uniform_ptr(b_tile + (int64_t)b_tiles_here * sb);
+    pa_n_u = uniform_ptr(pa_n);
+    pb_n_u = uniform_ptr(pb_n);
     const CTile c_in = c_tile(p, m0, n0, 4);
     const auto c_rsrc = c_in.rsrc;
 
@@ -340,7 +352,7 @@ __global__ void __launch_bounds__(256, 1) gemm_mfma16w4_kernel(GemmArgs p)
       [b_rd4] "v"(b_rd[4]), [b_rd5] "v"(b_rd[5]), [b_rd6] "v"(b_rd[6]), [b_rd7] "v"(b_rd[7]), [a_off] "v"(a_off),        \
       [b_off0] "v"(b_off0), [b_off1] "v"(b_off1), [pa] "s"(pa), [pb] "s"(pb), [da] "s"(da), [db] "s"(db), [sa] "s"(sa),   \
       [sb] "s"(sb), [ldsb] "s"(ldsb), [groups] "s"(groups), [accum] "s"(accum), [c_off] "v"(c_off), [p0] "s"(p0),       \
-      [c_rsrc] "s"(c_rsrc), [c_row16] "s"(c_row16), [pa_n] "s"(pa_n), [pb_n] "s"(pb_n), [flags] "s"(flags)               \
+      [c_rsrc] "s"(c_rsrc), [c_row16] "s"(c_row16), [pa_n] "s"(pa_n_u), [pb_n] "s"(pb_n_u), [flags] "s"(flags)               \
     : "memory", "scc", "s72", "s73", "s74", "s75", "s76", "s77", "s78", "s79", "s80", "s81", ACC950_W4_V(10), ACC950_W4_V(11), \
       ACC950_W4_V(12), ACC950_W4_V(13), ACC950_W4_V(14), ACC950_W4_V(15), ACC950_W4_V(16), ACC950_W4_V(17),             \
       ACC950_W4_V(18), ACC950_W4_V(19), ACC950_W4_V(20), ACC950_W4_V(21), ACC950_W4_V(22), ACC950_W4_V(23),             \
@@ -381,14 +393,19 @@ __global__ void __launch_bounds__(256, 1) gemm_mfma16w4_kernel(GemmArgs p)
 
     // ---- write-back: block (i, j) leaves the AGPR file just before its store.  Lane l holds row
     // i*16 + l%16 and columns j*16 + (l/16)*4 .. +3 of the wave tile.
-    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+    // (In a workgroup that walks several tiles the write-back's addresses do not change from tile to tile; computed from
+    // an opaque copy of the lane id they are recomputed per tile instead of being kept in registers across the K loop,
+    // where only v0-v99 are free.)
+    int lane_wb = lane, wave_wb = wave;
+    if constexpr (Cfg::PERSIST) asm volatile("" : "+v"(lane_wb), "+v"(wave_wb));
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave_wb);
     // One copy of the stores per epilogue (a uniform branch).
     // (epi_tag: 0 nothing, 1 ReLU, 2 the other epilogue ops, applied element by element from the call's arguments)
-    auto write_back = [&](auto epi_tag) {
+    auto write_back = [&](auto epi_tag) __attribute__((always_inline)) {
         constexpr int EPI = decltype(epi_tag)::value;
         constexpr bool RELU = EPI == 1;
         // row i of the wave tile's blocks, epilogue applied
-        auto load_row = [&](auto i_tag, acc_t (&row)[TN]) {
+        auto load_row = [&](auto i_tag, acc_t (&row)[TN]) __attribute__((always_inline)) {
             constexpr int i = decltype(i_tag)::value;
             w4_static_for<0, TN / 2>([&](auto h) {
                 const W4BlockPair pr = w4_acc_pair<i * TN + h.value * 2>();
@@ -416,8 +433,15 @@ __global__ void __launch_bounds__(256, 1) gemm_mfma16w4_kernel(GemmArgs p)
             // whole rows of a narrow type) passes through a CU's memory pipeline more than twice as fast as one that writes
             // the accumulator layout's 16 rows x 64 bytes (measured: 256 KB per CU in 2.4-2.9 us against 6.2-7.0 us)
             __syncthreads();
-            auto staged = [&](auto os_tag, auto&& pack) {
+            // (the lambdas of the write-back are always inlined: left as functions they would take the kernel's state by
+            // reference through memory, and everything they capture -- tile origin, descriptors, the call's arguments -- would
+            // live in scratch and come back in vector registers)
+            auto staged = [&](auto os_tag, auto&& pack) __attribute__((always_inline)) {
                 constexpr int OS = decltype(os_tag)::value;
+                // Non-temporal stores: C is written once and not read again by this launch, and lines of it kept in the L2
+                // would push out the A and B panels the workgroups of the XCD share (measured: int8 8192^3 4 % faster, fp16
+                // 4096^3 0.8 %, with the `nt` bit; `sc1` alone changes nothing)
+                constexpr int AUX = 2;
                 constexpr int ROW = WTN * OS;
                 // 16 bytes past a row: the 16 row starts are an odd number of 4-bank steps apart, so a lane group's
                 // 8- or 4-byte pieces of 16 rows land on 64 different banks
@@ -431,7 +455,7 @@ __global__ void __launch_bounds__(256, 1) gemm_mfma16w4_kernel(GemmArgs p)
                 const unsigned row_bytes = (unsigned)p.c_rs * OS;
                 constexpr int CPRW = ROW / 16;
                 constexpr int PIECES = (16 * CPRW + 63) / 64;
-                char* mine = slab + (lane & 15) * PITCH + ((lane >> 4) * 4) * OS;
+                char* mine = slab + (lane_wb & 15) * PITCH + ((lane_wb >> 4) * 4) * OS;
                 // (the accumulator reads of the next row are issued between this row's LDS writes and reads)
                 acc_t row[TN], next_row[TN];
                 load_row(std::integral_constant<int, 0>{}, row);
@@ -444,12 +468,12 @@ __global__ void __launch_bounds__(256, 1) gemm_mfma16w4_kernel(GemmArgs p)
                     if constexpr (i.value + 1 < TM) load_row(std::integral_constant<int, i.value + 1>{}, next_row);
 #pragma unroll
                     for (int it = 0; it < PIECES; ++it) {
-                        const int id = it * 64 + lane;
+                        const int id = it * 64 + lane_wb;
                         if ((16 * CPRW) % 64 != 0 && id >= 16 * CPRW) break;
                         const int r = id / CPRW, cc = id % CPRW;
                         const i32x4 v = *(const i32x4*)(slab + r * PITCH + cc * 16);
                         __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), tile.rsrc, (unsigned)r * row_bytes + cc * 16,
-                                                               (unsigned)(i.value * 16) * row_bytes, 0);
+                                                               (unsigned)(i.value * 16) * row_bytes, AUX);
                     }
                     if constexpr (i.value + 1 < TM) {
 #pragma unroll
@@ -501,17 +525,16 @@ __global__ void __launch_bounds__(256, 1) gemm_mfma16w4_kernel(GemmArgs p)
         stamp(0);
     }
     if constexpr (!Cfg::PERSIST) break;
-    if (!has_next) break;
-    if (!prefetch_next) {
+    if (tile_id + (int)gridDim.x >= total_tiles) break;
+    came_prefetched = TAIL_PREFETCH && p0 == 0; // (what this trip's closing steps did, as there is a next tile)
+    tile_id += (int)gridDim.x;
+    tile_origin(tile_id, m0, n0); // (computed again rather than carried across the loop and the write-back in scalar registers)
+    a_tile = a_panel(m0);
+    b_tile = b_panel(n0);
+    if (!came_prefetched) {
         __syncthreads(); // every wave has read its last fragments (stage 3) and is done with its slab
-        first_fills(pa_n, pb_n);
+        first_fills(a_tile, b_tile);
     }
-    came_prefetched = prefetch_next;
-    tile_id = next_id;
-    m0 = m0_next;
-    n0 = n0_next;
-    a_tile = pa_n;
-    b_tile = pb_n;
     } // tiles
 
 }
@@ -530,10 +553,10 @@ hipError_t launch_mfma16w4(const GemmArgs& a, hipStream_t stream, LaunchGeom* ge
     if (Cfg::PERSIST && grid_x > (unsigned)kComputeUnits) grid_x = kComputeUnits;
     args.stagger_groups = args.stagger_ticks = 0;
     if (Cfg::PERSIST && args.tiles_m * args.tiles_n > kComputeUnits) {
-        // measured on int8 8192^3 (four rounds): four groups 3 us apart gain 0.5 %; eight groups, or more than about
+        // measured on int8 8192^3 (four rounds): four groups 1.5 us apart gain 2 %; eight groups, or more than about
         // 10 us in all, lose several per cent (workgroups of an XCD then no longer share their panels in its L2)
         args.stagger_groups = 4;
-        args.stagger_ticks = 300;
+        args.stagger_ticks = 150;
     }
     if (geom) {
         geom->grid[0] = grid_x;
