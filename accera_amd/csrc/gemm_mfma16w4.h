@@ -404,34 +404,27 @@ __global__ void __launch_bounds__(256, 1) gemm_mfma16w4_kernel(GemmArgs p)
     auto write_back = [&](auto epi_tag) __attribute__((always_inline)) {
         constexpr int EPI = decltype(epi_tag)::value;
         constexpr bool RELU = EPI == 1;
-        // row i of the wave tile's blocks, epilogue applied
-        auto load_row = [&](auto i_tag, acc_t (&row)[TN]) __attribute__((always_inline)) {
-            constexpr int i = decltype(i_tag)::value;
-            w4_static_for<0, TN / 2>([&](auto h) {
-                const W4BlockPair pr = w4_acc_pair<i * TN + h.value * 2>();
-                row[h.value * 2] = __builtin_bit_cast(acc_t, pr.a);
-                row[h.value * 2 + 1] = __builtin_bit_cast(acc_t, pr.b);
-            });
-            if constexpr (RELU) {
+        // the epilogue on four finished sums
+        auto finish = [&](acc_t v) __attribute__((always_inline)) {
 #pragma unroll
-                for (int j = 0; j < TN; ++j)
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        if constexpr (IN == IN_I8) row[j][e] = row[j][e] > 0 ? row[j][e] : 0;
-                        else row[j][e] = __builtin_fmaxf(row[j][e], 0.f);
-                    }
-            } else if constexpr (EPI == 2) {
-#pragma unroll
-                for (int j = 0; j < TN; ++j)
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) row[j][e] = apply_epilogue<scalar_t>(row[j][e], p.epilogue, p.epilogue_arg);
+            for (int e = 0; e < 4; ++e) {
+                if constexpr (RELU) {
+                    if constexpr (IN == IN_I8) v[e] = v[e] > 0 ? v[e] : 0;
+                    else v[e] = __builtin_fmaxf(v[e], 0.f);
+                } else if constexpr (EPI == 2) {
+                    v[e] = apply_epilogue<scalar_t>(v[e], p.epilogue, p.epilogue_arg);
+                }
             }
+            return v;
         };
         {
-            // 16 rows of the wave tile are put together in a wave-private slab of the (now idle) tile buffers and leave as
-            // 16-byte pieces that cover whole rows of the wave tile: a store instruction that writes 2 rows x 512 bytes (or
-            // whole rows of a narrow type) passes through a CU's memory pipeline more than twice as fast as one that writes
-            // the accumulator layout's 16 rows x 64 bytes (measured: 256 KB per CU in 2.4-2.9 us against 6.2-7.0 us)
+            // 16 rows of the wave tile (one row of blocks) go from the accumulator registers into a wave-private slab of the
+            // (now idle) tile buffers as they are -- LDS stores take their data from the accumulator file directly, which
+            // saves the 256 register-file moves per wave that every other way out needs -- and come back as whole stretches of
+            // a row: 4 / 8 / 16 neighbouring sums per lane, which get the epilogue, are narrowed to the output type and leave
+            // as one 16-byte store.  A store instruction that writes 2 rows x 512 bytes (or whole rows of a narrow type)
+            // passes through a CU's memory pipeline more than twice as fast as one that writes the accumulator layout's
+            // 16 rows x 64 bytes (measured: 256 KB per CU in 2.4-2.9 us against 6.2-7.0 us).
             __syncthreads();
             // (the lambdas of the write-back are always inlined: left as functions they would take the kernel's state by
             // reference through memory, and everything they capture -- tile origin, descriptors, the call's arguments -- would
@@ -442,60 +435,66 @@ __global__ void __launch_bounds__(256, 1) gemm_mfma16w4_kernel(GemmArgs p)
                 // would push out the A and B panels the workgroups of the XCD share (measured: int8 8192^3 4 % faster, fp16
                 // 4096^3 0.8 %, with the `nt` bit; `sc1` alone changes nothing)
                 constexpr int AUX = 2;
-                constexpr int ROW = WTN * OS;
-                // 16 bytes past a row: the 16 row starts are an odd number of 4-bank steps apart, so a lane group's
-                // 8- or 4-byte pieces of 16 rows land on 64 different banks
-                constexpr int PITCH = ROW + 16;
-                static_assert(ROW % 32 == 0, "(ROW / 16 + 1) must be odd for the 16 row starts to differ mod 64 banks");
-                // (a workgroup that walks several tiles keeps the slabs in stage 3, the stage of the last k-step: the others
-                // may already be receiving the next tile)
+                constexpr int RAW_ROW = WTN * 4;      // a row of the wave tile as 32-bit sums
+                // 16 bytes past a row: the 16 row starts are an odd number of 4-bank steps apart
+                constexpr int PITCH = RAW_ROW + 16;
+                static_assert(RAW_ROW % 32 == 0, "(RAW_ROW / 16 + 1) must be odd for the 16 row starts to differ mod 64 banks");
+                // (a workgroup that walks several tiles keeps the slabs behind stage 2: stage 3 is the stage of the last k-step,
+                // the others may already be receiving the next tile)
                 static_assert((Cfg::PERSIST ? 3 * STAGE_BYTES : 0) + 4 * 16 * PITCH <= Cfg::LDS_BYTES, "four slabs fit (behind the first three stages)");
-                char* slab = smem + (Cfg::PERSIST ? 3 * STAGE_BYTES : 0) + wave_u * (16 * PITCH);
+                const unsigned slab_off = (Cfg::PERSIST ? 3 * STAGE_BYTES : 0) + wave_u * (16 * PITCH);
+                const char* slab = smem + slab_off;
+                const unsigned mine = smem_addr + slab_off + (unsigned)((lane_wb & 15) * PITCH + (lane_wb >> 4) * 16);
                 const CTile tile = c_tile(p, m0 + (wave_u / WAVES_N) * WTM, n0 + (wave_u % WAVES_N) * WTN, OS);
                 const unsigned row_bytes = (unsigned)p.c_rs * OS;
-                constexpr int CPRW = ROW / 16;
-                constexpr int PIECES = (16 * CPRW + 63) / 64;
-                char* mine = slab + (lane_wb & 15) * PITCH + ((lane_wb >> 4) * 4) * OS;
-                // (the accumulator reads of the next row are issued between this row's LDS writes and reads)
-                acc_t row[TN], next_row[TN];
-                load_row(std::integral_constant<int, 0>{}, row);
+                constexpr int VPL = 16 / OS;                 // sums per lane and store
+                constexpr int GPR = WTN / VPL;               // 16-byte pieces of the output per row of the wave tile
+                constexpr int PIECES = (16 * GPR + 63) / 64; // stores per lane and row of blocks
                 w4_static_for<0, TM>([&](auto i) {
-#pragma unroll
-                    for (int j = 0; j < TN; ++j) {
-                        auto w = pack(row[j]);
-                        *(decltype(w)*)(mine + j * 16 * OS) = w;
-                    }
-                    if constexpr (i.value + 1 < TM) load_row(std::integral_constant<int, i.value + 1>{}, next_row);
+                    w4_static_for<0, TN>([&](auto j) {
+                        constexpr int n = (i.value * TN + j.value) * 4;
+                        const unsigned at = mine; // (asm operands do not capture on their own)
+                        asm volatile("ds_write_b128 %0, a[%1:%2] offset:%3" : : "v"(at), "n"(n), "n"(n + 3), "n"(j.value * 64) : "memory");
+                    });
 #pragma unroll
                     for (int it = 0; it < PIECES; ++it) {
                         const int id = it * 64 + lane_wb;
-                        if ((16 * CPRW) % 64 != 0 && id >= 16 * CPRW) break;
-                        const int r = id / CPRW, cc = id % CPRW;
-                        const i32x4 v = *(const i32x4*)(slab + r * PITCH + cc * 16);
-                        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), tile.rsrc, (unsigned)r * row_bytes + cc * 16,
-                                                               (unsigned)(i.value * 16) * row_bytes, AUX);
-                    }
-                    if constexpr (i.value + 1 < TM) {
+                        if ((16 * GPR) % 64 != 0 && id >= 16 * GPR) break;
+                        const int r = id / GPR, g = id % GPR;
+                        acc_t v[VPL / 4];
 #pragma unroll
-                        for (int j = 0; j < TN; ++j) row[j] = next_row[j];
+                        for (int q = 0; q < VPL / 4; ++q) v[q] = finish(*(const acc_t*)(slab + r * PITCH + g * (VPL * 4) + q * 16));
+                        __builtin_amdgcn_raw_buffer_store_b128(pack(v), tile.rsrc, (unsigned)r * row_bytes + g * 16,
+                                                               (unsigned)(i.value * 16) * row_bytes, AUX);
                     }
                 });
             };
-            auto pack_f16 = [](const acc_t& v) -> i32x2 {
-                typedef _Float16 h4 __attribute__((ext_vector_type(4)));
-                return __builtin_bit_cast(i32x2, h4{(_Float16)v[0], (_Float16)v[1], (_Float16)v[2], (_Float16)v[3]});
+            typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+            typedef __bf16 b8 __attribute__((ext_vector_type(8)));
+            auto pack_f16 = [](const acc_t (&v)[2]) -> u32x4 {
+                return __builtin_bit_cast(u32x4, h8{(_Float16)v[0][0], (_Float16)v[0][1], (_Float16)v[0][2], (_Float16)v[0][3],
+                                                    (_Float16)v[1][0], (_Float16)v[1][1], (_Float16)v[1][2], (_Float16)v[1][3]});
             };
-            auto pack_bf16 = [](const acc_t& v) -> i32x2 {
-                typedef __bf16 b4 __attribute__((ext_vector_type(4)));
-                return __builtin_bit_cast(i32x2, b4{(__bf16)v[0], (__bf16)v[1], (__bf16)v[2], (__bf16)v[3]});
+            auto pack_bf16 = [](const acc_t (&v)[2]) -> u32x4 {
+                return __builtin_bit_cast(u32x4, b8{(__bf16)v[0][0], (__bf16)v[0][1], (__bf16)v[0][2], (__bf16)v[0][3],
+                                                    (__bf16)v[1][0], (__bf16)v[1][1], (__bf16)v[1][2], (__bf16)v[1][3]});
             };
-            auto pack_i16 = [](const acc_t& v) -> i32x2 {
-                return i32x2{(int)(((unsigned)v[0] & 0xffffu) | ((unsigned)v[1] << 16)), (int)(((unsigned)v[2] & 0xffffu) | ((unsigned)v[3] << 16))};
+            auto pack_i16 = [](const acc_t (&v)[2]) -> u32x4 {
+                u32x4 w;
+#pragma unroll
+                for (int q = 0; q < 2; ++q)
+#pragma unroll
+                    for (int h = 0; h < 2; ++h) w[q * 2 + h] = ((unsigned)v[q][2 * h] & 0xffffu) | ((unsigned)v[q][2 * h + 1] << 16);
+                return w;
             };
-            auto pack_i8 = [](const acc_t& v) -> int {
-                return (int)(((unsigned)v[0] & 0xffu) | (((unsigned)v[1] & 0xffu) << 8) | (((unsigned)v[2] & 0xffu) << 16) | ((unsigned)v[3] << 24));
+            auto pack_i8 = [](const acc_t (&v)[4]) -> u32x4 {
+                u32x4 w;
+#pragma unroll
+                for (int q = 0; q < 4; ++q)
+                    w[q] = ((unsigned)v[q][0] & 0xffu) | (((unsigned)v[q][1] & 0xffu) << 8) | (((unsigned)v[q][2] & 0xffu) << 16) | ((unsigned)v[q][3] << 24);
+                return w;
             };
-            auto pack_32 = [](const acc_t& v) -> i32x4 { return __builtin_bit_cast(i32x4, v); };
+            auto pack_32 = [](const acc_t (&v)[1]) -> u32x4 { return __builtin_bit_cast(u32x4, v[0]); };
             if (os == 4) staged(std::integral_constant<int, 4>{}, pack_32);
             else if constexpr (IN == IN_I8) {
                 if (os == 2) staged(std::integral_constant<int, 2>{}, pack_i16);
