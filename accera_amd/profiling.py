@@ -41,7 +41,9 @@ def _dominant(acc, counter):
             continue
         if not any(s in k for s in ("gemm_mfma_kernel", "gemm_mfma16_kernel", "gemm_mfma16w4_kernel", "gemm_skinny", "gemm_f32_kernel", "gemm_generic_kernel")):
             continue
-        if re.search(r"Config<[^>]*, true>\s*>", k):  # the build with clock stamps (last template argument), run by the phase probe
+        # the builds with clock stamps, run by the phase probe: third argument of Mfma16W4Config, last one of the others
+        if re.search(r"Mfma16W4Config<[^,>]*,[^,>]*, true\b", k) or (
+                "Mfma16W4Config" not in k and re.search(r"Config<[^>]*, true>\s*>", k)):
             continue
         tot = sum(cs[counter])
         if best is None or tot > best[1]:
