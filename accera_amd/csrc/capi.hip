@@ -142,7 +142,7 @@ bool mfma_can_take(const MfmaVariant& v, const Problem& pb)
         if (pb.have_pointers && !aligned16(g.C)) return false;
         // any M, N >= one tile when C is only written: the last row / column of tiles is moved to end at M / N
         // (its first column must still be 16 bytes aligned in B's and C's rows)
-        if (g.M % v.bm && (g.M < v.bm || g.prologue != PRO_SET)) return false;
+        if (g.M % v.bm && (g.M < v.bm || g.prologue != PRO_SET || (!v.a_kc && g.M % vec))) return false;
         if (g.N % v.bn && (g.N < v.bn || g.prologue != PRO_SET || g.N % vec || (g.N * os) % 16)) return false;
         if (g.K % bk) return false;
     }

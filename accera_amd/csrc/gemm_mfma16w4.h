@@ -13,7 +13,8 @@
 // moves accumulators between the register files and spills.  Tile staging, the LDS layout and
 // the stores are those of gemm_mfma16.h.
 //
-// Takes: A row-major, M and N multiples of the tile (any M >= 256 and any 16-byte-aligned N >= the tile width
+// Takes: A row-major (or column-major, in the one-tile-per-workgroup form with 256-wide tiles: staged as it lies in memory and
+// read with the transposing LDS loads, like a row-major B), M and N multiples of the tile (any M >= 256 and any 16-byte-aligned N >= the tile width
 // when C is not read: the last row / column of tiles then overlaps the one before), K a multiple of one k-step (64 bytes)
 // and at least four of them, rows of C 16 bytes aligned;
 // every prologue / epilogue op (an int8 C is only written, never read): C = A*B starts from zeros, C += A*B with a
@@ -28,12 +29,13 @@ namespace acc950 {
 // BN: 256, or 192 (K-contiguous B only; N = 3072 = 16 x 192 gives one tile per CU) with 128x96 wave tiles
 // PERSIST: one workgroup per CU walks several output tiles (grid = min(tiles, CUs)); the closing k-steps of a tile
 // fetch the first K tiles of the next one, and that tile's loop starts while this tile's stores are still on their way.
-template <int IN_, bool B_KC_, bool TIMED_ = false, int BN_ = 256, bool PERSIST_ = false>
+template <int IN_, bool B_KC_, bool TIMED_ = false, int BN_ = 256, bool PERSIST_ = false, bool A_KC_ = true>
 struct Mfma16W4Config {
     static constexpr bool TIMED = TIMED_, PERSIST = PERSIST_;
     static_assert(!PERSIST_ || BN_ == 256, "the 192-wide tile is for problems of one tile per CU");
     static constexpr int IN = IN_, BM = 256, BN = BN_, WAVES_M = 2, WAVES_N = 2, KB = 64, STAGES = 4, NT = 256;
-    static constexpr bool A_KC = true, B_KC = B_KC_;
+    static constexpr bool A_KC = A_KC_, B_KC = B_KC_;
+    static_assert(A_KC_ || (BN_ == 256 && !PERSIST_), "column-major A: 256-wide tiles, one per workgroup");
     // (a workgroup that walks several tiles stages its write-back behind the last LDS stage while the others already receive
     // the next tile: it asks for the whole LDS of the CU)
     static constexpr int LDS_BYTES = PERSIST_ ? 160 * 1024 : STAGES * (BM + BN) * KB;
@@ -68,13 +70,13 @@ template <typename Cfg>
 __global__ void __launch_bounds__(256, 1) gemm_mfma16w4_kernel(GemmArgs p)
 {
     constexpr int IN = Cfg::IN, BM = 256, BN = Cfg::BN, NT = 256, KB = 64, WAVES_N = 2;
-    constexpr bool B_KC = Cfg::B_KC;
+    constexpr bool A_KC = Cfg::A_KC, B_KC = Cfg::B_KC;
     constexpr int ES = InTraits<IN>::ES;
     constexpr int BK = KB / ES;
     constexpr int WTM = 128, WTN = BN / 2, TM = 8, TN = WTN / 16;
     constexpr int FILLS_B = BN * KB / (NT * 16), FILLS = 4 + FILLS_B; // fill instructions per thread and K tile
     // (swizzle and address arithmetic only: these are the tiles of the eight-wave kernel)
-    using TA = OperandTile<IN, BM, true, 512, KB, true>;
+    using TA = OperandTile<IN, BM, A_KC, 512, KB, true>;
     using TB = OperandTile<IN, BN, B_KC, 512, KB, true>;
     using acc_t = typename In16Traits<IN>::acc_t;
     using scalar_t = typename In16Traits<IN>::scalar_t;
@@ -131,7 +133,7 @@ __global__ void __launch_bounds__(256, 1) gemm_mfma16w4_kernel(GemmArgs p)
 
     const char* Ab = (const char*)p.A;
     const char* Bb = (const char*)p.B;
-    const int64_t lda = p.a_rs;
+    const int64_t lda = A_KC ? p.a_rs : p.a_cs;
     const int64_t ldb = B_KC ? p.b_cs : p.b_rs;
     const int KT = p.K / BK;
 
@@ -146,7 +148,15 @@ __global__ void __launch_bounds__(256, 1) gemm_mfma16w4_kernel(GemmArgs p)
     // the 16-row ds_read_b128 of a fragment is free of bank conflicts (the row/4 map of the eight-wave
     // kernel costs two passes; there the sibling wave's MFMAs hide it, here nothing does).
     auto kc_swz = [](int row) { return ((row >> 1) & 1) | ((((row >> 1) ^ (row >> 2)) & 1) << 1); };
-    const unsigned a_off = (unsigned)TA::global_off(tid / 4, (tid % 4) ^ kc_swz(tid / 4), 0, 0, lda);
+    constexpr int A_CPR = TA::CPR;
+    constexpr int A_RPP = NT / A_CPR;
+    unsigned a_off, a_off1;
+    if constexpr (A_KC) {
+        a_off = a_off1 = (unsigned)TA::global_off(tid / 4, (tid % 4) ^ kc_swz(tid / 4), 0, 0, lda);
+    } else {
+        a_off = (unsigned)TA::global_off(tid / A_CPR, TA::swizzle(tid / A_CPR, tid % A_CPR), 0, 0, lda);
+        a_off1 = (unsigned)TA::global_off(tid / A_CPR, TA::swizzle(tid / A_CPR + A_RPP, tid % A_CPR), 0, 0, lda);
+    }
     unsigned b_off0, b_off1;
     if constexpr (B_KC) {
         b_off0 = b_off1 = (unsigned)TB::global_off(tid / 4, (tid % 4) ^ kc_swz(tid / 4), 0, 0, ldb);
@@ -154,11 +164,11 @@ __global__ void __launch_bounds__(256, 1) gemm_mfma16w4_kernel(GemmArgs p)
         b_off0 = (unsigned)TB::global_off(tid / B_CPR, TB::swizzle(tid / B_CPR, tid % B_CPR), 0, 0, ldb);
         b_off1 = (unsigned)TB::global_off(tid / B_CPR, TB::swizzle(tid / B_CPR + B_RPP, tid % B_CPR), 0, 0, ldb);
     }
-    const unsigned da = __builtin_amdgcn_readfirstlane((unsigned)(64 * lda * ES));
+    const unsigned da = __builtin_amdgcn_readfirstlane((unsigned)((A_KC ? 64 : A_RPP) * lda * ES));
     const unsigned db = __builtin_amdgcn_readfirstlane((unsigned)((B_KC ? 64 : B_RPP) * ldb * ES));
-    const unsigned sa = KB;
+    const unsigned sa = __builtin_amdgcn_readfirstlane(A_KC ? (unsigned)KB : (unsigned)(BK * lda * ES));
     const unsigned sb = __builtin_amdgcn_readfirstlane(B_KC ? (unsigned)KB : (unsigned)(BK * ldb * ES));
-    auto a_panel = [&](int r0) __attribute__((always_inline)) { return Ab + (int64_t)r0 * lda * ES; };
+    auto a_panel = [&](int r0) __attribute__((always_inline)) { return Ab + (A_KC ? (int64_t)r0 * lda * ES : (int64_t)r0 * ES); };
     auto b_panel = [&](int c0) __attribute__((always_inline)) { return Bb + (B_KC ? (int64_t)c0 * ldb * ES : (int64_t)c0 * ES); };
     const char* a_tile = a_panel(m0);
     const char* b_tile = b_panel(n0);
@@ -169,7 +179,7 @@ __global__ void __launch_bounds__(256, 1) gemm_mfma16w4_kernel(GemmArgs p)
     // With paired fills a K-contiguous B is fetched two K tiles at a time on the even positions of the loop's pattern
     // (both 64-byte halves of a cache line in neighbouring requests), so its third tile is issued here only when the
     // first k-step sits at an odd position; otherwise the loop's first step fetches tiles 2 and 3.
-    constexpr bool B_PAIRED = B_KC && (BN == 192 || IN == IN_I8); // measured: behind the plain scheme for 16-bit inputs on 256-wide tiles
+    constexpr bool B_PAIRED = A_KC && B_KC && (BN == 192 || IN == IN_I8); // measured: behind the plain scheme for 16-bit inputs on 256-wide tiles
     const unsigned b_tiles_here = B_PAIRED ? 2u + (p0 & 1u) : 3u;
     // the first three K tiles of an output tile, issued ahead of its loop
     // (always inline: the panel addresses are scalar-register operands of the fill instructions)
@@ -179,7 +189,7 @@ __global__ void __launch_bounds__(256, 1) gemm_mfma16w4_kernel(GemmArgs p)
             const unsigned stage = ldsb + ((s + p0) & 3) * STAGE_BYTES;
 #pragma unroll
             for (int f = 0; f < 4; ++f)
-                TA::direct_issue_uniform(stage + f * 4096, a_off, a_src + (int64_t)s * sa + (int64_t)f * da);
+                TA::direct_issue_uniform(stage + f * 4096, (f & 1) ? a_off1 : a_off, a_src + (int64_t)s * sa + (int64_t)f * da);
             if ((unsigned)s < b_tiles_here) {
 #pragma unroll
                 for (int f = 0; f < FILLS_B; ++f)
@@ -192,7 +202,17 @@ __global__ void __launch_bounds__(256, 1) gemm_mfma16w4_kernel(GemmArgs p)
 
     // ---- LDS addresses of the fragment reads (stage 0; the loop adds stage and block offsets)
     const int kg = lane >> 4, li = lane & 15;
-    const unsigned a_rd = smem_addr + (unsigned)((wr0 + li) * 64 + (kg ^ kc_swz(li)) * 16);
+    // (a column-major A: the address of the wave's first block of rows; the loop derives the other seven from it, which
+    // differ in the bits of the block number only -- the swizzle is an XOR and every k row of the tile starts on a multiple of its length)
+    unsigned a_rd;
+    if constexpr (A_KC) a_rd = smem_addr + (unsigned)((wr0 + li) * 64 + (kg ^ kc_swz(li)) * 16);
+    else if constexpr (ES == 2) {
+        const int col_byte = (wr0 + (li & 3) * 4) * 2, k = kg * 8 + (li >> 2);
+        a_rd = smem_addr + (unsigned)(k * TA::ROW_BYTES + TA::swizzle(k, col_byte >> 4) * 16 + (col_byte & 15));
+    } else {
+        const int col_byte = wr0 + (li & 1) * 8, k = kg * 16 + (li >> 1);
+        a_rd = smem_addr + (unsigned)(k * TA::ROW_BYTES + TA::swizzle(k, col_byte >> 4) * 16 + (col_byte & 15));
+    }
     unsigned b_rd[8];
     if constexpr (B_KC) {
 #pragma unroll
@@ -350,6 +370,7 @@ __global__ void __launch_bounds__(256, 1) gemm_mfma16w4_kernel(GemmArgs p)
 #define ACC950_W4_OPERANDS                                                                                              \
     : [a_rd] "v"(a_rd), [b_rd0] "v"(b_rd[0]), [b_rd1] "v"(b_rd[1]), [b_rd2] "v"(b_rd[2]), [b_rd3] "v"(b_rd[3]),          \
       [b_rd4] "v"(b_rd[4]), [b_rd5] "v"(b_rd[5]), [b_rd6] "v"(b_rd[6]), [b_rd7] "v"(b_rd[7]), [a_off] "v"(a_off),        \
+      [a_off1] "v"(a_off1),                                                                                               \
       [b_off0] "v"(b_off0), [b_off1] "v"(b_off1), [pa] "s"(pa), [pb] "s"(pb), [da] "s"(da), [db] "s"(db), [sa] "s"(sa),   \
       [sb] "s"(sb), [ldsb] "s"(ldsb), [groups] "s"(groups), [accum] "s"(accum), [c_off] "v"(c_off), [p0] "s"(p0),       \
       [c_rsrc] "s"(c_rsrc), [c_row16] "s"(c_row16), [pa_n] "s"(pa_n_u), [pb_n] "s"(pb_n_u), [flags] "s"(flags)               \
@@ -365,7 +386,18 @@ __global__ void __launch_bounds__(256, 1) gemm_mfma16w4_kernel(GemmArgs p)
 #define ACC950_W4_R(f, d) f #d "0", f #d "1", f #d "2", f #d "3", f #d "4", f #d "5", f #d "6", f #d "7", f #d "8", f #d "9"
 #define ACC950_W4_V(d) ACC950_W4_R("v", d)
 #define ACC950_W4_A(d) ACC950_W4_R("a", d)
-    if constexpr (B_KC && BN == 192) {
+    if constexpr (!A_KC) {
+        if constexpr (IN == IN_I8) {
+            if constexpr (B_KC) asm volatile(ACC950_W4_LOOP_KC_AMC8("v_mfma_i32_16x16x64_i8") : ACC950_W4_OPERANDS);
+            else asm volatile(ACC950_W4_LOOP_MC8_AMC8("v_mfma_i32_16x16x64_i8") : ACC950_W4_OPERANDS);
+        } else if constexpr (B_KC) {
+            if constexpr (IN == IN_F16) asm volatile(ACC950_W4_LOOP_KC_AMC16("v_mfma_f32_16x16x32_f16") : ACC950_W4_OPERANDS);
+            else asm volatile(ACC950_W4_LOOP_KC_AMC16("v_mfma_f32_16x16x32_bf16") : ACC950_W4_OPERANDS);
+        } else {
+            if constexpr (IN == IN_F16) asm volatile(ACC950_W4_LOOP_MC16_AMC16("v_mfma_f32_16x16x32_f16") : ACC950_W4_OPERANDS);
+            else asm volatile(ACC950_W4_LOOP_MC16_AMC16("v_mfma_f32_16x16x32_bf16") : ACC950_W4_OPERANDS);
+        }
+    } else if constexpr (B_KC && BN == 192) {
         if constexpr (IN == IN_F16) asm volatile(ACC950_W4_LOOP_KCP6("v_mfma_f32_16x16x32_f16") : ACC950_W4_OPERANDS);
         else if constexpr (IN == IN_BF16) asm volatile(ACC950_W4_LOOP_KCP6("v_mfma_f32_16x16x32_bf16") : ACC950_W4_OPERANDS);
         else asm volatile(ACC950_W4_LOOP_KCP6("v_mfma_i32_16x16x64_i8") : ACC950_W4_OPERANDS);

@@ -30,6 +30,9 @@ namespace acc950 {
 // the same, one workgroup per CU walking several output tiles
 #define V16W4P(BKC) \
     { 256, 256, 2, 2, true, BKC, true, false, 64, 4, false, true, true, true, &launch_mfma16w4<Mfma16W4Config<ACC950_IN, BKC, false, 256, true>>, nullptr }
+// the same kernel for a column-major A (one tile per workgroup)
+#define V16W4A(BKC) \
+    { 256, 256, 2, 2, false, BKC, true, false, 64, 4, false, true, true, false, &launch_mfma16w4<Mfma16W4Config<ACC950_IN, BKC, false, 256, false, false>>, nullptr }
 #define V(BM, BN, WM, WN, BKC, DIRECT, EDGE, KB, STAGES) VA(true, BM, BN, WM, WN, BKC, DIRECT, EDGE, KB, STAGES)
 #define VP(BM, BN, WM, WN, BKC, KB, STAGES) VPA(true, BM, BN, WM, WN, BKC, KB, STAGES)
 // column-major A (M contiguous; the "transA" shapes of the reference's sweep lists,
@@ -76,6 +79,8 @@ static const MfmaVariant kVariants[] = {
     V16W4_192,
     V16W4P(false),
     V16W4P(true),
+    V16W4A(false),
+    V16W4A(true),
 };
 #undef LAYOUT_AT
 #undef VA
@@ -84,6 +89,7 @@ static const MfmaVariant kVariants[] = {
 #undef V16W4
 #undef V16W4_192
 #undef V16W4P
+#undef V16W4A
 #undef LAYOUT
 #undef V
 #undef VP

@@ -26,6 +26,7 @@ Register use (besides the operands the C++ side passes in):
     v[128:191]  fragments of even steps: B blocks 0..7 (v128..), A blocks 0..7 (v160..)
     v[192:255]  fragments of odd steps
     v[104:121]  LDS read addresses of the upper two stages (the 16-bit offset field reaches 64 KB)
+    v[114:127], v103  column-major A only: the read addresses of A's blocks 1..7 (lower two stages) and 0..7 (upper two)
     s[72:73], s[74:75]  fill pointers of A and B (the next tile to fetch); s[76:77], s[80:81] scratch pointers; s78 loop count;
     s79 row offset while C is loaded
 """
@@ -34,6 +35,8 @@ FRAG = 1024        # 16 rows x 64 bytes (K-contiguous operand)
 TN = 8             # blocks of 16 columns per wave: 8 (256-wide tile) or 6 (192-wide, K-contiguous B only)
 STAGE = 32768      # A's tile + B's tile (2 * TN * 16 rows x 64 bytes)
 RELAX_STORES = 47  # stores per thread the relaxed first k-steps of a later tile count on (see loop(): 2 tiles' fills + 47 = 63)
+A_LAYOUT = "kc"    # "kc": A row-major (K contiguous); "mc16" / "mc8": A as it lies in memory when column-major (M contiguous)
+A_LOW = ["%[a_rd]", "v122", "v123", "v124", "v125", "v126", "v127", "v103"]  # column-major A: read addresses of the lower two stages
 
 
 def set_width(tn):
@@ -67,10 +70,19 @@ def line(s):
 
 
 def read_a(x, stage, buf):
-    base = "%[a_rd]" if stage < 2 else "v104"
-    off = (stage & 1) * STAGE + x * FRAG
     n = afrag(buf, x)
-    return [line(f"ds_read_b128 v[{n}:{n + 3}], {base} offset:{off}")]
+    if A_LAYOUT == "kc":
+        base = "%[a_rd]" if stage < 2 else "v104"
+        off = (stage & 1) * STAGE + x * FRAG
+        return [line(f"ds_read_b128 v[{n}:{n + 3}], {base} offset:{off}")]
+    # column-major A is staged as it lies in memory (M contiguous) and read like a row-major B
+    op = "ds_read_b64_tr_b16" if A_LAYOUT == "mc16" else "ds_read_b64_tr_b8"
+    base = A_LOW[x] if stage < 2 else f"v{114 + x}"
+    out = []
+    for q in range(2):
+        off = (stage & 1) * STAGE + q * 2048
+        out.append(line(f"{op} v[{n + 2 * q}:{n + 2 * q + 1}], {base} offset:{off}"))
+    return out
 
 
 def read_b(x, stage, buf, b_layout):
@@ -94,7 +106,8 @@ def fill(f, stage, b_layout):
     """Fill instruction f (0..3 A, 4.. B) of a K tile as a list of MFMA slots: pointer, M0, the load (the MFMA
     between the M0 write and the load is the wait state M0 needs; the last pass also advances the pointer)."""
     if f < 4:
-        ptr, d, s, lane, tile, g, last = "s[72:73]", "%[da]", "%[sa]", "%[a_off]", 0, f, 3
+        ptr, d, s, tile, g, last = "s[72:73]", "%[da]", "%[sa]", 0, f, 3
+        lane = "%[a_off]" if (A_LAYOUT == "kc" or g % 2 == 0) else "%[a_off1]"
     else:
         g = f - 4
         ptr, d, s, tile, last = "s[74:75]", "%[db]", "%[sb]", B_TILE, (2 * TN * FRAG) // 4096 - 1
@@ -207,8 +220,17 @@ def loop(b_layout, persist=False):
            that does not know of the stores would wait for nearly all of them).  Entry at position 0 and at least one
            trip through the body (the copy counts as one)."""
     assert not (persist and b_layout == "kcp")
-    out = [line("s_mov_b64 s[72:73], %[pa]"), line("s_mov_b64 s[74:75], %[pb]"), line("s_mov_b32 s78, %[groups]"),
-           line(f"v_add_u32 v104, {2 * STAGE}, %[a_rd]")]
+    out = [line("s_mov_b64 s[72:73], %[pa]"), line("s_mov_b64 s[74:75], %[pb]"), line("s_mov_b32 s78, %[groups]")]
+    if A_LAYOUT == "kc":
+        out.append(line(f"v_add_u32 v104, {2 * STAGE}, %[a_rd]"))
+    else:
+        # block x of the wave's rows lies x * 32 (16-bit) or x * 16 (8-bit) bytes further along every k row of the tile, and
+        # the swizzle is an XOR on those address bits (rows of the tile start on multiples of their length)
+        assert not persist and TN == 8
+        for x in range(1, 8):
+            out.append(line(f"v_xor_b32 {A_LOW[x]}, {x * (32 if A_LAYOUT == 'mc16' else 16)}, %[a_rd]"))
+        for x in range(8):
+            out.append(line(f"v_add_u32 v{114 + x}, {2 * STAGE}, {A_LOW[x]}"))
     if b_layout in ("kc", "kcp"):
         out.append(line(f"v_add_u32 v105, {2 * STAGE}, %[b_rd0]"))
     else:
@@ -293,6 +315,20 @@ def main():
         set_width(8)
         body = loop(name, persist=True)
         print(f"#define ACC950_W4_LOOP_{name.upper()}_P(MFMA) \\")
+        print(" \\\n".join("    " + s for s in body))
+        print()
+    main_a_mc()
+
+
+def main_a_mc():
+    """The loops for a column-major A (one macro per pair of layouts; one workgroup per tile only)."""
+    global A_LAYOUT
+    for a_name, b_name in (("mc16", "kc"), ("mc16", "mc16"), ("mc8", "kc"), ("mc8", "mc8")):
+        set_width(8)
+        A_LAYOUT = a_name
+        body = loop(b_name)
+        A_LAYOUT = "kc"
+        print(f"#define ACC950_W4_LOOP_{b_name.upper()}_A{a_name.upper()}(MFMA) \\")
         print(" \\\n".join("    " + s for s in body))
         print()
 

@@ -14,7 +14,7 @@ struct MfmaVariant {
     int stages;          // LDS buffers
     bool pingpong;       // sibling waves alternate memory and compute clusters
     bool mi16;           // 16x16 MFMA shapes (else 32x32)
-    bool w4;             // four waves with 128x128 wave tiles and the hand-laid K loop: row-major A, at least four K tiles, an int8 C only written
+    bool w4;             // four waves with 128x128 wave tiles and the hand-laid K loop: at least four K tiles, an int8 C only written
     bool persist;        // w4 only: one workgroup per CU walks several output tiles, the next tile's first fills overlap this tile's end
     LaunchFn launch;
     LaunchFn launch_general; // build that carries every prologue / epilogue op, when `launch` is a lean build (else null)

@@ -91,8 +91,8 @@ def test_mfma_all_variants_narrow_integer_outputs(out_type):
             bm, bn = map(int, re.search(r"mfma (\d+)x(\d+)", name).groups())
             M, N = max(512, 2 * bm), (max(512, 2 * bn) if 512 % bn == 0 else 3 * bn)
             if "hand-laid" in name:  # C = A*B and relu(A*B) only, K in steps of four tiles
-                run_case("i8", out_type, M, N, 4 * kb, b_layout=b_layout, variant=v, seed=v)
-                run_case("i8", out_type, M, N, 12 * kb, b_layout=b_layout, variant=v, seed=v + 1, epilogue=ora.EPI_NONE)
+                run_case("i8", out_type, M, N, 4 * kb, b_layout=b_layout, variant=v, seed=v, a_layout=a_layout)
+                run_case("i8", out_type, M, N, 12 * kb, b_layout=b_layout, variant=v, seed=v + 1, epilogue=ora.EPI_NONE, a_layout=a_layout)
                 continue
             run_case("i8", out_type, M, N, 2 * kb, b_layout=b_layout, variant=v, seed=v, a_layout=a_layout)
             run_case("i8", out_type, M, N, 3 * kb, b_layout=b_layout, variant=v, seed=v + 1, a_layout=a_layout, prologue=ora.PRO_NONE)
@@ -140,7 +140,49 @@ def test_column_major_a_takes_the_mfma_kernels():
             run_case(in_type, out_type, 512, 768, 1024, a_layout="col", b_layout=b_layout, seed=11)
             run_case(in_type, out_type, 384, 128, 256, a_layout="col", b_layout=b_layout, seed=12, prologue=ora.PRO_NONE)
     g, b, lds, v = _lib.launch_geometry(_lib.F16, _lib.F32, 4096, 4096, 4096, (1, 4096), (4096, 1), (4096, 1))
-    assert "A=col-major" in _lib.variant_name(v) and "pingpong" in _lib.variant_name(v)
+    assert "A=col-major" in _lib.variant_name(v) and "hand-laid" in _lib.variant_name(v)
+
+
+@pytest.mark.parametrize("in_type,out_type", [("f16", "f32"), ("f16", "f16"), ("bf16", "bf16"), ("i8", "i32"), ("i8", "i8")])
+@pytest.mark.parametrize("b_layout", ["row", "col"])
+def test_four_wave_kernel_column_major_a(in_type, out_type, b_layout):
+    """The hand-laid kernel's form for a column-major A (staged as it lies in memory, read with the transposing LDS
+    loads), named explicitly: every position the K loop can be entered at, both wave rows and columns, C overwritten
+    and accumulated into, ragged M and N, and views of larger matrices (fill strides that differ from the extents)."""
+    import accera_amd as acc
+    import torch
+    from accera_amd import _lib
+    kb = 64 if in_type == "i8" else 32
+    vec = 16 if in_type == "i8" else 8
+    variants = [v for v, n in _variants(b_layout) if "hand-laid" in n and "A=col-major" in n]
+    assert len(variants) == 1
+    v = variants[0]
+    for k_tiles, epi in ((4, ora.EPI_RELU), (5, ora.EPI_NONE), (6, ora.EPI_RELU), (7, ora.EPI_RELU), (8, ora.EPI_NONE), (21, ora.EPI_RELU)):
+        print("variant", v, in_type, out_type, b_layout, "k tiles", k_tiles, flush=True)
+        run_case(in_type, out_type, 512, 768, k_tiles * kb, a_layout="col", b_layout=b_layout, variant=v, seed=900 + k_tiles, epilogue=epi)
+    if out_type != "i8":
+        print("variant", v, in_type, out_type, b_layout, "accumulating", flush=True)
+        run_case(in_type, out_type, 512, 512, 6 * kb, a_layout="col", b_layout=b_layout, variant=v, seed=931, prologue=ora.PRO_NONE)
+    # ragged M (a multiple of the 16-byte vector: the last row of tiles starts at M - 256) and ragged N
+    print("variant", v, in_type, out_type, b_layout, "ragged", flush=True)
+    run_case(in_type, out_type, 256 + 5 * vec, 512 + 3 * 16, 8 * kb, a_layout="col", b_layout=b_layout, variant=v, seed=932)
+    with pytest.raises(_lib.Acc950Error):  # the last row of tiles would start in the middle of a 16-byte piece of A's columns
+        run_case(in_type, out_type, 256 + vec // 2, 512, 8 * kb, a_layout="col", b_layout=b_layout, variant=v, seed=933)
+    # views: A is the transpose of the first M columns of a wider K x (M + pad) array
+    rng = np.random.default_rng(934)
+    M, N, K = 512, 512, 6 * kb
+    Abig = make_input(rng, (K, M + 3 * vec), in_type)
+    Bbig = make_input(rng, (N, K + vec) if b_layout == "col" else (K, N + 2 * vec), in_type)
+    Bview = Bbig[:, :K].T if b_layout == "col" else Bbig[:, :N]
+    Cbig = make_c0(rng, (M, N + 16), out_type)
+    dA, dB, dC = to_device(Abig, in_type), to_device(Bbig, in_type), to_device(Cbig, out_type)
+    print("variant", v, in_type, out_type, b_layout, "views", flush=True)
+    acc.gemm_relu(dA[:, :M].t(), dB[:, :K].t() if b_layout == "col" else dB[:, :N], dC[:, :N], variant=v)
+    torch.cuda.synchronize()
+    got = to_host(dC, out_type)
+    want = ora.gemm_relu_exact(np.ascontiguousarray(Abig[:, :M].T), np.ascontiguousarray(Bview), None, in_type, out_type)
+    assert_matches(got[:, :N], want, out_type, K)
+    assert np.array_equal(got[:, N:], Cbig[:, N:]), "columns beside the view were written"
 
 
 def test_mfma_single_k_tile_and_many_tiles():
@@ -237,7 +279,7 @@ def test_large_tile_kernels_on_padded_output_rows(in_type, out_type, pad):
 
 def _hand_laid(b_layout):
     from accera_amd import _lib
-    return next(v for v, n in _variants(b_layout) if "hand-laid" in n)
+    return next(v for v, n in _variants(b_layout) if "hand-laid" in n and "A=col-major" not in n)
 
 
 @pytest.mark.parametrize("in_type,out_type", [("f16", "f32"), ("f16", "f16"), ("bf16", "bf16"), ("bf16", "f32"),
@@ -249,7 +291,7 @@ def test_four_wave_kernel_every_output_type(in_type, out_type, b_layout):
     LDS), 6 output tiles so that the tile map and both wave rows / columns are exercised, K at one,
     two and five rounds of the four LDS stages."""
     kb = 64 if in_type == "i8" else 32
-    for v in [v for v, n in _variants(b_layout) if "hand-laid" in n]:  # 256x256, and 256x192 for column-major B
+    for v in [v for v, n in _variants(b_layout) if "hand-laid" in n and "A=col-major" not in n]:  # 256x256, and 256x192 for column-major B
         for k_tiles, epi in ((4, ora.EPI_RELU), (8, ora.EPI_NONE), (20, ora.EPI_RELU)):
             print("variant", v, in_type, out_type, b_layout, "k tiles", k_tiles, flush=True)
             run_case(in_type, out_type, 512, 768, k_tiles * kb, b_layout=b_layout, variant=v, seed=700 + k_tiles, epilogue=epi)
@@ -270,7 +312,7 @@ def test_four_wave_kernel_on_views_of_larger_matrices(in_type, out_type, b_layou
     rng = np.random.default_rng(41)
     M, N, K = 512, 768, 256 if in_type == "i8" else 384
     esz = 1 if in_type == "i8" else 2
-    for v in [v for v, n in _variants(b_layout) if "hand-laid" in n]:
+    for v in [v for v, n in _variants(b_layout) if "hand-laid" in n and "A=col-major" not in n]:
         Abig = make_input(rng, (M, K + 128 // esz), in_type)
         Bbig = make_input(rng, (N, K + 64 // esz) if b_layout == "col" else (K, N + 256 // esz), in_type)
         Bview = Bbig[:, :K].T if b_layout == "col" else Bbig[:, :N]
@@ -297,7 +339,7 @@ def test_four_wave_kernel_any_number_of_rows(in_type, out_type, M):
     from accera_amd import _lib
     kb = 64 if in_type == "i8" else 32
     for b_layout in ("row", "col"):
-        for v in [v for v, n in _variants(b_layout) if "hand-laid" in n]:
+        for v in [v for v, n in _variants(b_layout) if "hand-laid" in n and "A=col-major" not in n]:
             print("variant", v, in_type, out_type, b_layout, "M", M, flush=True)
             run_case(in_type, out_type, M, 768, 8 * kb, b_layout=b_layout, variant=v, seed=M)
             run_case(in_type, out_type, M, 768 + 16 + 64 * (M % 3), 4 * kb, b_layout=b_layout, variant=v, seed=M + 1)  # N ragged too
@@ -744,7 +786,7 @@ def test_random_problems_on_the_four_wave_kernel():
     for case in range(48):
         in_type, out_type = pairs[rng.integers(len(pairs))]
         b_layout = ("row", "col")[rng.integers(2)]
-        variants = [v for v, n in _variants(b_layout) if "hand-laid" in n]
+        variants = [v for v, n in _variants(b_layout) if "hand-laid" in n and "A=col-major" not in n]
         v = variants[rng.integers(len(variants))]
         kb = 64 if in_type == "i8" else 32
         pro, pa, epi, ea = ops[rng.integers(len(ops))]

@@ -342,3 +342,84 @@ def test_relaxed_first_steps_need_the_stores_they_count_on():
     g = _gen()
     with pytest.raises(AssertionError):
         _run_fills(g, "mc8", 8, 8, 3, persist=True, flags=2, stores_in_flight=40)
+
+
+@pytest.mark.parametrize("a_layout,b_layout", [("mc16", "kc"), ("mc16", "mc16"), ("mc8", "kc"), ("mc8", "mc8")])
+def test_loops_for_a_column_major_a(a_layout, b_layout):
+    """A staged as it lies in memory (M contiguous): its fragments come from transposing reads, two per block, from
+    per-block addresses the preamble derives from block 0's; its fill passes alternate between two lane offsets."""
+    g = _gen()
+    g.set_width(8)
+    g.A_LAYOUT = a_layout
+    try:
+        ins = _text(g.loop(b_layout))
+        steps = {pos: _text(g.step(pos, True, 16, False, b_layout)) for pos in range(4)}
+    finally:
+        g.A_LAYOUT = "kc"
+    # ---- preamble: blocks 1..7 of the lower stages by XOR, all eight of the upper stages 2 * STAGE further
+    pre = ins[:ins.index("4:")]
+    unit = 32 if a_layout == "mc16" else 16
+    low = ["%[a_rd]"] + [None] * 7
+    for i in pre:
+        m = re.match(r"v_xor_b32 (v\d+), (\d+), %\[a_rd\]$", i)
+        if m:
+            x = int(m.group(2)) // unit
+            assert int(m.group(2)) == x * unit and 1 <= x <= 7 and low[x] is None
+            low[x] = m.group(1)
+    assert None not in low and len(set(low)) == 8
+    up = {}
+    for i in pre:
+        m = re.match(rf"v_add_u32 (v\d+), {2 * g.STAGE}, (\S+)$", i)
+        if m and m.group(2) in low:
+            up[low.index(m.group(2))] = m.group(1)
+    assert sorted(up) == list(range(8))
+    regs = [int(r[1:]) for r in low[1:] + list(up.values())]
+    b_regs = set(range(106, 114)) if b_layout != "kc" else {105}
+    assert len(set(regs)) == 15 and all(100 <= r < 128 for r in regs) and not set(regs) & b_regs, "registers the loop owns, none shared with B's"
+    assert not any("v104" in i for i in ins)
+    # ---- every step: 16 reads of A into the other register set, inside A's tile of the next stage
+    op = "ds_read_b64_tr_b16" if a_layout == "mc16" else "ds_read_b64_tr_b8"
+    for pos, st in steps.items():
+        buf, nxt = pos % 2, (pos + 1) % 4
+        assert st[0] == "s_waitcnt lgkmcnt(4)"
+        reads = [i for i in st if i.startswith("ds_read")]
+        assert len(reads) == 16 + (8 if b_layout == "kc" else 16) and len(reads) <= 32
+        assert all(st[n - 1].startswith("MFMA") for n, i in enumerate(st) if i.startswith("ds_read")), "one read per MFMA slot"
+        a_reads = []
+        for r in reads:
+            m = re.match(r"(\S+) v\[(\d+):(\d+)\], (\S+) offset:(\d+)$", r)
+            v0 = int(m.group(2))
+            if v0 >= 160 + (buf ^ 1) * 64 and v0 < 192 + (buf ^ 1) * 64:
+                a_reads.append((m.group(1), v0, int(m.group(3)), m.group(4), int(m.group(5))))
+        assert len(a_reads) == 16 and reads[-4:] == [r for r in reads if any(f"v[{a[1]}:" in r for a in a_reads[-4:])], "A's last reads close the step"
+        for n, (o, v0, v1, base, off) in enumerate(a_reads):
+            x, q = divmod(n, 2)
+            assert o == op and v0 == 160 + (buf ^ 1) * 64 + x * 4 + 2 * q and v1 == v0 + 1
+            assert base == (low[x] if nxt < 2 else up[x])
+            assert off == (nxt & 1) * g.STAGE + q * 2048 and off + 2048 <= (nxt & 1) * g.STAGE + g.B_TILE
+        # fills of A: passes 0..3 in order, even passes with one lane offset, odd ones with the other
+        lanes = [i.split()[1].rstrip(",") for i in st if i.startswith("global_load_lds") and "a_off" in i]
+        assert lanes == ["%[a_off]", "%[a_off1]", "%[a_off]", "%[a_off1]"]
+
+
+def test_block_addresses_of_a_column_major_tile_differ_by_an_xor():
+    """What the preamble above relies on: with the tile's k rows starting on multiples of their length, the LDS address
+    of block x's transposing read is block 0's with x * 32 (16-bit) or x * 16 (8-bit) XORed in, for every lane."""
+    for es, row_bytes in ((2, 512), (1, 256)):
+        cpr = row_bytes // 16
+        def swizzle(row, c):
+            if es == 2:
+                return c ^ ((((row & 3) << 2) | (((row >> 3) & 1) << 1)) & (cpr - 1))
+            return c ^ ((((row & 7) << 1) | ((row >> 4) & 1)) & (cpr - 1))
+        for base in (0, 1024, 32768, 5 * 16384):      # start of the tile in LDS
+            for wr0 in (0, 128):
+                for lane in range(64):
+                    kg, li = lane >> 4, lane & 15
+                    def addr(x):
+                        if es == 2:
+                            col_byte, k = (wr0 + x * 16 + (li & 3) * 4) * 2, kg * 8 + (li >> 2)
+                        else:
+                            col_byte, k = wr0 + x * 16 + (li & 1) * 8, kg * 16 + (li >> 1)
+                        return base + k * row_bytes + swizzle(k, col_byte >> 4) * 16 + (col_byte & 15)
+                    for x in range(8):
+                        assert addr(x) == addr(0) ^ (x * 16 * es)
