@@ -30,4 +30,4 @@ def __getattr__(name):
 
 
 _LANG_NAMES = {"Array", "Role", "ScalarType", "Nest", "fuse", "Package", "Target", "MMAShape", "MMAFragmentOp",
-               "MMASchedulingPolicy", "CacheStrategy", "max", "min", "cast", "Schedule", "Plan"}
+               "MMASchedulingPolicy", "CacheStrategy", "max", "min", "cast", "Schedule", "Plan", "Cache", "AUTO"}

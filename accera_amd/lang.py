@@ -103,6 +103,14 @@ class MMASchedulingPolicy(enum.Enum):
     BLOCK_ORDER = 1
 
 
+class _Auto:
+    def __repr__(self):
+        return "AUTO"
+
+
+AUTO = _Auto()  # "let the compiler decide" default of cache arguments (the reference's accera.AUTO)
+
+
 class CacheStrategy(enum.Enum):
     BLOCKED = 0
     STRIPED = 1
@@ -366,7 +374,7 @@ class Schedule:
     def split(self, index, size):
         inner = Index(f"{index.name}i")
         self.indices.insert(self.indices.index(index) + 1, inner)
-        self.commands.append(("split", index, size))
+        self.commands.append(("split", index, size, inner))
         return inner
 
     def tile(self, shape):
@@ -397,9 +405,9 @@ def fuse(*schedules, partial=None):
 
 class Plan:
     """Execution-plan calls of the reference (Plan.py:134-703, 793-956).  `tensorize` carries semantics (prologue /
-    epilogue op) and its `mma_shape` selects the kernel family; the block tile comes from the schedule's splits; the
-    rest (cache, bind, unroll, ...) selects nothing here -- the kernels always stage A and B through LDS several K
-    tiles deep and keep C in accumulator registers -- and is recorded."""
+    epilogue op) and its `mma_shape` selects the kernel family; the block tile comes from the schedule's splits, its K
+    depth from the split of k inside a SHARED cache of A or B; `cache` and `bind` check their arguments as the
+    reference does; the rest (unroll, vectorize, ...) selects nothing here and is recorded."""
 
     def __init__(self, schedule, target):
         self.schedule = schedule
@@ -408,6 +416,7 @@ class Plan:
         self.prologue_op, self.prologue_arg = MMAFragmentOp.NONE, 0
         self.epilogue_op, self.epilogue_arg = MMAFragmentOp.NONE, 0
         self.mma_shape, self.num_total_passes = None, 1
+        self.caches = []
 
     def tensorize(self, indices, mma_shape=None, use_static_offsets=False, num_total_passes=1, num_fused_passes=None,
                   scheduling_policy=MMASchedulingPolicy.PASS_ORDER, prologue_op=MMAFragmentOp.NONE, prologue_arg=0,
@@ -434,19 +443,97 @@ class Plan:
         self.epilogue_op, self.epilogue_arg = epilogue_op, epilogue_arg
         self.commands.append(("tensorize", mma_shape, num_total_passes))
 
+    def cache(self, source, index=None, trigger_index=None, layout=None, max_elements=None, element_type=None, thrifty=None,
+              location=_MemorySpace.NONE, level=None, trigger_level=None, double_buffer=False, double_buffer_location=AUTO,
+              vectorize=AUTO, strategy=AUTO, **_):
+        """The reference's `Plan.cache` (lang/Plan.py:381-703): same arguments, same argument checks.  What a cache means
+        here: the kernels always stage blocks of A and B in LDS (the reference's SHARED caches) several K tiles deep
+        (its double buffering, one tile deeper) and keep C in accumulator registers (its MMA_FRAGMENT cache), so a
+        cache call does not switch staging on or off.  A SHARED cache of A or B does name the K depth of the staged block:
+        the extent of the split of k inside the cache index -- the `k_split` axis of the reference's sweep
+        (tools/benchmarkers/accera_gemm.py:281-293, 554-555) -- and a depth the library has kernels for (64 or 128 bytes
+        of K) binds the package function to one of them."""
+        if sum(x is not None for x in (index, level, max_elements)) != 1:
+            raise ValueError("Specify one and only one of index, level, or max_elements")
+        if max_elements is not None and max_elements <= 0:
+            raise ValueError("Max element count specified as a cache budget must be greater than 0")
+        target_array = source.array if isinstance(source, Cache) else source
+        if not isinstance(target_array, Array):
+            raise ValueError("the source of a cache is an Array or a Cache")
+        if double_buffer and target_array.role not in (Role.CONST, Role.INPUT):
+            raise ValueError("Double-buffering is only supported for CONST and INPUT arrays")
+        if not double_buffer and double_buffer_location is not AUTO:
+            raise ValueError("double_buffer_location is only valid to specify when double_buffer is set to True")
+        gpu = self.target.category == Target.Category.GPU
+        if gpu and location == _MemorySpace.GLOBAL:
+            raise ValueError("Global memory caches are not yet supported on GPU targets.")
+        if not gpu and strategy is not AUTO:
+            raise ValueError("Only AUTO strategy is supported on the CPU")
+        if double_buffer and location == _MemorySpace.MMA_FRAGMENT:
+            raise ValueError("Double buffering is not supported with Tensor caching")
+        if index is not None and (level is not None or trigger_level is not None):
+            raise ValueError("Can't specify both a cache index and a cache level or trigger level")
+        if level is not None and trigger_index is not None:
+            raise ValueError("Can't specify both a cache level and a cache index or trigger index")
+        order = self.schedule.indices
+        if max_elements is None:
+            if level is not None:
+                if not 0 < level <= len(order):
+                    raise ValueError("cache level out of range of the schedule's indices")
+                index = order[-level]
+            elif index not in order:
+                raise ValueError("the cache index is not an index of this plan's schedule")
+            if (trigger_level or trigger_index is not None) and target_array.role not in (Role.CONST, Role.INPUT):
+                raise ValueError("Multicaching is only supported for CONST and INPUT arrays")
+            if trigger_index is not None:
+                if trigger_index not in order:
+                    raise ValueError("the trigger index is not an index of this plan's schedule")
+                if order.index(trigger_index) > order.index(index):
+                    raise ValueError("Trigger index must be at or outside of the cache index")
+            if trigger_level is not None and trigger_level < len(order) - order.index(index):
+                raise ValueError("Trigger level must be greater than or equal to the cache level")
+        if double_buffer_location is AUTO:
+            double_buffer_location = ((_MemorySpace.PRIVATE if gpu and location == _MemorySpace.SHARED else location)
+                                      if double_buffer else _MemorySpace.NONE)
+        c = Cache(target_array, index, location, bool(double_buffer), double_buffer_location, layout,
+                  CacheStrategy.STRIPED if strategy is AUTO else strategy)
+        self.caches.append(c)
+        self.commands.append(("cache", target_array.name, location.name, bool(double_buffer)))
+        return c
+
+    def bind(self, mapping):
+        """The reference's `Plan.bind` (lang/Plan.py:793-878): indices (or tuples of indices) to the target's grid units.
+        GPU targets only, indices of this plan only.  The launch geometry itself belongs to the kernel the block tile
+        selects (one workgroup per tile, or per compute unit for the multi-tile form); the binding is recorded."""
+        if self.target.category != Target.Category.GPU:
+            raise ValueError("Only supported on plans with GPU targets")
+        for ix, unit in dict(mapping).items():
+            for one in (ix if isinstance(ix, (tuple, list)) else (ix,)):
+                if one not in self.schedule.indices:
+                    raise ValueError("bind: not an index of this plan's schedule")
+            if not isinstance(unit[0] if isinstance(unit, (tuple, list)) else unit, Target._GridUnit):
+                raise ValueError("bind: not a grid unit of the target")
+        self.commands.append(("bind", len(dict(mapping))))
+
     def _record(name):
         def f(self, *a, **k):
             self.commands.append((name, a, k))
             return None
         return f
 
-    cache = _record("cache")
-    bind = _record("bind")
     unroll = _record("unroll")
     vectorize = _record("vectorize")
     parallelize = _record("parallelize")
     kernelize = _record("kernelize")
     del _record
+
+
+class Cache:
+    """Handle a `Plan.cache` call returns (usable as the source of a further cache: lang/Cache.py in the reference)."""
+
+    def __init__(self, array, index, location, double_buffer, double_buffer_location, layout, strategy):
+        self.array, self.index, self.location = array, index, location
+        self.double_buffer, self.double_buffer_location, self.layout, self.strategy = double_buffer, double_buffer_location, layout, strategy
 
 
 # ---- pattern match to the GEMM (+ReLU) hot path -------------------------------------------------
@@ -460,6 +547,7 @@ class _GemmSpec:
         self.block_tile = None               # (bm, bn) when a GPU plan's outermost splits of i and j name one
         self.mma_shape = None                # the tensorized plan's instruction shape
         self.gpu_target = False              # the function was added from a plan for a GPU target
+        self.k_tile_bytes = None             # K depth of the block a SHARED cache of A or B stages, when the library has kernels of that depth
         self.variant = _lib.VARIANT_AUTO     # kernel instantiation picked from the block tile, else automatic
 
 
@@ -552,8 +640,24 @@ def _match(source):
                 family = "mi16" if plan.mma_shape.dims[0] == 16 else "mi32"
         if i in first and j in first:
             spec.block_tile = (first[i], first[j])
-        if family or spec.block_tile:
-            spec.variant = _variant_for(spec, spec.block_tile, family)
+        # K depth of the staged block: the split of k inside the index of a SHARED cache of A or B (the cached block
+        # then spans that many k); 64 or 128 bytes of K are depths the library has kernels for
+        k_bytes = None
+        shared = [c for c in plan.caches if c.location == _MemorySpace.SHARED and c.array in (A, B) and c.index is not None]
+        if shared:
+            order = sched.indices
+            for cmd in sched.commands:
+                if cmd[0] == "split" and cmd[1] is k:
+                    # (the block cached at an index spans the loops at and inside it: the outer k loop runs over blocks,
+                    # the inner one inside them)
+                    inside = all(order.index(k) < order.index(c.index) <= order.index(cmd[3]) for c in shared
+                                 if k in order and cmd[3] in order and c.index in order)
+                    if inside:
+                        k_bytes = int(cmd[2]) * {ScalarType.int8: 1, ScalarType.float32: 4}.get(A.element_type, 2)
+                    break
+        spec.k_tile_bytes = k_bytes if k_bytes in (64, 128) else None
+        if family or spec.block_tile or spec.k_tile_bytes:
+            spec.variant = _variant_for(spec, spec.block_tile, family, spec.k_tile_bytes)
     if spec.variant == _lib.VARIANT_AUTO and spec.batch is None:
         # no tile named by the plan: a choice recorded for this very shape by `accera_amd.tune --save`, if any
         from . import tuned
@@ -565,11 +669,12 @@ def _match(source):
     return spec
 
 
-def _variant_for(spec, tile=None, family=None):
-    """MFMA variant for a plan that names a block tile (bm, bn) and / or an instruction-shape family ("mi16": the
-    16x16 shapes, "mi32": the 32x32 ones).  Among the variants that accept the problem: those of the named tile if
-    there are any (else any tile), of the named family if there are any; the library's own choice when it is one of
-    them, else the best-ranked.  VARIANT_AUTO when nothing matches."""
+def _variant_for(spec, tile=None, family=None, k_bytes=None):
+    """MFMA variant for a plan that names a block tile (bm, bn), an instruction-shape family ("mi16": the
+    16x16 shapes, "mi32": the 32x32 ones) and / or the K depth of the staged block in bytes.  Among the variants that
+    accept the problem: those of the named tile if there are any (else any tile), of the named family if there are
+    any, of the named depth if there are any; the library's own choice when it is one of them, else the best-ranked.
+    VARIANT_AUTO when nothing matches."""
     lean = spec.prologue == _lib.PROLOGUE_SET and spec.prologue_arg == 0 and spec.epilogue in (_lib.EPILOGUE_RELU, _lib.EPILOGUE_NONE)
     geometry = (spec.A.element_type.lib_id, spec.C.element_type.lib_id, spec.M, spec.N, spec.K,
                 spec.A.strides[-2:], spec.B.strides[-2:], spec.C.strides[-2:])
@@ -586,11 +691,13 @@ def _variant_for(spec, tile=None, family=None):
     named = []
     if tile:
         named = [(v, n) for v, n in cands if f"mfma {tile[0]}x{tile[1]} " in n]
-        if not named and not family:
+        if not named and not family and not k_bytes:
             return _lib.VARIANT_AUTO
         cands = named or cands
     if family:
         cands = [(v, n) for v, n in cands if ("mi16" in n) == (family == "mi16")] or cands
+    if k_bytes:
+        cands = [(v, n) for v, n in cands if f" kb{k_bytes} " in n] or cands
     if not cands:
         return _lib.VARIANT_AUTO
     try:

@@ -482,3 +482,89 @@ def test_run_benchmark_times_gpu_functions_device_resident(tmp_path):
     tflops = 2 * 2048 ** 3 / r.min_of_means / 1e12
     assert 100 < tflops < 2500, tflops          # a kernel time, not a copy time (PCIe alone takes milliseconds here)
     assert host[0].min_of_means > 5 * r.min_of_means
+
+
+def test_cache_and_bind_check_their_arguments_and_the_cached_k_depth_selects_the_kernel(tmp_path):
+    """Plan.cache / Plan.bind of the reference (lang/Plan.py:381-703, 793-878): the same argument checks; and the split of
+    k inside a SHARED cache of A or B -- the K depth of the staged block, the `k_split` axis of the reference's sweep
+    (tools/benchmarkers/accera_gemm.py:281-293, 554-555) -- picks a kernel with K tiles of that many bytes."""
+    T = acc.ScalarType
+    target = acc.Target(acc.Target.Model.AMD_MI355X)
+    SHARED, GLOBAL, FRAG = target.MemorySpace.SHARED, target.MemorySpace.GLOBAL, target.MemorySpace.MMA_FRAGMENT
+
+    def plan_for(k_split, tgt=target, in_t=T.float16):
+        A = acc.Array(role=acc.Role.INPUT, element_type=in_t, shape=(1024, 1024))
+        B = acc.Array(role=acc.Role.INPUT, element_type=in_t, shape=(1024, 1024))
+        C = acc.Array(role=acc.Role.INPUT_OUTPUT, element_type=T.float32 if in_t != T.int8 else T.int32, shape=(1024, 1024))
+        nest = acc.Nest(shape=(1024, 1024, 1024))
+        i, j, k = nest.get_indices()
+
+        @nest.iteration_logic
+        def _():
+            C[i, j] += A[i, k] * B[k, j]
+
+        schedule = nest.create_schedule()
+        ii, jj, kk = schedule.tile({i: 256, j: 256, k: k_split})
+        schedule.reorder(i, j, k, ii, jj, kk)
+        return schedule.create_plan(tgt), (i, j, k, ii, jj, kk), (A, B, C)
+
+    plan, (i, j, k, ii, jj, kk), (A, B, C) = plan_for(32)
+    with pytest.raises(ValueError, match="one and only one of index, level, or max_elements"):
+        plan.cache(A, location=SHARED)
+    with pytest.raises(ValueError, match="one and only one of index, level, or max_elements"):
+        plan.cache(A, index=ii, level=2, location=SHARED)
+    with pytest.raises(ValueError, match="greater than 0"):
+        plan.cache(A, max_elements=0)
+    with pytest.raises(ValueError, match="only supported for CONST and INPUT"):
+        plan.cache(C, index=ii, double_buffer=True, location=SHARED)
+    with pytest.raises(ValueError, match="double_buffer_location is only valid"):
+        plan.cache(A, index=ii, double_buffer_location=target.MemorySpace.PRIVATE)
+    with pytest.raises(ValueError, match="Global memory caches are not yet supported on GPU"):
+        plan.cache(A, index=ii, location=GLOBAL)
+    with pytest.raises(ValueError, match="not supported with Tensor caching"):
+        plan.cache(A, index=ii, double_buffer=True, location=FRAG)
+    with pytest.raises(ValueError, match="cache index and a cache level or trigger level"):
+        plan.cache(A, index=ii, trigger_level=4, location=SHARED)
+    with pytest.raises(ValueError, match="at or outside"):
+        plan.cache(A, index=ii, trigger_index=kk, location=SHARED)
+    with pytest.raises(ValueError, match="Multicaching is only supported"):
+        plan.cache(C, index=ii, trigger_index=i, location=SHARED)
+    with pytest.raises(ValueError, match="not an index of this plan"):
+        plan.cache(A, index=acc.Nest(shape=(4, 4, 4)).get_indices()[0], location=SHARED)
+    host_plan, hidx, harr = plan_for(32, acc.Target.HOST)
+    with pytest.raises(ValueError, match="Only AUTO strategy"):
+        host_plan.cache(harr[0], index=hidx[3], strategy=acc.CacheStrategy.BLOCKED)
+    with pytest.raises(ValueError, match="GPU targets"):
+        host_plan.bind({hidx[0]: target.GridUnit.BLOCK_Y})
+    with pytest.raises(ValueError, match="not an index"):
+        plan.bind({acc.Nest(shape=(4, 4, 4)).get_indices()[0]: target.GridUnit.BLOCK_X})
+    with pytest.raises(ValueError, match="not a grid unit"):
+        plan.bind({i: "BLOCK_X"})
+    # what the checks let through returns a handle with the reference's defaults resolved
+    c = plan.cache(A, index=ii, double_buffer=True, location=SHARED)
+    assert c.double_buffer and c.double_buffer_location == target.MemorySpace.PRIVATE and c.strategy == acc.CacheStrategy.STRIPED
+    assert plan.cache(B, level=3, location=SHARED).index is ii                    # level 3 of (i, j, k, ii, jj, kk) is ii
+    assert plan.cache(C, index=ii, location=FRAG).double_buffer_location == target.MemorySpace.NONE
+    plan.bind({i: target.GridUnit.BLOCK_Y, j: target.GridUnit.BLOCK_X, (ii, jj): target.GridUnit.WARP_X})
+
+    # ---- K depth of the cached block -> K tile of the kernel
+    package = acc.Package()
+    names = {}
+    for tag, in_t, k_split, cached in (("f16_k32", T.float16, 32, True), ("f16_k64", T.float16, 64, True), ("i8_k128", T.int8, 128, True),
+                                       ("f16_k64_uncached", T.float16, 64, False), ("f16_k16", T.float16, 16, True)):
+        p, (i, j, k, ii, jj, kk), arr = plan_for(k_split, in_t=in_t)
+        p.bind({i: target.GridUnit.BLOCK_Y, j: target.GridUnit.BLOCK_X})
+        p.tensorize(indices=(ii, jj, kk), mma_shape=acc.MMAShape.M16xN16xK64_B1 if in_t == T.int8 else acc.MMAShape.M16xN16xK32_B1,
+                    prologue_op=acc.MMAFragmentOp.SET, prologue_arg=0, epilogue_op=acc.MMAFragmentOp.ReLU)
+        if cached:
+            p.cache(arr[0], index=ii, double_buffer=True, location=SHARED)
+            p.cache(arr[1], index=ii, double_buffer=True, location=SHARED)
+        names[tag] = package.add(p, args=arr, base_name=tag)
+    files = package.build(name="kdepth", format=acc.Package.Format.HAT_DYNAMIC, output_dir=str(tmp_path))
+    fns = hat.parse(files[0])["functions"]
+    kernel = lambda tag: fns[names[tag]]["auxiliary"]["accera_mi355x"]["kernel"]
+    assert " kb64 " in kernel("f16_k32") and "mfma 256x256" in kernel("f16_k32")      # 32 fp16 = 64 bytes of K
+    assert " kb128 " in kernel("f16_k64") and "mfma 256x256" in kernel("f16_k64") and "mi16" in kernel("f16_k64")
+    assert " kb128 " in kernel("i8_k128")
+    assert " kb64 " in kernel("f16_k64_uncached")      # no cache call: the library's choice for the tile
+    assert " kb64 " in kernel("f16_k16")               # a depth no kernel has: the library's choice
