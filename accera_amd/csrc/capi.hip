@@ -125,9 +125,12 @@ bool mfma_can_take(const MfmaVariant& v, const Problem& pb)
     if (v.a_kc ? g.a_cs != 1 : g.a_rs != 1) return false;   // A with K contiguous (row-major) or M contiguous
     if (v.b_kc ? g.b_rs != 1 : g.b_cs != 1) return false;
     const int64_t lda = v.a_kc ? g.a_rs : g.a_cs, ldb = v.b_kc ? g.b_cs : g.b_rs;
-    if (lda % vec || ldb % vec) return false;
-    if (pb.have_pointers && (!aligned16(g.A) || !aligned16(g.B))) return false;
-    if (g.batch > 1 && (g.a_bs % vec || g.b_bs % vec)) return false; // every problem of the batch 16-byte aligned
+    // (the any-shape edge kernels load unaligned chunks: no condition on leading dimensions, pointers or batch strides)
+    if (!v.any) {
+        if (lda % vec || ldb % vec) return false;
+        if (pb.have_pointers && (!aligned16(g.A) || !aligned16(g.B))) return false;
+        if (g.batch > 1 && (g.a_bs % vec || g.b_bs % vec)) return false; // every problem of the batch 16-byte aligned
+    }
     // int8 outputs need rows of C that start 16 bytes apart: byte-wise stores to rows at odd distances
     // are switched off (that path faulted on the device in its first run and the cause is not known)
     if (g.out_type == T_I8) {
@@ -147,9 +150,7 @@ bool mfma_can_take(const MfmaVariant& v, const Problem& pb)
         if (g.K % bk) return false;
     }
     if (v.edge) {
-        if (g.K % vec) return false;
-        if (!v.b_kc && g.N % vec) return false;
-        if (!v.a_kc && g.M % vec) return false;
+        if (!v.any && (g.K % vec || (!v.b_kc && g.N % vec) || (!v.a_kc && g.M % vec))) return false;
     } else {
         if (!v.w4 && (g.M % v.bm || g.N % v.bn || g.K % bk)) return false;
     }
@@ -295,7 +296,7 @@ int auto_mfma_variant(const Problem& pb)
                                 2 * v.stages * (v.bm + v.bn) * v.kb <= 160 * 1024 && v.bm * v.bn <= 256 * 128) ? 2 : 1;
         const int64_t rounds = (tiles + 256 * wgs_per_cu - 1) / (256 * wgs_per_cu);
         double cost = (double)rounds * wgs_per_cu * v.bm * v.bn;
-        if (v.edge) cost *= 1.5;                 // register-staged fill, bounds checks
+        if (v.edge) cost *= v.any ? 2.0 : 1.5;   // register-staged fill, bounds checks (unaligned chunks cost more requests)
         if (!v.direct) cost *= 1.2;
         // measured on sweeps: 4-wave tiles reach about 85 % of the ping-pong kernel's rate when two
         // workgroups share a CU and about 70 % when a workgroup has the CU to itself
@@ -319,6 +320,69 @@ int auto_mfma_variant(const Problem& pb)
     return best;
 }
 
+// ---- K split of an MFMA variant: the kernel runs as a batch of partial products over consecutive ranges of K into a
+// workspace of 32-bit sums, and a second kernel adds the slices in order and does the prologue / epilogue ops
+// (gemm_splitk.hip).  Every slice but the last spans `ks` elements of K (whole K tiles), the last what is left.
+struct SplitPlan {
+    int splits, ks, k_last;
+};
+constexpr size_t kMaxSplitFloats = (size_t)1 << 28; // 1 GiB of partial sums
+
+GemmArgs split_first_step(const GemmArgs& g, const SplitPlan& sp, void* ws)
+{
+    GemmArgs q = g;
+    q.C = ws;
+    q.c_rs = g.N; q.c_cs = 1;
+    q.out_type = g.in_type == T_I8 ? T_I32 : T_F32;
+    q.prologue = PRO_SET; q.prologue_arg = 0.f;
+    q.epilogue = EPI_NONE; q.epilogue_arg = 0.f;
+    q.K = sp.ks; q.k_last = sp.k_last;
+    q.batch = sp.splits;
+    q.a_bs = (int64_t)sp.ks * g.a_cs; q.b_bs = (int64_t)sp.ks * g.b_rs; q.c_bs = (int64_t)g.M * g.N;
+    return q;
+}
+
+// Slices for `want` splits of this problem on variant v (fewer when K has too few K tiles); false when the variant
+// cannot run the problem split (a batch, one slice only, partial products it does not take).
+bool plan_split(const MfmaVariant& v, const Problem& pb, int want, SplitPlan* sp)
+{
+    const GemmArgs& g = pb.g;
+    if (g.batch > 1 || want <= 1) return false;
+    const int bk = v.kb / elem_size(g.in_type);
+    const int kt = (g.K + bk - 1) / bk, least = v.w4 ? 4 : 1; // K tiles in all; K tiles a slice needs
+    int splits = want < kt / least ? want : kt / least;
+    if (splits <= 1) return false;
+    const int per = (kt + splits - 1) / splits;
+    splits = (kt + per - 1) / per;
+    if (splits > 1 && g.K - (splits - 1) * per * bk < least * bk) --splits; // (the last slice takes what a too short one would have left)
+    if (splits <= 1) return false;
+    if ((size_t)splits * (size_t)g.M * (size_t)g.N > kMaxSplitFloats) return false;
+    sp->splits = splits;
+    sp->ks = per * bk;
+    sp->k_last = g.K - (splits - 1) * sp->ks;
+    Problem q{split_first_step(g, *sp, nullptr), pb.have_pointers};
+    if (!mfma_can_take(v, q)) return false;
+    q.g.K = sp->k_last;
+    return mfma_can_take(v, q);
+}
+
+// Splits the library takes by itself: only when the tiles leave at least half of the compute units idle and K is long
+// enough for the second kernel (a few microseconds) to pay.
+int auto_mfma_splits(const MfmaVariant& v, const Problem& pb)
+{
+    const GemmArgs& g = pb.g;
+    if (g.batch > 1) return 1;
+    const int64_t tiles = (((int64_t)g.M + v.bm - 1) / v.bm) * (((int64_t)g.N + v.bn - 1) / v.bn);
+    if (tiles * 2 > kComputeUnits) return 1;
+    const int64_t steps = (int64_t)g.K * elem_size(g.in_type) / 64; // k-steps of 64 bytes
+    if (steps < 32) return 1;
+    int64_t want = kComputeUnits / tiles < steps / 8 ? kComputeUnits / tiles : steps / 8;
+    if (want > 32) want = 32;
+    if ((size_t)want * (size_t)g.M * (size_t)g.N > ((size_t)1 << 24)) return 1; // 64 MiB of partial sums at most without being asked
+    SplitPlan sp;
+    return want > 1 && plan_split(v, pb, (int)want, &sp) ? sp.splits : 1;
+}
+
 struct Choice {
     int variant;
     int splits;
@@ -337,6 +401,13 @@ int choose(const Problem& pb, int variant, int k_splits, Choice* c)
         if (f32_can_take(pb.g)) { c->variant = ACC950_VARIANT_F32_MFMA; return ACC950_OK; }
         int mv = auto_mfma_variant(pb);
         c->variant = mv >= 0 ? mv : ACC950_VARIANT_GENERIC;
+        if (mv >= 0) {
+            int n = 0;
+            const MfmaVariant& v = mfma_table(pb.g.in_type, &n)[mv];
+            SplitPlan sp;
+            if (k_splits > 1) c->splits = plan_split(v, pb, k_splits, &sp) ? sp.splits : 1;
+            else if (k_splits == 0) c->splits = auto_mfma_splits(v, pb);
+        }
         return ACC950_OK;
     }
     if (variant == ACC950_VARIANT_GENERIC) { c->variant = variant; return ACC950_OK; }
@@ -361,6 +432,12 @@ int choose(const Problem& pb, int variant, int k_splits, Choice* c)
     if (variant < 0 || variant >= n) return fail(ACC950_INVALID_ARGUMENT, "unknown kernel variant");
     if (!mfma_can_take(tab[variant], pb)) return fail(ACC950_UNSUPPORTED, "MFMA variant cannot take this shape / layout / alignment");
     c->variant = variant;
+    if (k_splits > 1) { // (a named variant is split only when asked)
+        SplitPlan sp;
+        if (!plan_split(tab[variant], pb, k_splits, &sp))
+            return fail(ACC950_UNSUPPORTED, "this MFMA variant cannot run the problem with K split (a batch, too few K tiles, or partial products it does not take)");
+        c->splits = sp.splits;
+    }
     return ACC950_OK;
 }
 
@@ -423,7 +500,28 @@ int run(const Problem& pb, const Choice& c, hipStream_t stream, LaunchGeom* geom
         // kernels with a lean build take C = A*B and C = relu(A*B) there, everything else in the full build
         const MfmaVariant& mv = tab[c.variant];
         const bool lean = g.prologue == PRO_SET && g.prologue_arg == 0.f && (g.epilogue == EPI_RELU || g.epilogue == EPI_NONE);
-        e = (mv.launch_general && !lean ? mv.launch_general : mv.launch)(g, stream, geom, dry_run);
+        SplitPlan sp;
+        if (c.splits > 1 && plan_split(mv, pb, c.splits, &sp)) {
+            float* ws = nullptr;
+            if (!dry_run) {
+                const size_t floats = (size_t)sp.splits * (size_t)g.M * (size_t)g.N;
+                unsigned* unused = nullptr;
+                if (static_ws) {
+                    if (floats > kStaticFloats)
+                        return fail(ACC950_UNSUPPORTED, "this problem's K split needs " + std::to_string(floats * sizeof(float)) +
+                                    " bytes of partial sums; the built-in workspace holds " + std::to_string(kStaticFloats * sizeof(float)) + " bytes");
+                    e = static_workspace(&ws);
+                    if (e != hipSuccess) return fail_hip(e, "address of the built-in workspace");
+                } else {
+                    e = workspace_for(stream, floats, 0, &ws, &unused);
+                    if (e != hipSuccess) return fail_hip(e, "workspace allocation");
+                }
+            }
+            e = mv.launch(split_first_step(g, sp, ws), stream, geom, dry_run); // partial products: C = A*B, nothing else
+            if (e == hipSuccess && !dry_run) e = launch_splitk_reduce(g, ws, sp.splits, stream);
+        } else {
+            e = (mv.launch_general && !lean ? mv.launch_general : mv.launch)(g, stream, geom, dry_run);
+        }
     }
     if (e != hipSuccess) return fail_hip(e, "kernel launch");
     return ACC950_OK;
@@ -611,7 +709,7 @@ int acc950_mfma_phase_probe(int in_type, int out_type, int M, int N, int K, cons
     Problem pb;
     int rc = make_problem(in_type, out_type, M, N, K, A, K, 1, B, N, 1, C, N, 1, PRO_SET0, EPI_RELU, true, &pb);
     if (rc) return rc;
-    const MfmaVariant probe = {256, 256, 2, 4, true, false, true, false, 64, 4, true, false, false, false, nullptr, nullptr};
+    const MfmaVariant probe = {256, 256, 2, 4, true, false, true, false, 64, 4, true, false, false, false, false, nullptr, nullptr};
     int n_unused = 0;
     if (M < 256 || N < 256 || K < 1 || !mfma_table(pb.g.in_type, &n_unused) || !mfma_can_take(probe, pb))
         return fail(ACC950_UNSUPPORTED, "the phase probe runs the 256x256 kernels: 8/16-bit inputs, dense row-major A, B, C, M and N multiples of 256, K of 64 bytes");
@@ -760,7 +858,7 @@ int acc950_variant_name(int variant, char* buf, size_t buf_len)
     const MfmaVariant& v = tab[variant];
     std::snprintf(buf, buf_len, "mfma %dx%d kb%d waves %dx%d %sB=%s fill=%s stages=%d%s%s%s", v.bm, v.bn, v.kb, v.waves_m, v.waves_n,
                   v.a_kc ? "" : "A=col-major ", v.b_kc ? "col-major" : "row-major", v.direct ? "direct" : "registers", v.stages,
-                  v.edge ? " edge" : "", v.pingpong ? " pingpong" : "", v.w4 ? (v.persist ? " mi16 hand-laid loop multi-tile" : " mi16 hand-laid loop") : v.mi16 ? " mi16" : "");
+                  v.edge ? (v.any ? " edge any-alignment" : " edge") : "", v.pingpong ? " pingpong" : "", v.w4 ? (v.persist ? " mi16 hand-laid loop multi-tile" : " mi16 hand-laid loop") : v.mi16 ? " mi16" : "");
     return ACC950_OK;
 }
 

@@ -32,6 +32,7 @@ struct GemmArgs {
     int tiles_m, tiles_n; // workgroup grid in tiles (MFMA kernels)
     int batch;                  // independent problems, one per blockIdx.z (1 for a plain GEMM)
     int64_t a_bs, b_bs, c_bs;   // element distance between consecutive problems of a batch
+    int k_last;                 // > 0: K of the last problem of the batch (a K split run as a batch of partial products: the last slice is what is left)
     int stagger_groups, stagger_ticks; // multi-tile kernels: workgroup group g of stagger_groups starts g * stagger_ticks * 10 ns late (0: no stagger)
     unsigned long long* stamps; // timed MFMA instantiation only: [workgroup][4 points][shader clock, 100 MHz clock]
 };
@@ -136,6 +137,7 @@ __device__ __forceinline__ void select_batch(GemmArgs& p)
     p.A = (const char*)p.A + z * p.a_bs * elem_bytes(p.in_type);
     p.B = (const char*)p.B + z * p.b_bs * elem_bytes(p.in_type);
     p.C = (char*)p.C + z * p.c_bs * elem_bytes(p.out_type);
+    if (p.k_last > 0 && (int)z == p.batch - 1) p.K = p.k_last;
 }
 
 // MI355X: 256 compute units in 8 XCDs (the library runs on gfx950 only; the launch geometry of the kernels that keep

@@ -117,15 +117,43 @@ struct OperandTile {
     }
 
     // ---- register-staged fill ----
-    template <bool EDGE>
+    // EDGE 0: full tiles.  1: tiles that end past M / N / K, every row of the operand 16 bytes aligned and K (and the
+    // contiguous extent) a multiple of the 16-byte vector: chunks are in or out as a whole.  2: any sizes, leading
+    // dimensions and pointers: chunks lie anywhere (the loads are declared unaligned; the hardware takes them), and the
+    // chunk that straddles the end of a row is put together from single elements.
+    template <int EDGE>
     __device__ static __forceinline__ void load_global(i32x4 (&regs)[PER_THREAD], const char* base, int r0, int k0,
                                                        int64_t ld, int rmax, int K, int tid)
     {
+        typedef i32x4 __attribute__((aligned(1))) i32x4_any;
+        constexpr int VEC = 16 / ES;
 #pragma unroll
         for (int i = 0; i < PER_THREAD; ++i) {
             int id = tid + i * NT;
             int row = id / CPR, c = id % CPR;
-            if constexpr (EDGE) {
+            if constexpr (EDGE == 2) {
+                // elements of this chunk inside the matrix: all of them, the first few, or none
+                const bool row_in = KC ? (r0 + row) < rmax : (k0 + row) < K;
+                const int left = KC ? K - (k0 + c * VEC) : rmax - (r0 + c * VEC);
+                const int n = row_in ? (left < 0 ? 0 : left) : 0;
+                const char* src = base + global_off(row, c, r0, k0, ld);
+                if (n >= VEC) regs[i] = *(const i32x4_any*)src;
+                else {
+                    i32x4 v = {0, 0, 0, 0};
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) {
+                        if (e >= n) break;
+                        if constexpr (ES == 2) {
+                            const unsigned x = *(const unsigned short*)(src + 2 * e);
+                            v[e >> 1] |= (int)(x << ((e & 1) * 16));
+                        } else {
+                            const unsigned x = *(const unsigned char*)(src + e);
+                            v[e >> 2] |= (int)(x << ((e & 3) * 8));
+                        }
+                    }
+                    regs[i] = v;
+                }
+            } else if constexpr (EDGE == 1) {
                 if (in_bounds(row, c, r0, k0, rmax, K))
                     regs[i] = *(const i32x4*)(base + global_off(row, c, r0, k0, ld));
                 else
@@ -292,8 +320,11 @@ __device__ __forceinline__ void tile_coords(int pid, int tiles_m, int tiles_n, i
 
 // Compile-time description of one kernel instantiation.
 template <int IN_, int BM_, int BN_, int WAVES_M_, int WAVES_N_, bool A_KC_, bool B_KC_, bool DIRECT_, bool EDGE_, int KB_, int STAGES_,
-          bool PINGPONG_ = false, bool TIMED_ = false>
+          bool PINGPONG_ = false, bool TIMED_ = false, bool ANY_ = false>
 struct MfmaConfig {
+    // ANY (an EDGE build): operands of any size, leading dimension and alignment (see OperandTile::load_global)
+    static constexpr bool ANY = ANY_;
+    static_assert(!ANY_ || EDGE_, "the any-shape fill is a form of the edge fill");
     static constexpr bool PINGPONG = PINGPONG_;
     // TIMED: wave 0 of every workgroup reads the shader-clock counter and the constant
     // 100 MHz counter at kernel entry, after the prologue, after the main loop and at the
@@ -326,7 +357,9 @@ struct CTile {
 __device__ __forceinline__ CTile c_tile(const GemmArgs& p, int row, int col, unsigned os, unsigned back = 0)
 {
     char* base = (char*)p.C + ((int64_t)row * p.c_rs + col) * os - back;
-    const int64_t bytes = ((int64_t)(p.M - 1 - row) * p.c_rs + (p.N - col)) * os + back;
+    // (rounded up to the end of the dword that holds the last element: reads of sub-dword elements fetch the aligned dword
+    // around them, and the range check is on the whole access)
+    const int64_t bytes = ((((int64_t)(p.M - 1 - row) * p.c_rs + (p.N - col)) * os + back) + 3) & ~(int64_t)3;
     const unsigned records = bytes <= 0 ? 0u : bytes > 0xffffffffll ? 0xffffffffu : (unsigned)bytes;
     return CTile{__builtin_amdgcn_make_buffer_rsrc(base, 0, records, 0x00020000)};
 }
@@ -351,6 +384,7 @@ __global__ void __launch_bounds__(Cfg::NT, Cfg::WGS_PER_CU) gemm_mfma_kernel(Gem
     constexpr int IN = Cfg::IN, BM = Cfg::BM, BN = Cfg::BN, WAVES_M = Cfg::WAVES_M, WAVES_N = Cfg::WAVES_N;
     constexpr int KB = Cfg::KB, STAGES = Cfg::STAGES, NT = Cfg::NT;
     constexpr bool A_KC = Cfg::A_KC, B_KC = Cfg::B_KC, DIRECT = Cfg::DIRECT, EDGE = Cfg::EDGE;
+    constexpr int FILL_MODE = Cfg::ANY ? 2 : (EDGE ? 1 : 0);
     constexpr int ES = InTraits<IN>::ES;
     constexpr int BK = KB / ES;
     constexpr int KSTEPS = KB / 32;
@@ -593,8 +627,8 @@ __global__ void __launch_bounds__(Cfg::NT, Cfg::WGS_PER_CU) gemm_mfma_kernel(Gem
         }
     } else {
         i32x4 ra[TA::PER_THREAD], rb[TB::PER_THREAD];
-        TA::template load_global<EDGE>(ra, Ab, m0, 0, lda, p.M, p.K, tid);
-        TB::template load_global<EDGE>(rb, Bb, n0, 0, ldb, p.N, p.K, tid);
+        TA::template load_global<FILL_MODE>(ra, Ab, m0, 0, lda, p.M, p.K, tid);
+        TB::template load_global<FILL_MODE>(rb, Bb, n0, 0, ldb, p.N, p.K, tid);
         TA::store_lds(ra, smem, tid);
         TB::store_lds(rb, smem + TA::TILE_BYTES, tid);
         __syncthreads();
@@ -602,8 +636,8 @@ __global__ void __launch_bounds__(Cfg::NT, Cfg::WGS_PER_CU) gemm_mfma_kernel(Gem
             char* cur = smem + (kt & 1) * STAGE_BYTES;
             char* nxt = smem + ((kt + 1) & 1) * STAGE_BYTES;
             if (kt + 1 < KT) {
-                TA::template load_global<EDGE>(ra, Ab, m0, (kt + 1) * BK, lda, p.M, p.K, tid);
-                TB::template load_global<EDGE>(rb, Bb, n0, (kt + 1) * BK, ldb, p.N, p.K, tid);
+                TA::template load_global<FILL_MODE>(ra, Ab, m0, (kt + 1) * BK, lda, p.M, p.K, tid);
+                TB::template load_global<FILL_MODE>(rb, Bb, n0, (kt + 1) * BK, ldb, p.N, p.K, tid);
             }
             load_first_frags(cur, cur + TA::TILE_BYTES);
             mma_tile(cur, cur + TA::TILE_BYTES, cur, cur + TA::TILE_BYTES, std::false_type{}, std::false_type{}, 0, 0);

@@ -12,27 +12,32 @@
 namespace acc950 {
 
 #define VA(AKC, BM, BN, WM, WN, BKC, DIRECT, EDGE, KB, STAGES)                                         \
-    { BM, BN, WM, WN, AKC, BKC, DIRECT, EDGE, KB, STAGES, false, false, false, false,                  \
+    { BM, BN, WM, WN, AKC, BKC, DIRECT, EDGE, KB, STAGES, false, false, false, false, false,           \
       &launch_mfma<MfmaConfig<ACC950_IN, BM, BN, WM, WN, AKC, BKC, DIRECT, EDGE, KB, STAGES>>, nullptr }
 #define VPA(AKC, BM, BN, WM, WN, BKC, KB, STAGES)                                                       \
-    { BM, BN, WM, WN, AKC, BKC, true, false, KB, STAGES, true, false, false, false,                    \
+    { BM, BN, WM, WN, AKC, BKC, true, false, KB, STAGES, true, false, false, false, false,             \
       &launch_mfma<MfmaConfig<ACC950_IN, BM, BN, WM, WN, AKC, BKC, true, false, KB, STAGES, true>>, nullptr }
 // ping-pong on the 16x16 MFMA shapes
 #define V16(AKC, BM, BN, WM, WN, BKC, KB, STAGES)                                                       \
-    { BM, BN, WM, WN, AKC, BKC, true, false, KB, STAGES, true, true, false, false,                     \
+    { BM, BN, WM, WN, AKC, BKC, true, false, KB, STAGES, true, true, false, false, false,              \
       &launch_mfma16<Mfma16Config<ACC950_IN, BM, BN, WM, WN, AKC, BKC, KB, STAGES, false>>,           \
       &launch_mfma16<Mfma16Config<ACC950_IN, BM, BN, WM, WN, AKC, BKC, KB, STAGES, true>> }
 // four waves, 128x128 wave tiles, hand-laid K loop
 #define V16W4(BKC) \
-    { 256, 256, 2, 2, true, BKC, true, false, 64, 4, false, true, true, false, &launch_mfma16w4<Mfma16W4Config<ACC950_IN, BKC>>, nullptr }
+    { 256, 256, 2, 2, true, BKC, true, false, 64, 4, false, true, true, false, false, &launch_mfma16w4<Mfma16W4Config<ACC950_IN, BKC>>, nullptr }
 #define V16W4_192 \
-    { 256, 192, 2, 2, true, true, true, false, 64, 4, false, true, true, false, &launch_mfma16w4<Mfma16W4Config<ACC950_IN, true, false, 192>>, nullptr }
+    { 256, 192, 2, 2, true, true, true, false, 64, 4, false, true, true, false, false, &launch_mfma16w4<Mfma16W4Config<ACC950_IN, true, false, 192>>, nullptr }
 // the same, one workgroup per CU walking several output tiles
 #define V16W4P(BKC) \
-    { 256, 256, 2, 2, true, BKC, true, false, 64, 4, false, true, true, true, &launch_mfma16w4<Mfma16W4Config<ACC950_IN, BKC, false, 256, true>>, nullptr }
+    { 256, 256, 2, 2, true, BKC, true, false, 64, 4, false, true, true, true, false, &launch_mfma16w4<Mfma16W4Config<ACC950_IN, BKC, false, 256, true>>, nullptr }
 // the same kernel for a column-major A (one tile per workgroup)
 #define V16W4A(BKC) \
-    { 256, 256, 2, 2, false, BKC, true, false, 64, 4, false, true, true, false, &launch_mfma16w4<Mfma16W4Config<ACC950_IN, BKC, false, 256, false, false>>, nullptr }
+    { 256, 256, 2, 2, false, BKC, true, false, 64, 4, false, true, true, false, false, &launch_mfma16w4<Mfma16W4Config<ACC950_IN, BKC, false, 256, false, false>>, nullptr }
+// any sizes, leading dimensions and alignments (the odd shapes of the reference's sweep lists, e.g.
+// /root/reference/tools/benchmarkers/gemm_resnet_inception.csv): register-staged 128x128 tiles whose fill takes unaligned chunks
+#define VANY(AKC, BKC)                                                                                  \
+    { 128, 128, 2, 2, AKC, BKC, false, true, 128, 2, false, false, false, false, true,                 \
+      &launch_mfma<MfmaConfig<ACC950_IN, 128, 128, 2, 2, AKC, BKC, false, true, 128, 2, false, false, true>>, nullptr }
 #define V(BM, BN, WM, WN, BKC, DIRECT, EDGE, KB, STAGES) VA(true, BM, BN, WM, WN, BKC, DIRECT, EDGE, KB, STAGES)
 #define VP(BM, BN, WM, WN, BKC, KB, STAGES) VPA(true, BM, BN, WM, WN, BKC, KB, STAGES)
 // column-major A (M contiguous; the "transA" shapes of the reference's sweep lists,
@@ -81,6 +86,10 @@ static const MfmaVariant kVariants[] = {
     V16W4P(true),
     V16W4A(false),
     V16W4A(true),
+    VANY(true, false),
+    VANY(true, true),
+    VANY(false, false),
+    VANY(false, true),
 };
 #undef LAYOUT_AT
 #undef VA
@@ -90,6 +99,7 @@ static const MfmaVariant kVariants[] = {
 #undef V16W4_192
 #undef V16W4P
 #undef V16W4A
+#undef VANY
 #undef LAYOUT
 #undef V
 #undef VP

@@ -1,0 +1,82 @@
+// Second step of a K split of the MFMA kernels: C = epilogue(prologue(C) + slice 0 + slice 1 + ...).
+//
+// The first step is the GEMM kernel itself, launched as a batch of `splits` partial products over consecutive ranges of
+// K (blockIdx.z picks the range) that writes 32-bit sums into a workspace, slice after slice, each an M x N row-major
+// matrix.  This kernel adds the slices of every element in slice order -- a fixed order, so the result does not depend
+// on which workgroup finished first -- and then does what the GEMM kernel's write-back does for an unsplit problem: the
+// prologue op on the old C, the epilogue op (the fused ReLU comes after the whole sum), the narrowing store.
+//
+// The reference has no counterpart (its `k_split` is the K depth of the block tile); shapes of its sweep lists with a
+// small output and a long K (/root/reference/tools/benchmarkers/gemm_bert_assorted.csv: 768 x 320 x 30522,
+// gemm_resnet_inception.csv: 288 x 64 x 21609) are the ones that leave most compute units idle without it.
+#include "common.h"
+#include "variants.h"
+
+namespace acc950 {
+
+struct SplitReduceArgs {
+    const void* ws;       // [splits][M][N] float or int
+    int splits, M, N;
+    void* C;
+    int64_t c_rs, c_cs;
+    int out_type, is_int;
+    int prologue, epilogue;
+    float prologue_arg, epilogue_arg;
+};
+
+// one thread per four consecutive columns of a row (N is padded up to a multiple of four by the test below)
+__global__ void __launch_bounds__(256) splitk_reduce_kernel(SplitReduceArgs p)
+{
+    const int groups_n = (p.N + 3) / 4;
+    const int64_t id = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (id >= (int64_t)p.M * groups_n) return;
+    const int row = (int)(id / groups_n), col0 = (int)(id % groups_n) * 4;
+    const int64_t slice = (int64_t)p.M * p.N;
+    const int64_t at = (int64_t)row * p.N + col0;
+    const int cols = p.N - col0 < 4 ? p.N - col0 : 4;
+    if (p.is_int) {
+        int sum[4] = {0, 0, 0, 0};
+        const int* w = (const int*)p.ws + at;
+        for (int s = 0; s < p.splits; ++s)
+            for (int e = 0; e < cols; ++e) sum[e] = wrap_add(sum[e], w[(int64_t)s * slice + e]);
+        for (int e = 0; e < cols; ++e) {
+            const int64_t idx = (int64_t)row * p.c_rs + (int64_t)(col0 + e) * p.c_cs;
+            const int v = apply_prologue<int>(sum[e], p.prologue, p.prologue_arg, [&]() { return load_out_int(p.C, p.out_type, idx); });
+            store_out_int(p.C, p.out_type, idx, apply_epilogue<int>(v, p.epilogue, p.epilogue_arg));
+        }
+    } else {
+        float sum[4] = {0.f, 0.f, 0.f, 0.f};
+        const float* w = (const float*)p.ws + at;
+        if (cols == 4 && (at & 3) == 0) {
+            for (int s = 0; s < p.splits; ++s) {
+                const f32x4 x = *(const f32x4*)(w + (int64_t)s * slice);
+                for (int e = 0; e < 4; ++e) sum[e] += x[e];
+            }
+        } else {
+            for (int s = 0; s < p.splits; ++s)
+                for (int e = 0; e < cols; ++e) sum[e] += w[(int64_t)s * slice + e];
+        }
+        for (int e = 0; e < cols; ++e) {
+            const int64_t idx = (int64_t)row * p.c_rs + (int64_t)(col0 + e) * p.c_cs;
+            const float v = apply_prologue<float>(sum[e], p.prologue, p.prologue_arg, [&]() { return load_out(p.C, p.out_type, idx); });
+            store_out(p.C, p.out_type, idx, apply_epilogue<float>(v, p.epilogue, p.epilogue_arg));
+        }
+    }
+}
+
+// g: the caller's problem (its C, strides, output type and ops); ws: the slices the first step wrote
+hipError_t launch_splitk_reduce(const GemmArgs& g, const void* ws, int splits, hipStream_t stream)
+{
+    SplitReduceArgs a{};
+    a.ws = ws; a.splits = splits; a.M = g.M; a.N = g.N;
+    a.C = g.C; a.c_rs = g.c_rs; a.c_cs = g.c_cs;
+    a.out_type = g.out_type; a.is_int = g.in_type == T_I8;
+    a.prologue = g.prologue; a.epilogue = g.epilogue; a.prologue_arg = g.prologue_arg; a.epilogue_arg = g.epilogue_arg;
+    const int64_t threads = (int64_t)g.M * ((g.N + 3) / 4);
+    const int64_t blocks = (threads + 255) / 256;
+    if (blocks <= 0 || blocks > 0x7fffffffll) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, a);
+    return hipGetLastError();
+}
+
+} // namespace acc950

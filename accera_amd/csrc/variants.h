@@ -16,6 +16,7 @@ struct MfmaVariant {
     bool mi16;           // 16x16 MFMA shapes (else 32x32)
     bool w4;             // four waves with 128x128 wave tiles and the hand-laid K loop: at least four K tiles, an int8 C only written
     bool persist;        // w4 only: one workgroup per CU walks several output tiles, the next tile's first fills overlap this tile's end
+    bool any;            // edge only: operands of any size, leading dimension and alignment (unaligned loads, row ends put together from elements)
     LaunchFn launch;
     LaunchFn launch_general; // build that carries every prologue / epilogue op, when `launch` is a lean build (else null)
 };
@@ -28,6 +29,9 @@ const MfmaVariant* mfma_variants_i8(int* count);
 hipError_t launch_mfma_timed_f16(const GemmArgs& a, hipStream_t stream, LaunchGeom* geom, bool dry_run);
 hipError_t launch_mfma_timed_bf16(const GemmArgs& a, hipStream_t stream, LaunchGeom* geom, bool dry_run);
 hipError_t launch_mfma_timed_i8(const GemmArgs& a, hipStream_t stream, LaunchGeom* geom, bool dry_run);
+
+// second step of a K split of the MFMA kernels (gemm_splitk.hip)
+hipError_t launch_splitk_reduce(const GemmArgs& g, const void* ws, int splits, hipStream_t stream);
 
 bool f32_can_take(const GemmArgs& g);
 hipError_t launch_f32(const GemmArgs& a, hipStream_t stream, LaunchGeom* geom, bool dry_run);

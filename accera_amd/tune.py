@@ -49,14 +49,22 @@ def _make(torch, rows, cols, t, col_major, gen):
     return x.t() if col_major else x
 
 
-def candidates(in_id, out_id, M, N, K, sa, sb, sc, splits_for_skinny=(0, 2, 4, 8)):
-    """(variant, k_splits) pairs the library accepts for this problem."""
+def candidates(in_id, out_id, M, N, K, sa, sb, sc, splits_for_skinny=(0, 2, 4, 8), splits_for_mfma=(0, 2, 4, 8, 16, 32)):
+    """(variant, k_splits) pairs the library accepts for this problem.  MFMA variants are tried with K split over workgroups
+    only when the output is small (at most 128 tiles of 128 x 128): elsewhere the partial sums cost more than the idle
+    compute units."""
     L = _lib.lib()
     ids = list(range(_lib.num_variants())) + [_lib.VARIANT_SKINNY_BASE + i for i in range(_lib.num_skinny_variants())]
     ids += [_lib.VARIANT_F32_MFMA, _lib.VARIANT_GENERIC]
     out = []
     for v in ids:
-        for sp in (splits_for_skinny if v >= _lib.VARIANT_SKINNY_BASE and v < _lib.VARIANT_GENERIC else (0,)):
+        if _lib.VARIANT_SKINNY_BASE <= v < _lib.VARIANT_GENERIC:
+            sweep = splits_for_skinny
+        elif v < _lib.num_variants() and -(-M // 128) * -(-N // 128) <= 128:
+            sweep = splits_for_mfma
+        else:
+            sweep = (0,)
+        for sp in sweep:
             try:
                 _lib.launch_geometry(in_id, out_id, M, N, K, sa, sb, sc, v, sp)
             except _lib.Acc950Error:

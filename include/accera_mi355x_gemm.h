@@ -88,8 +88,12 @@ int acc950_gemm_relu(int in_type, int out_type, int M, int N, int K,
  * point of the reference's tuning space (tile sizes, cache strategy, double buffering:
  * /root/reference/tools/benchmarkers/accera_gemm.py:187-348).  `variant` is
  * ACC950_VARIANT_AUTO, an index < acc950_num_variants() into the MFMA table,
- * ACC950_VARIANT_SKINNY_BASE + i, ACC950_VARIANT_F32_MFMA or ACC950_VARIANT_GENERIC.  `k_splits` (skinny
- * kernels only; 0 = automatic) splits K over workgroups.  A named variant that does not take the
+ * ACC950_VARIANT_SKINNY_BASE + i, ACC950_VARIANT_F32_MFMA or ACC950_VARIANT_GENERIC.  `k_splits` splits K
+ * over workgroups (skinny and MFMA kernels; 0 = the library decides -- for a named MFMA variant: no split --,
+ * 1 = no split, n > 1 = at most n slices).  The slices are added in a fixed order, so a split result does not
+ * vary from run to run; an MFMA kernel's split goes through a workspace of 4 * slices * M * N bytes (held per
+ * stream, or the built-in one of acc950_gemm_ops_static) and a second kernel that adds the slices and applies
+ * the prologue / epilogue ops.  A named variant that does not take the
  * problem -- its sizes, layouts, alignment, or its prologue / epilogue ops (the four-wave kernels
  * do not read an int8 C) -- returns ACC950_UNSUPPORTED; nothing runs.
  */

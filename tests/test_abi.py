@@ -53,8 +53,11 @@ def test_launch_geometry_of_the_configs():
     assert "skinny" in _lib.variant_name(v) and g[0] * g[1] >= 43 and b[0] % 64 == 0
     g, b, lds, v = _lib.launch_geometry(_lib.F32, _lib.F32, 512, 512, 512, (512, 1), (512, 1), (512, 1))
     assert v == _lib.VARIANT_F32_MFMA and g[:2] == [16, 16]
-    # unaligned shapes fall to the thread-bound kernel, explicit variants refuse them
+    # sizes that are not multiples of the 16-byte vector take the MFMA kernel whose fill accepts unaligned chunks; an operand with
+    # no unit stride falls to the thread-bound kernel; explicit variants refuse what they do not take
     g, b, lds, v = _lib.launch_geometry(_lib.F16, _lib.F32, 100, 71, 40, (40, 1), (71, 1), (71, 1))
+    assert "any-alignment" in _lib.variant_name(v) and g == [1, 1, 1]
+    g, b, lds, v = _lib.launch_geometry(_lib.F16, _lib.F32, 100, 71, 40, (80, 2), (71, 1), (71, 1))
     assert v == _lib.VARIANT_GENERIC and g[:2] == [2, 2]
     with pytest.raises(_lib.Acc950Error) as e:
         _lib.launch_geometry(_lib.F16, _lib.F32, 100, 71, 40, (40, 1), (71, 1), (71, 1), variant=0)

@@ -892,3 +892,125 @@ def test_skinny_workspaces_are_per_stream():
     for i in range(2):
         want = ora.gemm_relu_exact(A, Bs[i], out_zeros(M, N, "f16"), "f16", "f16", ora.PRO_SET0, ora.EPI_RELU)
         assert_matches(to_host(dCs[i], "f16"), want, "f16", K)
+
+
+@pytest.mark.parametrize("in_type,out_type", [("f16", "f32"), ("f16", "f16"), ("bf16", "bf16"), ("i8", "i32"), ("i8", "i16")])
+@pytest.mark.parametrize("a_layout,b_layout", [("row", "row"), ("row", "col"), ("col", "row"), ("col", "col")])
+def test_any_alignment_mfma_kernel(in_type, out_type, a_layout, b_layout):
+    """Sizes, leading dimensions and pointers that are not multiples of the 16-byte vector (the odd shapes of the
+    reference's sweep lists, tools/benchmarkers/gemm_resnet_inception.csv: K = 1225, 3025, 5329, M = 27, 147, 363 ...):
+    the edge kernel whose fill takes unaligned chunks, named explicitly; C overwritten and read; then operands that are
+    views into larger arrays starting at an odd element."""
+    import accera_amd as acc
+    import torch
+    from accera_amd import _lib
+    key = (" A=col-major" if a_layout == "col" else " waves 2x2 B="), (" B=col-major" if b_layout == "col" else " B=row-major")
+    variants = [v for v in range(_lib.num_variants()) if "any-alignment" in _lib.variant_name(v) and all(k in _lib.variant_name(v) for k in key)
+                and ("A=col-major" in _lib.variant_name(v)) == (a_layout == "col")]
+    assert len(variants) == 1, [_lib.variant_name(v) for v in variants]
+    v = variants[0]
+    for n, (M, N, K) in enumerate([(363, 64, 3025), (192, 48, 1225), (27, 32, 2201), (196, 600, 64), (100, 72, 41), (129, 257, 131), (1, 1, 1), (5, 300, 7)]):
+        print("variant", v, in_type, out_type, a_layout, b_layout, M, N, K, flush=True)
+        run_case(in_type, out_type, M, N, K, a_layout=a_layout, b_layout=b_layout, variant=v, seed=1200 + n)
+        run_case(in_type, out_type, M, N, K, a_layout=a_layout, b_layout=b_layout, variant=v, seed=1300 + n, prologue=ora.PRO_NONE,
+                 epilogue=ora.EPI_NONE)
+    # views that start at an odd element of larger arrays (pointers aligned to the element only, odd leading dimensions)
+    rng = np.random.default_rng(1400)
+    M, N, K = 150, 203, 333
+    Abig = make_input(rng, (K + 3, M + 5) if a_layout == "col" else (M + 3, K + 5), in_type)
+    Bbig = make_input(rng, (N + 3, K + 7) if b_layout == "col" else (K + 3, N + 7), in_type)
+    Cbig = make_c0(rng, (M + 2, N + 3), out_type)
+    dA, dB, dC = to_device(Abig, in_type), to_device(Bbig, in_type), to_device(Cbig, out_type)
+    Av = Abig[1:K + 1, 3:M + 3].T if a_layout == "col" else Abig[1:M + 1, 3:K + 3]
+    Bv = Bbig[1:N + 1, 5:K + 5].T if b_layout == "col" else Bbig[1:K + 1, 5:N + 5]
+    dAv = dA[1:K + 1, 3:M + 3].t() if a_layout == "col" else dA[1:M + 1, 3:K + 3]
+    dBv = dB[1:N + 1, 5:K + 5].t() if b_layout == "col" else dB[1:K + 1, 5:N + 5]
+    for prologue in (ora.PRO_SET0, ora.PRO_NONE):
+        dC.copy_(to_device(Cbig, out_type))
+        print("variant", v, in_type, out_type, a_layout, b_layout, "views, prologue", prologue, flush=True)
+        acc.gemm_relu(dAv, dBv, dC[1:M + 1, 1:N + 1], prologue=prologue, variant=v)
+        torch.cuda.synchronize()
+        got = to_host(dC, out_type)
+        want = ora.gemm_relu_exact(np.ascontiguousarray(Av), np.ascontiguousarray(Bv), np.ascontiguousarray(Cbig[1:M + 1, 1:N + 1]),
+                                   in_type, out_type, prologue, ora.EPI_RELU)
+        assert_matches(got[1:M + 1, 1:N + 1], want, out_type, K)
+        rest = np.ones(Cbig.shape, bool)
+        rest[1:M + 1, 1:N + 1] = False
+        assert np.array_equal(got[rest], Cbig[rest]), "elements around the view were written"
+
+
+def test_odd_sizes_take_an_mfma_kernel_automatically():
+    """K, N or leading dimensions that are not multiples of the 16-byte vector no longer fall to the thread-bound kernel."""
+    from accera_amd import _lib
+    for in_t, out_t, M, N, K in ((_lib.I8, _lib.I32, 1000, 1000, 1000), (_lib.F16, _lib.F32, 363, 64, 3025), (_lib.BF16, _lib.BF16, 289, 384, 2593)):
+        g, b, lds, v = _lib.launch_geometry(in_t, out_t, M, N, K, (K, 1), (N, 1), (N, 1))
+        assert "any-alignment" in _lib.variant_name(v), _lib.variant_name(v)
+    run_case("i8", "i32", 1000, 1000, 1000, seed=77, expect_variant=None)
+    run_case("f16", "f16", 289, 384, 2593, seed=78, a_layout="col")
+
+
+def _named(*keys, b_layout="row"):
+    """The first variant whose description holds every key."""
+    return next(v for v, n in _variants(b_layout) if all(k in n for k in keys))
+
+
+@pytest.mark.parametrize("in_type,out_type", [("f16", "f32"), ("f16", "f16"), ("bf16", "bf16"), ("i8", "i32"), ("i8", "i8")])
+def test_k_split_of_the_mfma_kernels(in_type, out_type):
+    """K split over workgroups: the kernel runs as a batch of partial products into a workspace, a second kernel adds the
+    slices in slice order and applies the ops (the ReLU after the whole sum).  Per kernel family and split count, slices
+    of equal and unequal length, C overwritten and read, every op; integer results bit-exact; two runs give the same bits."""
+    import accera_amd as acc
+    import torch
+    from accera_amd import _lib
+    kb = 64 if in_type == "i8" else 32
+    families = [("hand-laid", "row", "row", ("mfma 256x256", "hand-laid loop")), ("hand-laid, B col-major", "row", "col", ("mfma 256x256", "hand-laid loop")),
+                ("hand-laid, A col-major", "col", "row", ("A=col-major", "hand-laid loop")),
+                ("ping-pong 16x16", "row", "row", ("mfma 256x256 kb64", "pingpong mi16")), ("128x128 direct", "row", "row", ("mfma 128x128 kb64", "fill=direct")),
+                ("any alignment", "row", "row", ("any-alignment",))]
+    for label, a_layout, b_layout, keys in families:
+        v = next(v for v, n in _variants(b_layout) if all(k in n for k in keys) and ("A=col-major" in n) == (a_layout == "col")
+                 and "multi-tile" not in n)
+        for splits, k_tiles in ((2, 8), (3, 40), (5, 21), (8, 40)):
+            print(label, "variant", v, in_type, out_type, "splits", splits, "k tiles", k_tiles, flush=True)
+            g = _lib.launch_geometry(ora.TYPE_IDS[in_type], ora.TYPE_IDS[out_type], 256, 512, k_tiles * kb,
+                                     (1, 256) if a_layout == "col" else (k_tiles * kb, 1), (1, k_tiles * kb) if b_layout == "col" else (512, 1), (512, 1), v, splits)[0]
+            assert 1 < g[2] <= splits, g
+            run_case(in_type, out_type, 256, 512, k_tiles * kb, a_layout=a_layout, b_layout=b_layout, variant=v, splits=splits, seed=1500 + splits)
+            if out_type != "i8" or "hand-laid" not in label:
+                run_case(in_type, out_type, 256, 512, k_tiles * kb, a_layout=a_layout, b_layout=b_layout, variant=v, splits=splits, seed=1510 + splits,
+                         prologue=ora.PRO_NONE, epilogue=ora.EPI_RELU_NOCOND)
+    # odd sizes on the any-alignment kernel; SCALE / SET ops with their operands; the same bits on a second run
+    v = _named("any-alignment")
+    rng = np.random.default_rng(1520)
+    M, N, K = 147, 64 if out_type == "i8" else 65, 3025   # (rows of an int8 C must be 16 bytes apart for the MFMA kernels)
+    A, B = make_input(rng, (M, K), in_type), make_input(rng, (K, N), in_type)
+    C0 = make_c0(rng, (M, N), out_type, scale=100)
+    for pro, pa, epi, ea in ((ora.PRO_SCALE, 0.5, ora.EPI_SCALE, 2.0), (ora.PRO_SET, 3.0, ora.EPI_RELU, 0.0), (ora.PRO_NONE, 0.0, ora.EPI_SET, 1.0)):
+        outs = []
+        for _ in range(2):
+            dC = to_device(C0, out_type)
+            acc.gemm_relu(to_device(A, in_type), to_device(B, in_type), dC, prologue=pro, prologue_arg=pa, epilogue=epi, epilogue_arg=ea,
+                          variant=v, k_splits=4)
+            torch.cuda.synchronize()
+            outs.append(to_host(dC, out_type))
+        assert np.array_equal(outs[0].view(np.uint8), outs[1].view(np.uint8)), "a K split must add its slices in a fixed order"
+        want = ora.gemm_relu_exact(A, B, C0, in_type, out_type, pro, epi, prologue_arg=pa, epilogue_arg=ea)
+        assert_matches(outs[0], want, out_type, K)
+
+
+def test_k_split_is_chosen_for_small_outputs_with_a_long_k_and_refused_where_it_cannot_run():
+    """Shapes of the reference's sweep lists that leave most compute units idle (gemm_bert_assorted.csv: 768 x 320 x 30522;
+    gemm_resnet_inception.csv: 288 x 64 x 21609) are split by the library itself; the benchmark configurations are not."""
+    import accera_amd as acc
+    from accera_amd import _lib
+    g, b, lds, v = _lib.launch_geometry(_lib.F16, _lib.F32, 768, 320, 30522, (30522, 1), (320, 1), (320, 1))
+    assert "mfma" in _lib.variant_name(v) and g[2] > 1, (g, _lib.variant_name(v))
+    run_case("f16", "f32", 768, 320, 30522, seed=1530, dist="normal")
+    run_case("i8", "i32", 288, 64, 21609, seed=1531)
+    run_case("bf16", "bf16", 512, 256, 8192, seed=1532, prologue=ora.PRO_NONE)
+    for M, N, K, sa, sb, sc, t_in, t_out in ((4096, 4096, 4096, (4096, 1), (4096, 1), (4096, 1), _lib.F16, _lib.F32),
+                                             (4096, 3072, 768, (768, 1), (1, 768), (3072, 1), _lib.BF16, _lib.BF16),
+                                             (8192, 8192, 8192, (8192, 1), (8192, 1), (8192, 1), _lib.I8, _lib.I32)):
+        assert _lib.launch_geometry(t_in, t_out, M, N, K, sa, sb, sc)[0][2] == 1
+    with pytest.raises(_lib.Acc950Error):  # three K tiles cannot be split for a kernel whose slices need four each
+        _lib.launch_geometry(_lib.F16, _lib.F32, 256, 256, 224, (224, 1), (256, 1), (256, 1), _hand_laid("row"), 2)
