@@ -367,7 +367,9 @@ bool plan_split(const MfmaVariant& v, const Problem& pb, int want, SplitPlan* sp
 }
 
 // Splits the library takes by itself: only when the tiles leave at least half of the compute units idle and K is long
-// enough for the second kernel (a few microseconds) to pay.
+// enough for the second kernel (a few microseconds) to pay.  Measured on small outputs with a long K (512 x 512 x 8192,
+// 256 x 256 x 16384, 1024 x 1024 x 4096, 768 x 320 x 30522, 1024 x 80 x 30522; 16-bit inputs): the best split brings the
+// workgroups to about one per compute unit and leaves a slice 16 to 60 k-steps of 64 bytes.
 int auto_mfma_splits(const MfmaVariant& v, const Problem& pb)
 {
     const GemmArgs& g = pb.g;
@@ -376,7 +378,7 @@ int auto_mfma_splits(const MfmaVariant& v, const Problem& pb)
     if (tiles * 2 > kComputeUnits) return 1;
     const int64_t steps = (int64_t)g.K * elem_size(g.in_type) / 64; // k-steps of 64 bytes
     if (steps < 32) return 1;
-    int64_t want = kComputeUnits / tiles < steps / 8 ? kComputeUnits / tiles : steps / 8;
+    int64_t want = kComputeUnits / tiles < steps / 16 ? kComputeUnits / tiles : steps / 16;
     if (want > 32) want = 32;
     if ((size_t)want * (size_t)g.M * (size_t)g.N > ((size_t)1 << 24)) return 1; // 64 MiB of partial sums at most without being asked
     SplitPlan sp;
