@@ -503,15 +503,15 @@ int run(const Problem& pb, const Choice& c, hipStream_t stream, LaunchGeom* geom
         const MfmaVariant& mv = tab[c.variant];
         const bool lean = g.prologue == PRO_SET && g.prologue_arg == 0.f && (g.epilogue == EPI_RELU || g.epilogue == EPI_NONE);
         SplitPlan sp;
-        if (c.splits > 1 && plan_split(mv, pb, c.splits, &sp)) {
+        bool split = c.splits > 1 && plan_split(mv, pb, c.splits, &sp);
+        // (slices that do not fit the built-in workspace: the problem runs unsplit, which every variant that can be split also takes)
+        if (split && static_ws && (size_t)sp.splits * (size_t)g.M * (size_t)g.N > kStaticFloats) split = false;
+        if (split) {
             float* ws = nullptr;
             if (!dry_run) {
                 const size_t floats = (size_t)sp.splits * (size_t)g.M * (size_t)g.N;
                 unsigned* unused = nullptr;
                 if (static_ws) {
-                    if (floats > kStaticFloats)
-                        return fail(ACC950_UNSUPPORTED, "this problem's K split needs " + std::to_string(floats * sizeof(float)) +
-                                    " bytes of partial sums; the built-in workspace holds " + std::to_string(kStaticFloats * sizeof(float)) + " bytes");
                     e = static_workspace(&ws);
                     if (e != hipSuccess) return fail_hip(e, "address of the built-in workspace");
                 } else {

@@ -129,11 +129,12 @@ int acc950_gemm_ops_host(int in_type, int out_type, int M, int N, int K,
  * acc950_gemm_ops for callers that cannot allocate device memory (code under HIP graph capture, tight serving
  * loops, harnesses that forbid it).  It has no counterpart in the reference.  Same arguments, same kernels, same
  * results; the difference is where the skinny kernels' partial sums and arrival counters live when workgroups
- * combine their sums (a K split, or the shared column blocks of the default decode kernel): in a fixed array of
+ * combine their sums (a K split, or the shared column blocks of the default decode kernel), and the slices of an
+ * MFMA kernel's K split: in a fixed array of
  * ACC950_STATIC_WORKSPACE_BYTES inside the library's device image (each GPU the library runs on holds its own
  * copy until the process ends) instead of a per-stream allocation.  The call makes no hipMalloc / hipFree and no
- * other allocating call; a problem whose workspace would not fit returns ACC950_UNSUPPORTED and runs nothing
- * (8 x 11008 x 4096 needs 2.7 MiB).  All calls on one GPU share that array: calls that overlap on a GPU (different
+ * other allocating call; a skinny problem whose workspace would not fit returns ACC950_UNSUPPORTED and runs nothing
+ * (8 x 11008 x 4096 needs 2.7 MiB), an MFMA problem whose slices would not fit runs unsplit.  All calls on one GPU share that array: calls that overlap on a GPU (different
  * streams, different host threads) race on it -- keep them on one stream or use acc950_gemm_ops.  The kernels leave
  * the counters at zero, which is how the array starts.  Launch each kernel once outside a capture first: the first
  * launch of a kernel loads its code and may raise its LDS limit.

@@ -24,8 +24,9 @@ def test_static_workspace_entry_point_matches_the_allocating_one():
     stream = torch.cuda.current_stream().cuda_stream
     rng = np.random.default_rng(2024)
     # decode shape first (its slow-phase column blocks are shared by two workgroups each: 2.7 MiB of partial sums),
-    # then a smaller problem with an explicit K split over four workgroups per column block
-    cases = [(8, 11008, 4096, 0), (4, 2048, 1024, 4)]
+    # then a smaller problem with an explicit K split over four workgroups per column block; then a small square output
+    # with a long K, which the library splits by itself on an MFMA kernel (8 slices of 256 KiB of partial sums)
+    cases = [(8, 11008, 4096, 0), (4, 2048, 1024, 4), (256, 256, 4096, 0)]
     data = []
     for M, N, K, ks in cases:
         A = make_input(rng, (M, K), "f16", "normal")
@@ -35,6 +36,7 @@ def test_static_workspace_entry_point_matches_the_allocating_one():
         _lib.check(_call(L.acc950_gemm_ops, dA, dB, d_ref, M, N, K, ks, stream))
         data.append((A, B, dA, dB, d_ref, d_new))
     torch.cuda.synchronize()
+    assert _lib.launch_geometry(_lib.F16, _lib.F16, 256, 256, 4096, (4096, 1), (256, 1), (256, 1))[0][2] > 1
     allocations_before = _lib.allocation_probe()
     assert allocations_before >= 2  # the allocating entry point made this stream's workspace
     for rep in range(2):  # the pair of calls twice: the second round finds the array as the first left it
@@ -56,3 +58,15 @@ def test_static_workspace_entry_point_matches_the_allocating_one():
     assert rc == _lib.UNSUPPORTED and b"built-in workspace" in L.acc950_last_error()
     torch.cuda.synchronize()
     assert (to_host(d_new, "f16") == 9).all()
+    # an MFMA kernel's K split that does not fit runs unsplit instead (1024 x 1024 x 4096: four slices would be 16 MiB)
+    M = N = 1024
+    K = 4096
+    A = make_input(rng, (M, K), "f16", "normal")
+    B = (make_input(rng, (K, N), "f16", "normal").astype(np.float32) * 0.05).astype(np.float16)
+    dA, dB, dC = to_device(A, "f16"), to_device(B, "f16"), to_device(np.full((M, N), 9, np.float16), "f16")
+    assert _lib.launch_geometry(_lib.F16, _lib.F16, M, N, K, (K, 1), (N, 1), (N, 1))[0][2] > 1
+    _lib.check(_call(L.acc950_gemm_ops_static, dA, dB, dC, M, N, K, 0, stream))
+    torch.cuda.synchronize()
+    assert _lib.allocation_probe() == allocations_before
+    rows = rng.choice(M, 16, replace=False)
+    assert_matches(to_host(dC, "f16")[rows], ora.gemm_relu_exact(A[rows], B, out_zeros(16, N, "f16"), "f16", "f16", ora.PRO_SET0, ora.EPI_RELU), "f16", K)
