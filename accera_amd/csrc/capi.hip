@@ -9,6 +9,7 @@
 
 #include <atomic>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <map>
 #include <mutex>
@@ -143,10 +144,10 @@ bool mfma_can_take(const MfmaVariant& v, const Problem& pb)
         const bool lean = g.prologue == PRO_SET || os >= 2;
         if (!lean || g.K % bk || g.K < 4 * bk || (g.c_rs * os) % 16 || (g.batch > 1 && (g.c_bs * os) % 16)) return false;
         if (pb.have_pointers && !aligned16(g.C)) return false;
-        // any M, N >= one tile when C is only written: the last row / column of tiles is moved to end at M / N
-        // (its first column must still be 16 bytes aligned in B's and C's rows)
-        if (g.M % v.bm && (g.M < v.bm || g.prologue != PRO_SET || (!v.a_kc && g.M % vec))) return false;
-        if (g.N % v.bn && (g.N < v.bn || g.prologue != PRO_SET || g.N % vec || (g.N * os) % 16)) return false;
+        // any M, N >= one tile: the last row / column of tiles is moved to end at M / N (its first column must still be
+        // 16 bytes aligned in B's and C's rows); when C is read, the moved tile does not store what it shares with its neighbour
+        if (g.M % v.bm && (g.M < v.bm || (!v.a_kc && g.M % vec))) return false;
+        if (g.N % v.bn && (g.N < v.bn || g.N % vec || (g.N * os) % 16)) return false;
         if (g.K % bk) return false;
     }
     if (v.edge) {
@@ -474,6 +475,12 @@ int run(const Problem& pb, const Choice& c, hipStream_t stream, LaunchGeom* geom
             skinny_column_blocks(sv, g.N) >= 128 && skinny_column_blocks(sv, g.N) <= 200 && g.K >= 512 &&
             (g.batch <= 1 || (g.b_bs * 2) % 512 == 0))
             s.extra_phase = (int)((3u - (unsigned)(reinterpret_cast<uintptr_t>(g.B) >> 7)) & 3u);
+        // (measurement aid: ACC950_SKINNY_SHARED_PHASE = -1 switches the sharing off, 0..3 shares the blocks of that phase instead)
+        static const char* const phase_override = std::getenv("ACC950_SKINNY_SHARED_PHASE");
+        if (phase_override && s.extra_phase >= 0) {
+            const int v = std::atoi(phase_override);
+            s.extra_phase = v < 0 ? -1 : (int)(((unsigned)v - (unsigned)(reinterpret_cast<uintptr_t>(g.B) >> 7)) & 3u);
+        }
         const int ws_splits = s.extra_phase >= 0 ? 2 : c.splits;
         if (!dry_run && ws_splits > 1) {
             const size_t nb = g.batch > 1 ? (size_t)g.batch : 1;

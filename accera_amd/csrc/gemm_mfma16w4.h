@@ -14,8 +14,8 @@
 // the stores are those of gemm_mfma16.h.
 //
 // Takes: A row-major (or column-major, in the one-tile-per-workgroup form with 256-wide tiles: staged as it lies in memory and
-// read with the transposing LDS loads, like a row-major B), M and N multiples of the tile (any M >= 256 and any 16-byte-aligned N >= the tile width
-// when C is not read: the last row / column of tiles then overlaps the one before), K a multiple of one k-step (64 bytes)
+// read with the transposing LDS loads, like a row-major B), any M >= 256 and any 16-byte-aligned N >= the tile width
+// (the last row / column of tiles overlaps the one before), K a multiple of one k-step (64 bytes)
 // and at least four of them, rows of C 16 bytes aligned;
 // every prologue / epilogue op (an int8 C is only written, never read): C = A*B starts from zeros, C += A*B with a
 // 32-bit C loads the tile of C straight into the accumulator registers, everything else (a 16-bit C, beta * C,
@@ -104,8 +104,9 @@ __global__ void __launch_bounds__(256, 1) gemm_mfma16w4_kernel(GemmArgs p)
     stamp(0);
 
     // M and N need not be multiples of the tile: the last row / column of tiles ends at M / N and overlaps its
-    // neighbour.  What both compute gets the same bits from both (the host allows this only when C is not read,
-    // and only for N whose last tile still starts on a 16-byte boundary of B's and C's rows).
+    // neighbour (the host allows this only for N whose last tile still starts on a 16-byte boundary of B's and C's
+    // rows).  What both compute gets the same bits from both; when C is read, the moved tile leaves the rows and
+    // columns it shares with its neighbour to the neighbour (see the write-back), so that no element is added to twice.
     auto tile_origin = [&](int id, int& r0, int& c0) __attribute__((always_inline)) {
         int tile_m, tile_n;
         tile_coords(id, p.tiles_m, p.tiles_n, tile_m, tile_n);
@@ -480,6 +481,16 @@ __global__ void __launch_bounds__(256, 1) gemm_mfma16w4_kernel(GemmArgs p)
                 const unsigned mine = smem_addr + slab_off + (unsigned)((lane_wb & 15) * PITCH + (lane_wb >> 4) * 16);
                 const CTile tile = c_tile(p, m0 + (wave_u / WAVES_N) * WTM, n0 + (wave_u % WAVES_N) * WTN, OS);
                 const unsigned row_bytes = (unsigned)p.c_rs * OS;
+                // A tile that was moved up / left to end at M / N, of a problem that reads C: its first rows / columns belong
+                // to the neighbouring tile, which may or may not have written them yet -- they are not stored from here.
+                // (first row / column of the wave tile this workgroup owns; 0 wherever nothing is shared)
+                int own_row = 0, own_col = 0;
+                if (p.prologue != PRO_SET) {
+                    int tm, tn;
+                    tile_coords(tile_id, p.tiles_m, p.tiles_n, tm, tn);
+                    own_row = tm * BM - m0 - (wave_u / WAVES_N) * WTM;
+                    own_col = tn * BN - n0 - (wave_u % WAVES_N) * WTN;
+                }
                 constexpr int VPL = 16 / OS;                 // sums per lane and store
                 constexpr int GPR = WTN / VPL;               // 16-byte pieces of the output per row of the wave tile
                 constexpr int PIECES = (16 * GPR + 63) / 64; // stores per lane and row of blocks
@@ -497,8 +508,9 @@ __global__ void __launch_bounds__(256, 1) gemm_mfma16w4_kernel(GemmArgs p)
                         acc_t v[VPL / 4];
 #pragma unroll
                         for (int q = 0; q < VPL / 4; ++q) v[q] = finish(*(const acc_t*)(slab + r * PITCH + g * (VPL * 4) + q * 16));
-                        __builtin_amdgcn_raw_buffer_store_b128(pack(v), tile.rsrc, (unsigned)r * row_bytes + g * 16,
-                                                               (unsigned)(i.value * 16) * row_bytes, AUX);
+                        if (i.value * 16 + r >= own_row && g * VPL >= own_col)
+                            __builtin_amdgcn_raw_buffer_store_b128(pack(v), tile.rsrc, (unsigned)r * row_bytes + g * 16,
+                                                                   (unsigned)(i.value * 16) * row_bytes, AUX);
                     }
                 });
             };

@@ -334,7 +334,7 @@ def test_four_wave_kernel_on_views_of_larger_matrices(in_type, out_type, b_layou
 @pytest.mark.parametrize("in_type,out_type,M", [("f16", "f32", 600), ("bf16", "bf16", 1000), ("i8", "i32", 257), ("f16", "f16", 511)])
 def test_four_wave_kernel_any_number_of_rows(in_type, out_type, M):
     """M and N that are not multiples of the tile: the last row / column of tiles ends at M / N and overlaps the
-    one before it (allowed when C is only written).  Accumulating into C with such sizes is refused."""
+    one before it, overwriting C and accumulating into it."""
     import accera_amd as acc
     from accera_amd import _lib
     kb = 64 if in_type == "i8" else 32
@@ -343,8 +343,10 @@ def test_four_wave_kernel_any_number_of_rows(in_type, out_type, M):
             print("variant", v, in_type, out_type, b_layout, "M", M, flush=True)
             run_case(in_type, out_type, M, 768, 8 * kb, b_layout=b_layout, variant=v, seed=M)
             run_case(in_type, out_type, M, 768 + 16 + 64 * (M % 3), 4 * kb, b_layout=b_layout, variant=v, seed=M + 1)  # N ragged too
-            with pytest.raises(_lib.Acc950Error):
-                run_case(in_type, out_type, M, 768, 8 * kb, b_layout=b_layout, variant=v, seed=M, prologue=ora.PRO_NONE)
+            # C += A*B with such sizes: the moved tiles leave what they share with their neighbours to the neighbours
+            run_case(in_type, out_type, M, 768, 8 * kb, b_layout=b_layout, variant=v, seed=M + 2, prologue=ora.PRO_NONE)
+            run_case(in_type, out_type, M, 768 + 16 + 64 * (M % 3), 5 * kb, b_layout=b_layout, variant=v, seed=M + 3, prologue=ora.PRO_NONE,
+                     epilogue=ora.EPI_NONE)
     with pytest.raises(_lib.Acc950Error):  # fewer rows than one tile
         run_case(in_type, out_type, 200, 768, 8 * kb, variant=_hand_laid("row"))
 
@@ -790,7 +792,7 @@ def test_random_problems_on_the_four_wave_kernel():
         v = variants[rng.integers(len(variants))]
         kb = 64 if in_type == "i8" else 32
         pro, pa, epi, ea = ops[rng.integers(len(ops))]
-        whole = pro != ora.PRO_SET or rng.integers(2) == 0          # ragged sizes only when C is not read
+        whole = rng.integers(2) == 0
         tile_n = 192 if "256x192" in _lib.variant_name(v) else 256
         M = int(rng.integers(1, 5)) * 256 if whole else int(rng.integers(256, 1100))
         N = int(rng.integers(1, 5)) * tile_n if whole else int(rng.integers(tile_n // 16, 70)) * 16
@@ -833,6 +835,9 @@ def test_random_problems_on_the_four_wave_kernel():
     # C is read: C += A*B straight into the accumulators (32-bit C), and widened / scaled by ordinary code
     ("i8", "i32", "row", 4352, 4096, 512, "none", "relu"),
     ("f16", "f16", "row", 4352, 4096, 256, "scale", "scale"),
+    # ragged sizes and C read: moved tiles do not store what their neighbours own
+    ("f16", "f32", "row", 4400, 4112, 256, "none", "relu"),
+    ("bf16", "bf16", "col", 4400, 4112, 384, "scale", "none"),
     # three rounds over the workgroups
     ("i8", "i32", "row", 8192, 6144, 256, "set0", "relu"),
 ])
