@@ -70,3 +70,55 @@ def test_static_workspace_entry_point_matches_the_allocating_one():
     assert _lib.allocation_probe() == allocations_before
     rows = rng.choice(M, 16, replace=False)
     assert_matches(to_host(dC, "f16")[rows], ora.gemm_relu_exact(A[rows], B, out_zeros(16, N, "f16"), "f16", "f16", ora.PRO_SET0, ora.EPI_RELU), "f16", K)
+
+
+def test_static_workspace_entry_point_under_graph_capture():
+    """What the entry point is for: a chain of launches recorded into a HIP graph (no allocation may happen while a
+    stream is capturing) and replayed.  A two-layer decode step -- skinny GEMM + ReLU, then a second skinny GEMM on its
+    output -- plus a small-output GEMM that the library splits over K (two kernels); every replay is checked against the
+    same calls made eagerly, with the program's own work and synchronisations between the replays."""
+    import torch
+    from accera_amd import _lib
+    L = _lib.lib()
+    _lib.check(L.acc950_init(0))
+    rng = np.random.default_rng(77)
+    M, H, F = 8, 4096, 11008
+    X = make_input(rng, (M, H), "f16", "normal")
+    W1 = (make_input(rng, (H, F), "f16", "normal").astype(np.float32) * 0.03).astype(np.float16)
+    W2 = (make_input(rng, (F, H), "f16", "normal").astype(np.float32) * 0.03).astype(np.float16)
+    P, Q = make_input(rng, (256, 4096), "f16", "normal"), (make_input(rng, (4096, 256), "f16", "normal").astype(np.float32) * 0.05).astype(np.float16)
+    dX, dW1, dW2, dP, dQ = (to_device(a, "f16") for a in (X, W1, W2, P, Q))
+    mk = lambda r, c: to_device(np.zeros((r, c), np.float16), "f16")
+    hid_e, out_e, sq_e, hid_g, out_g, sq_g = mk(M, F), mk(M, H), mk(256, 256), mk(M, F), mk(M, H), mk(256, 256)
+
+    def step(entry, hid, out, sq, stream):
+        args = lambda A, B, C, m, n, k, epi: (_lib.F16, _lib.F16, m, n, k, A.data_ptr(), k, 1, B.data_ptr(), n, 1, C.data_ptr(), n, 1,
+                                              _lib.PROLOGUE_SET0, 0.0, epi, 0.0, _lib.VARIANT_AUTO, 0, stream)
+        _lib.check(entry(*args(dX, dW1, hid, M, F, H, _lib.EPILOGUE_RELU)))
+        _lib.check(entry(*args(hid, dW2, out, M, H, F, _lib.EPILOGUE_NONE)))
+        _lib.check(entry(*args(dP, dQ, sq, 256, 256, 4096, _lib.EPILOGUE_RELU)))
+
+    # eager, on the current stream (also loads every kernel's code and sets its LDS limit before the capture)
+    step(L.acc950_gemm_ops_static, hid_e, out_e, sq_e, torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    want = [to_host(t, "f16").copy() for t in (hid_e, out_e, sq_e)]
+    assert_matches(want[0], ora.gemm_relu_exact(X, W1, out_zeros(M, F, "f16"), "f16", "f16", ora.PRO_SET0, ora.EPI_RELU), "f16", H)
+    before = _lib.allocation_probe()
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            step(L.acc950_gemm_ops_static, hid_g, out_g, sq_g, side.cuda_stream)
+    assert _lib.allocation_probe() == before
+    for replay in range(4):
+        for t in (hid_g, out_g, sq_g):
+            t.fill_(3)                                   # eager work between the replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for got, ref in zip((hid_g, out_g, sq_g), want):
+            assert np.array_equal(to_host(got, "f16").view(np.uint16), ref.view(np.uint16)), replay
+        if replay == 1:                                  # the same entry point eagerly, between replays: the array is shared
+            step(L.acc950_gemm_ops_static, hid_e, out_e, sq_e, torch.cuda.current_stream().cuda_stream)
+            torch.cuda.synchronize()
