@@ -29,12 +29,12 @@ def test_shape_list_fixture():
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("in_type,out_type", [("f16", "f16"), ("i8", "i32")])
+@pytest.mark.parametrize("in_type,out_type", [("f16", "f16"), ("bf16", "f32"), ("i8", "i32")])
 def test_every_shape_of_the_reference_sweep_lists(in_type, out_type):
     import accera_amd as acc
     import torch
     from accera_amd import _lib
-    tdt = {"f16": torch.float16, "i8": torch.int8, "i32": torch.int32}
+    tdt = {"f16": torch.float16, "bf16": torch.bfloat16, "f32": torch.float32, "i8": torch.int8, "i32": torch.int32}
     gen = torch.Generator(device="cuda")
     gen.manual_seed(339)
     kinds = {}
@@ -61,8 +61,9 @@ def test_every_shape_of_the_reference_sweep_lists(in_type, out_type):
         idx = np.arange(M) if M <= 48 else np.random.default_rng(n).choice(M, 24, replace=False)
         sel = torch.as_tensor(idx, device="cuda")
         torch.cuda.synchronize()
-        want = ora.gemm_relu_exact(A[sel].cpu().numpy(), B.cpu().numpy(), C0[sel].cpu().numpy(), in_type, out_type, prologue, ora.EPI_RELU)
-        assert_matches(C[sel].cpu().numpy(), want, out_type, K)
+        host = lambda x, t: x.cpu().view(torch.int16).numpy().view(np.uint16) if t == "bf16" else x.cpu().numpy()  # (bf16 travels as its bits)
+        want = ora.gemm_relu_exact(host(A[sel], in_type), host(B, in_type), host(C0[sel], out_type), in_type, out_type, prologue, ora.EPI_RELU)
+        assert_matches(host(C[sel], out_type), want, out_type, K)
     print(kinds)
     assert kinds.get("any-alignment", 0) + kinds.get("any-alignment, K split", 0) >= 90
     assert sum(c for k, c in kinds.items() if "K split" in k) >= 20
