@@ -153,7 +153,15 @@ bool mfma_can_take(const MfmaVariant& v, const Problem& pb)
     if (v.edge) {
         if (!v.any && (g.K % vec || (!v.b_kc && g.N % vec) || (!v.a_kc && g.M % vec))) return false;
     } else {
-        if (!v.w4 && (g.M % v.bm || g.N % v.bn || g.K % bk)) return false;
+        if (!v.w4 && g.K % bk) return false;
+        if (!v.w4) {
+            // the 32x32-shape kernels move the last row / column of tiles to end at M / N when C is only written; the
+            // eight-wave kernels on the 16x16 shapes take whole tiles only
+            const int os = elem_size(g.out_type);
+            const bool movable = !v.mi16 && g.prologue == PRO_SET;
+            if (g.M % v.bm && (!movable || g.M < v.bm || (!v.a_kc && g.M % vec))) return false;
+            if (g.N % v.bn && (!movable || g.N < v.bn || g.N % vec || (g.N * os) % 16)) return false;
+        }
     }
     // offsets inside one output tile are 32-bit in the write-back
     if ((int64_t)v.bm * g.c_rs * 4 >= (1ll << 32)) return false;

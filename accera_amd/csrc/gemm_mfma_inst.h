@@ -90,6 +90,12 @@ static const MfmaVariant kVariants[] = {
     VANY(true, true),
     VANY(false, false),
     VANY(false, true),
+    // 128x128 tiles with four stages of 128 bytes of K: 96 KB on their way to a CU at a time (medium-sized problems of one
+    // tile per CU are bound by the latency of their fills, not by the matrix cores)
+    V(128, 128, 2, 2, false, true, false, 128, 4),
+    V(128, 128, 2, 2, true, true, false, 128, 4),
+    VA(false, 128, 128, 2, 2, false, true, false, 128, 4),
+    VA(false, 128, 128, 2, 2, true, true, false, 128, 4),
 };
 #undef LAYOUT_AT
 #undef VA

@@ -1019,3 +1019,30 @@ def test_k_split_is_chosen_for_small_outputs_with_a_long_k_and_refused_where_it_
         assert _lib.launch_geometry(t_in, t_out, M, N, K, sa, sb, sc)[0][2] == 1
     with pytest.raises(_lib.Acc950Error):  # three K tiles cannot be split for a kernel whose slices need four each
         _lib.launch_geometry(_lib.F16, _lib.F32, 256, 256, 224, (224, 1), (256, 1), (256, 1), _hand_laid("row"), 2)
+
+
+@pytest.mark.parametrize("in_type,out_type", [("f16", "f32"), ("bf16", "bf16"), ("i8", "i32")])
+def test_full_tile_kernels_on_sizes_that_are_not_tile_multiples(in_type, out_type):
+    """The direct-fill kernels on the 32x32 instruction shapes take any M, N of at least one tile when C is only written:
+    the last row / column of tiles is moved to end at M / N.  Every such variant, both layouts of B, column-major A;
+    reading C with such sizes is refused (the edge kernels take it)."""
+    from accera_amd import _lib
+    vec = 16 if in_type == "i8" else 8
+    seen = 0
+    for b_layout in ("row", "col"):
+        for v, name in _variants(b_layout):
+            if "fill=direct" not in name or "mi16" in name:
+                continue
+            bm, bn = map(int, re.search(r"mfma (\d+)x(\d+)", name).groups())
+            kb = int(re.search(r"kb(\d+)", name).group(1)) // (1 if in_type == "i8" else 2)
+            a_layout = "col" if "A=col-major" in name else "row"
+            M, N = 2 * bm + 5 * vec, bn + 3 * 16
+            print("variant", v, name, in_type, M, N, flush=True)
+            run_case(in_type, out_type, M, N, 5 * kb, a_layout=a_layout, b_layout=b_layout, variant=v, seed=1600 + v)
+            run_case(in_type, out_type, bm, N, 3 * kb, a_layout=a_layout, b_layout=b_layout, variant=v, seed=1700 + v, epilogue=ora.EPI_NONE)
+            with pytest.raises(_lib.Acc950Error):
+                run_case(in_type, out_type, M, N, 5 * kb, a_layout=a_layout, b_layout=b_layout, variant=v, seed=1, prologue=ora.PRO_NONE)
+            with pytest.raises(_lib.Acc950Error):   # less than one tile
+                run_case(in_type, out_type, bm - vec, N, 5 * kb, a_layout=a_layout, b_layout=b_layout, variant=v, seed=1)
+            seen += 1
+    assert seen >= 20
