@@ -25,7 +25,7 @@ EXPORTS = [
     "acc950_variant_name", "acc950_last_error",
 ]
 # measurement aids (include/accera_mi355x_probes.h): not part of the product ABI
-PROBE_EXPORTS = ["acc950_mfma_ceiling", "acc950_mfma_phase_probe", "acc950_copy_probe", "acc950_stream_read_probe", "acc950_workspace_probe", "acc950_allocation_probe"]
+PROBE_EXPORTS = ["acc950_mfma_ceiling", "acc950_mfma_traffic_probe", "acc950_mfma_phase_probe", "acc950_copy_probe", "acc950_stream_read_probe", "acc950_workspace_probe", "acc950_allocation_probe"]
 
 
 class Acc950Error(RuntimeError):
@@ -67,6 +67,7 @@ def lib():
                                                                            ctypes.POINTER(cu), ctypes.POINTER(ci)]
     L.acc950_variant_name.argtypes = [ci, ctypes.c_char_p, ctypes.c_size_t]
     L.acc950_mfma_ceiling.argtypes = [ci, ci, ci, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double)]
+    L.acc950_mfma_traffic_probe.argtypes = [ci, ci, ci, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double)]
     L.acc950_mfma_phase_probe.argtypes = [ci, ci, ci, ci, ci, vp, vp, vp, ctypes.POINTER(ctypes.c_double)]
     L.acc950_copy_probe.argtypes = [vp, vp, ctypes.c_size_t, vp]
     L.acc950_stream_read_probe.argtypes = [vp, ctypes.c_size_t, vp, vp]
@@ -99,6 +100,14 @@ def mfma_ceiling(in_type, data_mode=2, iters=20000):
     data_mode 0 zeros, 1 constant, 2 random operands."""
     t, g = ctypes.c_double(), ctypes.c_double()
     check(lib().acc950_mfma_ceiling(in_type, data_mode, iters, ctypes.byref(t), ctypes.byref(g)))
+    return t.value, g.value
+
+
+def mfma_traffic_probe(in_type, traffic, iters=2000):
+    """(tera-ops/s, sustained shader clock in GHz) of the four-wave loop's MFMAs with its traffic added piece by piece:
+    traffic 0 none, 1 its LDS reads, 2 also its direct-to-LDS fills from the caches, 3 the fills from a 1 GiB buffer."""
+    t, g = ctypes.c_double(), ctypes.c_double()
+    check(lib().acc950_mfma_traffic_probe(in_type, traffic, iters, ctypes.byref(t), ctypes.byref(g)))
     return t.value, g.value
 
 

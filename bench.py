@@ -214,8 +214,13 @@ def machine_ceiling(c):
         t = getattr(_lib, c["in_type"].upper())
         rnd, ghz = _lib.mfma_ceiling(t, 2, 20000)
         cool, ghz0 = _lib.mfma_ceiling(t, 0, 20000)
-        return {"mfma_only_random_operands": round(rnd, 1), "clock_ghz_random": round(ghz, 3),
-                "mfma_only_zero_operands": round(cool, 1), "clock_ghz_zero": round(ghz0, 3), "unit": "TFLOP/s" if t != _lib.I8 else "TOP/s"}
+        out = {"mfma_only_random_operands": round(rnd, 1), "clock_ghz_random": round(ghz, 3),
+               "mfma_only_zero_operands": round(cool, 1), "clock_ghz_zero": round(ghz0, 3), "unit": "TFLOP/s" if t != _lib.I8 else "TOP/s"}
+        # the four-wave loop's MFMAs with its traffic added piece by piece: which traffic the sustained clock follows
+        for key, traffic in (("four_wave_issue_no_traffic", 0), ("plus_lds_reads", 1), ("plus_fills_from_cache", 2), ("plus_fills_from_hbm", 3)):
+            rate, clock = _lib.mfma_traffic_probe(t, traffic, 3000)
+            out[key] = {"rate": round(rate, 1), "clock_ghz": round(clock, 3)}
+        return out
     if c["bound"] == "hbm":
         nbytes = c["K"] * c["N"] * ES[c["in_type"]]
         bufs = [torch.empty(nbytes, dtype=torch.uint8, device="cuda").fill_(i + 1) for i in range(8)]

@@ -24,6 +24,11 @@ extern "C" {
  * The sustained clock under MFMA load depends on the operand data, so the random-data
  * figure is the practical compute roof for random GEMM inputs on the device at hand.
  *
+ * acc950_mfma_traffic_probe: the same MFMAs, one wave per SIMD and 64 per step as in the four-wave GEMM loop, on random
+ * operands, with that loop's traffic added piece by piece: traffic 0 none, 1 its 24 LDS reads per step, 2 also its
+ * direct-to-LDS fills (32 KB per step and workgroup) from a buffer that stays in the caches, 3 the fills from a 1 GiB
+ * buffer.  Shows which traffic the sustained clock follows.
+ *
  * acc950_mfma_phase_probe: runs a build of the 256x256 MFMA kernel the automatic choice takes
  * for large aligned problems (four waves with the hand-laid K loop when K has at least four
  * K tiles of 64 bytes, else the eight-wave ping-pong form) that reads the shader-clock counter
@@ -41,6 +46,7 @@ extern "C" {
  * byte counters and for the achievable HBM rate.  `scratch4` is 4 bytes of device memory.
  */
 int acc950_mfma_ceiling(int in_type, int data_mode, int iters, double* tera_ops, double* clock_ghz);
+int acc950_mfma_traffic_probe(int in_type, int traffic, int iters, double* tera_ops, double* clock_ghz);
 int acc950_mfma_phase_probe(int in_type, int out_type, int M, int N, int K, const void* A, const void* B, void* C, double out[8]);
 int acc950_copy_probe(void* dst, const void* src, size_t bytes, void* stream);
 int acc950_stream_read_probe(const void* src, size_t bytes, void* scratch4, void* stream);
