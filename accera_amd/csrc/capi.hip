@@ -313,6 +313,9 @@ int auto_mfma_variant(const Problem& pb)
         // rank inside one tile shape: ping-pong kb64 x4 > ping-pong others > 8-wave > 4-wave (kb64 x4 first)
         int rank = v.pingpong ? (v.kb == 64 && v.stages == 4 ? 8 : 6) : (v.waves_m * v.waves_n == 8 ? 4 : 2);
         if (!v.pingpong && v.kb == 64 && v.stages == 4) rank += 1;
+        // one tile per CU at most: the deepest prefetch wins (four stages of 128 bytes of K; 2048^3: 21.8 against 25-26 us), where
+        // more tiles than CUs want two workgroups per CU, which only the smaller stages leave room for
+        if (!v.pingpong && v.direct && v.kb == 128 && v.stages == 4 && tiles <= kComputeUnits) rank += 2;
         // 16x16 shapes: measured 4-9 % faster than the 32x32 shapes on every large problem, in the lean build
         // (C = A*B, C = relu(A*B)); their full build reads C element by element and lost 20 % to the 32x32 form
         const bool lean = pb.g.prologue == PRO_SET && pb.g.prologue_arg == 0.f && (pb.g.epilogue == EPI_RELU || pb.g.epilogue == EPI_NONE);
@@ -386,7 +389,7 @@ int auto_mfma_splits(const MfmaVariant& v, const Problem& pb)
     const int64_t tiles = (((int64_t)g.M + v.bm - 1) / v.bm) * (((int64_t)g.N + v.bn - 1) / v.bn);
     if (tiles * 2 > kComputeUnits) return 1;
     const int64_t steps = (int64_t)g.K * elem_size(g.in_type) / 64; // k-steps of 64 bytes
-    if (steps < 32) return 1;
+    if (steps < 64) return 1; // (1024^3, 32 k-steps: 9.8 us unsplit, 15.1 us in two slices -- the second kernel costs about 5 us)
     int64_t want = kComputeUnits / tiles < steps / 16 ? kComputeUnits / tiles : steps / 16;
     if (want > 32) want = 32;
     if ((size_t)want * (size_t)g.M * (size_t)g.N > ((size_t)1 << 24)) return 1; // 64 MiB of partial sums at most without being asked
