@@ -56,6 +56,7 @@ const MfmaVariant* mfma_table(int in_type, int* n)
     case T_F16: return mfma_variants_f16(n);
     case T_BF16: return mfma_variants_bf16(n);
     case T_I8: return mfma_variants_i8(n);
+    case T_F32: return mfma_variants_f32(n);
     default: *n = 0; return nullptr;
     }
 }
@@ -120,6 +121,7 @@ int make_problem(int in_type, int out_type, int M, int N, int K,
 bool mfma_can_take(const MfmaVariant& v, const Problem& pb)
 {
     const GemmArgs& g = pb.g;
+    if (!v.launch) return false; // (a place in the table this input type has no kernel for)
     if (g.M <= 0 || g.N <= 0 || g.K <= 0) return false;
     const int es = elem_size(g.in_type), vec = 16 / es, bk = v.kb / es;
     if (g.c_cs != 1) return false;                          // C row-major
@@ -412,8 +414,21 @@ int choose(const Problem& pb, int variant, int k_splits, Choice* c)
             c->splits = k_splits > 0 ? k_splits : auto_skinny_splits(sv, pb.g);
             return ACC950_OK;
         }
-        if (f32_can_take(pb.g)) { c->variant = ACC950_VARIANT_F32_MFMA; return ACC950_OK; }
         int mv = auto_mfma_variant(pb);
+        if (pb.g.in_type == T_F32 && f32_can_take(pb.g)) {
+            // fp32: the LDS-tiled kernels when their workgroups (tiles x K slices) fill at least half of the chip, else the kernel
+            // of 32 x 32 blocks (512^3: 16 tiles of 128 x 128 would keep 16 CUs busy)
+            int slices = 1;
+            if (mv >= 0) {
+                int n = 0;
+                const MfmaVariant& v = mfma_table(pb.g.in_type, &n)[mv];
+                SplitPlan sp;
+                slices = k_splits > 1 ? (plan_split(v, pb, k_splits, &sp) ? sp.splits : 1) : k_splits == 0 ? auto_mfma_splits(v, pb) : 1;
+                const int64_t tiles = (((int64_t)pb.g.M + v.bm - 1) / v.bm) * (((int64_t)pb.g.N + v.bn - 1) / v.bn);
+                if (tiles * slices * 2 < kComputeUnits) mv = -1;
+            }
+            if (mv < 0) { c->variant = ACC950_VARIANT_F32_MFMA; return ACC950_OK; }
+        }
         c->variant = mv >= 0 ? mv : ACC950_VARIANT_GENERIC;
         if (mv >= 0) {
             int n = 0;

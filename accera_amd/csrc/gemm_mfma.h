@@ -34,10 +34,11 @@
 
 namespace acc950 {
 
-enum : int { IN_F16 = 0, IN_BF16 = 1, IN_I8 = 2 };
+enum : int { IN_F16 = 0, IN_BF16 = 1, IN_I8 = 2, IN_F32 = 3 };
 
 template <int IN> struct InTraits { static constexpr int ES = 2; using acc_t = f32x16; using scalar_t = float; };
 template <> struct InTraits<IN_I8> { static constexpr int ES = 1; using acc_t = i32x16; using scalar_t = int; };
+template <> struct InTraits<IN_F32> { static constexpr int ES = 4; using acc_t = f32x16; using scalar_t = float; };
 
 template <int IN>
 __device__ __forceinline__ void mfma32(const i32x4& a, const i32x4& b, typename InTraits<IN>::acc_t& c)
@@ -46,7 +47,16 @@ __device__ __forceinline__ void mfma32(const i32x4& a, const i32x4& b, typename 
         c = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
     else if constexpr (IN == IN_BF16)
         c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
-    else
+    else if constexpr (IN == IN_F32) {
+        // fp32: v_mfma_f32_32x32x2_f32 sums two k per instruction, one from each half of the wave.  A fragment holds four
+        // consecutive k of its row per lane (k 0..3 in lanes 0-31, k 4..7 in lanes 32-63 of the 32-byte step), the same for
+        // both operands, so instruction e pairs k = e with k = 4 + e and four of them sum the step.
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int ai = a[e], bi = b[e]; // (into scalars first: a bit cast applied to the element expression itself reads element 0)
+            c = __builtin_amdgcn_mfma_f32_32x32x2f32(__int_as_float(ai), __int_as_float(bi), c, 0, 0, 0);
+        }
+    } else
         c = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c, 0, 0, 0);
 }
 
@@ -89,7 +99,12 @@ struct OperandTile {
     __device__ static __forceinline__ int swizzle(int row, int c)
     {
         if constexpr (KC) return KB == 128 ? c ^ ((row >> 1) & 7) : c ^ ((row >> 2) & 3);
-        else if constexpr (!MI16) {
+        else if constexpr (ES == 4) {
+            // 32-bit elements are read one per lane (32 neighbouring columns of a k row = 128 bytes: all banks of one half); the
+            // two halves of a wave read k rows four apart and share their banks -- two passes per read, which the 64-cycle
+            // fp32 instructions hide, so there is no swizzle to keep in step with the fills
+            return c;
+        } else if constexpr (!MI16) {
             if constexpr (ES == 2) return c ^ (((row & 3) << 2) & (CPR - 1));
             else return c ^ (((row & 7) << 1) & (CPR - 1));
         } else {
@@ -99,7 +114,7 @@ struct OperandTile {
             else return c ^ ((((row & 7) << 1) | ((row >> 4) & 1)) & (CPR - 1));
         }
     }
-    static constexpr int SWIZZLE_PERIOD = KC ? 16 : (ES == 2 ? (MI16 ? 16 : 4) : (MI16 ? 32 : 8)); // rows after which it repeats
+    static constexpr int SWIZZLE_PERIOD = KC ? 16 : ES == 4 ? 1 : (ES == 2 ? (MI16 ? 16 : 4) : (MI16 ? 32 : 8)); // rows after which it repeats
 
     // Byte offset in global memory of logical chunk (row, c) of the tile whose first
     // row is r0 (M/N index) and first K element is k0.  ld = leading dimension in elements.
@@ -143,7 +158,9 @@ struct OperandTile {
 #pragma unroll
                     for (int e = 0; e < VEC; ++e) {
                         if (e >= n) break;
-                        if constexpr (ES == 2) {
+                        if constexpr (ES == 4) {
+                            v[e] = *(const int*)(src + 4 * e);
+                        } else if constexpr (ES == 2) {
                             const unsigned x = *(const unsigned short*)(src + 2 * e);
                             v[e >> 1] |= (int)(x << ((e & 1) * 16));
                         } else {
@@ -222,6 +239,17 @@ struct OperandTile {
             int row = row0 + (lane & 31);
             int c = ks * 2 + (lane >> 5);
             return *(const i32x4*)(lds + row * ROW_BYTES + swizzle(row, c) * 16);
+        } else if constexpr (ES == 4) {
+            // 32-bit elements, staged [k][row]: the lane's column (row0 + lane % 32) of the four k rows of its half
+            const int col_byte = (row0 + (lane & 31)) * 4;
+            const int c = col_byte >> 4, within = col_byte & 15;
+            i32x4 out;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int k = ks * 8 + (lane >> 5) * 4 + e;
+                out[e] = *(const int*)(lds + k * ROW_BYTES + swizzle(k, c) * 16 + within);
+            }
+            return out;
         } else if constexpr (ES == 2) {
             // ds_read_b64_tr_b16: in each group of 16 lanes, lanes 4j..4j+3 point at k-row j
             // (4 x 8 bytes = 16 columns); lane i receives column i of those 4 rows.

@@ -17,6 +17,15 @@ namespace acc950 {
 #define VPA(AKC, BM, BN, WM, WN, BKC, KB, STAGES)                                                       \
     { BM, BN, WM, WN, AKC, BKC, true, false, KB, STAGES, true, false, false, false, false,             \
       &launch_mfma<MfmaConfig<ACC950_IN, BM, BN, WM, WN, AKC, BKC, true, false, KB, STAGES, true>>, nullptr }
+// (the fp32 unit has the 32x32 instruction shape only: its table keeps the places of the other kernels, so that a variant
+// number means the same kernel geometry for every input type, with no launcher behind them)
+#ifdef ACC950_NO_MI16
+#define V16(AKC, BM, BN, WM, WN, BKC, KB, STAGES) { BM, BN, WM, WN, AKC, BKC, true, false, KB, STAGES, true, true, false, false, false, nullptr, nullptr }
+#define V16W4(BKC) { 256, 256, 2, 2, true, BKC, true, false, 64, 4, false, true, true, false, false, nullptr, nullptr }
+#define V16W4_192 { 256, 192, 2, 2, true, true, true, false, 64, 4, false, true, true, false, false, nullptr, nullptr }
+#define V16W4P(BKC) { 256, 256, 2, 2, true, BKC, true, false, 64, 4, false, true, true, true, false, nullptr, nullptr }
+#define V16W4A(BKC) { 256, 256, 2, 2, false, BKC, true, false, 64, 4, false, true, true, false, false, nullptr, nullptr }
+#else
 // ping-pong on the 16x16 MFMA shapes
 #define V16(AKC, BM, BN, WM, WN, BKC, KB, STAGES)                                                       \
     { BM, BN, WM, WN, AKC, BKC, true, false, KB, STAGES, true, true, false, false, false,              \
@@ -33,6 +42,7 @@ namespace acc950 {
 // the same kernel for a column-major A (one tile per workgroup)
 #define V16W4A(BKC) \
     { 256, 256, 2, 2, false, BKC, true, false, 64, 4, false, true, true, false, false, &launch_mfma16w4<Mfma16W4Config<ACC950_IN, BKC, false, 256, false, false>>, nullptr }
+#endif
 // any sizes, leading dimensions and alignments (the odd shapes of the reference's sweep lists, e.g.
 // /root/reference/tools/benchmarkers/gemm_resnet_inception.csv): register-staged 128x128 tiles whose fill takes unaligned chunks
 #define VANY(AKC, BKC)                                                                                  \
@@ -113,6 +123,7 @@ static const MfmaVariant kVariants[] = {
 // Timed build of the kernel the automatic choice takes for large aligned problems with row-major B:
 // the four-wave kernel when K has at least four K tiles, else the 256x256 ping-pong kernel on the
 // 16x16 MFMA shapes.  Same code plus four clock stamps per workgroup.
+#ifdef ACC950_TIMED_FN
 hipError_t ACC950_TIMED_FN(const GemmArgs& a, hipStream_t stream, LaunchGeom* geom, bool dry_run)
 {
     constexpr int K4 = 4 * 64 / InTraits<ACC950_IN>::ES;
@@ -121,6 +132,7 @@ hipError_t ACC950_TIMED_FN(const GemmArgs& a, hipStream_t stream, LaunchGeom* ge
     if (a.K >= K4) return launch_mfma16w4<Mfma16W4Config<ACC950_IN, false, true>>(a, stream, geom, dry_run);
     return launch_mfma16<Mfma16Config<ACC950_IN, 256, 256, 2, 4, true, false, 64, 4, false, true>>(a, stream, geom, dry_run);
 }
+#endif
 
 const MfmaVariant* ACC950_TABLE_FN(int* count)
 {

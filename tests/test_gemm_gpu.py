@@ -1046,3 +1046,49 @@ def test_full_tile_kernels_on_sizes_that_are_not_tile_multiples(in_type, out_typ
                 run_case(in_type, out_type, bm - vec, N, 5 * kb, a_layout=a_layout, b_layout=b_layout, variant=v, seed=1)
             seen += 1
     assert seen >= 20
+
+
+@pytest.mark.parametrize("b_layout", ["row", "col"])
+def test_fp32_on_the_tiled_mfma_kernels(b_layout):
+    """fp32 inputs on the LDS-tiled kernels (v_mfma_f32_32x32x2_f32; four instructions per 32-byte k-step): every variant
+    that has a launcher for fp32 -- the 32x32-shape ones; the 16x16-shape places of the table refuse -- at K tile counts
+    below, at and above the pipeline depth, column-major A, edges, odd sizes, C read, and a K split."""
+    from accera_amd import _lib
+    seen = 0
+    for v, name in _variants(b_layout):
+        kb = int(re.search(r"kb(\d+)", name).group(1)) // 4
+        a_layout = "col" if "A=col-major" in name else "row"
+        bm, bn = map(int, re.search(r"mfma (\d+)x(\d+)", name).groups())
+        M, N = max(512, 2 * bm), (max(512, 2 * bn) if 512 % bn == 0 else 3 * bn)
+        if "mi16" in name:
+            with pytest.raises(_lib.Acc950Error):
+                run_case("f32", "f32", M, N, 4 * kb, a_layout=a_layout, b_layout=b_layout, variant=v, seed=v)
+            continue
+        print("variant", v, name, flush=True)
+        for k_tiles in (1, 2, 3, 7):
+            run_case("f32", "f32", M, N, k_tiles * kb, a_layout=a_layout, b_layout=b_layout, variant=v, seed=1800 + v + k_tiles)
+        run_case("f32", "f32", M, N, 5 * kb, a_layout=a_layout, b_layout=b_layout, variant=v, seed=1900 + v, prologue=ora.PRO_NONE,
+                 epilogue=ora.EPI_RELU_NOCOND)
+        if "edge" in name:
+            odd = "any-alignment" in name
+            run_case("f32", "f32", 204 if a_layout == "col" and not odd else 203 if odd else 200, 145 if odd else 144, 171 if odd else 172,
+                     a_layout=a_layout, b_layout=b_layout, variant=v, seed=2000 + v)
+        if "fill=direct" in name and "pingpong" not in name:
+            run_case("f32", "f32", M, N, 12 * kb, a_layout=a_layout, b_layout=b_layout, variant=v, splits=3, seed=2100 + v)
+        seen += 1
+    assert seen >= 12
+
+
+def test_fp32_automatic_choice():
+    """Small fp32 problems stay with the kernel of 32 x 32 blocks; large ones take the tiled kernels, split over K where the
+    tiles alone would leave the chip idle."""
+    from accera_amd import _lib
+    g, b, lds, v = _lib.launch_geometry(_lib.F32, _lib.F32, 512, 512, 512, (512, 1), (512, 1), (512, 1))
+    assert v == _lib.VARIANT_F32_MFMA
+    g, b, lds, v = _lib.launch_geometry(_lib.F32, _lib.F32, 1024, 1024, 1024, (1024, 1), (1024, 1), (1024, 1))
+    assert "mfma 128x128" in _lib.variant_name(v) and g[2] > 1, (g, _lib.variant_name(v))
+    g, b, lds, v = _lib.launch_geometry(_lib.F32, _lib.F32, 4096, 4096, 4096, (4096, 1), (4096, 1), (4096, 1))
+    assert "mfma" in _lib.variant_name(v) and "thread-bound" not in _lib.variant_name(v) and g[2] == 1
+    run_case("f32", "f32", 1024, 1024, 1024, seed=2200)
+    run_case("f32", "f32", 2048, 1536, 1000, seed=2201, b_layout="col", prologue=ora.PRO_NONE)
+    run_case("f32", "f32", 363, 64, 3025, seed=2202, a_layout="col")

@@ -29,7 +29,7 @@ def test_shape_list_fixture():
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("in_type,out_type", [("f16", "f16"), ("bf16", "f32"), ("i8", "i32")])
+@pytest.mark.parametrize("in_type,out_type", [("f16", "f16"), ("bf16", "f32"), ("i8", "i32"), ("f32", "f32")])
 def test_every_shape_of_the_reference_sweep_lists(in_type, out_type):
     import accera_amd as acc
     import torch
@@ -54,7 +54,7 @@ def test_every_shape_of_the_reference_sweep_lists(in_type, out_type):
         grid, block, lds, v = _lib.launch_geometry(ora.TYPE_IDS[in_type], ora.TYPE_IDS[out_type], M, N, K, sa, sb, (N, 1))
         name = _lib.variant_name(v)
         assert v != _lib.VARIANT_GENERIC, (M, N, K, ta, tb, name)
-        kind = "skinny" if "skinny" in name else ("any-alignment" if "any-alignment" in name else "mfma") + (", K split" if grid[2] > 1 else "")
+        kind = "fp32 32x32 blocks" if v == _lib.VARIANT_F32_MFMA else "skinny" if "skinny" in name else ("any-alignment" if "any-alignment" in name else "mfma") + (", K split" if grid[2] > 1 else "")
         kinds[kind] = kinds.get(kind, 0) + 1
         print(n, (M, N, K, ta, tb, beta), name, "slices", grid[2], flush=True)
         acc.gemm_relu(A, B, C, prologue=prologue, epilogue=ora.EPI_RELU)
@@ -65,5 +65,6 @@ def test_every_shape_of_the_reference_sweep_lists(in_type, out_type):
         want = ora.gemm_relu_exact(host(A[sel], in_type), host(B, in_type), host(C0[sel], out_type), in_type, out_type, prologue, ora.EPI_RELU)
         assert_matches(host(C[sel], out_type), want, out_type, K)
     print(kinds)
-    assert kinds.get("any-alignment", 0) + kinds.get("any-alignment, K split", 0) >= 90
+    if in_type != "f32":  # (small fp32 problems stay with the kernel of 32 x 32 blocks, which takes any size)
+        assert kinds.get("any-alignment", 0) + kinds.get("any-alignment, K split", 0) >= 90
     assert sum(c for k, c in kinds.items() if "K split" in k) >= 10
