@@ -744,7 +744,8 @@ int acc950_mfma_phase_probe(int in_type, int out_type, int M, int N, int K, cons
     Problem pb;
     int rc = make_problem(in_type, out_type, M, N, K, A, K, 1, B, N, 1, C, N, 1, PRO_SET0, EPI_RELU, true, &pb);
     if (rc) return rc;
-    const MfmaVariant probe = {256, 256, 2, 4, true, false, true, false, 64, 4, true, false, false, false, false, nullptr, nullptr};
+    // (the shape conditions of the timed kernel, which is no row of the variant table: any launcher stands for "exists")
+    const MfmaVariant probe = {256, 256, 2, 4, true, false, true, false, 64, 4, true, false, false, false, false, launch_mfma_timed_f16, nullptr};
     int n_unused = 0;
     if (M < 256 || N < 256 || K < 1 || !mfma_table(pb.g.in_type, &n_unused) || !mfma_can_take(probe, pb))
         return fail(ACC950_UNSUPPORTED, "the phase probe runs the 256x256 kernels: 8/16-bit inputs, dense row-major A, B, C, M and N multiples of 256, K of 64 bytes");

@@ -99,6 +99,18 @@ __device__ __forceinline__ T apply_prologue(T sum, int pro, float arg, LoadC&& l
     return wrap_add(sum, load_c());
 }
 
+// Cache policy of the stores to C in the LDS-tiled MFMA kernels of the 32x32 shapes and the eight-wave 16x16 ones:
+// `sc1 nt` (bit 4 and bit 1 of a buffer instruction's aux operand).  A store whose line is already in the L2 -- a C
+// that the same launch has read for its prologue -- otherwise leaves a dirty line there, and all of them are written
+// back only when the kernel ends, after the last wave, at about 1 us per MB: 2048^3 fp16 with beta = 1 took 27.1 us
+// against 20.8 with beta = 0 on every kernel of the library, the thread-bound one included.  With `sc1` the store goes
+// through to memory while the kernel still runs (22.1 us); `nt` keeps the line from taking room that the operand
+// panels use (worth 0.5 - 1 us by itself on problems of 20 us that only write C).  Not for everything: the small fp32
+// kernel, whose stores are the last thing a 9 us launch does, loses 2.6 us waiting for them to reach memory, and the
+// four-wave kernels (a C far larger than the L2, lines gone before the kernel ends) keep `nt` alone: with `sc1` they
+// measured 1 % slower when C is only written and 0 - 1 % faster when it is read.
+constexpr int C_STORE_AUX = 16 | 2;
+
 // Store one float accumulator as the output element type.
 __device__ __forceinline__ void store_out(void* C, int out_type, int64_t idx, float v)
 {

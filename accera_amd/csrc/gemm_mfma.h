@@ -401,9 +401,9 @@ __device__ __forceinline__ T c_load(CTile t, unsigned voff, unsigned soff)
 template <typename T>
 __device__ __forceinline__ void c_store(CTile t, unsigned voff, unsigned soff, T v)
 {
-    if constexpr (sizeof(T) == 4) __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v), t.rsrc, voff, soff, 0);
-    else if constexpr (sizeof(T) == 2) __builtin_amdgcn_raw_buffer_store_b16(__builtin_bit_cast(unsigned short, v), t.rsrc, voff, soff, 0);
-    else __builtin_amdgcn_raw_buffer_store_b8(__builtin_bit_cast(unsigned char, v), t.rsrc, voff, soff, 0);
+    if constexpr (sizeof(T) == 4) __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v), t.rsrc, voff, soff, C_STORE_AUX);
+    else if constexpr (sizeof(T) == 2) __builtin_amdgcn_raw_buffer_store_b16(__builtin_bit_cast(unsigned short, v), t.rsrc, voff, soff, C_STORE_AUX);
+    else __builtin_amdgcn_raw_buffer_store_b8(__builtin_bit_cast(unsigned char, v), t.rsrc, voff, soff, C_STORE_AUX);
 }
 
 template <typename Cfg>
@@ -835,7 +835,7 @@ __global__ void __launch_bounds__(Cfg::NT, Cfg::WGS_PER_CU) gemm_mfma_kernel(Gem
             const int row = id / CPRW, cc = id % CPRW;
             const i32x4 v = *(const i32x4*)(slab + row * PITCH_B + cc * 16);
             __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), tile.rsrc, (unsigned)row * row_bytes + cc * 16,
-                                                   (unsigned)(i * 32) * row_bytes, 0);
+                                                   (unsigned)(i * 32) * row_bytes, C_STORE_AUX);
         }
     };
     // fp16 / bf16: two columns packed per dword after a swap with the neighbouring lane

@@ -245,7 +245,7 @@ __global__ void __launch_bounds__(Cfg::NT, 1) gemm_mfma16_kernel(GemmArgs p)
 #pragma unroll
             for (int j = 0; j < TN; ++j)
                 __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, fin4(acc[i][j])), tile.rsrc, lane_off + j * 64,
-                                                       (unsigned)(i * 16) * row_bytes, 0);
+                                                       (unsigned)(i * 16) * row_bytes, C_STORE_AUX);
     } else if ((p.c_rs * os) % 16 == 0 && ((size_t)p.C & 15) == 0) {
         // narrow outputs: 16 rows of the wave tile are put together in a wave-private slab of the
         // (now idle) tile buffers and leave as 16-byte pieces that cover whole rows
@@ -275,7 +275,7 @@ __global__ void __launch_bounds__(Cfg::NT, 1) gemm_mfma16_kernel(GemmArgs p)
                     const int row = id / CPRW, cc = id % CPRW;
                     const i32x4 v = *(const i32x4*)(slab + row * PITCH + cc * 16);
                     __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), tile.rsrc, (unsigned)row * row_bytes + cc * 16,
-                                                           (unsigned)(i * 16) * row_bytes, 0);
+                                                           (unsigned)(i * 16) * row_bytes, C_STORE_AUX);
                 }
             }
         };
@@ -302,7 +302,7 @@ __global__ void __launch_bounds__(Cfg::NT, 1) gemm_mfma16_kernel(GemmArgs p)
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
                         static_assert(OS == 2, "16-bit elements");
-                        __builtin_amdgcn_raw_buffer_store_b16((unsigned short)((unsigned)w[e >> 1] >> ((e & 1) * 16)), tile.rsrc, lane_off + e * 2, so, 0);
+                        __builtin_amdgcn_raw_buffer_store_b16((unsigned short)((unsigned)w[e >> 1] >> ((e & 1) * 16)), tile.rsrc, lane_off + e * 2, so, C_STORE_AUX);
                     }
                 }
         };

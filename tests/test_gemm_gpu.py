@@ -1092,3 +1092,36 @@ def test_fp32_automatic_choice():
     run_case("f32", "f32", 1024, 1024, 1024, seed=2200)
     run_case("f32", "f32", 2048, 1536, 1000, seed=2201, b_layout="col", prologue=ora.PRO_NONE)
     run_case("f32", "f32", 363, 64, 3025, seed=2202, a_layout="col")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("in_type,out_type", [("f16", "f32"), ("bf16", "bf16"), ("i8", "i32")])
+def test_measurement_aids_of_the_benchmark(in_type, out_type):
+    """The in-kernel phase times and the MFMA ceilings that bench.py reports beside every figure: the calls succeed on a
+    small problem and what they return is plausible (positive times that add up to less than the kernel's span, a clock
+    between 0.5 and 3 GHz, a pipe occupancy between 0 and 1, a rate below the nominal peak)."""
+    import torch
+    from accera_amd import _lib
+    _lib.check(_lib.lib().acc950_init(0))
+    tin = {"f16": torch.float16, "bf16": torch.bfloat16, "i8": torch.int8}[in_type]
+    tout = {"f32": torch.float32, "bf16": torch.bfloat16, "i32": torch.int32}[out_type]
+    M, N, K = 512, 768, 1024
+    if in_type == "i8":
+        A = torch.randint(-128, 128, (M, K), device="cuda", dtype=tin)
+        B = torch.randint(-128, 128, (K, N), device="cuda", dtype=tin)
+    else:
+        A = torch.randn((M, K), device="cuda").to(tin)
+        B = torch.randn((K, N), device="cuda").to(tin)
+    C = torch.zeros((M, N), device="cuda", dtype=tout)
+    lid = {"f16": _lib.F16, "bf16": _lib.BF16, "i8": _lib.I8, "f32": _lib.F32, "i32": _lib.I32}
+    r = _lib.mfma_phase_probe(lid[in_type], lid[out_type], M, N, K, A.data_ptr(), B.data_ptr(), C.data_ptr())
+    torch.cuda.synchronize()
+    assert r["prologue_us"] > 0 and r["main_loop_us"] > 0 and r["write_back_us"] > 0
+    assert r["prologue_us"] + r["main_loop_us"] + r["write_back_us"] <= r["kernel_span_us"] * 1.001
+    assert 0.5 < r["clock_ghz_main_loop"] < 3.0 and 0.0 < r["mfma_pipe_busy_main_loop"] <= 1.0
+    peak = 5000.0 if in_type == "i8" else 2500.0
+    rate, clock = _lib.mfma_ceiling(lid[in_type], 2, 2000)
+    assert 0.2 * peak < rate < peak * 1.02 and 0.5 < clock < 3.0
+    for traffic in range(4):
+        rate, clock = _lib.mfma_traffic_probe(lid[in_type], traffic, 300)
+        assert 0.1 * peak < rate < peak * 1.02 and 0.5 < clock < 3.0
