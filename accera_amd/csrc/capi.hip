@@ -303,21 +303,30 @@ int auto_mfma_variant(const Problem& pb)
         const MfmaVariant& v = tab[i];
         if (!mfma_can_take(v, pb)) continue;
         const int64_t tiles = (((int64_t)pb.g.M + v.bm - 1) / v.bm) * (((int64_t)pb.g.N + v.bn - 1) / v.bn);
-        const int wgs_per_cu = (tiles > 256 && v.waves_m * v.waves_n <= 4 &&
+        // what one compute unit has to get through: its share of the tiles, one after the other as far as the matrix cores
+        // are concerned; two workgroups side by side (when the tile leaves room for two) only hide each other's waits
+        const int64_t per_cu = (tiles + kComputeUnits - 1) / kComputeUnits;
+        const int wgs_per_cu = (per_cu >= 2 && v.waves_m * v.waves_n <= 4 &&
                                 2 * v.stages * (v.bm + v.bn) * v.kb <= 160 * 1024 && v.bm * v.bn <= 256 * 128) ? 2 : 1;
-        const int64_t rounds = (tiles + 256 * wgs_per_cu - 1) / (256 * wgs_per_cu);
-        double cost = (double)rounds * wgs_per_cu * v.bm * v.bn;
+        double cost = (double)per_cu * v.bm * v.bn;
         if (v.edge) cost *= v.any ? 2.0 : 1.5;   // register-staged fill, bounds checks (unaligned chunks cost more requests)
         if (!v.direct) cost *= 1.2;
         // measured on sweeps: 4-wave tiles reach about 85 % of the ping-pong kernel's rate when two
         // workgroups share a CU and about 70 % when a workgroup has the CU to itself
         if (v.waves_m * v.waves_n <= 4 && !v.w4) cost /= wgs_per_cu == 2 ? 0.85 : 0.7;
+        // smaller tiles fetch more bytes and read more fragments per MFMA
+        // (measured, 64x64 against 128x128 tiles: fp32, bound by its slow MFMAs, 1024^3 20.7 against 63.7 us and 3072x1024x1024
+        // 53 against 66; 8- and 16-bit inputs win while a CU has at most two of them -- fp16 1024^3 6.6 against 9.5 us,
+        // 1536x1152x2048 14.4 against 17.0 -- and lose beyond: 3072x1024x1024 13.1 against 9.8, 2048^3 30.3 against 21.2)
+        if (v.bm * v.bn <= 64 * 64) cost /= pb.g.in_type == T_F32 ? 0.9 : per_cu <= 2 ? 0.75 : 0.5;
+        else if (v.bm * v.bn <= 128 * 64) cost /= 0.8;
         // rank inside one tile shape: ping-pong kb64 x4 > ping-pong others > 8-wave > 4-wave (kb64 x4 first)
         int rank = v.pingpong ? (v.kb == 64 && v.stages == 4 ? 8 : 6) : (v.waves_m * v.waves_n == 8 ? 4 : 2);
         if (!v.pingpong && v.kb == 64 && v.stages == 4) rank += 1;
         // one tile per CU at most: the deepest prefetch wins (four stages of 128 bytes of K; 2048^3: 21.8 against 25-26 us), where
-        // more tiles than CUs want two workgroups per CU, which only the smaller stages leave room for
-        if (!v.pingpong && v.direct && v.kb == 128 && v.stages == 4 && tiles <= kComputeUnits) rank += 2;
+        // more tiles than CUs want two workgroups per CU, which only the smaller stages leave room for; below 32 tiles of K the
+        // four stages of 64 bytes are ahead (2048x2048x512 fp16: 7.5 against 8.2 us)
+        if (!v.pingpong && v.direct && v.kb == 128 && v.stages == 4 && tiles <= kComputeUnits && (int64_t)pb.g.K * elem_size(pb.g.in_type) >= 4096) rank += 2;
         // 16x16 shapes: measured 4-9 % faster than the 32x32 shapes on every large problem, in the lean build
         // (C = A*B, C = relu(A*B)); their full build reads C element by element and lost 20 % to the 32x32 form
         const bool lean = pb.g.prologue == PRO_SET && pb.g.prologue_arg == 0.f && (pb.g.epilogue == EPI_RELU || pb.g.epilogue == EPI_NONE);

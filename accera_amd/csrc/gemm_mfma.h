@@ -398,12 +398,15 @@ __device__ __forceinline__ T c_load(CTile t, unsigned voff, unsigned soff)
     else if constexpr (sizeof(T) == 2) return __builtin_bit_cast(T, __builtin_amdgcn_raw_buffer_load_b16(t.rsrc, voff, soff, 0));
     else return __builtin_bit_cast(T, __builtin_amdgcn_raw_buffer_load_b8(t.rsrc, voff, soff, 0));
 }
-template <typename T>
+// (AUX: the cache policy.  Only stores that write whole 128-byte lines go through the L2 -- see C_STORE_AUX; pieces of
+// lines, as the edge kernels and the element-wise narrow stores write them, would each become a read-modify-write in
+// memory: 600x64x196 fp16 with beta = 1 on the any-alignment kernel took 20 us that way instead of 10.)
+template <typename T, int AUX = 0>
 __device__ __forceinline__ void c_store(CTile t, unsigned voff, unsigned soff, T v)
 {
-    if constexpr (sizeof(T) == 4) __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v), t.rsrc, voff, soff, C_STORE_AUX);
-    else if constexpr (sizeof(T) == 2) __builtin_amdgcn_raw_buffer_store_b16(__builtin_bit_cast(unsigned short, v), t.rsrc, voff, soff, C_STORE_AUX);
-    else __builtin_amdgcn_raw_buffer_store_b8(__builtin_bit_cast(unsigned char, v), t.rsrc, voff, soff, C_STORE_AUX);
+    if constexpr (sizeof(T) == 4) __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v), t.rsrc, voff, soff, AUX);
+    else if constexpr (sizeof(T) == 2) __builtin_amdgcn_raw_buffer_store_b16(__builtin_bit_cast(unsigned short, v), t.rsrc, voff, soff, AUX);
+    else __builtin_amdgcn_raw_buffer_store_b8(__builtin_bit_cast(unsigned char, v), t.rsrc, voff, soff, AUX);
 }
 
 template <typename Cfg>
@@ -504,7 +507,7 @@ __global__ void __launch_bounds__(Cfg::NT, Cfg::WGS_PER_CU) gemm_mfma_kernel(Gem
     // sched_barrier after every slot pins this order against the machine scheduler.
     constexpr int SLOTS = TM * TN;
     constexpr int FILLS_PER_SLOT = (FILLS + SLOTS - 1) / SLOTS; // all fills within the first k-step
-    static_assert(TM + TN <= SLOTS, "not enough MFMA slots to prefetch the next fragments");
+    constexpr int READS_PER_SLOT = (TM + TN + SLOTS - 1) / SLOTS; // (more than one only for wave tiles of one or two blocks)
     static_assert(KSTEPS % 2 == 0, "fragment buffers alternate per k-step and must line up across tiles");
     i32x4 af[2][TM], bf[2][TN];
     auto load_first_frags = [&](const char* sa, const char* sb) {
@@ -531,8 +534,12 @@ __global__ void __launch_bounds__(Cfg::NT, Cfg::WGS_PER_CU) gemm_mfma_kernel(Gem
                     mfma32<IN>(af[ks & 1][i], bf[ks & 1][j], acc[i][j]);
                     if (!last || cross) {
                         // B fragments first: the first MFMAs of the next step need bf[0] and af[0]
-                        if (slot < TN) bf[(ks + 1) & 1][slot] = TB::read_frag(rb, wc0 + slot * 32, rks, lane);
-                        else if (slot - TN < TM) af[(ks + 1) & 1][slot - TN] = TA::read_frag(ra, wr0 + (slot - TN) * 32, rks, lane);
+#pragma unroll
+                        for (int u = 0; u < READS_PER_SLOT; ++u) {
+                            const int q = slot * READS_PER_SLOT + u;
+                            if (q < TN) bf[(ks + 1) & 1][q] = TB::read_frag(rb, wc0 + q * 32, rks, lane);
+                            else if (q - TN < TM) af[(ks + 1) & 1][q - TN] = TA::read_frag(ra, wr0 + (q - TN) * 32, rks, lane);
+                        }
                     }
                     if constexpr (DIRECT && fill) {
                         if (ks == 0) {
@@ -897,7 +904,7 @@ __global__ void __launch_bounds__(Cfg::NT, Cfg::WGS_PER_CU) gemm_mfma_kernel(Gem
         const unsigned os = p.out_type == T_I8 ? 1 : (p.out_type == T_F32 || p.out_type == T_I32) ? 4 : 2;
         const bool staged = CAN_STAGE && (p.c_rs * os) % 16 == 0 && ((size_t)p.C & 15) == 0;
         if constexpr (IN == IN_I8) {
-            if (p.out_type == T_I32) for_each_element(int{}, [&](CTile t, unsigned vo, unsigned so, int v) { c_store<int>(t, vo, so, fin(v)); return v; });
+            if (p.out_type == T_I32) for_each_element(int{}, [&](CTile t, unsigned vo, unsigned so, int v) { c_store<int, EDGE ? 0 : C_STORE_AUX>(t, vo, so, fin(v)); return v; });
             else if (CAN_STAGE && staged) {
                 if constexpr (CAN_STAGE) {
                     __syncthreads(); // every wave is done reading the tile buffers
@@ -906,7 +913,7 @@ __global__ void __launch_bounds__(Cfg::NT, Cfg::WGS_PER_CU) gemm_mfma_kernel(Gem
                 }
             } else if (p.out_type == T_I16) for_each_element(int16_t{}, [&](CTile t, unsigned vo, unsigned so, int v) { c_store<int16_t>(t, vo, so, (int16_t)fin(v)); return v; });
             else for_each_element(int8_t{}, [&](CTile t, unsigned vo, unsigned so, int v) { c_store<int8_t>(t, vo, so, (int8_t)fin(v)); return v; });
-        } else if (p.out_type == T_F32) for_each_element(float{}, [&](CTile t, unsigned vo, unsigned so, float v) { c_store<float>(t, vo, so, fin(v)); return v; });
+        } else if (p.out_type == T_F32) for_each_element(float{}, [&](CTile t, unsigned vo, unsigned so, float v) { c_store<float, EDGE ? 0 : C_STORE_AUX>(t, vo, so, fin(v)); return v; });
         else if (CAN_STAGE && staged) {
             if constexpr (CAN_STAGE) {
                 __syncthreads(); // every wave is done reading the tile buffers

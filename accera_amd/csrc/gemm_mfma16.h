@@ -302,7 +302,7 @@ __global__ void __launch_bounds__(Cfg::NT, 1) gemm_mfma16_kernel(GemmArgs p)
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
                         static_assert(OS == 2, "16-bit elements");
-                        __builtin_amdgcn_raw_buffer_store_b16((unsigned short)((unsigned)w[e >> 1] >> ((e & 1) * 16)), tile.rsrc, lane_off + e * 2, so, C_STORE_AUX);
+                        __builtin_amdgcn_raw_buffer_store_b16((unsigned short)((unsigned)w[e >> 1] >> ((e & 1) * 16)), tile.rsrc, lane_off + e * 2, so, 0);
                     }
                 }
         };

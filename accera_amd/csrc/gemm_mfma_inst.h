@@ -106,6 +106,16 @@ static const MfmaVariant kVariants[] = {
     V(128, 128, 2, 2, true, true, false, 128, 4),
     VA(false, 128, 128, 2, 2, false, true, false, 128, 4),
     VA(false, 128, 128, 2, 2, true, true, false, 128, 4),
+    // small tiles for problems whose 128x128 tiles would leave most of the chip idle and whose K is too short to split:
+    // 64x64 (a wave has one 32x32 block) and 128x64, deep prefetch, two or more workgroups per CU
+    V(64, 64, 2, 2, false, true, false, 128, 4),
+    V(64, 64, 2, 2, true, true, false, 128, 4),
+    VA(false, 64, 64, 2, 2, false, true, false, 128, 4),
+    VA(false, 64, 64, 2, 2, true, true, false, 128, 4),
+    V(128, 64, 2, 2, false, true, false, 128, 3),
+    V(128, 64, 2, 2, true, true, false, 128, 3),
+    VA(false, 128, 64, 2, 2, false, true, false, 128, 3),
+    VA(false, 128, 64, 2, 2, true, true, false, 128, 3),
 };
 #undef LAYOUT_AT
 #undef VA

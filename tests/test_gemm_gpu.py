@@ -1080,13 +1080,15 @@ def test_fp32_on_the_tiled_mfma_kernels(b_layout):
 
 
 def test_fp32_automatic_choice():
-    """Small fp32 problems stay with the kernel of 32 x 32 blocks; large ones take the tiled kernels, split over K where the
-    tiles alone would leave the chip idle."""
+    """Small fp32 problems stay with the kernel of 32 x 32 blocks; large ones take the tiled kernels -- 64 x 64 tiles while
+    larger ones would leave compute units idle -- split over K where the tiles alone would not fill the chip."""
     from accera_amd import _lib
     g, b, lds, v = _lib.launch_geometry(_lib.F32, _lib.F32, 512, 512, 512, (512, 1), (512, 1), (512, 1))
     assert v == _lib.VARIANT_F32_MFMA
     g, b, lds, v = _lib.launch_geometry(_lib.F32, _lib.F32, 1024, 1024, 1024, (1024, 1), (1024, 1), (1024, 1))
-    assert "mfma 128x128" in _lib.variant_name(v) and g[2] > 1, (g, _lib.variant_name(v))
+    assert "mfma 64x64" in _lib.variant_name(v) and g[2] == 1, (g, _lib.variant_name(v))   # one small tile per compute unit
+    g, b, lds, v = _lib.launch_geometry(_lib.F32, _lib.F32, 256, 256, 4096, (4096, 1), (256, 1), (256, 1))
+    assert "mfma 64x64" in _lib.variant_name(v) and g[2] > 1, (g, _lib.variant_name(v))    # 16 tiles: split over K
     g, b, lds, v = _lib.launch_geometry(_lib.F32, _lib.F32, 4096, 4096, 4096, (4096, 1), (4096, 1), (4096, 1))
     assert "mfma" in _lib.variant_name(v) and "thread-bound" not in _lib.variant_name(v) and g[2] == 1
     run_case("f32", "f32", 1024, 1024, 1024, seed=2200)
@@ -1125,3 +1127,19 @@ def test_measurement_aids_of_the_benchmark(in_type, out_type):
     for traffic in range(4):
         rate, clock = _lib.mfma_traffic_probe(lid[in_type], traffic, 300)
         assert 0.1 * peak < rate < peak * 1.02 and 0.5 < clock < 3.0
+
+
+@pytest.mark.gpu
+def test_small_tiles_are_chosen_for_problems_that_would_not_fill_the_chip():
+    """64 x 64 tiles (a wave has one 32 x 32 block) while 128 x 128 tiles would leave most compute units idle; the larger
+    tiles again once a compute unit would get more than two of the small ones (8- and 16-bit inputs)."""
+    from accera_amd import _lib
+    for t, o in ((_lib.F16, _lib.F16), (_lib.BF16, _lib.F32), (_lib.I8, _lib.I32)):
+        for (M, N, K), want in (((1024, 1024, 1024), "mfma 64x64"), ((1536, 1152, 2048), "mfma 64x64"), ((512, 512, 512), "mfma 64x64"),
+                                ((2048, 2048, 2048), "mfma 128x128"), ((3072, 1024, 1024), "mfma 128x128")):
+            g, b, lds, v = _lib.launch_geometry(t, o, M, N, K, (K, 1), (N, 1), (N, 1))
+            assert want in _lib.variant_name(v), (M, N, K, _lib.variant_name(v))
+    run_case("f16", "f16", 1024, 1024, 1024, seed=2300)
+    run_case("bf16", "f32", 1536, 1152, 2048, seed=2301, b_layout="col", prologue=ora.PRO_NONE)
+    run_case("i8", "i32", 1024, 960, 1024, seed=2302, a_layout="col")
+    run_case("i8", "i8", 1000, 1024, 512, seed=2303)

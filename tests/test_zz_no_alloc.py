@@ -58,11 +58,11 @@ def test_static_workspace_entry_point_matches_the_allocating_one():
     assert rc == _lib.UNSUPPORTED and b"built-in workspace" in L.acc950_last_error()
     torch.cuda.synchronize()
     assert (to_host(d_new, "f16") == 9).all()
-    # an MFMA kernel's K split that does not fit runs unsplit instead (1024 x 1024 x 4096: four slices would be 16 MiB)
-    M = N = 1024
-    K = 4096
+    # an MFMA kernel's K split that does not fit runs unsplit instead (512 x 1024 x 8192: two slices of 2 MiB are the whole
+    # array, part of which holds the counters)
+    M, N, K = 512, 1024, 8192
     A = make_input(rng, (M, K), "f16", "normal")
-    B = (make_input(rng, (K, N), "f16", "normal").astype(np.float32) * 0.05).astype(np.float16)
+    B = (make_input(rng, (K, N), "f16", "normal").astype(np.float32) * 0.03).astype(np.float16)
     dA, dB, dC = to_device(A, "f16"), to_device(B, "f16"), to_device(np.full((M, N), 9, np.float16), "f16")
     assert _lib.launch_geometry(_lib.F16, _lib.F16, M, N, K, (K, 1), (N, 1), (N, 1))[0][2] > 1
     _lib.check(_call(L.acc950_gemm_ops_static, dA, dB, dC, M, N, K, 0, stream))
