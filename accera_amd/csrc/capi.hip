@@ -434,7 +434,9 @@ int choose(const Problem& pb, int variant, int k_splits, Choice* c)
                 SplitPlan sp;
                 slices = k_splits > 1 ? (plan_split(v, pb, k_splits, &sp) ? sp.splits : 1) : k_splits == 0 ? auto_mfma_splits(v, pb) : 1;
                 const int64_t tiles = (((int64_t)pb.g.M + v.bm - 1) / v.bm) * (((int64_t)pb.g.N + v.bn - 1) / v.bn);
-                if (tiles * slices * 2 < kComputeUnits) mv = -1;
+                // (or more workgroups than there are 32 x 32 blocks: a small output with a long K, which only the tiled kernels split)
+                const int64_t blocks = (((int64_t)pb.g.M + 31) / 32) * (((int64_t)pb.g.N + 31) / 32);
+                if (tiles * slices * 2 < kComputeUnits && tiles * slices <= blocks) mv = -1;
             }
             if (mv < 0) { c->variant = ACC950_VARIANT_F32_MFMA; return ACC950_OK; }
         }

@@ -48,6 +48,9 @@ namespace acc950 {
 #define VANY(AKC, BKC)                                                                                  \
     { 128, 128, 2, 2, AKC, BKC, false, true, 128, 2, false, false, false, false, true,                 \
       &launch_mfma<MfmaConfig<ACC950_IN, 128, 128, 2, 2, AKC, BKC, false, true, 128, 2, false, false, true>>, nullptr }
+#define VANY64(AKC, BKC)                                                                                \
+    { 64, 64, 2, 2, AKC, BKC, false, true, 128, 2, false, false, false, false, true,                   \
+      &launch_mfma<MfmaConfig<ACC950_IN, 64, 64, 2, 2, AKC, BKC, false, true, 128, 2, false, false, true>>, nullptr }
 #define V(BM, BN, WM, WN, BKC, DIRECT, EDGE, KB, STAGES) VA(true, BM, BN, WM, WN, BKC, DIRECT, EDGE, KB, STAGES)
 #define VP(BM, BN, WM, WN, BKC, KB, STAGES) VPA(true, BM, BN, WM, WN, BKC, KB, STAGES)
 // column-major A (M contiguous; the "transA" shapes of the reference's sweep lists,
@@ -116,6 +119,11 @@ static const MfmaVariant kVariants[] = {
     V(128, 64, 2, 2, true, true, false, 128, 3),
     VA(false, 128, 64, 2, 2, false, true, false, 128, 3),
     VA(false, 128, 64, 2, 2, true, true, false, 128, 3),
+    // and the any-alignment form on 64x64 tiles (the odd shapes of the reference's lists are mostly small)
+    VANY64(true, false),
+    VANY64(true, true),
+    VANY64(false, false),
+    VANY64(false, true),
 };
 #undef LAYOUT_AT
 #undef VA
@@ -126,6 +134,7 @@ static const MfmaVariant kVariants[] = {
 #undef V16W4P
 #undef V16W4A
 #undef VANY
+#undef VANY64
 #undef LAYOUT
 #undef V
 #undef VP

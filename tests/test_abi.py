@@ -56,7 +56,7 @@ def test_launch_geometry_of_the_configs():
     # sizes that are not multiples of the 16-byte vector take the MFMA kernel whose fill accepts unaligned chunks; an operand with
     # no unit stride falls to the thread-bound kernel; explicit variants refuse what they do not take
     g, b, lds, v = _lib.launch_geometry(_lib.F16, _lib.F32, 100, 71, 40, (40, 1), (71, 1), (71, 1))
-    assert "any-alignment" in _lib.variant_name(v) and g == [1, 1, 1]
+    assert "any-alignment" in _lib.variant_name(v) and "mfma 64x64" in _lib.variant_name(v) and g == [4, 1, 1]
     g, b, lds, v = _lib.launch_geometry(_lib.F16, _lib.F32, 100, 71, 40, (80, 2), (71, 1), (71, 1))
     assert v == _lib.VARIANT_GENERIC and g[:2] == [2, 2]
     with pytest.raises(_lib.Acc950Error) as e:

@@ -912,8 +912,14 @@ def test_any_alignment_mfma_kernel(in_type, out_type, a_layout, b_layout):
     key = (" A=col-major" if a_layout == "col" else " waves 2x2 B="), (" B=col-major" if b_layout == "col" else " B=row-major")
     variants = [v for v in range(_lib.num_variants()) if "any-alignment" in _lib.variant_name(v) and all(k in _lib.variant_name(v) for k in key)
                 and ("A=col-major" in _lib.variant_name(v)) == (a_layout == "col")]
-    assert len(variants) == 1, [_lib.variant_name(v) for v in variants]
-    v = variants[0]
+    assert len(variants) == 2, [_lib.variant_name(v) for v in variants]   # 128 x 128 and 64 x 64 tiles
+    for v in variants:
+        _any_alignment_cases(v, in_type, out_type, a_layout, b_layout)
+
+
+def _any_alignment_cases(v, in_type, out_type, a_layout, b_layout):
+    import accera_amd as acc
+    import torch
     for n, (M, N, K) in enumerate([(363, 64, 3025), (192, 48, 1225), (27, 32, 2201), (196, 600, 64), (100, 72, 41), (129, 257, 131), (1, 1, 1), (5, 300, 7)]):
         print("variant", v, in_type, out_type, a_layout, b_layout, M, N, K, flush=True)
         run_case(in_type, out_type, M, N, K, a_layout=a_layout, b_layout=b_layout, variant=v, seed=1200 + n)
