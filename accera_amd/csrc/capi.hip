@@ -303,12 +303,17 @@ int auto_mfma_variant(const Problem& pb)
         const MfmaVariant& v = tab[i];
         if (!mfma_can_take(v, pb)) continue;
         const int64_t tiles = (((int64_t)pb.g.M + v.bm - 1) / v.bm) * (((int64_t)pb.g.N + v.bn - 1) / v.bn);
-        // what one compute unit has to get through: its share of the tiles, one after the other as far as the matrix cores
-        // are concerned; two workgroups side by side (when the tile leaves room for two) only hide each other's waits
+        // 8- and 16-bit inputs: rounds of workgroups over the compute units, two side by side where the tile leaves room and
+        // there are more tiles than units (a workgroup of the 4-wave kernels is bound by its own waits, so two run almost as
+        // fast as one; 4096x2304x768 fp16: 576 tiles of 128x128 take 23.9 us, 144 of 256x256 18.9).  fp32, bound by its slow
+        // MFMAs: what one unit has to get through, its share of the tiles one after the other (3072x1024x1024: 768 tiles of
+        // 64x64, three per unit, 53 us; 192 of 128x128 on 192 units 66 us).
+        const bool fp32 = pb.g.in_type == T_F32;
         const int64_t per_cu = (tiles + kComputeUnits - 1) / kComputeUnits;
-        const int wgs_per_cu = (per_cu >= 2 && v.waves_m * v.waves_n <= 4 &&
+        const int wgs_per_cu = ((fp32 ? per_cu >= 2 : tiles > kComputeUnits) && v.waves_m * v.waves_n <= 4 &&
                                 2 * v.stages * (v.bm + v.bn) * v.kb <= 160 * 1024 && v.bm * v.bn <= 256 * 128) ? 2 : 1;
-        double cost = (double)per_cu * v.bm * v.bn;
+        const int64_t rounds = (tiles + kComputeUnits * wgs_per_cu - 1) / (kComputeUnits * wgs_per_cu);
+        double cost = fp32 ? (double)per_cu * v.bm * v.bn : (double)rounds * wgs_per_cu * v.bm * v.bn;
         if (v.edge) cost *= v.any ? 2.0 : 1.5;   // register-staged fill, bounds checks (unaligned chunks cost more requests)
         if (!v.direct) cost *= 1.2;
         // measured on sweeps: 4-wave tiles reach about 85 % of the ping-pong kernel's rate when two
@@ -391,8 +396,8 @@ bool plan_split(const MfmaVariant& v, const Problem& pb, int want, SplitPlan* sp
 
 // Splits the library takes by itself: only when the tiles leave at least half of the compute units idle and K is long
 // enough for the second kernel (a few microseconds) to pay.  Measured on small outputs with a long K (512 x 512 x 8192,
-// 256 x 256 x 16384, 1024 x 1024 x 4096, 768 x 320 x 30522, 1024 x 80 x 30522; 16-bit inputs): the best split brings the
-// workgroups to about one per compute unit and leaves a slice 16 to 60 k-steps of 64 bytes.
+// 256 x 256 x 16384, 1024 x 1024 x 4096, 768 x 320 x 30522, 1024 x 80 x 30522; 16-bit inputs): the best split fills the
+// compute units once and leaves a slice 12 to 64 k-steps of 64 bytes.
 int auto_mfma_splits(const MfmaVariant& v, const Problem& pb)
 {
     const GemmArgs& g = pb.g;
@@ -400,8 +405,17 @@ int auto_mfma_splits(const MfmaVariant& v, const Problem& pb)
     const int64_t tiles = (((int64_t)g.M + v.bm - 1) / v.bm) * (((int64_t)g.N + v.bn - 1) / v.bn);
     if (tiles * 2 > kComputeUnits) return 1;
     const int64_t steps = (int64_t)g.K * elem_size(g.in_type) / 64; // k-steps of 64 bytes
-    if (steps < 64) return 1; // (1024^3, 32 k-steps: 9.8 us unsplit, 15.1 us in two slices -- the second kernel costs about 5 us)
-    int64_t want = kComputeUnits / tiles < steps / 16 ? kComputeUnits / tiles : steps / 16;
+    // (1024^3, 32 k-steps, on 64 tiles: 9.8 us unsplit, 15.1 us in two slices -- the second kernel costs about 5 us; with a
+    // handful of tiles a short K is still worth splitting: int8 363x64x3025, 6 tiles and 47 k-steps, 46.9 us unsplit, 15.7 in eight)
+    if (steps < 64 && tiles * 8 > kComputeUnits) return 1;
+    // a slice of about 64 k-steps, shorter ones (down to 12) only while the tiles are few; never more workgroups than the
+    // compute units hold at once (two of the 64 x 64 tiles each), never more than 32 slices.  Measured with 64 x 64 tiles, fp16,
+    // us by slices 4 / 8 / 16 / 32: 768x320x30522 82 / 52 / 50 / 57; 1024x80x30522 79 / 50 / 37 / 41; 288x64x21609 59 / 36 / 24 / 21;
+    // 363x64x3025 17 / 13 / 13 / 15; 512x512x8192 16 / 17 / 22 / 31; 256x256x16384 23 / 18 / 19 / 22.
+    const int64_t slots = kComputeUnits * (v.bm * v.bn <= 64 * 64 ? 2 : 1);
+    const int64_t few = steps / 12 < 192 / tiles ? steps / 12 : 192 / tiles;
+    int64_t want = steps / 64 > few ? steps / 64 : few;
+    if (want > slots / tiles) want = slots / tiles;
     if (want > 32) want = 32;
     if ((size_t)want * (size_t)g.M * (size_t)g.N > ((size_t)1 << 24)) return 1; // 64 MiB of partial sums at most without being asked
     SplitPlan sp;

@@ -165,12 +165,14 @@ def test_block_tile_of_a_gpu_plan_selects_the_kernel(tmp_path):
     package = acc.Package()
     n256 = package.add(plan_with((256, 256)), args=(A, B, C), base_name="tile256")
     n128 = package.add(plan_with((128, 128)), args=(A, B, C), base_name="tile128")
+    n64 = package.add(plan_with((64, 64)), args=(A, B, C), base_name="tile64")    # (the reference's MFMA tests tile 64 x 64: mfma_tests.py:89-97)
     n48 = package.add(plan_with((48, 80)), args=(A, B, C), base_name="tile_other")   # no such kernel: automatic choice
     files = package.build(name="tiles", format=acc.Package.Format.HAT_DYNAMIC, output_dir=str(tmp_path))
     fns = hat.parse(files[0])["functions"]
     rec = lambda n: fns[n]["auxiliary"]["accera_mi355x"]
     assert "mfma 256x256" in rec(n256)["kernel"] and rec(n256)["launch_parameters"][:3] == [16, 1, 1]
     assert "mfma 128x128" in rec(n128)["kernel"] and rec(n128)["launch_parameters"][:3] == [64, 1, 1]
+    assert "mfma 64x64" in rec(n64)["kernel"] and rec(n64)["launch_parameters"][:3] == [256, 1, 1]
     assert "mfma" in rec(n48)["kernel"]
 
 
