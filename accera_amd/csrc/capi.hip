@@ -302,7 +302,8 @@ int auto_mfma_variant(const Problem& pb)
     for (int i = 0; i < n; ++i) {
         const MfmaVariant& v = tab[i];
         if (!mfma_can_take(v, pb)) continue;
-        const int64_t tiles = (((int64_t)pb.g.M + v.bm - 1) / v.bm) * (((int64_t)pb.g.N + v.bn - 1) / v.bn);
+        // (a batch is one launch: its problems' tiles fill the chip together)
+        const int64_t tiles = (((int64_t)pb.g.M + v.bm - 1) / v.bm) * (((int64_t)pb.g.N + v.bn - 1) / v.bn) * (pb.g.batch > 1 ? pb.g.batch : 1);
         // 8- and 16-bit inputs: rounds of workgroups over the compute units, two side by side where the tile leaves room and
         // there are more tiles than units (a workgroup of the 4-wave kernels is bound by its own waits, so two run almost as
         // fast as one; 4096x2304x768 fp16: 576 tiles of 128x128 take 23.9 us, 144 of 256x256 18.9).  fp32, bound by its slow
@@ -339,7 +340,7 @@ int auto_mfma_variant(const Problem& pb)
         // four waves with 128x128 wave tiles: measured 3-9 % faster than the eight-wave form on large problems
         // (a third less LDS traffic, and the part is at its power limit there)
         // (walking several tiles per workgroup pays when there is more than one round of tiles over the CUs)
-        if (v.w4) rank = v.persist ? (tiles > kComputeUnits ? 14 : 12) : 13;
+        if (v.w4) rank = v.persist ? (tiles / (pb.g.batch > 1 ? pb.g.batch : 1) > kComputeUnits ? 14 : 12) : 13; // (tiles of one problem: a workgroup walks inside its own)
         const bool better = best < 0 || cost < best_cost * 0.999 ||
                             (cost <= best_cost * 1.001 && ((int64_t)v.bm * v.bn > (int64_t)tab[best].bm * tab[best].bn ||
                                                            ((int64_t)v.bm * v.bn == (int64_t)tab[best].bm * tab[best].bn && rank > best_rank)));
