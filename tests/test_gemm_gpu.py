@@ -977,10 +977,13 @@ def test_k_split_of_the_mfma_kernels(in_type, out_type):
     families = [("hand-laid", "row", "row", ("mfma 256x256", "hand-laid loop")), ("hand-laid, B col-major", "row", "col", ("mfma 256x256", "hand-laid loop")),
                 ("hand-laid, A col-major", "col", "row", ("A=col-major", "hand-laid loop")),
                 ("ping-pong 16x16", "row", "row", ("mfma 256x256 kb64", "pingpong mi16")), ("128x128 direct", "row", "row", ("mfma 128x128 kb64", "fill=direct")),
-                ("any alignment", "row", "row", ("any-alignment",))]
+                ("any alignment", "row", "row", ("mfma 128x128", "any-alignment")),
+                ("64x64 direct", "row", "row", ("mfma 64x64", "fill=direct")), ("64x64 direct, A and B col-major", "col", "col", ("mfma 64x64", "fill=direct")),
+                ("128x64 direct", "row", "col", ("mfma 128x64", "fill=direct")), ("64x64 any alignment", "col", "row", ("mfma 64x64", "any-alignment"))]
     for label, a_layout, b_layout, keys in families:
         v = next(v for v, n in _variants(b_layout) if all(k in n for k in keys) and ("A=col-major" in n) == (a_layout == "col")
                  and "multi-tile" not in n)
+        kb = int(re.search(r"kb(\d+)", _lib.variant_name(v)).group(1)) // (1 if in_type == "i8" else 2) if "64 " in label or "128x64" in label else kb
         for splits, k_tiles in ((2, 8), (3, 40), (5, 21), (8, 40)):
             print(label, "variant", v, in_type, out_type, "splits", splits, "k tiles", k_tiles, flush=True)
             g = _lib.launch_geometry(ora.TYPE_IDS[in_type], ora.TYPE_IDS[out_type], 256, 512, k_tiles * kb,
