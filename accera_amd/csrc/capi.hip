@@ -398,7 +398,7 @@ bool plan_split(const MfmaVariant& v, const Problem& pb, int want, SplitPlan* sp
 // Splits the library takes by itself: only when the tiles leave at least half of the compute units idle and K is long
 // enough for the second kernel (a few microseconds) to pay.  Measured on small outputs with a long K (512 x 512 x 8192,
 // 256 x 256 x 16384, 1024 x 1024 x 4096, 768 x 320 x 30522, 1024 x 80 x 30522; 16-bit inputs): the best split fills the
-// compute units once and leaves a slice 12 to 64 k-steps of 64 bytes.
+// compute units once or twice and leaves a slice 4 to 60 k-steps of 64 bytes.
 int auto_mfma_splits(const MfmaVariant& v, const Problem& pb)
 {
     const GemmArgs& g = pb.g;
@@ -406,16 +406,18 @@ int auto_mfma_splits(const MfmaVariant& v, const Problem& pb)
     const int64_t tiles = (((int64_t)g.M + v.bm - 1) / v.bm) * (((int64_t)g.N + v.bn - 1) / v.bn);
     if (tiles * 2 > kComputeUnits) return 1;
     const int64_t steps = (int64_t)g.K * elem_size(g.in_type) / 64; // k-steps of 64 bytes
-    // (1024^3, 32 k-steps, on 64 tiles: 9.8 us unsplit, 15.1 us in two slices -- the second kernel costs about 5 us; with a
-    // handful of tiles a short K is still worth splitting: int8 363x64x3025, 6 tiles and 47 k-steps, 46.9 us unsplit, 15.7 in eight)
-    if (steps < 64 && tiles * 8 > kComputeUnits) return 1;
-    // a slice of about 64 k-steps, shorter ones (down to 12) only while the tiles are few; never more workgroups than the
-    // compute units hold at once (two of the 64 x 64 tiles each), never more than 32 slices.  Measured with 64 x 64 tiles, fp16,
-    // us by slices 4 / 8 / 16 / 32: 768x320x30522 82 / 52 / 50 / 57; 1024x80x30522 79 / 50 / 37 / 41; 288x64x21609 59 / 36 / 24 / 21;
-    // 363x64x3025 17 / 13 / 13 / 15; 512x512x8192 16 / 17 / 22 / 31; 256x256x16384 23 / 18 / 19 / 22.
+    // (1024^3, 32 k-steps, on 64 tiles of 128 x 128: 9.8 us unsplit, 15.1 us in two slices -- the second kernel costs 3 to 5 us;
+    // with a handful of tiles a short K is still worth splitting: int8 363x64x3025, 6 tiles and 47 k-steps, 46.9 us unsplit,
+    // 10.8 in sixteen slices; a k-step of the register-staged kernels takes about four times as long as one of the direct ones)
+    if (steps * (v.direct ? 1 : 4) < 64 && tiles * 8 > kComputeUnits) return 1;
+    // Slices of about 32 k-steps; shorter ones, down to 4, while that keeps the workgroups at or below one per compute unit;
+    // never more workgroups than the compute units hold at once (two of the 64 x 64 tiles each), never more than 32 slices.
+    // Measured with 64 x 64 tiles, fp16, us by slices 4 / 8 / 16 / 32: 768x320x30522 84 / 53 / 49 / 53; 1024x80x30522
+    // 81 / 49 / 33 / 36; 288x64x21609 61 / 35 / 22 / 16; 363x64x3025 16 / 11 / 10 / 11; 576x96x5329 18 / 13 / 12 / 14;
+    // 512x512x8192 15 / 15 / 18 / 25; 256x256x16384 22 / 15 / 15 / 17; 384x96x1225 7.9 / 6.9 / 7.2 / 6.9.
     const int64_t slots = kComputeUnits * (v.bm * v.bn <= 64 * 64 ? 2 : 1);
-    const int64_t few = steps / 12 < 192 / tiles ? steps / 12 : 192 / tiles;
-    int64_t want = steps / 64 > few ? steps / 64 : few;
+    const int64_t few = steps / 4 < kComputeUnits / tiles ? steps / 4 : kComputeUnits / tiles;
+    int64_t want = steps / 32 > few ? steps / 32 : few;
     if (want > slots / tiles) want = slots / tiles;
     if (want > 32) want = 32;
     if ((size_t)want * (size_t)g.M * (size_t)g.N > ((size_t)1 << 24)) return 1; // 64 MiB of partial sums at most without being asked

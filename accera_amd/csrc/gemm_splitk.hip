@@ -34,28 +34,42 @@ __global__ void __launch_bounds__(256) splitk_reduce_kernel(SplitReduceArgs p)
     const int64_t slice = (int64_t)p.M * p.N;
     const int64_t at = (int64_t)row * p.N + col0;
     const int cols = p.N - col0 < 4 ? p.N - col0 : 4;
+    // The loads of eight slices are issued together (one trip through memory per batch instead of one per slice); the adds
+    // stay in slice order.
+    const bool vec = cols == 4 && (at & 3) == 0;
+    auto add_slices = [&](auto zero, auto&& add) {
+        using T = decltype(zero);
+        typedef T T4 __attribute__((ext_vector_type(4)));
+        T4 sum = {zero, zero, zero, zero};
+        const T* w = (const T*)p.ws + at;
+        for (int s0 = 0; s0 < p.splits; s0 += 8) {
+            T4 x[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                x[u] = T4{zero, zero, zero, zero};
+                if (s0 + u < p.splits) {
+                    const T* src = w + (int64_t)(s0 + u) * slice;
+                    if (vec) x[u] = *(const T4*)src;
+                    else
+                        for (int e = 0; e < cols; ++e) x[u][e] = src[e];
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+                if (s0 + u < p.splits)
+                    for (int e = 0; e < 4; ++e) sum[e] = add(sum[e], x[u][e]);
+        }
+        return sum;
+    };
     if (p.is_int) {
-        int sum[4] = {0, 0, 0, 0};
-        const int* w = (const int*)p.ws + at;
-        for (int s = 0; s < p.splits; ++s)
-            for (int e = 0; e < cols; ++e) sum[e] = wrap_add(sum[e], w[(int64_t)s * slice + e]);
+        const auto sum = add_slices(0, [](int a, int b) { return wrap_add(a, b); });
         for (int e = 0; e < cols; ++e) {
             const int64_t idx = (int64_t)row * p.c_rs + (int64_t)(col0 + e) * p.c_cs;
             const int v = apply_prologue<int>(sum[e], p.prologue, p.prologue_arg, [&]() { return load_out_int(p.C, p.out_type, idx); });
             store_out_int(p.C, p.out_type, idx, apply_epilogue<int>(v, p.epilogue, p.epilogue_arg));
         }
     } else {
-        float sum[4] = {0.f, 0.f, 0.f, 0.f};
-        const float* w = (const float*)p.ws + at;
-        if (cols == 4 && (at & 3) == 0) {
-            for (int s = 0; s < p.splits; ++s) {
-                const f32x4 x = *(const f32x4*)(w + (int64_t)s * slice);
-                for (int e = 0; e < 4; ++e) sum[e] += x[e];
-            }
-        } else {
-            for (int s = 0; s < p.splits; ++s)
-                for (int e = 0; e < cols; ++e) sum[e] += w[(int64_t)s * slice + e];
-        }
+        const auto sum = add_slices(0.f, [](float a, float b) { return a + b; });
         for (int e = 0; e < cols; ++e) {
             const int64_t idx = (int64_t)row * p.c_rs + (int64_t)(col0 + e) * p.c_cs;
             const float v = apply_prologue<float>(sum[e], p.prologue, p.prologue_arg, [&]() { return load_out(p.C, p.out_type, idx); });

@@ -25,8 +25,8 @@ def test_static_workspace_entry_point_matches_the_allocating_one():
     rng = np.random.default_rng(2024)
     # decode shape first (its slow-phase column blocks are shared by two workgroups each: 2.7 MiB of partial sums),
     # then a smaller problem with an explicit K split over four workgroups per column block; then a small square output
-    # with a long K, which the library splits by itself on an MFMA kernel (8 slices of 256 KiB of partial sums)
-    cases = [(8, 11008, 4096, 0), (4, 2048, 1024, 4), (256, 256, 4096, 0)]
+    # with a long K, which the library splits by itself on an MFMA kernel (32 slices of 64 KiB of partial sums)
+    cases = [(8, 11008, 4096, 0), (4, 2048, 1024, 4), (128, 128, 8192, 0)]
     data = []
     for M, N, K, ks in cases:
         A = make_input(rng, (M, K), "f16", "normal")
@@ -36,7 +36,7 @@ def test_static_workspace_entry_point_matches_the_allocating_one():
         _lib.check(_call(L.acc950_gemm_ops, dA, dB, d_ref, M, N, K, ks, stream))
         data.append((A, B, dA, dB, d_ref, d_new))
     torch.cuda.synchronize()
-    assert _lib.launch_geometry(_lib.F16, _lib.F16, 256, 256, 4096, (4096, 1), (256, 1), (256, 1))[0][2] > 1
+    assert _lib.launch_geometry(_lib.F16, _lib.F16, 128, 128, 8192, (8192, 1), (128, 1), (128, 1))[0][2] > 1
     allocations_before = _lib.allocation_probe()
     assert allocations_before >= 2  # the allocating entry point made this stream's workspace
     for rep in range(2):  # the pair of calls twice: the second round finds the array as the first left it
@@ -86,17 +86,17 @@ def test_static_workspace_entry_point_under_graph_capture():
     X = make_input(rng, (M, H), "f16", "normal")
     W1 = (make_input(rng, (H, F), "f16", "normal").astype(np.float32) * 0.03).astype(np.float16)
     W2 = (make_input(rng, (F, H), "f16", "normal").astype(np.float32) * 0.03).astype(np.float16)
-    P, Q = make_input(rng, (256, 4096), "f16", "normal"), (make_input(rng, (4096, 256), "f16", "normal").astype(np.float32) * 0.05).astype(np.float16)
+    P, Q = make_input(rng, (128, 8192), "f16", "normal"), (make_input(rng, (8192, 128), "f16", "normal").astype(np.float32) * 0.03).astype(np.float16)
     dX, dW1, dW2, dP, dQ = (to_device(a, "f16") for a in (X, W1, W2, P, Q))
     mk = lambda r, c: to_device(np.zeros((r, c), np.float16), "f16")
-    hid_e, out_e, sq_e, hid_g, out_g, sq_g = mk(M, F), mk(M, H), mk(256, 256), mk(M, F), mk(M, H), mk(256, 256)
+    hid_e, out_e, sq_e, hid_g, out_g, sq_g = mk(M, F), mk(M, H), mk(128, 128), mk(M, F), mk(M, H), mk(128, 128)
 
     def step(entry, hid, out, sq, stream):
         args = lambda A, B, C, m, n, k, epi: (_lib.F16, _lib.F16, m, n, k, A.data_ptr(), k, 1, B.data_ptr(), n, 1, C.data_ptr(), n, 1,
                                               _lib.PROLOGUE_SET0, 0.0, epi, 0.0, _lib.VARIANT_AUTO, 0, stream)
         _lib.check(entry(*args(dX, dW1, hid, M, F, H, _lib.EPILOGUE_RELU)))
         _lib.check(entry(*args(hid, dW2, out, M, H, F, _lib.EPILOGUE_NONE)))
-        _lib.check(entry(*args(dP, dQ, sq, 256, 256, 4096, _lib.EPILOGUE_RELU)))
+        _lib.check(entry(*args(dP, dQ, sq, 128, 128, 8192, _lib.EPILOGUE_RELU)))
 
     # eager, on the current stream (also loads every kernel's code and sets its LDS limit before the capture)
     step(L.acc950_gemm_ops_static, hid_e, out_e, sq_e, torch.cuda.current_stream().cuda_stream)
