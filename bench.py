@@ -152,12 +152,14 @@ def cpu_baseline(c, threads, budget_rows=None):
         B = np.asfortranarray(B)
     C = np.zeros((M, N), ora.NP_STORAGE[c["out_type"]])
     ora.gemm_relu(A[:16], B, C[:16], t, c["out_type"], threads=threads)  # warm-up (page faults, OpenMP pool)
-    t0 = time.perf_counter()
-    ora.gemm_relu(A, B, C, t, c["out_type"], schedule=ora.SCHED_TRANSFORMED, threads=threads)
-    dt = time.perf_counter() - t0
+    passes, dt = 3, float("inf")
+    for _ in range(passes):
+        t0 = time.perf_counter()
+        ora.gemm_relu(A, B, C, t, c["out_type"], schedule=ora.SCHED_TRANSFORMED, threads=threads)
+        dt = min(dt, time.perf_counter() - t0)
     return dict(value=round(2 * M * N * K / dt / 1e12, 5), unit="TFLOP/s" if t != "i8" else "TOP/s", cores=threads,
                 kind="port", seconds=round(dt, 3),
-                sample=f"rows 0..{M - 1} of A against all of B ({M}x{N}x{K}), one pass, OpenMP over column tiles")
+                sample=f"rows 0..{M - 1} of A against all of B ({M}x{N}x{K}), best of {passes} passes, OpenMP over column tiles")
 
 
 def vendor_library(c, first_set, steps):
