@@ -1,4 +1,6 @@
-"""ctypes binding of libaccera_mi355x.so (the C ABI declared in include/accera_mi355x_gemm.h, the measurement aids in include/accera_mi355x_probes.h).
+"""ctypes binding of libaccera_mi355x.so (the C ABI declared in include/accera_mi355x_gemm.h) and of
+libaccera_mi355x_probes.so (the measurement aids of include/accera_mi355x_probes.h, a library of its own that only the
+benchmark and the tests of its aids load).
 
 There is no CPU fallback: if the shared library is missing, loading raises with the
 build command; if a call fails, the library's own error text is raised.
@@ -9,6 +11,7 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_DIR = os.path.join(_HERE, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libaccera_mi355x.so")
+PROBES_LIB_PATH = os.path.join(LIB_DIR, "libaccera_mi355x_probes.so")
 INCLUDE_DIR = os.path.join(os.path.dirname(_HERE), "include")
 
 # element types / ops / status codes / variant ids (accera_mi355x_gemm.h)
@@ -23,9 +26,11 @@ EXPORTS = [
     "acc950_gemm_batched", "acc950_gemm_batched_host", "acc950_bind", "acc950_launch", "acc950_unbind",
     "acc950_launch_geometry", "acc950_num_variants", "acc950_num_skinny_variants",
     "acc950_variant_name", "acc950_last_error",
+    "acc950_bound_choice", "acc950_workspace_probe", "acc950_allocation_probe", "acc950_release_workspaces",
 ]
-# measurement aids (include/accera_mi355x_probes.h): not part of the product ABI
-PROBE_EXPORTS = ["acc950_mfma_ceiling", "acc950_mfma_traffic_probe", "acc950_mfma_phase_probe", "acc950_copy_probe", "acc950_stream_read_probe", "acc950_workspace_probe", "acc950_allocation_probe"]
+# measurement aids (include/accera_mi355x_probes.h, libaccera_mi355x_probes.so): not part of the product
+PROBE_EXPORTS = ["acc950_mfma_ceiling", "acc950_mfma_traffic_probe", "acc950_mfma_phase_probe", "acc950_copy_probe", "acc950_stream_read_probe",
+                 "acc950_probes_last_error"]
 
 
 class Acc950Error(RuntimeError):
@@ -66,18 +71,40 @@ def lib():
     L.acc950_launch_geometry.argtypes = [ci, ci, ci, ci, ci] + [i64] * 6 + [ci, ci, ctypes.POINTER(cu), ctypes.POINTER(cu),
                                                                            ctypes.POINTER(cu), ctypes.POINTER(ci)]
     L.acc950_variant_name.argtypes = [ci, ctypes.c_char_p, ctypes.c_size_t]
+    L.acc950_allocation_probe.argtypes = [ctypes.POINTER(ctypes.c_ulonglong)]
+    L.acc950_workspace_probe.argtypes = [vp, ctypes.POINTER(vp), ctypes.POINTER(vp)]
+    L.acc950_bound_choice.argtypes = [ci, ctypes.POINTER(ci), ctypes.POINTER(ci)]
+    L.acc950_release_workspaces.argtypes = []
+    L.acc950_last_error.restype = ctypes.c_char_p
+    for name in EXPORTS:
+        if name != "acc950_last_error":
+            getattr(L, name).restype = ci
+    _lib = L
+    return L
+
+
+_probes = None
+
+
+def probes():
+    """The measurement-aid library (loads it on first use): machine ceilings, copy / read probes, the in-kernel phase probe."""
+    global _probes
+    if _probes is not None:
+        return _probes
+    if not os.path.exists(PROBES_LIB_PATH):
+        raise RuntimeError(f"{PROBES_LIB_PATH} is missing: build it with `make -C accera_amd/csrc`")
+    L = ctypes.CDLL(PROBES_LIB_PATH, mode=ctypes.RTLD_GLOBAL)
+    ci, vp = ctypes.c_int, ctypes.c_void_p
     L.acc950_mfma_ceiling.argtypes = [ci, ci, ci, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double)]
     L.acc950_mfma_traffic_probe.argtypes = [ci, ci, ci, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double)]
     L.acc950_mfma_phase_probe.argtypes = [ci, ci, ci, ci, ci, vp, vp, vp, ctypes.POINTER(ctypes.c_double)]
     L.acc950_copy_probe.argtypes = [vp, vp, ctypes.c_size_t, vp]
     L.acc950_stream_read_probe.argtypes = [vp, ctypes.c_size_t, vp, vp]
-    L.acc950_allocation_probe.argtypes = [ctypes.POINTER(ctypes.c_ulonglong)]
-    L.acc950_workspace_probe.argtypes = [vp, ctypes.POINTER(vp), ctypes.POINTER(vp)]
-    L.acc950_last_error.restype = ctypes.c_char_p
-    for name in EXPORTS + PROBE_EXPORTS:
-        if name != "acc950_last_error":
+    L.acc950_probes_last_error.restype = ctypes.c_char_p
+    for name in PROBE_EXPORTS:
+        if name != "acc950_probes_last_error":
             getattr(L, name).restype = ci
-    _lib = L
+    _probes = L
     return L
 
 
@@ -86,10 +113,15 @@ def check(rc):
         raise Acc950Error(rc, lib().acc950_last_error().decode())
 
 
+def check_probe(rc):
+    if rc != OK:
+        raise Acc950Error(rc, probes().acc950_probes_last_error().decode() or "probe failed")
+
+
 def mfma_phase_probe(in_type, out_type, M, N, K, a_ptr, b_ptr, c_ptr):
     """In-kernel phase times of the 256x256 kernel the automatic choice takes, on device operands; returns a dict."""
     out = (ctypes.c_double * 8)()
-    check(lib().acc950_mfma_phase_probe(in_type, out_type, M, N, K, a_ptr, b_ptr, c_ptr, out))
+    check_probe(probes().acc950_mfma_phase_probe(in_type, out_type, M, N, K, a_ptr, b_ptr, c_ptr, out))
     return {"prologue_us": out[0] / 1e3, "main_loop_us": out[1] / 1e3, "write_back_us": out[2] / 1e3,
             "clock_ghz_prologue": out[3], "clock_ghz_main_loop": out[4], "clock_ghz_write_back": out[5],
             "kernel_span_us": out[6] / 1e3, "mfma_pipe_busy_main_loop": out[7]}
@@ -99,7 +131,7 @@ def mfma_ceiling(in_type, data_mode=2, iters=20000):
     """(tera-ops/s, sustained shader clock in GHz) of a pure MFMA loop on this GPU;
     data_mode 0 zeros, 1 constant, 2 random operands."""
     t, g = ctypes.c_double(), ctypes.c_double()
-    check(lib().acc950_mfma_ceiling(in_type, data_mode, iters, ctypes.byref(t), ctypes.byref(g)))
+    check_probe(probes().acc950_mfma_ceiling(in_type, data_mode, iters, ctypes.byref(t), ctypes.byref(g)))
     return t.value, g.value
 
 
@@ -107,7 +139,7 @@ def mfma_traffic_probe(in_type, traffic, iters=2000):
     """(tera-ops/s, sustained shader clock in GHz) of the four-wave loop's MFMAs with its traffic added piece by piece:
     traffic 0 none, 1 its LDS reads, 2 also its direct-to-LDS fills from the caches, 3 the fills from a 1 GiB buffer."""
     t, g = ctypes.c_double(), ctypes.c_double()
-    check(lib().acc950_mfma_traffic_probe(in_type, traffic, iters, ctypes.byref(t), ctypes.byref(g)))
+    check_probe(probes().acc950_mfma_traffic_probe(in_type, traffic, iters, ctypes.byref(t), ctypes.byref(g)))
     return t.value, g.value
 
 
@@ -123,6 +155,11 @@ def workspace_probe(stream):
     a, b = ctypes.c_void_p(), ctypes.c_void_p()
     check(lib().acc950_workspace_probe(stream, ctypes.byref(a), ctypes.byref(b)))
     return a.value, b.value
+
+
+def release_workspaces():
+    """Frees the K-split workspaces of the current device (all streams) after waiting for the device to go idle."""
+    check(lib().acc950_release_workspaces())
 
 
 def variant_name(variant):

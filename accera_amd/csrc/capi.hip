@@ -1,7 +1,6 @@
 // C ABI of the library (include/accera_mi355x_gemm.h): argument checking, kernel
 // selection, the host-pointer path and the launch-geometry query.
 #include "../../include/accera_mi355x_gemm.h"
-#include "../../include/accera_mi355x_probes.h"
 #include "common.h"
 #include "skinny.h"
 #include <vector>
@@ -200,8 +199,9 @@ int auto_skinny_variant(const Problem& pb)
 // ---- workspace of the skinny kernels' K split ------------------------------------------
 // Partial sums (fp32) and one arrival counter per column block.  One workspace per (device, stream): launches on one
 // stream run one after the other and may share it, launches on different streams may overlap and must not.  A
-// workspace only grows, and an outgrown block stays allocated until the process ends, because launches queued
-// earlier may still be using it.  The pointers are copied out while the lock is held.
+// workspace only grows, and an outgrown block stays allocated, because launches queued earlier may still be using
+// it, until acc950_release_workspaces frees everything on an idle device.  The pointers are copied out while the
+// lock is held.
 struct Workspace {
     float* scratch = nullptr;
     size_t floats = 0;
@@ -210,6 +210,7 @@ struct Workspace {
 };
 std::mutex g_ws_mutex;
 std::map<std::pair<int, hipStream_t>, Workspace> g_ws;
+std::vector<std::pair<int, void*>> g_ws_retired; // (device, block) outgrown by its workspace: freed by acc950_release_workspaces
 std::atomic<unsigned long long> g_device_allocations{0}; // hipMalloc calls made by the GEMM entry points (acc950_allocation_probe)
 
 hipError_t workspace_for(hipStream_t stream, size_t floats, size_t counters, float** scratch, unsigned** cnt)
@@ -225,7 +226,8 @@ hipError_t workspace_for(hipStream_t stream, size_t floats, size_t counters, flo
         e = hipMalloc((void**)&p, want * sizeof(float));
         if (e != hipSuccess) return e;
         ++g_device_allocations;
-        w.scratch = p; // (the block it replaces is left to earlier launches)
+        if (w.scratch) g_ws_retired.emplace_back(dev, (void*)w.scratch); // (left to the launches queued earlier)
+        w.scratch = p;
         w.floats = want;
     }
     if (counters > w.n_counters) {
@@ -236,6 +238,7 @@ hipError_t workspace_for(hipStream_t stream, size_t floats, size_t counters, flo
         ++g_device_allocations;
         e = hipMemset(p, 0, want * sizeof(unsigned));
         if (e != hipSuccess) { (void)hipFree(p); return e; }
+        if (w.counters) g_ws_retired.emplace_back(dev, (void*)w.counters);
         w.counters = p;
         w.n_counters = want;
     }
@@ -373,10 +376,14 @@ GemmArgs split_first_step(const GemmArgs& g, const SplitPlan& sp, void* ws)
 
 // Slices for `want` splits of this problem on variant v (fewer when K has too few K tiles); false when the variant
 // cannot run the problem split (a batch, one slice only, partial products it does not take).
-bool plan_split(const MfmaVariant& v, const Problem& pb, int want, SplitPlan* sp)
+bool plan_split(const MfmaVariant& v, const Problem& pb, int want, SplitPlan* sp, size_t max_floats = kMaxSplitFloats)
 {
     const GemmArgs& g = pb.g;
     if (g.batch > 1 || want <= 1) return false;
+    // (never more slices than the workspace at hand holds)
+    const size_t per_slice = (size_t)g.M * (size_t)g.N;
+    if (per_slice == 0 || max_floats / per_slice < 2) return false;
+    if ((size_t)want > max_floats / per_slice) want = (int)(max_floats / per_slice);
     const int bk = v.kb / elem_size(g.in_type);
     const int kt = (g.K + bk - 1) / bk, least = v.w4 ? 4 : 1; // K tiles in all; K tiles a slice needs
     int splits = want < kt / least ? want : kt / least;
@@ -385,7 +392,7 @@ bool plan_split(const MfmaVariant& v, const Problem& pb, int want, SplitPlan* sp
     splits = (kt + per - 1) / per;
     if (splits > 1 && g.K - (splits - 1) * per * bk < least * bk) --splits; // (the last slice takes what a too short one would have left)
     if (splits <= 1) return false;
-    if ((size_t)splits * (size_t)g.M * (size_t)g.N > kMaxSplitFloats) return false;
+    if ((size_t)splits * per_slice > max_floats) return false;
     sp->splits = splits;
     sp->ks = per * bk;
     sp->k_last = g.K - (splits - 1) * sp->ks;
@@ -399,7 +406,7 @@ bool plan_split(const MfmaVariant& v, const Problem& pb, int want, SplitPlan* sp
 // enough for the second kernel (a few microseconds) to pay.  Measured on small outputs with a long K (512 x 512 x 8192,
 // 256 x 256 x 16384, 1024 x 1024 x 4096, 768 x 320 x 30522, 1024 x 80 x 30522; 16-bit inputs): the best split fills the
 // compute units once or twice and leaves a slice 4 to 60 k-steps of 64 bytes.
-int auto_mfma_splits(const MfmaVariant& v, const Problem& pb)
+int auto_mfma_splits(const MfmaVariant& v, const Problem& pb, size_t max_floats = kMaxSplitFloats)
 {
     const GemmArgs& g = pb.g;
     if (g.batch > 1) return 1;
@@ -422,7 +429,7 @@ int auto_mfma_splits(const MfmaVariant& v, const Problem& pb)
     if (want > 32) want = 32;
     if ((size_t)want * (size_t)g.M * (size_t)g.N > ((size_t)1 << 24)) return 1; // 64 MiB of partial sums at most without being asked
     SplitPlan sp;
-    return want > 1 && plan_split(v, pb, (int)want, &sp) ? sp.splits : 1;
+    return want > 1 && plan_split(v, pb, (int)want, &sp, max_floats) ? sp.splits : 1;
 }
 
 struct Choice {
@@ -430,7 +437,9 @@ struct Choice {
     int splits;
 };
 
-int choose(const Problem& pb, int variant, int k_splits, Choice* c)
+// max_split_floats: 32-bit partial sums the workspace of this call holds (the built-in array of acc950_gemm_ops_static
+// is smaller than what the allocating entry points may ask for): an MFMA kernel's K split never plans more slices.
+int choose(const Problem& pb, int variant, int k_splits, Choice* c, size_t max_split_floats = kMaxSplitFloats)
 {
     c->splits = 1;
     if (variant == ACC950_VARIANT_AUTO) {
@@ -449,7 +458,7 @@ int choose(const Problem& pb, int variant, int k_splits, Choice* c)
                 int n = 0;
                 const MfmaVariant& v = mfma_table(pb.g.in_type, &n)[mv];
                 SplitPlan sp;
-                slices = k_splits > 1 ? (plan_split(v, pb, k_splits, &sp) ? sp.splits : 1) : k_splits == 0 ? auto_mfma_splits(v, pb) : 1;
+                slices = k_splits > 1 ? (plan_split(v, pb, k_splits, &sp, max_split_floats) ? sp.splits : 1) : k_splits == 0 ? auto_mfma_splits(v, pb, max_split_floats) : 1;
                 const int64_t tiles = (((int64_t)pb.g.M + v.bm - 1) / v.bm) * (((int64_t)pb.g.N + v.bn - 1) / v.bn);
                 // (or more workgroups than there are 32 x 32 blocks: a small output with a long K, which only the tiled kernels split)
                 const int64_t blocks = (((int64_t)pb.g.M + 31) / 32) * (((int64_t)pb.g.N + 31) / 32);
@@ -462,8 +471,8 @@ int choose(const Problem& pb, int variant, int k_splits, Choice* c)
             int n = 0;
             const MfmaVariant& v = mfma_table(pb.g.in_type, &n)[mv];
             SplitPlan sp;
-            if (k_splits > 1) c->splits = plan_split(v, pb, k_splits, &sp) ? sp.splits : 1;
-            else if (k_splits == 0) c->splits = auto_mfma_splits(v, pb);
+            if (k_splits > 1) c->splits = plan_split(v, pb, k_splits, &sp, max_split_floats) ? sp.splits : 1;
+            else if (k_splits == 0) c->splits = auto_mfma_splits(v, pb, max_split_floats);
         }
         return ACC950_OK;
     }
@@ -491,8 +500,8 @@ int choose(const Problem& pb, int variant, int k_splits, Choice* c)
     c->variant = variant;
     if (k_splits > 1) { // (a named variant is split only when asked)
         SplitPlan sp;
-        if (!plan_split(tab[variant], pb, k_splits, &sp))
-            return fail(ACC950_UNSUPPORTED, "this MFMA variant cannot run the problem with K split (a batch, too few K tiles, or partial products it does not take)");
+        if (!plan_split(tab[variant], pb, k_splits, &sp, max_split_floats))
+            return fail(ACC950_UNSUPPORTED, "this MFMA variant cannot run the problem with K split (a batch, too few K tiles, partial products it does not take, or slices the workspace does not hold)");
         c->splits = sp.splits;
     }
     return ACC950_OK;
@@ -525,16 +534,12 @@ int run(const Problem& pb, const Choice& c, hipStream_t stream, LaunchGeom* geom
         // 128-byte lines have address bits 8:7 = 11 stream ~25 % slower (measured), so they are
         // shared by two workgroups each; the otherwise idle CUs take the second halves.
         const SkinnyVariant& skv = skinny_variant(sv);
-        if (skv.mfma && skv.cols == 64 && c.splits == 1 && pb.have_pointers && (g.b_rs * 2) % 512 == 0 &&
+        // (Which blocks those are follows B's address.  A query without pointers reports phase 0: no phase has more blocks,
+        // so the grid it names is what launches or one workgroup more.)
+        if (skv.mfma && skv.cols == 64 && c.splits == 1 && (g.b_rs * 2) % 512 == 0 &&
             skinny_column_blocks(sv, g.N) >= 128 && skinny_column_blocks(sv, g.N) <= 200 && g.K >= 512 &&
             (g.batch <= 1 || (g.b_bs * 2) % 512 == 0))
-            s.extra_phase = (int)((3u - (unsigned)(reinterpret_cast<uintptr_t>(g.B) >> 7)) & 3u);
-        // (measurement aid: ACC950_SKINNY_SHARED_PHASE = -1 switches the sharing off, 0..3 shares the blocks of that phase instead)
-        static const char* const phase_override = std::getenv("ACC950_SKINNY_SHARED_PHASE");
-        if (phase_override && s.extra_phase >= 0) {
-            const int v = std::atoi(phase_override);
-            s.extra_phase = v < 0 ? -1 : (int)(((unsigned)v - (unsigned)(reinterpret_cast<uintptr_t>(g.B) >> 7)) & 3u);
-        }
+            s.extra_phase = pb.have_pointers ? (int)((3u - (unsigned)(reinterpret_cast<uintptr_t>(g.B) >> 7)) & 3u) : 0;
         const int ws_splits = s.extra_phase >= 0 ? 2 : c.splits;
         if (!dry_run && ws_splits > 1) {
             const size_t nb = g.batch > 1 ? (size_t)g.batch : 1;
@@ -564,9 +569,8 @@ int run(const Problem& pb, const Choice& c, hipStream_t stream, LaunchGeom* geom
         const MfmaVariant& mv = tab[c.variant];
         const bool lean = g.prologue == PRO_SET && g.prologue_arg == 0.f && (g.epilogue == EPI_RELU || g.epilogue == EPI_NONE);
         SplitPlan sp;
-        bool split = c.splits > 1 && plan_split(mv, pb, c.splits, &sp);
-        // (slices that do not fit the built-in workspace: the problem runs unsplit, which every variant that can be split also takes)
-        if (split && static_ws && (size_t)sp.splits * (size_t)g.M * (size_t)g.N > kStaticFloats) split = false;
+        // (the choice was made for the workspace of this call: the same plan comes out again)
+        const bool split = c.splits > 1 && plan_split(mv, pb, c.splits, &sp, static_ws ? kStaticFloats : kMaxSplitFloats);
         if (split) {
             float* ws = nullptr;
             if (!dry_run) {
@@ -655,7 +659,7 @@ int acc950_gemm_ops_static(int in_type, int out_type, int M, int N, int K,
                           prologue_arg, epilogue_arg);
     if (rc) return rc;
     Choice c;
-    rc = choose(pb, variant, k_splits, &c);
+    rc = choose(pb, variant, k_splits, &c, kStaticFloats);
     if (rc) return rc;
     return run(pb, c, (hipStream_t)stream, nullptr, false, true);
 }
@@ -722,6 +726,15 @@ int acc950_launch(int handle)
     return run(bc.pb, bc.choice, bc.stream, nullptr, false);
 }
 
+int acc950_bound_choice(int handle, int* variant, int* k_splits)
+{
+    std::lock_guard<std::mutex> lock(g_bound_mutex);
+    if (handle < 0 || (size_t)handle >= g_bound.size() || !g_bound[handle].live) return fail(ACC950_INVALID_ARGUMENT, "unknown call handle");
+    if (variant) *variant = g_bound[handle].choice.variant;
+    if (k_splits) *k_splits = g_bound[handle].choice.splits;
+    return ACC950_OK;
+}
+
 int acc950_unbind(int handle)
 {
     std::lock_guard<std::mutex> lock(g_bound_mutex);
@@ -754,6 +767,31 @@ int acc950_allocation_probe(unsigned long long* count)
     return ACC950_OK;
 }
 
+int acc950_release_workspaces(void)
+{
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return fail_hip(e, "hipGetDevice");
+    e = hipDeviceSynchronize(); // nothing queued earlier still uses a block
+    if (e != hipSuccess) return fail_hip(e, "hipDeviceSynchronize");
+    std::lock_guard<std::mutex> lock(g_ws_mutex);
+    hipError_t first = hipSuccess;
+    auto release = [&](void* p) { if (p) { hipError_t r = hipFree(p); if (r != hipSuccess && first == hipSuccess) first = r; } };
+    for (auto it = g_ws.begin(); it != g_ws.end();) {
+        if (it->first.first != dev) { ++it; continue; }
+        release(it->second.scratch);
+        release(it->second.counters);
+        it = g_ws.erase(it);
+    }
+    for (auto it = g_ws_retired.begin(); it != g_ws_retired.end();) {
+        if (it->first != dev) { ++it; continue; }
+        release(it->second);
+        it = g_ws_retired.erase(it);
+    }
+    if (first != hipSuccess) return fail_hip(first, "hipFree");
+    return ACC950_OK;
+}
+
 int acc950_workspace_probe(void* stream, void** partial_sums, void** counters)
 {
     if (!partial_sums || !counters) return fail(ACC950_INVALID_ARGUMENT, "null output");
@@ -763,57 +801,6 @@ int acc950_workspace_probe(void* stream, void** partial_sums, void** counters)
     if (e != hipSuccess) return fail_hip(e, "workspace allocation");
     *partial_sums = f;
     *counters = c;
-    return ACC950_OK;
-}
-
-int acc950_mfma_phase_probe(int in_type, int out_type, int M, int N, int K, const void* A, const void* B, void* C, double* out)
-{
-    if (!out) return fail(ACC950_INVALID_ARGUMENT, "null output");
-    Problem pb;
-    int rc = make_problem(in_type, out_type, M, N, K, A, K, 1, B, N, 1, C, N, 1, PRO_SET0, EPI_RELU, true, &pb);
-    if (rc) return rc;
-    // (the shape conditions of the timed kernel, which is no row of the variant table: any launcher stands for "exists")
-    const MfmaVariant probe = {256, 256, 2, 4, true, false, true, false, 64, 4, true, false, false, false, false, launch_mfma_timed_f16, nullptr};
-    int n_unused = 0;
-    if (M < 256 || N < 256 || K < 1 || !mfma_table(pb.g.in_type, &n_unused) || !mfma_can_take(probe, pb))
-        return fail(ACC950_UNSUPPORTED, "the phase probe runs the 256x256 kernels: 8/16-bit inputs, dense row-major A, B, C, M and N multiples of 256, K of 64 bytes");
-    GemmArgs g = pb.g;
-    const int tiles = (M / 256) * (N / 256);
-    hipError_t e = hipMalloc((void**)&g.stamps, (size_t)tiles * 8 * sizeof(unsigned long long));
-    if (e != hipSuccess) return fail_hip(e, "stamp buffer");
-    std::vector<unsigned long long> h((size_t)tiles * 8);
-    const int reps = 20; // the last launch is the one read back; the others settle the clocks
-    for (int i = 0; i < reps && e == hipSuccess; ++i) {
-        e = g.in_type == T_I8 ? launch_mfma_timed_i8(g, nullptr, nullptr, false)
-            : g.in_type == T_BF16 ? launch_mfma_timed_bf16(g, nullptr, nullptr, false) : launch_mfma_timed_f16(g, nullptr, nullptr, false);
-    }
-    if (e == hipSuccess) e = hipDeviceSynchronize();
-    if (e == hipSuccess) e = hipMemcpy(h.data(), g.stamps, h.size() * sizeof(unsigned long long), hipMemcpyDeviceToHost);
-    hipError_t e2 = hipFree(g.stamps);
-    if (e != hipSuccess) return fail_hip(e, "phase probe");
-    if (e2 != hipSuccess) return fail_hip(e2, "phase probe");
-    // per phase: average wall time (100 MHz counter) and average shader cycles over the workgroups
-    unsigned long long first = ~0ull, last = 0;
-    double ns[3] = {0, 0, 0}, cyc[3] = {0, 0, 0};
-    for (int t = 0; t < tiles; ++t) {
-        const unsigned long long* w = &h[(size_t)t * 8];
-        first = w[1] < first ? w[1] : first;
-        last = w[7] > last ? w[7] : last;
-        for (int q = 0; q < 3; ++q) {
-            ns[q] += (double)(w[(q + 1) * 2 + 1] - w[q * 2 + 1]) * 10.0;
-            cyc[q] += (double)(w[(q + 1) * 2] - w[q * 2]);
-        }
-    }
-    for (int q = 0; q < 3; ++q) {
-        out[q] = ns[q] / tiles;                       // prologue, main loop, write-back [ns]
-        out[3 + q] = ns[q] > 0 ? cyc[q] / ns[q] : 0;  // shader clock in that phase [GHz]
-    }
-    out[6] = (double)(last - first) * 10.0;           // first workgroup start to last workgroup end [ns]
-    // MFMA pipe occupancy of the main loop: per SIMD, 512 MFMA cycles per 32 bytes of K (two waves x 8 MFMAs of 32 cycles,
-    // or one wave x 32 MFMAs of 16 cycles)
-    const int es = g.in_type == T_I8 ? 1 : 2;
-    const double mfma_cycles = 2.0 * 8.0 * 32.0 * ((double)K * es / 32.0);
-    out[7] = cyc[1] > 0 ? mfma_cycles / (cyc[1] / tiles) : 0;
     return ACC950_OK;
 }
 

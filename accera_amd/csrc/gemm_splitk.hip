@@ -36,7 +36,8 @@ __global__ void __launch_bounds__(256) splitk_reduce_kernel(SplitReduceArgs p)
     const int cols = p.N - col0 < 4 ? p.N - col0 : 4;
     // The loads of eight slices are issued together (one trip through memory per batch instead of one per slice); the adds
     // stay in slice order.
-    const bool vec = cols == 4 && (at & 3) == 0;
+    // (a slice starts M * N elements after the one before: every slice's piece is 16 bytes aligned only when that is a multiple of four too)
+    const bool vec = cols == 4 && (at & 3) == 0 && (slice & 3) == 0;
     auto add_slices = [&](auto zero, auto&& add) {
         using T = decltype(zero);
         typedef T T4 __attribute__((ext_vector_type(4)));
@@ -61,8 +62,25 @@ __global__ void __launch_bounds__(256) splitk_reduce_kernel(SplitReduceArgs p)
         }
         return sum;
     };
+    // Four finished outputs that lie side by side, aligned, in a C that is only written leave as one store.
+    const int os = p.out_type == T_I8 ? 1 : (p.out_type == T_F32 || p.out_type == T_I32) ? 4 : 2;
+    const int64_t idx0 = (int64_t)row * p.c_rs + col0;
+    const bool vec_out = cols == 4 && p.c_cs == 1 && p.prologue == PRO_SET && (((size_t)p.C + (size_t)idx0 * os) & (size_t)(4 * os - 1)) == 0;
+    typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+    typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
     if (p.is_int) {
         const auto sum = add_slices(0, [](int a, int b) { return wrap_add(a, b); });
+        if (vec_out) {
+            int r[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) r[e] = apply_epilogue<int>(wrap_add(sum[e], (int)p.prologue_arg), p.epilogue, p.epilogue_arg);
+            if (p.out_type == T_I32) *(i32x4*)((int*)p.C + idx0) = i32x4{r[0], r[1], r[2], r[3]};
+            else if (p.out_type == T_I16)
+                *(u32x2*)((int16_t*)p.C + idx0) = u32x2{((unsigned)r[0] & 0xffffu) | ((unsigned)r[1] << 16), ((unsigned)r[2] & 0xffffu) | ((unsigned)r[3] << 16)};
+            else
+                *(unsigned*)((int8_t*)p.C + idx0) = ((unsigned)r[0] & 0xffu) | (((unsigned)r[1] & 0xffu) << 8) | (((unsigned)r[2] & 0xffu) << 16) | ((unsigned)r[3] << 24);
+            return;
+        }
         for (int e = 0; e < cols; ++e) {
             const int64_t idx = (int64_t)row * p.c_rs + (int64_t)(col0 + e) * p.c_cs;
             const int v = apply_prologue<int>(sum[e], p.prologue, p.prologue_arg, [&]() { return load_out_int(p.C, p.out_type, idx); });
@@ -70,6 +88,19 @@ __global__ void __launch_bounds__(256) splitk_reduce_kernel(SplitReduceArgs p)
         }
     } else {
         const auto sum = add_slices(0.f, [](float a, float b) { return a + b; });
+        if (vec_out) {
+            float r[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) r[e] = apply_epilogue<float>(sum[e] + p.prologue_arg, p.epilogue, p.epilogue_arg);
+            if (p.out_type == T_F32) *(f32x4*)((float*)p.C + idx0) = f32x4{r[0], r[1], r[2], r[3]};
+            else if (p.out_type == T_F16)
+                *(u32x2*)((uint16_t*)p.C + idx0) = u32x2{(unsigned)float_to_f16_bits(r[0]) | ((unsigned)float_to_f16_bits(r[1]) << 16),
+                                                         (unsigned)float_to_f16_bits(r[2]) | ((unsigned)float_to_f16_bits(r[3]) << 16)};
+            else
+                *(u32x2*)((uint16_t*)p.C + idx0) = u32x2{(unsigned)float_to_bf16_bits(r[0]) | ((unsigned)float_to_bf16_bits(r[1]) << 16),
+                                                         (unsigned)float_to_bf16_bits(r[2]) | ((unsigned)float_to_bf16_bits(r[3]) << 16)};
+            return;
+        }
         for (int e = 0; e < cols; ++e) {
             const int64_t idx = (int64_t)row * p.c_rs + (int64_t)(col0 + e) * p.c_cs;
             const float v = apply_prologue<float>(sum[e], p.prologue, p.prologue_arg, [&]() { return load_out(p.C, p.out_type, idx); });

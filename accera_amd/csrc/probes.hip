@@ -1,3 +1,6 @@
+// libaccera_mi355x_probes.so: measurement aids used by the benchmark and by the tests of the benchmark's aids; the product
+// library (libaccera_mi355x.so) holds none of this.
+//
 // Measurement aids used by the benchmark: what this particular GPU can sustain, so that
 // a kernel's distance from the nominal peak can be split into "kernel" and "machine".
 //
@@ -11,13 +14,17 @@
 #include "../../include/accera_mi355x_gemm.h"
 #include "../../include/accera_mi355x_probes.h"
 #include "common.h"
+#include "probe_timed.h"
 
 #include <cstdlib>
+#include <string>
 #include <vector>
 
 using namespace acc950;
 
 namespace {
+
+thread_local std::string t_probe_error; // why the phase probe refused its last call on this thread
 
 // 8 waves per workgroup (two per SIMD, as in the GEMM kernels), 16 independent 16x16 accumulators
 // per wave, the instruction written out so that every MFMA accumulates in place.
@@ -263,6 +270,72 @@ int acc950_stream_read_probe(const void* src, size_t bytes, void* scratch4, void
     if (!src || !scratch4 || bytes % 16) return ACC950_INVALID_ARGUMENT;
     hipLaunchKernelGGL(acc950_stream_read_kernel, dim3(512), dim3(256), 0, (hipStream_t)stream, (const i32x4*)src, (int*)scratch4, bytes / 16);
     return hipGetLastError() == hipSuccess ? ACC950_OK : ACC950_HIP_ERROR;
+}
+
+const char* acc950_probes_last_error(void) { return t_probe_error.c_str(); }
+
+int acc950_mfma_phase_probe(int in_type, int out_type, int M, int N, int K, const void* A, const void* B, void* C, double* out)
+{
+    // The timed kernels take whole 256x256 tiles of dense row-major operands only (the four-wave form from four K tiles of
+    // 64 bytes up, the eight-wave form below): everything else is refused here, before anything is sized or launched.
+    auto refuse = [&](int code, const char* why) { t_probe_error = why; return code; };
+    if (!out || !A || !B || !C) return refuse(ACC950_INVALID_ARGUMENT, "null pointer");
+    if (in_type != T_F16 && in_type != T_BF16 && in_type != T_I8) return refuse(ACC950_UNSUPPORTED, "the phase probe runs the 256x256 kernels: 8/16-bit inputs");
+    const bool out_ok = in_type == T_I8 ? (out_type == T_I32 || out_type == T_I16 || out_type == T_I8) : (out_type == T_F32 || out_type == T_F16 || out_type == T_BF16);
+    if (!out_ok) return refuse(ACC950_INVALID_ARGUMENT, "unsupported input/output element type pair");
+    const int es = in_type == T_I8 ? 1 : 2, bk = 64 / es;
+    if (M < 256 || N < 256 || K < bk || M % 256 || N % 256 || K % bk)
+        return refuse(ACC950_UNSUPPORTED, "the phase probe runs the 256x256 kernels: dense row-major A, B, C, M and N multiples of 256, K a multiple of 64 bytes");
+    if (((uintptr_t)A | (uintptr_t)B | (uintptr_t)C) & 15) return refuse(ACC950_UNSUPPORTED, "the phase probe needs 16-byte aligned operands");
+    // (32-bit offsets inside a tile, as the product's own check has them)
+    if ((int64_t)256 * N * 4 >= (1ll << 32) || (int64_t)256 * K * es >= (1ll << 31) || (int64_t)bk * N * es >= (1ll << 31))
+        return refuse(ACC950_UNSUPPORTED, "the phase probe's tiles use 32-bit offsets: rows too long");
+    GemmArgs g{};
+    g.A = A; g.B = B; g.C = C; g.M = M; g.N = N; g.K = K;
+    g.a_rs = K; g.a_cs = 1; g.b_rs = N; g.b_cs = 1; g.c_rs = N; g.c_cs = 1;
+    g.in_type = in_type; g.out_type = out_type;
+    g.prologue = PRO_SET0; g.epilogue = EPI_RELU;
+    g.batch = 1;
+    // one record of four stamps per tile the launcher walks: its own count of tiles
+    LaunchGeom geom{};
+    auto launch = [&](bool dry) {
+        return in_type == T_I8 ? launch_mfma_timed_i8(g, nullptr, &geom, dry)
+               : in_type == T_BF16 ? launch_mfma_timed_bf16(g, nullptr, &geom, dry) : launch_mfma_timed_f16(g, nullptr, &geom, dry);
+    };
+    const int tiles = (M / 256) * (N / 256);
+    hipError_t e = hipMalloc((void**)&g.stamps, (size_t)tiles * 8 * sizeof(unsigned long long));
+    if (e != hipSuccess) return refuse(ACC950_HIP_ERROR, hipGetErrorString(e));
+    std::vector<unsigned long long> h((size_t)tiles * 8);
+    const int reps = 20; // the last launch is the one read back; the others settle the clocks
+    for (int i = 0; i < reps && e == hipSuccess; ++i) e = launch(false);
+    if (e == hipSuccess) e = hipDeviceSynchronize();
+    if (e == hipSuccess) e = hipMemcpy(h.data(), g.stamps, h.size() * sizeof(unsigned long long), hipMemcpyDeviceToHost);
+    hipError_t e2 = hipFree(g.stamps);
+    if (e != hipSuccess) return refuse(ACC950_HIP_ERROR, hipGetErrorString(e));
+    if (e2 != hipSuccess) return refuse(ACC950_HIP_ERROR, hipGetErrorString(e2));
+    // per phase: average wall time (100 MHz counter) and average shader cycles over the workgroups
+    unsigned long long first = ~0ull, last = 0;
+    double ns[3] = {0, 0, 0}, cyc[3] = {0, 0, 0};
+    for (int t = 0; t < tiles; ++t) {
+        const unsigned long long* w = &h[(size_t)t * 8];
+        first = w[1] < first ? w[1] : first;
+        last = w[7] > last ? w[7] : last;
+        for (int q = 0; q < 3; ++q) {
+            ns[q] += (double)(w[(q + 1) * 2 + 1] - w[q * 2 + 1]) * 10.0;
+            cyc[q] += (double)(w[(q + 1) * 2] - w[q * 2]);
+        }
+    }
+    for (int q = 0; q < 3; ++q) {
+        out[q] = ns[q] / tiles;                       // prologue, main loop, write-back [ns]
+        out[3 + q] = ns[q] > 0 ? cyc[q] / ns[q] : 0;  // shader clock in that phase [GHz]
+    }
+    out[6] = (double)(last - first) * 10.0;           // first workgroup start to last workgroup end [ns]
+    // MFMA pipe occupancy of the main loop: per SIMD, 512 MFMA cycles per 32 bytes of K (two waves x 8 MFMAs of 32 cycles,
+    // or one wave x 32 MFMAs of 16 cycles)
+    const double mfma_cycles = 2.0 * 8.0 * 32.0 * ((double)K * es / 32.0);
+    out[7] = cyc[1] > 0 ? mfma_cycles / (cyc[1] / tiles) : 0;
+    t_probe_error.clear();
+    return ACC950_OK;
 }
 
 } // extern "C"

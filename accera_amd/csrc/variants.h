@@ -26,11 +26,6 @@ const MfmaVariant* mfma_variants_bf16(int* count);
 const MfmaVariant* mfma_variants_i8(int* count);
 const MfmaVariant* mfma_variants_f32(int* count); // (32x32-shape entries only; the others have no launcher)
 
-// timed build of the 256x256 ping-pong kernel (row-major B, full tiles only)
-hipError_t launch_mfma_timed_f16(const GemmArgs& a, hipStream_t stream, LaunchGeom* geom, bool dry_run);
-hipError_t launch_mfma_timed_bf16(const GemmArgs& a, hipStream_t stream, LaunchGeom* geom, bool dry_run);
-hipError_t launch_mfma_timed_i8(const GemmArgs& a, hipStream_t stream, LaunchGeom* geom, bool dry_run);
-
 // second step of a K split of the MFMA kernels (gemm_splitk.hip)
 hipError_t launch_splitk_reduce(const GemmArgs& g, const void* ws, int splits, hipStream_t stream);
 

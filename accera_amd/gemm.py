@@ -73,6 +73,10 @@ class GemmCall:
         _lib.check(rc)
         self._handle = handle.value
         self._launch, self._unbind = L.acc950_launch, L.acc950_unbind
+        # what the library bound for this very call (its ops and pointers): kernel variant and number of K slices
+        v, ks = ctypes.c_int(), ctypes.c_int()
+        _lib.check(L.acc950_bound_choice(self._handle, ctypes.byref(v), ctypes.byref(ks)))
+        self.chosen = (v.value, ks.value)
 
     def __call__(self):
         rc = self._launch(self._handle)

@@ -792,15 +792,19 @@ class Package:
                 "    return rc;", "}", ""]
         return "\n".join(lines)
 
-    def build(self, name, format=None, mode=None, platform=None, tolerance=1e-5, output_dir=None, gpu_records=True, **_):
+    def build(self, name, format=None, mode=None, platform=None, tolerance=1e-5, output_dir=None, gpu_records=False, **_):
         """Emit `<output_dir>/<name>.hat` and `<name>.so` (HAT_DYNAMIC).  Returns the list of
-        files written (Package.py:551-788 returns the same kind of list).
+        files written (Package.py:551-788 returns the same kind of list): the .hat, the .so, and -- when the package
+        holds functions of GPU-target plans and gpu_records is False -- `<name>_gpu.hat` as a third entry.
 
-        gpu_records: functions added from a plan for a GPU target get the records the reference writes for such targets
-        (Package.py:714-743): `runtime = "ROCM"` and `launches = "<fn>__gpu__"` on the function and a
-        `[device_functions.<fn>__gpu__]` table with its `launch_parameters`, `dynamic_shared_mem_bytes` and `provider`.
-        Functions of HOST-target plans (the quick-start form) never do.  The host symbol `<fn>` takes host pointers
-        either way; False leaves the GPU records out altogether (a plain host-convention package)."""
+        `<name>.hat` is by default a plain host-convention package: every function is a cdecl symbol of `<name>.so` that
+        takes host pointers, with nothing a stock loader would hand to a run-time compiler (hatlib compiles the `provider`
+        of a function that `launches` a device function, /root/reference/accera/python/accera/Package.py:714-743).  The
+        records the reference writes for GPU targets -- `runtime = "ROCM"` and `launches = "<fn>__gpu__"` on the function,
+        a `[device_functions.<fn>__gpu__]` table with `launch_parameters`, `dynamic_shared_mem_bytes` and `provider` --
+        go into the sibling `<name>_gpu.hat` over the same library, for loaders that know the provider is prebuilt
+        (accera_amd.hat does).  gpu_records=True puts them into `<name>.hat` itself instead and writes no sibling.
+        Functions of HOST-target plans (the quick-start form) never carry them."""
         fmt = format or Package.Format.DEFAULT
         if not (fmt & Package.Format.HAT_DYNAMIC):
             raise NotImplementedError("only Package.Format.HAT_DYNAMIC is produced by this build")
@@ -818,6 +822,26 @@ class Package:
                "-laccera_mi355x", f"-Wl,-rpath,$ORIGIN/{rel}", f"-Wl,-rpath,{_lib.LIB_DIR}"]
         subprocess.check_call(cmd)
 
+        required_gpu = {"runtime": "ROCM", "model": "AMD MI355X", "instruction_set_version": "gfx950"}
+        compiled_with = {"compiler": "hipcc (kernels), gcc (entry points)", "flags": "--offload-arch=gfx950 -O3",
+                         "libraries": ["libaccera_mi355x.so"]}
+
+        def write(path, with_gpu_records):
+            functions, device_functions = self._records(with_gpu_records)
+            _hat.write_hat(path, name, functions, link_target=f"{name}.so", device_functions=device_functions,
+                           author=self._description.get("author", ""), version=self._description.get("version", ""),
+                           license_url=self._description.get("license", ""), required_gpu=required_gpu, compiled_with=compiled_with)
+
+        write(hat_path, gpu_records)
+        files = [hat_path, so_path]
+        if not gpu_records and any(f["spec"].gpu_target for f in self._functions):
+            gpu_hat_path = os.path.join(output_dir, f"{name}_gpu.hat")
+            write(gpu_hat_path, True)
+            files.append(gpu_hat_path)
+        return files
+
+    def _records(self, gpu_records):
+        """(functions, device_functions) of the .hat; gpu_records: with the GPU-target records of Package.py:714-743."""
         functions, device_functions = [], []
         for f in self._functions:
             s = f["spec"]
@@ -849,10 +873,4 @@ class Package:
                     dynamic_shared_mem_bytes=lds, provider=os.path.basename(_lib.LIB_PATH), runtime="ROCM",
                     auxiliary={"accera_mi355x": {"kernel": _lib.variant_name(variant), "entry": f"{f['name']}__device"}}))
             functions.append(fn)
-        _hat.write_hat(hat_path, name, functions, link_target=f"{name}.so", device_functions=device_functions,
-                       author=self._description.get("author", ""), version=self._description.get("version", ""),
-                       license_url=self._description.get("license", ""),
-                       required_gpu={"runtime": "ROCM", "model": "AMD MI355X", "instruction_set_version": "gfx950"},
-                       compiled_with={"compiler": "hipcc (kernels), gcc (entry points)", "flags": "--offload-arch=gfx950 -O3",
-                                      "libraries": ["libaccera_mi355x.so"]})
-        return [hat_path, so_path]
+        return functions, device_functions

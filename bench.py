@@ -1,14 +1,15 @@
 #!/usr/bin/env python3
 """Benchmark of the matmul + fused-ReLU hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c2] [--no-cpu] [--only] [--all]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c2] [--no-cpu] [--only]
 
 A "step" is one GEMM+ReLU launch on device-resident synthetic inputs.  The default
 workload is the configuration the headline metric is quoted on: fp16 inputs, fp32
 accumulate / output, M=N=K=4096, C = max(A.B, 0).  The metric also names the int8 GEMM and
-the skinny decode GEMM, so the default run measures those two as well, the same way, and
-reports them under "other_configs", each with its own roofline block (`--only` leaves them
-out).  Before the W untimed warm-up steps of a configuration its kernel is launched for
+the skinny decode GEMM, and the benchmark has two more configurations (the fp32 quick-start
+problem and the bf16 FFN GEMM), so the default run measures all four others as well, the same
+way, and reports them under "other_configs", each with its own roofline block (`--only`
+leaves them out).  Before the W untimed warm-up steps of a configuration its kernel is launched for
 SETTLE_MS of wall time (reported as settle_ms): after idling the engine clock takes some tens
 of milliseconds of load to settle, whatever W is.  One JSON line is printed with
   value         whole-job TFLOP/s (2*M*N*K per step, the formula of the reference's
@@ -18,7 +19,7 @@ of milliseconds of load to settle, whatever W is.  One JSON line is printed with
   cpu_baseline  the CPU oracle (a restatement of the reference's HOST schedule, not an
                 Accera-generated package) timed on this box's host cores
 
-`--all` measures all five BASELINE configurations.
+(`--all` is accepted and means the default: all five configurations.)
 """
 import argparse
 import json
@@ -228,14 +229,14 @@ def machine_ceiling(c):
         bufs = [torch.empty(nbytes, dtype=torch.uint8, device="cuda").fill_(i + 1) for i in range(8)]
         out = torch.zeros(1, dtype=torch.int32, device="cuda")
         stream = torch.cuda.current_stream()
-        L = _lib.lib()
+        L = _lib.probes()
         for i in range(8):
-            _lib.check(L.acc950_stream_read_probe(bufs[i].data_ptr(), nbytes, out.data_ptr(), stream.cuda_stream))
+            _lib.check_probe(L.acc950_stream_read_probe(bufs[i].data_ptr(), nbytes, out.data_ptr(), stream.cuda_stream))
         torch.cuda.synchronize()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record(stream)
         for i in range(80):
-            _lib.check(L.acc950_stream_read_probe(bufs[i % 8].data_ptr(), nbytes, out.data_ptr(), stream.cuda_stream))
+            _lib.check_probe(L.acc950_stream_read_probe(bufs[i % 8].data_ptr(), nbytes, out.data_ptr(), stream.cuda_stream))
         e1.record(stream)
         torch.cuda.synchronize()
         return {"plain_streaming_read_same_bytes": round(nbytes / (e0.elapsed_time(e1) * 1e-3 / 80) / 1e9, 1), "unit": "GB/s"}
@@ -291,8 +292,8 @@ def main():
     ap.add_argument("--variant", type=int, default=-1)
     ap.add_argument("--k-splits", type=int, default=0)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", action="store_true", help="measure --config alone (default: c4 and c5 ride along with c2)")
-    ap.add_argument("--all", action="store_true", help="measure all five BASELINE configurations")
+    ap.add_argument("--only", action="store_true", help="measure --config alone (default: the four other configurations ride along)")
+    ap.add_argument("--all", action="store_true", help="all five BASELINE configurations (the default)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs on ONE GPU only (no collectives, no sharding); run with --gpus 1", file=sys.stderr)
@@ -308,7 +309,7 @@ def main():
     c = CONFIGS[args.config]
     # plain copy of known size: the reference point for scaling profiler byte counters
     probe = torch.empty(2, 64 << 20, dtype=torch.uint8, device="cuda")
-    _lib.check(_lib.lib().acc950_copy_probe(probe[1].data_ptr(), probe[0].data_ptr(), 64 << 20, torch.cuda.current_stream().cuda_stream))
+    _lib.check_probe(_lib.probes().acc950_copy_probe(probe[1].data_ptr(), probe[0].data_ptr(), 64 << 20, torch.cuda.current_stream().cuda_stream))
     torch.cuda.synchronize()
     del probe
     m = measure(args.config, args.steps, args.warmup, args.variant, args.k_splits)
@@ -332,9 +333,9 @@ def main():
         # bounded sample: about 10-30 s of single-core work spread over the host cores
         rows = {"c2": None, "c4": 2048, "c3": None, "c1": None, "c5": None}[args.config]
         out["cpu_baseline"] = cpu_baseline(c, threads, rows)
-    # the rest of the metric: int8 GEMM (TOP/s against the int8 MFMA peak) and the skinny decode GEMM (HBM GB/s)
-    others = [n for n in sorted(CONFIGS) if n != args.config] if args.all else \
-        ([] if args.only or args.variant >= 0 or args.k_splits else [n for n in ("c4", "c5") if n != args.config])
+    # the rest of the metric -- int8 GEMM (TOP/s against the int8 MFMA peak), skinny decode GEMM (HBM GB/s) -- and the two
+    # remaining configurations of the benchmark (bf16 FFN GEMM, fp32 quick-start problem)
+    others = [] if args.only or args.variant >= 0 or args.k_splits else [n for n in ("c4", "c5", "c3", "c1") if n != args.config]
     if others:
         out["other_configs"] = [measure(n, args.steps, args.warmup) for n in others]
     print(json.dumps(out), flush=True)

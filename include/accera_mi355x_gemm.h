@@ -134,7 +134,9 @@ int acc950_gemm_ops_host(int in_type, int out_type, int M, int N, int K,
  * ACC950_STATIC_WORKSPACE_BYTES inside the library's device image (each GPU the library runs on holds its own
  * copy until the process ends) instead of a per-stream allocation.  The call makes no hipMalloc / hipFree and no
  * other allocating call; a skinny problem whose workspace would not fit returns ACC950_UNSUPPORTED and runs nothing
- * (8 x 11008 x 4096 needs 2.7 MiB), an MFMA problem whose slices would not fit runs unsplit.  All calls on one GPU share that array: calls that overlap on a GPU (different
+ * (8 x 11008 x 4096 needs 2.7 MiB); an MFMA problem is split into as many slices as fit the array (the kernel is
+ * chosen for that number), so its sums can be added in a different order than acc950_gemm_ops adds them -- the
+ * results are the same bits only when the allocating entry point's split fits the array too.  All calls on one GPU share that array: calls that overlap on a GPU (different
  * streams, different host threads) race on it -- keep them on one stream or use acc950_gemm_ops.  The kernels leave
  * the counters at zero, which is how the array starts.  Launch each kernel once outside a capture first: the first
  * launch of a kernel loads its code and may raise its LDS limit.
@@ -221,6 +223,36 @@ int acc950_launch_geometry(int in_type, int out_type, int M, int N, int K,
 int acc950_num_variants(void);
 int acc950_num_skinny_variants(void);
 int acc950_variant_name(int variant, char* buf, size_t buf_len);
+
+/* ---- bookkeeping of the library itself (for tests and long-running hosts; no counterpart in the reference) ---- */
+
+/*
+ * The K-split workspace the skinny kernels would use for a launch on `stream` of the current device
+ * (partial sums and arrival counters; one workspace per device and stream, so that launches
+ * on different streams never share one).  Allocates it at its smallest size if the stream has
+ * none yet.  DEVICE addresses, for comparison only.
+ */
+int acc950_workspace_probe(void* stream, void** partial_sums, void** counters);
+
+/* Number of device allocations (hipMalloc) the GEMM entry points of this process have made so far: K-split
+ * workspaces and the device buffers of the host-pointer path.  A test of an entry point that must not allocate
+ * reads it before and after. */
+int acc950_allocation_probe(unsigned long long* count);
+
+/*
+ * Frees every K-split workspace the allocating entry points have made on the current device (all streams), the blocks
+ * they have outgrown included, after waiting for the device to go idle.  The next launch that needs a workspace
+ * allocates a new one.  For programs that create and destroy streams or sweep over growing problems; a workspace
+ * otherwise stays with its (device, stream) pair until the process ends (at least 4 MiB + 16 KiB per pair).  Must not
+ * run while another thread launches on the device.  No counterpart in the reference, whose functions own no device state.
+ */
+int acc950_release_workspaces(void);
+
+/*
+ * What a bound call (acc950_bind) runs: the kernel variant chosen and the number of K slices (1: no split).  The
+ * launch-geometry query above answers for the plain product; this answers for the call's own ops and pointers.
+ */
+int acc950_bound_choice(int handle, int* variant, int* k_splits);
 
 /* Text of the last error on the calling thread ("" if none). */
 const char* acc950_last_error(void);

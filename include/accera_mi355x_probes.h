@@ -1,10 +1,10 @@
 /*
- * accera_mi355x_probes.h -- measurement aids of libaccera_mi355x.so.
+ * accera_mi355x_probes.h -- measurement aids, exported by libaccera_mi355x_probes.so (a library of its own:
+ * the product library libaccera_mi355x.so holds none of them, nor the timed kernel builds behind them).
  *
  * Not part of the product ABI (that is accera_mi355x_gemm.h): nothing here computes a result a
  * caller of the library needs.  The benchmark and the tests use these entry points to tell what
- * the GPU at hand sustains, to scale profiler byte counters, and to look at the library's own
- * bookkeeping.  None has a counterpart in the reference, whose harness times whole package
+ * the GPU at hand sustains and to scale profiler byte counters.  None has a counterpart in the reference, whose harness times whole package
  * calls (/root/reference/tools/benchmarkers/accera_gemm.py:584-657).
  */
 #ifndef ACCERA_MI355X_PROBES_H
@@ -33,7 +33,8 @@ extern "C" {
  * for large aligned problems (four waves with the hand-laid K loop when K has at least four
  * K tiles of 64 bytes, else the eight-wave ping-pong form) that reads the shader-clock counter
  * and the constant 100 MHz counter at four points in every workgroup, on dense row-major
- * DEVICE operands (M, N multiples of 256, SET-0 prologue, ReLU epilogue), synchronously.
+ * DEVICE operands (M, N multiples of 256, K a multiple of 64 bytes, 16-byte aligned pointers; SET-0 prologue, ReLU
+ * epilogue), synchronously; anything else is refused with ACC950_UNSUPPORTED before anything is launched.
  * out[0..2] = average time of prologue / main loop / write-back in ns, out[3..5] = shader
  * clock in GHz during each phase, out[6] = first workgroup start to last workgroup end in
  * ns, out[7] = fraction of the main loop's cycles the MFMA pipe is busy (the cycles its
@@ -51,18 +52,8 @@ int acc950_mfma_phase_probe(int in_type, int out_type, int M, int N, int K, cons
 int acc950_copy_probe(void* dst, const void* src, size_t bytes, void* stream);
 int acc950_stream_read_probe(const void* src, size_t bytes, void* scratch4, void* stream);
 
-/*
- * The K-split workspace the skinny kernels would use for a launch on `stream` of the current device
- * (partial sums and arrival counters; one workspace per device and stream, so that launches
- * on different streams never share one).  Allocates it at its smallest size if the stream has
- * none yet.  DEVICE addresses, for comparison only.
- */
-int acc950_workspace_probe(void* stream, void** partial_sums, void** counters);
-
-/* Number of device allocations (hipMalloc) the GEMM entry points of this process have made so far: K-split
- * workspaces and the device buffers of the host-pointer path.  A test of an entry point that must not allocate
- * reads it before and after. */
-int acc950_allocation_probe(unsigned long long* count);
+/* Why acc950_mfma_phase_probe refused its last call on this thread (the product library's acc950_last_error knows nothing of it). */
+const char* acc950_probes_last_error(void);
 
 #if defined(__cplusplus)
 }

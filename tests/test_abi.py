@@ -21,10 +21,34 @@ def test_every_declared_symbol_is_exported():
     names = _declared()
     assert len(names) >= 9 and set(_lib.EXPORTS) == set(names)
     L = ctypes.CDLL(_lib.LIB_PATH)
+    for n in names:
+        assert getattr(L, n) is not None, n
+    # the measurement aids are a library of their own; the product library holds none of them
     probes = _declared("accera_mi355x_probes.h")
     assert set(_lib.PROBE_EXPORTS) == set(probes) and not set(probes) & set(names)
-    for n in names + probes:
-        assert getattr(L, n) is not None, n
+    P = ctypes.CDLL(_lib.PROBES_LIB_PATH)
+    for n in probes:
+        assert getattr(P, n) is not None, n
+        assert not hasattr(L, n), f"{n} belongs in the probes library only"
+
+
+def test_phase_probe_refuses_what_its_kernels_do_not_take_before_launching():
+    """The timed kernels take whole 256x256 tiles of dense, aligned operands only; the probe says so itself and runs nothing
+    (no GPU is needed to be refused)."""
+    P = _lib.probes()
+    out = (ctypes.c_double * 8)()
+    ok_ptrs = (0x10000, 0x20000, 0x30000)
+    for M, N, K in ((300, 512, 512), (512, 300, 512), (512, 512, 100), (128, 512, 512), (512, 512, 0)):
+        rc = P.acc950_mfma_phase_probe(_lib.F16, _lib.F32, M, N, K, *ok_ptrs, out)
+        assert rc == _lib.UNSUPPORTED and b"multiples of 256" in P.acc950_probes_last_error(), (M, N, K)
+    assert P.acc950_mfma_phase_probe(_lib.I8, _lib.I32, 512, 512, 96, *ok_ptrs, out) == _lib.UNSUPPORTED          # K of 64 bytes
+    assert P.acc950_mfma_phase_probe(_lib.F16, _lib.F32, 512, 512, 512, 0x10008, 0x20000, 0x30000, out) == _lib.UNSUPPORTED
+    assert P.acc950_mfma_phase_probe(_lib.F32, _lib.F32, 512, 512, 512, *ok_ptrs, out) == _lib.UNSUPPORTED
+    assert P.acc950_mfma_phase_probe(_lib.F16, _lib.I32, 512, 512, 512, *ok_ptrs, out) == _lib.INVALID_ARGUMENT
+    assert P.acc950_mfma_phase_probe(_lib.F16, _lib.F32, 512, 512, 512, None, 0x20000, 0x30000, out) == _lib.INVALID_ARGUMENT
+    with pytest.raises(_lib.Acc950Error) as e:
+        _lib.mfma_phase_probe(_lib.F16, _lib.F32, 300, 512, 512, *ok_ptrs)
+    assert e.value.code == _lib.UNSUPPORTED and "multiples of 256" in str(e.value)
 
 
 def test_variant_table_is_described():
@@ -107,8 +131,12 @@ def test_bound_call_handles_without_launching():
             _lib.PROLOGUE_SET0, 0.0, _lib.EPILOGUE_RELU, 0.0, _lib.VARIANT_AUTO, 0, None)
     assert L.acc950_bind(*args, ctypes.byref(h)) == _lib.OK and h.value >= 0
     first = h.value
+    v, ks = ctypes.c_int(-5), ctypes.c_int(-5)
+    assert L.acc950_bound_choice(first, ctypes.byref(v), ctypes.byref(ks)) == _lib.OK
+    assert "mfma" in _lib.variant_name(v.value) and ks.value >= 1
     assert L.acc950_unbind(first) == _lib.OK
     assert L.acc950_unbind(first) == _lib.INVALID_ARGUMENT and L.acc950_launch(first) == _lib.INVALID_ARGUMENT
+    assert L.acc950_bound_choice(first, ctypes.byref(v), ctypes.byref(ks)) == _lib.INVALID_ARGUMENT
     assert L.acc950_bind(*args, ctypes.byref(h)) == _lib.OK and h.value == first   # slot reused
     assert L.acc950_unbind(first) == _lib.OK
     bad = list(args)

@@ -897,6 +897,18 @@ def test_skinny_workspaces_are_per_stream():
     for i in range(2):
         want = ora.gemm_relu_exact(A, Bs[i], out_zeros(M, N, "f16"), "f16", "f16", ora.PRO_SET0, ora.EPI_RELU)
         assert_matches(to_host(dCs[i], "f16"), want, "f16", K)
+    # the workspaces can be handed back (a host that creates and destroys streams): the next launches make new ones
+    before = _lib.allocation_probe()
+    _lib.release_workspaces()
+    for d in dCs:
+        d.fill_(5)
+    for c in calls:
+        c()
+    torch.cuda.synchronize()
+    assert _lib.allocation_probe() >= before + 2
+    for i in range(2):
+        want = ora.gemm_relu_exact(A, Bs[i], out_zeros(M, N, "f16"), "f16", "f16", ora.PRO_SET0, ora.EPI_RELU)
+        assert_matches(to_host(dCs[i], "f16"), want, "f16", K)
 
 
 @pytest.mark.parametrize("in_type,out_type", [("f16", "f32"), ("f16", "f16"), ("bf16", "bf16"), ("i8", "i32"), ("i8", "i16")])

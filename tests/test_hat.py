@@ -54,8 +54,11 @@ def _native_shape(in_t, wide=False):
     return S.M32xN32xK16_B1 if wide else S.M16xN16xK32_B1
 
 
-def _gpu_plan_package(tmp, in_t, out_t, M, N, K, b_layout=None, epilogue=None, base_name="matmul_relu", mma_shape=None, **build_args):
-    """mfma_tests.py:359-432 (`_matmul_relu`): tensorized plan with SET prologue and ReLU epilogue."""
+def _gpu_plan_package(tmp, in_t, out_t, M, N, K, b_layout=None, epilogue=None, base_name="matmul_relu", mma_shape=None, which="gpu",
+                      **build_args):
+    """mfma_tests.py:359-432 (`_matmul_relu`): tensorized plan with SET prologue and ReLU epilogue.  Returns
+    ((hat, so), name): the .hat with the GPU-target records (`<name>_gpu.hat` of a default build), or with which="host"
+    the plain host-convention `<name>.hat`."""
     target = acc.Target(acc.Target.Model.AMD_MI355X)
     A = acc.Array(role=acc.Role.INPUT, element_type=in_t, shape=(M, K))
     B = acc.Array(role=acc.Role.INPUT, element_type=in_t, shape=(K, N), layout=b_layout or acc.Array.Layout.FIRST_MAJOR)
@@ -79,7 +82,8 @@ def _gpu_plan_package(tmp, in_t, out_t, M, N, K, b_layout=None, epilogue=None, b
     package = acc.Package()
     name = package.add(plan, args=(A, B, C), base_name=base_name)
     files = package.build(name="gpu_pkg", output_dir=str(tmp), **build_args)
-    return files, name
+    hat_path = files[2] if which == "gpu" and len(files) > 2 else files[0]
+    return (hat_path, files[1]), name
 
 
 def test_quickstart_builds_a_valid_hat(tmp_path):
@@ -200,11 +204,43 @@ def test_gpu_target_functions_carry_the_reference_device_records(tmp_path):
     # the loader pairs them
     _, functions = hat.load(hat_path)
     assert functions[name].launches == name + "__gpu__" and functions[name].device_record == dev
-    # gpu_records=False: the same function as a plain host-convention record
-    (hat2, _), name2 = _gpu_plan_package(tmp_path / "plain", acc.ScalarType.float16, acc.ScalarType.float32, 4096, 4096, 4096,
-                                         gpu_records=False)
-    doc2 = hat.parse(hat2)
-    assert name2 == name and "device_functions" not in doc2 and "launches" not in doc2["functions"][name]
+    # gpu_records=True: the same records in `<name>.hat` itself, and no sibling file
+    target = acc.Target(acc.Target.Model.AMD_MI355X)
+    (hat3, so3), name3 = _gpu_plan_package(tmp_path / "inline", acc.ScalarType.float16, acc.ScalarType.float32, 4096, 4096, 4096,
+                                           gpu_records=True)
+    assert os.path.basename(hat3) == "gpu_pkg.hat" and not os.path.exists(os.path.join(os.path.dirname(hat3), "gpu_pkg_gpu.hat"))
+    doc3 = hat.parse(hat3)
+    assert name3 == name and doc3["device_functions"][name + "__gpu__"] == dev and doc3["functions"][name]["launches"] == name + "__gpu__"
+
+
+def test_default_package_is_host_convention_with_nothing_for_a_run_time_compiler(tmp_path):
+    """What a stock loader does with a function that `launches` something is compile its `provider`
+    (Package.py:714-743); the kernels here are prebuilt, so `<name>.hat` of a default build carries no such record:
+    every function is a plain cdecl symbol on host pointers, and the GPU-target records sit in `<name>_gpu.hat`."""
+    import ctypes
+    (host_hat, so_path), name = _gpu_plan_package(tmp_path, acc.ScalarType.float16, acc.ScalarType.float32, 1024, 1024, 1024, which="host")
+    assert os.path.basename(host_hat) == "gpu_pkg.hat"
+    text = open(host_hat).read()
+    assert "device_functions" not in text and "launches" not in text and "provider" not in text
+    doc = hat.parse(host_hat)
+    fn = doc["functions"][name]
+    assert fn["calling_convention"] == "cdecl" and "runtime" not in fn
+    assert doc["dependencies"]["link_target"] == "gpu_pkg.so"
+    # the launch geometry is still on record, as auxiliary data a stock loader ignores
+    assert fn["auxiliary"]["accera_mi355x"]["device_entry"] == name + "__device"
+    # the sibling with the GPU records names the same library and the same function
+    gpu_hat = os.path.join(os.path.dirname(host_hat), "gpu_pkg_gpu.hat")
+    gdoc = hat.parse(gpu_hat)
+    assert gdoc["dependencies"]["link_target"] == "gpu_pkg.so" and gdoc["functions"][name]["launches"] == name + "__gpu__"
+    assert gdoc["functions"][name]["arguments"] == fn["arguments"]
+    assert getattr(ctypes.CDLL(so_path), name) is not None
+    # the loader gives a host-pointer callable for the default file and pairs the device entry for the sibling
+    _, host_functions = hat.load(host_hat)
+    _, gpu_functions = hat.load(gpu_hat)
+    assert host_functions[name].device_record is None and gpu_functions[name].device_record is not None
+    # a package of HOST-target plans only has no sibling
+    files = _quickstart_package(tmp_path / "host_only")
+    assert len(files) == 2
 
 
 def test_tensor_core_table_and_mma_shape_validation(tmp_path):

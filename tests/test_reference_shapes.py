@@ -50,14 +50,16 @@ def test_every_shape_of_the_reference_sweep_lists(in_type, out_type):
         C0 = draw(M, N, "i8" if out_type == "i32" else out_type, False).to(tdt[out_type])
         C = C0.clone()
         prologue = ora.PRO_SET0 if beta == 0 else ora.PRO_NONE
-        sa, sb = (A.stride(0), A.stride(1)), (B.stride(0), B.stride(1))
-        grid, block, lds, v = _lib.launch_geometry(ora.TYPE_IDS[in_type], ora.TYPE_IDS[out_type], M, N, K, sa, sb, (N, 1))
+        # the kernel and the K slices bound for this very call: its prologue (beta = 1 reads C) and its pointers
+        call = acc.GemmCall(A, B, C, prologue=prologue, epilogue=ora.EPI_RELU)
+        v, slices = call.chosen
         name = _lib.variant_name(v)
         assert v != _lib.VARIANT_GENERIC, (M, N, K, ta, tb, name)
-        kind = "fp32 32x32 blocks" if v == _lib.VARIANT_F32_MFMA else "skinny" if "skinny" in name else ("any-alignment" if "any-alignment" in name else "mfma") + (", K split" if grid[2] > 1 else "")
+        split = slices > 1 and "skinny" not in name
+        kind = "fp32 32x32 blocks" if v == _lib.VARIANT_F32_MFMA else "skinny" if "skinny" in name else ("any-alignment" if "any-alignment" in name else "mfma") + (", K split" if split else "")
         kinds[kind] = kinds.get(kind, 0) + 1
-        print(n, (M, N, K, ta, tb, beta), name, "slices", grid[2], flush=True)
-        acc.gemm_relu(A, B, C, prologue=prologue, epilogue=ora.EPI_RELU)
+        print(n, (M, N, K, ta, tb, beta), name, "slices", slices, flush=True)
+        call()
         idx = np.arange(M) if M <= 48 else np.random.default_rng(n).choice(M, 24, replace=False)
         sel = torch.as_tensor(idx, device="cuda")
         torch.cuda.synchronize()
