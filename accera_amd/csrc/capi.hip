@@ -3,6 +3,7 @@
 #include "../../include/accera_mi355x_gemm.h"
 #include "common.h"
 #include "skinny.h"
+#include "host_path.h"
 #include <vector>
 #include "variants.h"
 
@@ -594,19 +595,6 @@ int run(const Problem& pb, const Choice& c, hipStream_t stream, LaunchGeom* geom
     return ACC950_OK;
 }
 
-// ---- device buffers of the host-pointer path (grow-only, one set per process) --------
-std::mutex g_host_mutex;
-struct DevBuf { void* p = nullptr; size_t bytes = 0; } g_dA, g_dB, g_dC;
-
-hipError_t reserve(DevBuf& b, size_t bytes)
-{
-    if (bytes <= b.bytes) return hipSuccess;
-    if (b.p) { hipError_t e = hipFree(b.p); if (e != hipSuccess) return e; b.p = nullptr; b.bytes = 0; }
-    hipError_t e = hipMalloc(&b.p, bytes);
-    if (e == hipSuccess) { b.bytes = bytes; ++g_device_allocations; }
-    return e;
-}
-
 size_t extent_elems(int rows, int cols, int64_t rs, int64_t cs)
 {
     if (rows <= 0 || cols <= 0) return 0;
@@ -858,21 +846,18 @@ int acc950_gemm_batched_host(int in_type, int out_type, int batch, int M, int N,
     const size_t c_bytes = (nb * c_bs + c_elems) * elem_size(out_type);
     const bool c_dense = c_elems == (size_t)M * (size_t)N && (batch == 1 || (size_t)c_bs == c_elems);
 
-    std::lock_guard<std::mutex> lock(g_host_mutex);
-    hipError_t e;
-    if ((e = reserve(g_dA, a_bytes ? a_bytes : 16)) != hipSuccess) return fail_hip(e, "hipMalloc(A)");
-    if ((e = reserve(g_dB, b_bytes ? b_bytes : 16)) != hipSuccess) return fail_hip(e, "hipMalloc(B)");
-    if ((e = reserve(g_dC, c_bytes)) != hipSuccess) return fail_hip(e, "hipMalloc(C)");
-    if (a_bytes && (e = hipMemcpy(g_dA.p, A, a_bytes, hipMemcpyHostToDevice)) != hipSuccess) return fail_hip(e, "copy A to device");
-    if (b_bytes && (e = hipMemcpy(g_dB.p, B, b_bytes, hipMemcpyHostToDevice)) != hipSuccess) return fail_hip(e, "copy B to device");
-    // C travels to the device when it is read (prologue NONE / SCALE), or when its extent has
-    // gaps that the copy back must not clobber
-    if (prologue != PRO_SET || !c_dense)
-        if ((e = hipMemcpy(g_dC.p, C, c_bytes, hipMemcpyHostToDevice)) != hipSuccess) return fail_hip(e, "copy C to device");
-    rc = acc950_gemm_batched(in_type, out_type, batch, M, N, K, g_dA.p, a_bs, a_rs, a_cs, g_dB.p, b_bs, b_rs, b_cs, g_dC.p, c_bs, c_rs,
-                             c_cs, prologue, prologue_arg, epilogue, epilogue_arg, variant, k_splits, nullptr);
-    if (rc) return rc;
-    if ((e = hipMemcpy(C, g_dC.p, c_bytes, hipMemcpyDeviceToHost)) != hipSuccess) return fail_hip(e, "copy C to host");
+    // Through pinned staging on a context of this call's own (host_path.hip): calls from different host threads do not
+    // wait for each other.
+    static const bool counted = (host_path_count_allocations(&g_device_allocations), true);
+    (void)counted;
+    HostOperands h{A, B, C, a_bytes, b_bytes, c_bytes, prologue != PRO_SET || !c_dense};
+    int status = ACC950_OK;
+    const hipError_t e = host_path_run(h, [&](void* dA, void* dB, void* dC, hipStream_t stream) {
+        return acc950_gemm_batched(in_type, out_type, batch, M, N, K, dA, a_bs, a_rs, a_cs, dB, b_bs, b_rs, b_cs, dC, c_bs, c_rs, c_cs,
+                                   prologue, prologue_arg, epilogue, epilogue_arg, variant, k_splits, stream);
+    }, &status);
+    if (status != ACC950_OK) return status; // (the launcher's own error text stands)
+    if (e != hipSuccess) return fail_hip(e, "host-pointer path (allocation or copy)");
     return ACC950_OK;
 }
 

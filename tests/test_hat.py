@@ -365,6 +365,42 @@ def test_readme_quickstart_end_to_end(tmp_path):
 
 
 @pytest.mark.gpu
+def test_package_functions_called_from_two_host_threads_at_once(tmp_path):
+    """A package function takes host arrays (README.md:124-130) and may be called from any thread.  Each call in flight has
+    its own device buffers, staging buffers and stream, so calls from two threads overlap; both must be right, call after
+    call, on operands large enough for several staging pieces and on an accumulating (C is read) problem."""
+    import threading
+    (hat_a, _), name_a = _gpu_plan_package(tmp_path / "a", acc.ScalarType.float16, acc.ScalarType.float32, 1024, 2048, 3072, which="host")
+    (hat_b, _), name_b = _gpu_plan_package(tmp_path / "b", acc.ScalarType.int8, acc.ScalarType.int32, 2048, 1024, 4096, which="host",
+                                           mma_shape=acc.MMAShape.M16xN16xK64_B1)
+    fa, fb = hat.load(hat_a)[1][name_a], hat.load(hat_b)[1][name_b]
+    rng = np.random.default_rng(5)
+    from tests.util import assert_matches, make_input
+    Aa, Ba = make_input(rng, (1024, 3072), "f16"), make_input(rng, (3072, 2048), "f16")
+    Ab, Bb = make_input(rng, (2048, 4096), "i8"), make_input(rng, (4096, 1024), "i8")
+    want_a = ora.gemm_relu_exact(Aa, Ba, None, "f16", "f32")
+    want_b = ora.gemm_relu_exact(Ab, Bb, None, "i8", "i32")
+    errors = []
+
+    def worker(f, A, B, want, out_t, K, reps):
+        try:
+            for _ in range(reps):
+                C = np.full(want.shape, 3, want.dtype)
+                f(A, B, C)
+                assert_matches(C, want, out_t, K)
+        except BaseException as e:  # (reported by the main thread)
+            errors.append(e)
+
+    threads = [threading.Thread(target=worker, args=(fa, Aa, Ba, want_a, "f32", 3072, 6)),
+               threading.Thread(target=worker, args=(fb, Ab, Bb, want_b, "i32", 4096, 6))]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors[0]
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("in_t,out_t,shape,b_layout", [
     (acc.ScalarType.float16, acc.ScalarType.float32, (256, 384, 512), None),
     (acc.ScalarType.bfloat16, acc.ScalarType.bfloat16, (256, 256, 192), acc.Array.Layout.LAST_MAJOR),
