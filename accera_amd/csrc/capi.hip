@@ -176,15 +176,17 @@ bool skinny_can_take(const Problem& pb, int sv)
 {
     const GemmArgs& g = pb.g;
     const SkinnyVariant& v = skinny_variant(sv);
-    if (g.in_type != T_F16 && g.in_type != T_BF16) return false;
-    if (g.M < 1 || g.M > v.max_m || g.N < 8 || g.K < v.k_step) return false;
+    if (g.in_type != T_F16 && g.in_type != T_BF16 && !(g.in_type == T_I8 && v.i8)) return false;
+    const int es = elem_size(g.in_type), vec = 16 / es; // elements per 16-byte piece
+    const int k_step = skinny_k_step(v, g.in_type);
+    if (g.M < 1 || g.M > v.max_m || g.N < vec || g.K < k_step) return false;
     if (g.a_cs != 1 || g.b_cs != 1 || g.c_cs != 1) return false;
-    if (g.N % 8 || g.K % v.k_step || g.b_rs % 8) return false;
-    if (g.a_rs % (v.mfma ? 8 : 2)) return false; // A pieces are fetched 16 (4) bytes at a time
+    if (g.N % vec || g.K % k_step || g.b_rs % vec) return false;
+    if (g.a_rs % (v.mfma ? vec : 2)) return false; // A pieces are fetched 16 (4) bytes at a time
     // per-lane offsets of the direct-to-LDS fills are 32-bit
-    if ((int64_t)g.K * g.b_rs * 2 >= (1ll << 32) || (int64_t)v.max_m * g.a_rs * 2 >= (1ll << 32)) return false;
+    if ((int64_t)g.K * g.b_rs * es >= (1ll << 32) || (int64_t)v.max_m * g.a_rs * es >= (1ll << 32)) return false;
     if (pb.have_pointers && (!aligned16(g.B) || (reinterpret_cast<uintptr_t>(g.A) & (v.mfma ? 15u : 3u)))) return false;
-    if (g.batch > 1 && (g.b_bs % 8 || g.a_bs % (v.mfma ? 8 : 2))) return false;
+    if (g.batch > 1 && (g.b_bs % vec || g.a_bs % (v.mfma ? vec : 2))) return false;
     return true;
 }
 
@@ -486,11 +488,11 @@ int choose(const Problem& pb, int variant, int k_splits, Choice* c, size_t max_s
     if (variant >= ACC950_VARIANT_SKINNY_BASE && variant < ACC950_VARIANT_SKINNY_BASE + skinny_num_variants()) {
         const int sv = variant - ACC950_VARIANT_SKINNY_BASE;
         if (!skinny_can_take(pb, sv))
-            return fail(ACC950_UNSUPPORTED, "skinny kernel needs 16-bit inputs, row-major A/B/C, N % 8 == 0, and M <= 32, K % 16 == 0 (MFMA family) "
-                                            "or M <= 8, K % 2 == 0 (dot-product family)");
+            return fail(ACC950_UNSUPPORTED, "skinny kernel needs row-major A/B/C, rows of B in whole 16-byte pieces, and M <= 32, K a multiple of 32 bytes, 8- or 16-bit inputs (MFMA family) "
+                                            "or M <= 8, K % 2 == 0, 16-bit inputs (dot-product family)");
         c->variant = variant;
         c->splits = k_splits > 0 ? k_splits : auto_skinny_splits(sv, pb.g);
-        const int max_splits = pb.g.K / skinny_variant(sv).k_step;
+        const int max_splits = pb.g.K / skinny_k_step(skinny_variant(sv), pb.g.in_type);
         if (c->splits > max_splits) c->splits = max_splits;
         return ACC950_OK;
     }
@@ -537,7 +539,7 @@ int run(const Problem& pb, const Choice& c, hipStream_t stream, LaunchGeom* geom
         const SkinnyVariant& skv = skinny_variant(sv);
         // (Which blocks those are follows B's address.  A query without pointers reports phase 0: no phase has more blocks,
         // so the grid it names is what launches or one workgroup more.)
-        if (skv.mfma && skv.cols == 64 && c.splits == 1 && (g.b_rs * 2) % 512 == 0 &&
+        if (skv.mfma && skv.cols == 64 && g.in_type != T_I8 && c.splits == 1 && (g.b_rs * 2) % 512 == 0 &&
             skinny_column_blocks(sv, g.N) >= 128 && skinny_column_blocks(sv, g.N) <= 200 && g.K >= 512 &&
             (g.batch <= 1 || (g.b_bs * 2) % 512 == 0))
             s.extra_phase = pb.have_pointers ? (int)((3u - (unsigned)(reinterpret_cast<uintptr_t>(g.B) >> 7)) & 3u) : 0;

@@ -304,6 +304,7 @@ hipError_t launch_skinny(int v, const SkinnyArgs& a, hipStream_t stream, LaunchG
 {
     if (v < 0 || v >= skinny_num_variants()) return hipErrorInvalidValue;
     const SkinnyVariant& s = skinny_variant(v);
+    if (a.in_type == T_I8) return s.i8 ? s.i8(a, stream, geom, dry_run) : hipErrorInvalidValue;
     return a.in_type == T_BF16 ? s.bf16(a, stream, geom, dry_run) : s.f16(a, stream, geom, dry_run);
 }
 

@@ -39,6 +39,7 @@
 //     to occupy the chip unless N is large.
 #include "common.h"
 #include "skinny.h"
+#include <type_traits>
 
 namespace acc950 {
 
@@ -46,12 +47,20 @@ namespace {
 
 typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 
-template <bool BF16, int CB, int WAVES, int DEPTH>
+// IN: T_F16, T_BF16 (16 k rows per step, v_mfma_f32_32x32x16) or T_I8 (32 k rows per step, v_mfma_i32_32x32x32_i8, sums
+// that wrap around like the reference's int32 accumulator: /root/reference/accera/acc-translate/src/Target/Cpp/CppPrinterUtils.h:342-360).
+// A step has the same bytes either way: a 64-column block of int8 is 32 k rows x 64 bytes where fp16 has 16 x 128.
+template <int IN, int CB, int WAVES, int DEPTH>
 __global__ void __launch_bounds__(WAVES * 64) gemm_skinny_mfma_kernel(SkinnyArgs p)
 {
     static_assert(CB == 64 || CB == 256, "column block of 64 or 256");
-    constexpr int KS = 16;                        // k rows per step
-    constexpr int RB = CB * 2;                    // bytes of one B row piece
+    constexpr bool I8 = IN == T_I8, BF16 = IN == T_BF16;
+    constexpr int ES = I8 ? 1 : 2;                // bytes per input element
+    constexpr int KS = 32 / ES;                   // k rows per step (32 bytes of K per row of A)
+    constexpr int RB = CB * ES;                   // bytes of one B row piece
+    using sum_t = std::conditional_t<I8, int, float>;
+    typedef sum_t sum4 __attribute__((ext_vector_type(4)));
+    typedef sum_t sum16 __attribute__((ext_vector_type(16)));
     constexpr int CPR = RB / 16;                  // 16-byte chunks per row piece
     constexpr int RPF = 64 / CPR;                 // rows per fill instruction (1 KB)
     constexpr int BFILLS = KS / RPF;              // B fills per step
@@ -65,9 +74,9 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_skinny_mfma_kernel(SkinnyArgs
     extern __shared__ __attribute__((aligned(1024))) char smem[];
     { // batched launch: blockIdx.z picks the problem (and its slice of the K-split workspace)
         const int64_t z = blockIdx.z;
-        p.A = (const char*)p.A + z * p.a_bs * 2;
-        p.B = (const char*)p.B + z * p.b_bs * 2;
-        p.C = (char*)p.C + z * p.c_bs * (p.out_type == T_F32 ? 4 : 2);
+        p.A = (const char*)p.A + z * p.a_bs * ES;
+        p.B = (const char*)p.B + z * p.b_bs * ES;
+        p.C = (char*)p.C + z * p.c_bs * elem_bytes(p.out_type);
         p.scratch += z * p.scratch_bs;
         p.counters += z * p.counter_bs;
     }
@@ -107,26 +116,28 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_skinny_mfma_kernel(SkinnyArgs
 
     // B fill number f puts rows f*RPF .. of the step at the same LDS rows (RB bytes each):
     // lane l lands at row f*RPF + l/CPR, chunk position l%CPR, and fetches the logical chunk
-    // position ^ 2*(row%4) (the four k rows of one transposing read go to different banks).
-    const int64_t row_bytes = p.b_rs * 2;
+    // position ^ swz(row): the k rows of one transposing read go to different banks (16-bit: four rows of 128 bytes and
+    // more, x 2*(row%4); 8-bit: eight rows, of which rows j and j+4 of a 64-byte pitch share their banks, x 2*(row/4%2)).
+    auto swz = [](int row) { return I8 && CB == 64 ? ((row >> 2) & 1) << 1 : I8 ? (row & 7) << 1 : (row & 3) << 1; };
+    const int64_t row_bytes = p.b_rs * ES;
     const int fh = lane / CPR, fpos = lane % CPR;
     unsigned boff[BFILLS];
 #pragma unroll
     for (int f = 0; f < BFILLS; ++f) {
         const int row = RPF * f + fh;
-        const int col = col_base + ((fpos ^ ((row & 3) << 1)) << 3);
-        boff[f] = (unsigned)((int64_t)row * row_bytes + (int64_t)(col < p.N ? col : 0) * 2); // outside N: any valid address
+        const int col = col_base + ((fpos ^ swz(row)) << 4) / ES;
+        boff[f] = (unsigned)((int64_t)row * row_bytes + (int64_t)(col < p.N ? col : 0) * ES); // outside N: any valid address
     }
     const int am = lane >> 1;
     const bool a_active = am < p.M;
     // the two 16-byte halves of a row swap places in rows 8-15 and 24-31, so that the 16 lanes of one
     // read phase (32-byte row pitch) spread over all banks
-    const unsigned aoff = (unsigned)((int64_t)(a_active ? am : 0) * p.a_rs * 2 + ((lane & 1) ^ ((am >> 3) & 1)) * 16);
+    const unsigned aoff = (unsigned)((int64_t)(a_active ? am : 0) * p.a_rs * ES + ((lane & 1) ^ ((am >> 3) & 1)) * 16);
 
     auto issue = [&](int it, int slot) { // it < my_steps
         const int s = s_begin + wave + it * WAVES;
         const char* bsrc = (const char*)p.B + (int64_t)s * KS * row_bytes;
-        const char* asrc = (const char*)p.A + (int64_t)s * KS * 2;
+        const char* asrc = (const char*)p.A + (int64_t)s * KS * ES;
         const unsigned dst = ring_addr + slot * SLOT_BYTES;
 #pragma unroll
         for (int f = 0; f < BFILLS; f += 2)
@@ -146,15 +157,22 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_skinny_mfma_kernel(SkinnyArgs
     for (int j = 0; j < JB; ++j)
 #pragma unroll
         for (int q = 0; q < 2; ++q) {
-            const int k = h * 8 + q * 4 + (i16 >> 2);
-            const int chunk = j * 4 + g * 2 + ((i16 & 3) >> 1);
-            roff[j][q] = (unsigned)(k * RB + ((chunk ^ ((k & 3) << 1)) << 4) + (i16 & 1) * 8);
+            if constexpr (I8) {
+                // ds_read_b64_tr_b8: lanes 2j, 2j+1 of a group of 16 point at k row j (2 x 8 bytes = 16 columns), lane i gets column i of those 8 rows
+                const int k = h * 16 + q * 8 + (i16 >> 1);
+                const int chunk = j * 2 + g;
+                roff[j][q] = (unsigned)(k * RB + ((chunk ^ swz(k)) << 4) + (i16 & 1) * 8);
+            } else {
+                const int k = h * 8 + q * 4 + (i16 >> 2);
+                const int chunk = j * 4 + g * 2 + ((i16 & 3) >> 1);
+                roff[j][q] = (unsigned)(k * RB + ((chunk ^ swz(k)) << 4) + (i16 & 1) * 8);
+            }
         }
     const unsigned aread = B_BYTES + (lane & 31) * 32 + (h ^ (((lane & 31) >> 3) & 1)) * 16;
 
-    f32x16 acc[JB];
+    sum16 acc[JB];
 #pragma unroll
-    for (int j = 0; j < JB; ++j) acc[j] = f32x16{};
+    for (int j = 0; j < JB; ++j) acc[j] = sum16{};
 
     auto consume = [&](int slot_idx, auto refill) {
         const char* slot = ring + slot_idx * SLOT_BYTES;
@@ -163,8 +181,9 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_skinny_mfma_kernel(SkinnyArgs
         for (int j = 0; j < JB; ++j)
 #pragma unroll
             for (int q = 0; q < 2; ++q) {
-                s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((ACC950_LDS s16x4*)(slot + roff[j][q]));
-                i32x2 w = __builtin_bit_cast(i32x2, v);
+                i32x2 w;
+                if constexpr (I8) w = __builtin_amdgcn_ds_read_tr8_b64_v2i32((ACC950_LDS i32x2*)(slot + roff[j][q]));
+                else w = __builtin_bit_cast(i32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((ACC950_LDS s16x4*)(slot + roff[j][q])));
                 bfrag[j][q * 2] = w[0];
                 bfrag[j][q * 2 + 1] = w[1];
             }
@@ -173,7 +192,9 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_skinny_mfma_kernel(SkinnyArgs
         refill();
 #pragma unroll
         for (int j = 0; j < JB; ++j) {
-            if constexpr (BF16)
+            if constexpr (I8)
+                acc[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bfrag[j], afrag, acc[j], 0, 0, 0);
+            else if constexpr (BF16)
                 acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, bfrag[j]), __builtin_bit_cast(bf16x8, afrag), acc[j], 0, 0, 0);
             else
                 acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, bfrag[j]), __builtin_bit_cast(f16x8, afrag), acc[j], 0, 0, 0);
@@ -205,32 +226,38 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_skinny_mfma_kernel(SkinnyArgs
     // accumulator layout (C^T block j): register r of lane l = column j*32 + (r/4)*8 + (l/32)*4 + r%4,
     // row l%32 of A.  Reorder through LDS to [row][256 columns].
     __syncthreads(); // every wave is done with its ring
-    float* red = (float*)smem; // [wave][M][CB]
+    sum_t* red = (sum_t*)smem; // [wave][M][CB]
     const int m = lane & 31;
     if (m < p.M) {
-        float* mine = red + ((size_t)wave * p.M + m) * CB + h * 4;
+        sum_t* mine = red + ((size_t)wave * p.M + m) * CB + h * 4;
 #pragma unroll
         for (int j = 0; j < JB; ++j)
 #pragma unroll
             for (int q = 0; q < 4; ++q)
-                *(f32x4*)(mine + j * 32 + q * 8) = f32x4{acc[j][q * 4], acc[j][q * 4 + 1], acc[j][q * 4 + 2], acc[j][q * 4 + 3]};
+                *(sum4*)(mine + j * 32 + q * 8) = sum4{acc[j][q * 4], acc[j][q * 4 + 1], acc[j][q * 4 + 2], acc[j][q * 4 + 3]};
     }
     __syncthreads();
 
-    const int groups = p.M * (CB / 4); // float4 groups of the workgroup's block
-    // four adjacent columns of one row: one 8- or 16-byte store when C allows it
-    const bool vec_ok = p.prologue != PRO_SET ? false
-                        : (p.out_type == T_F32 ? (p.c_rs % 4 == 0 && ((size_t)p.C & 15) == 0) : (p.c_rs % 4 == 0 && ((size_t)p.C & 7) == 0));
-    auto finish4 = [&](int grp, f32x4 s) {
+    const int groups = p.M * (CB / 4); // groups of four sums of the workgroup's block
+    // four adjacent columns of one row: one 4-, 8- or 16-byte store when C allows it
+    const int os = elem_bytes(p.out_type);
+    const bool vec_ok = p.prologue == PRO_SET && p.c_rs % 4 == 0 && ((size_t)p.C & (size_t)(4 * os - 1)) == 0;
+    auto finish4 = [&](int grp, sum4 s) {
         const int row = grp / (CB / 4), n = col_base + (grp % (CB / 4)) * 4;
         if (n >= p.N) return; // N is a multiple of 8: a group is entirely inside or outside
         const int64_t idx = (int64_t)row * p.c_rs + n;
         if (vec_ok) {
-            f32x4 r;
+            sum_t r[4];
 #pragma unroll
-            for (int e = 0; e < 4; ++e) r[e] = apply_epilogue<float>(s[e] + p.prologue_arg, p.epilogue, p.epilogue_arg);
-            if (p.out_type == T_F32) {
-                *(f32x4*)((float*)p.C + idx) = r;
+            for (int e = 0; e < 4; ++e) r[e] = apply_epilogue<sum_t>(wrap_add(s[e], (sum_t)p.prologue_arg), p.epilogue, p.epilogue_arg);
+            if constexpr (I8) {
+                if (p.out_type == T_I32) *(i32x4*)((int*)p.C + idx) = i32x4{r[0], r[1], r[2], r[3]};
+                else if (p.out_type == T_I16)
+                    *(i32x2*)((int16_t*)p.C + idx) = i32x2{(int)(((unsigned)r[0] & 0xffffu) | ((unsigned)r[1] << 16)), (int)(((unsigned)r[2] & 0xffffu) | ((unsigned)r[3] << 16))};
+                else
+                    *(unsigned*)((int8_t*)p.C + idx) = ((unsigned)r[0] & 0xffu) | (((unsigned)r[1] & 0xffu) << 8) | (((unsigned)r[2] & 0xffu) << 16) | ((unsigned)r[3] << 24);
+            } else if (p.out_type == T_F32) {
+                *(f32x4*)((float*)p.C + idx) = f32x4{r[0], r[1], r[2], r[3]};
             } else if (p.out_type == T_F16) {
                 typedef _Float16 h4 __attribute__((ext_vector_type(4)));
                 *(h4*)((uint16_t*)p.C + idx) = h4{(_Float16)r[0], (_Float16)r[1], (_Float16)r[2], (_Float16)r[3]};
@@ -242,16 +269,20 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_skinny_mfma_kernel(SkinnyArgs
         }
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-            float v = s[e];
-            v = apply_prologue<float>(v, p.prologue, p.prologue_arg, [&]() { return load_out(p.C, p.out_type, idx + e); });
-            store_out(p.C, p.out_type, idx + e, apply_epilogue<float>(v, p.epilogue, p.epilogue_arg));
+            if constexpr (I8) {
+                const int v = apply_prologue<int>(s[e], p.prologue, p.prologue_arg, [&]() { return load_out_int(p.C, p.out_type, idx + e); });
+                store_out_int(p.C, p.out_type, idx + e, apply_epilogue<int>(v, p.epilogue, p.epilogue_arg));
+            } else {
+                const float v = apply_prologue<float>(s[e], p.prologue, p.prologue_arg, [&]() { return load_out(p.C, p.out_type, idx + e); });
+                store_out(p.C, p.out_type, idx + e, apply_epilogue<float>(v, p.epilogue, p.epilogue_arg));
+            }
         }
     };
 
     if (nsplit == 1) {
         for (int grp = tid; grp < groups; grp += NT) {
-            f32x4 s = *(const f32x4*)(red + (size_t)grp * 4);
-            for (int w = 1; w < WAVES; ++w) s += *(const f32x4*)(red + (size_t)w * p.M * CB + (size_t)grp * 4);
+            sum4 s = *(const sum4*)(red + (size_t)grp * 4);
+            for (int w = 1; w < WAVES; ++w) s += *(const sum4*)(red + (size_t)w * p.M * CB + (size_t)grp * 4);
             finish4(grp, s);
         }
         return;
@@ -260,10 +291,10 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_skinny_mfma_kernel(SkinnyArgs
     // ---- K split ----
     // The partial goes out as agent-scope relaxed atomic stores (written through to the level
     // all XCDs share) and only has to be acknowledged (vmcnt = 0) before the ticket is taken.
-    float* part = p.scratch + ((int64_t)split_idx * nblocks + bx) * (32 * CB);
+    sum_t* part = (sum_t*)p.scratch + ((int64_t)split_idx * nblocks + bx) * (32 * CB);
     for (int grp = tid; grp < groups; grp += NT) {
-        f32x4 s = *(const f32x4*)(red + (size_t)grp * 4);
-        for (int w = 1; w < WAVES; ++w) s += *(const f32x4*)(red + (size_t)w * p.M * CB + (size_t)grp * 4);
+        sum4 s = *(const sum4*)(red + (size_t)grp * 4);
+        for (int w = 1; w < WAVES; ++w) s += *(const sum4*)(red + (size_t)w * p.M * CB + (size_t)grp * 4);
 #pragma unroll
         for (int e = 0; e < 4; ++e) __hip_atomic_store(part + grp * 4 + e, s[e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
@@ -277,12 +308,12 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_skinny_mfma_kernel(SkinnyArgs
     const int64_t slice = (int64_t)nblocks * (32 * CB);
     for (int grp = tid; grp < groups; grp += NT) {
         // loads of 8 slices are issued together (one memory latency per batch); the adds stay in split order
-        const float* src = p.scratch + (int64_t)bx * (32 * CB) + (size_t)grp * 4;
-        f32x4 s = {0.f, 0.f, 0.f, 0.f};
+        const sum_t* src = (const sum_t*)p.scratch + (int64_t)bx * (32 * CB) + (size_t)grp * 4;
+        sum4 s = {0, 0, 0, 0};
         for (int sp0 = 0; sp0 < nsplit; sp0 += 8) {
-            f32x4 v[8];
+            sum4 v[8];
 #pragma unroll
-            for (int u = 0; u < 8; ++u) v[u] = sp0 + u < nsplit ? *(const f32x4*)(src + (sp0 + u) * slice) : f32x4{0.f, 0.f, 0.f, 0.f};
+            for (int u = 0; u < 8; ++u) v[u] = sp0 + u < nsplit ? *(const sum4*)(src + (sp0 + u) * slice) : sum4{0, 0, 0, 0};
 #pragma unroll
             for (int u = 0; u < 8; ++u)
                 if (sp0 + u < nsplit) s += v[u];
@@ -292,11 +323,11 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_skinny_mfma_kernel(SkinnyArgs
     if (tid == 0) p.counters[bx] = 0; // ready for the next launch
 }
 
-template <bool BF16, int CB, int WAVES, int DEPTH>
+template <int IN, int CB, int WAVES, int DEPTH>
 hipError_t launch_one(const SkinnyArgs& a, hipStream_t stream, LaunchGeom* geom, bool dry_run)
 {
-    auto kern = gemm_skinny_mfma_kernel<BF16, CB, WAVES, DEPTH>;
-    unsigned lds = WAVES * DEPTH * (16 * CB * 2 + 1024);
+    auto kern = gemm_skinny_mfma_kernel<IN, CB, WAVES, DEPTH>;
+    unsigned lds = WAVES * DEPTH * (32 * CB + 1024); // (a step's piece of B is 32 bytes of K for every column, whatever the type)
     const unsigned red = WAVES * a.M * CB * 4; // [wave][row of A][column] floats of the tail
     if (lds < red) lds = red;
     const int nblocks = (a.N + CB - 1) / CB;
@@ -318,7 +349,7 @@ hipError_t launch_one(const SkinnyArgs& a, hipStream_t stream, LaunchGeom* geom,
 }
 
 // narrow (64 columns, no K split needed from 128 blocks up) first, then wide
-#define SM(CB, W, D) { CB, W, D, true, 32, 16, 32 * CB, &launch_one<false, CB, W, D>, &launch_one<true, CB, W, D> }
+#define SM(CB, W, D) { CB, W, D, true, 32, 16, 32 * CB, &launch_one<T_F16, CB, W, D>, &launch_one<T_BF16, CB, W, D>, &launch_one<T_I8, CB, W, D> }
 const SkinnyVariant kSkinnyMfma[] = { SM(64, 4, 4), SM(64, 4, 8), SM(64, 2, 8), SM(64, 8, 4), SM(256, 4, 4), SM(256, 2, 4) };
 #undef SM
 

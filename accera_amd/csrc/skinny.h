@@ -6,7 +6,7 @@
 namespace acc950 {
 
 struct SkinnyArgs {
-    const void* A;  // M x K, row-major (K contiguous), 16-bit elements
+    const void* A;  // M x K, row-major (K contiguous), 16-bit elements (8-bit: MFMA family)
     const void* B;  // K x N, row-major (N contiguous)
     void* C;        // M x N, row-major
     int M, N, K;
@@ -34,10 +34,14 @@ struct SkinnyVariant {
     int waves, depth;  // waves per workgroup, ring slots (steps in flight) per wave
     bool mfma;
     int max_m;         // rows of A the kernel can take
-    int k_step;        // K rows per wave step; every K split is a whole number of steps
-    int block_floats;  // scratch floats per column block and split
+    int k_step;        // K rows per wave step for 16-bit inputs (int8: twice as many); every K split is a whole number of steps
+    int block_floats;  // scratch sums (32 bits each) per column block and split
     SkinnyLaunchFn f16, bf16;
+    SkinnyLaunchFn i8; // int8 inputs, int32 sums (MFMA family only; null otherwise)
 };
+
+// k rows per wave step of variant v for this input type
+inline int skinny_k_step(const SkinnyVariant& v, int in_type) { return in_type == T_I8 ? 2 * v.k_step : v.k_step; }
 
 // tables of the two families (gemm_skinny.hip, gemm_skinny_mfma.hip)
 const SkinnyVariant* skinny_dot2_table(int* count);

@@ -448,6 +448,36 @@ def test_skinny_all_variants_and_splits(in_type, out_type):
     run_case(in_type, out_type, 24, 2048, 512, seed=80, dist="normal", prologue=ora.PRO_NONE, epilogue=ora.EPI_RELU_NOCOND)
 
 
+@pytest.mark.parametrize("out_type", ["i32", "i16", "i8"])
+def test_skinny_int8_streaming_kernels(out_type):
+    """int8 rows of A against a large row-major int8 B on the streaming kernels of the matrix-core family
+    (v_mfma_i32_32x32x32_i8, 32 k rows per step), bit-exact against the oracle: every variant x K splits, ragged M / N, a K of
+    one step, accumulation into C, and the automatic choice for the decode shape."""
+    from accera_amd import _lib
+    names = [_lib.variant_name(100 + sv) for sv in range(_lib.num_skinny_variants())]
+    mfma = [100 + i for i, n in enumerate(names) if "mfma" in n]
+    for v in mfma:
+        for splits in (1, 3, 8):
+            print("skinny int8", v, names[v - 100], "splits", splits, flush=True)
+            run_case("i8", out_type, 8, 1024 + 64, 1024, variant=v, splits=splits, seed=v * 10 + splits)
+    run_case("i8", out_type, 32, 1024 + 64, 2048, variant=mfma[0], splits=2, seed=170)
+    run_case("i8", out_type, 17, 1008, 992, variant=mfma[0], splits=4, seed=171)
+    run_case("i8", out_type, 1, 16, 32, variant=mfma[0], splits=1, seed=172, epilogue=ora.EPI_NONE)
+    run_case("i8", out_type, 3, 80, 96, variant=mfma[0], splits=8, seed=173)
+    if out_type != "i8":  # (an int8 C is only written)
+        run_case("i8", out_type, 8, 2048, 512, seed=179, prologue=ora.PRO_NONE)
+        run_case("i8", out_type, 24, 2048, 512, seed=180, prologue=ora.PRO_NONE, epilogue=ora.EPI_RELU_NOCOND)
+    # the dot-product family has no int8 form
+    dot2 = 100 + next(i for i, n in enumerate(names) if "dot2" in n)
+    with pytest.raises(_lib.Acc950Error) as e:
+        _lib.launch_geometry(_lib.I8, _lib.I32, 8, 1024, 1024, (1024, 1), (1024, 1), (1024, 1), variant=dot2)
+    assert e.value.code == _lib.UNSUPPORTED
+    # automatic choice: the decode shape in int8 streams on the matrix-core family
+    grid, block, lds, v = _lib.launch_geometry(_lib.I8, getattr(_lib, out_type.upper()), 8, 11008, 4096, (4096, 1), (11008, 1), (11008, 1))
+    assert "skinny mfma" in _lib.variant_name(v)
+    run_case("i8", out_type, 8, 11008, 4096, seed=181)
+
+
 def test_skinny_repeated_launches_reuse_counters():
     """The K-split arrival counters must return to zero after every launch."""
     for rep in range(3):
