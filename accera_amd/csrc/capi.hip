@@ -346,7 +346,9 @@ int auto_mfma_variant(const Problem& pb)
         // four waves with 128x128 wave tiles: measured 3-9 % faster than the eight-wave form on large problems
         // (a third less LDS traffic, and the part is at its power limit there)
         // (walking several tiles per workgroup pays when there is more than one round of tiles over the CUs)
-        if (v.w4) rank = v.persist ? (tiles / (pb.g.batch > 1 ? pb.g.batch : 1) > kComputeUnits ? 14 : 12) : 13; // (tiles of one problem: a workgroup walks inside its own)
+        // (a column-major A: the two forms measured level -- 8192^3 tA fp16 774 against 784 us, int8 393 against 391,
+        // 8192 x 8192 x 4096 410 against 407 -- and the one-tile form stays the choice)
+        if (v.w4) rank = v.persist ? (v.a_kc && tiles / (pb.g.batch > 1 ? pb.g.batch : 1) > kComputeUnits ? 14 : 12) : 13; // (tiles of one problem: a workgroup walks inside its own)
         const bool better = best < 0 || cost < best_cost * 0.999 ||
                             (cost <= best_cost * 1.001 && ((int64_t)v.bm * v.bn > (int64_t)tab[best].bm * tab[best].bn ||
                                                            ((int64_t)v.bm * v.bn == (int64_t)tab[best].bm * tab[best].bn && rank > best_rank)));

@@ -13,7 +13,7 @@
 // moves accumulators between the register files and spills.  Tile staging, the LDS layout and
 // the stores are those of gemm_mfma16.h.
 //
-// Takes: A row-major (or column-major, in the one-tile-per-workgroup form with 256-wide tiles: staged as it lies in memory and
+// Takes: A row-major (or column-major, with 256-wide tiles: staged as it lies in memory and
 // read with the transposing LDS loads, like a row-major B), any M >= 256 and any 16-byte-aligned N >= the tile width
 // (the last row / column of tiles overlaps the one before), K a multiple of one k-step (64 bytes)
 // and at least four of them, rows of C 16 bytes aligned;
@@ -35,7 +35,7 @@ struct Mfma16W4Config {
     static_assert(!PERSIST_ || BN_ == 256, "the 192-wide tile is for problems of one tile per CU");
     static constexpr int IN = IN_, BM = 256, BN = BN_, WAVES_M = 2, WAVES_N = 2, KB = 64, STAGES = 4, NT = 256;
     static constexpr bool A_KC = A_KC_, B_KC = B_KC_;
-    static_assert(A_KC_ || (BN_ == 256 && !PERSIST_), "column-major A: 256-wide tiles, one per workgroup");
+    static_assert(A_KC_ || BN_ == 256, "column-major A: 256-wide tiles");
     // (a workgroup that walks several tiles stages its write-back behind the last LDS stage while the others already receive
     // the next tile: it asks for the whole LDS of the CU)
     static constexpr int LDS_BYTES = PERSIST_ ? 160 * 1024 : STAGES * (BM + BN) * KB;
@@ -387,7 +387,18 @@ __global__ void __launch_bounds__(256, 1) gemm_mfma16w4_kernel(GemmArgs p)
 #define ACC950_W4_R(f, d) f #d "0", f #d "1", f #d "2", f #d "3", f #d "4", f #d "5", f #d "6", f #d "7", f #d "8", f #d "9"
 #define ACC950_W4_V(d) ACC950_W4_R("v", d)
 #define ACC950_W4_A(d) ACC950_W4_R("a", d)
-    if constexpr (!A_KC) {
+    if constexpr (!A_KC && TAIL_PREFETCH) {
+        if constexpr (IN == IN_I8) {
+            if constexpr (B_KC) asm volatile(ACC950_W4_LOOP_KC_AMC8_P("v_mfma_i32_16x16x64_i8") : ACC950_W4_OPERANDS);
+            else asm volatile(ACC950_W4_LOOP_MC8_AMC8_P("v_mfma_i32_16x16x64_i8") : ACC950_W4_OPERANDS);
+        } else if constexpr (B_KC) {
+            if constexpr (IN == IN_F16) asm volatile(ACC950_W4_LOOP_KC_AMC16_P("v_mfma_f32_16x16x32_f16") : ACC950_W4_OPERANDS);
+            else asm volatile(ACC950_W4_LOOP_KC_AMC16_P("v_mfma_f32_16x16x32_bf16") : ACC950_W4_OPERANDS);
+        } else {
+            if constexpr (IN == IN_F16) asm volatile(ACC950_W4_LOOP_MC16_AMC16_P("v_mfma_f32_16x16x32_f16") : ACC950_W4_OPERANDS);
+            else asm volatile(ACC950_W4_LOOP_MC16_AMC16_P("v_mfma_f32_16x16x32_bf16") : ACC950_W4_OPERANDS);
+        }
+    } else if constexpr (!A_KC) {
         if constexpr (IN == IN_I8) {
             if constexpr (B_KC) asm volatile(ACC950_W4_LOOP_KC_AMC8("v_mfma_i32_16x16x64_i8") : ACC950_W4_OPERANDS);
             else asm volatile(ACC950_W4_LOOP_MC8_AMC8("v_mfma_i32_16x16x64_i8") : ACC950_W4_OPERANDS);

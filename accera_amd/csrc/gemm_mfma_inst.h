@@ -25,6 +25,7 @@ namespace acc950 {
 #define V16W4_192 { 256, 192, 2, 2, true, true, true, false, 64, 4, false, true, true, false, false, nullptr, nullptr }
 #define V16W4P(BKC) { 256, 256, 2, 2, true, BKC, true, false, 64, 4, false, true, true, true, false, nullptr, nullptr }
 #define V16W4A(BKC) { 256, 256, 2, 2, false, BKC, true, false, 64, 4, false, true, true, false, false, nullptr, nullptr }
+#define V16W4PA(BKC) { 256, 256, 2, 2, false, BKC, true, false, 64, 4, false, true, true, true, false, nullptr, nullptr }
 #else
 // ping-pong on the 16x16 MFMA shapes
 #define V16(AKC, BM, BN, WM, WN, BKC, KB, STAGES)                                                       \
@@ -42,6 +43,9 @@ namespace acc950 {
 // the same kernel for a column-major A (one tile per workgroup)
 #define V16W4A(BKC) \
     { 256, 256, 2, 2, false, BKC, true, false, 64, 4, false, true, true, false, false, &launch_mfma16w4<Mfma16W4Config<ACC950_IN, BKC, false, 256, false, false>>, nullptr }
+// ... walking several output tiles
+#define V16W4PA(BKC) \
+    { 256, 256, 2, 2, false, BKC, true, false, 64, 4, false, true, true, true, false, &launch_mfma16w4<Mfma16W4Config<ACC950_IN, BKC, false, 256, true, false>>, nullptr }
 #endif
 // any sizes, leading dimensions and alignments (the odd shapes of the reference's sweep lists, e.g.
 // /root/reference/tools/benchmarkers/gemm_resnet_inception.csv): register-staged 128x128 tiles whose fill takes unaligned chunks
@@ -124,6 +128,9 @@ static const MfmaVariant kVariants[] = {
     VANY64(true, true),
     VANY64(false, false),
     VANY64(false, true),
+    // four-wave kernel for a column-major A, one workgroup per CU walking several output tiles
+    V16W4PA(false),
+    V16W4PA(true),
 };
 #undef LAYOUT_AT
 #undef VA
@@ -133,6 +140,7 @@ static const MfmaVariant kVariants[] = {
 #undef V16W4_192
 #undef V16W4P
 #undef V16W4A
+#undef V16W4PA
 #undef VANY
 #undef VANY64
 #undef LAYOUT

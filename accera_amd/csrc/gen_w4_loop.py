@@ -226,7 +226,7 @@ def loop(b_layout, persist=False):
     else:
         # block x of the wave's rows lies x * 32 (16-bit) or x * 16 (8-bit) bytes further along every k row of the tile, and
         # the swizzle is an XOR on those address bits (rows of the tile start on multiples of their length)
-        assert not persist and TN == 8
+        assert TN == 8
         for x in range(1, 8):
             out.append(line(f"v_xor_b32 {A_LOW[x]}, {x * (32 if A_LAYOUT == 'mc16' else 16)}, %[a_rd]"))
         for x in range(8):
@@ -321,16 +321,18 @@ def main():
 
 
 def main_a_mc():
-    """The loops for a column-major A (one macro per pair of layouts; one workgroup per tile only)."""
+    """The loops for a column-major A (one macro per pair of layouts), for one tile per workgroup and for a workgroup that
+    walks several tiles (_P: closing steps that prefetch the next tile)."""
     global A_LAYOUT
-    for a_name, b_name in (("mc16", "kc"), ("mc16", "mc16"), ("mc8", "kc"), ("mc8", "mc8")):
-        set_width(8)
-        A_LAYOUT = a_name
-        body = loop(b_name)
-        A_LAYOUT = "kc"
-        print(f"#define ACC950_W4_LOOP_{b_name.upper()}_A{a_name.upper()}(MFMA) \\")
-        print(" \\\n".join("    " + s for s in body))
-        print()
+    for persist in (False, True):
+        for a_name, b_name in (("mc16", "kc"), ("mc16", "mc16"), ("mc8", "kc"), ("mc8", "mc8")):
+            set_width(8)
+            A_LAYOUT = a_name
+            body = loop(b_name, persist=persist)
+            A_LAYOUT = "kc"
+            print(f"#define ACC950_W4_LOOP_{b_name.upper()}_A{a_name.upper()}{'_P' if persist else ''}(MFMA) \\")
+            print(" \\\n".join("    " + s for s in body))
+            print()
 
 
 if __name__ == "__main__":

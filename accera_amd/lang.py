@@ -716,7 +716,8 @@ def _variant_for(spec, tile=None, family=None, k_bytes=None):
         # the hand-laid loop ahead of both (the multi-tile form when there is more than one round of tiles); then larger tiles
         r = 2 * ("pingpong" in name) + (1 if "mi16" in name and lean else -1 if "mi16" in name else 0)
         if "hand-laid loop" in name:
-            r = 4 + (("multi-tile" in name) == (tiles > 256))
+            # (multi-tile form when there is more than one round of tiles -- for a row-major A; the forms for a column-major A measured level)
+            r = 4 + (("multi-tile" in name) == (tiles > 256 and "A=col-major" not in name))
         return (r, bm * bn if tiles >= 256 else -bm * bn, "edge" not in name)
     return sorted(cands, key=lambda c: rank(c[1]))[-1][0]  # (`max` is the DSL's elementwise maximum in this module)
 

@@ -877,7 +877,7 @@ def test_four_wave_kernel_walking_several_tiles(in_type, out_type, b_layout, M, 
     import accera_amd as acc
     import torch
     from accera_amd import _lib
-    v = [v for v, n in _variants(b_layout) if "multi-tile" in n]
+    v = [v for v, n in _variants(b_layout) if "multi-tile" in n and "A=col-major" not in n]
     assert len(v) == 1
     pro_op, pa = {"set0": (ora.PRO_SET0, 0.0), "none": (ora.PRO_NONE, 0.0), "scale": (ora.PRO_SCALE, 0.5)}[pro]
     epi_op, ea = {"relu": (ora.EPI_RELU, 0.0), "none": (ora.EPI_NONE, 0.0), "scale": (ora.EPI_SCALE, 2.0)}[epi]
@@ -899,6 +899,45 @@ def test_four_wave_kernel_walking_several_tiles(in_type, out_type, b_layout, M, 
     if (M // 256) * (N // 256) % 256 == 0 and M % 256 == 0 and N % 256 == 0:
         # whole rounds of tiles over the compute units (with a nearly empty last round the cost model prefers smaller tiles)
         assert "multi-tile" in _lib.variant_name(chosen) and grid == [256, 1, 1]
+
+
+@pytest.mark.parametrize("in_type,out_type,b_layout,M,N,K,pro,epi", [
+    # two rounds over the workgroups, K of 8 and 12 k-steps (closing steps fetch the next tile)
+    ("f16", "f32", "row", 4096, 8192, 256, "set0", "relu"),
+    ("bf16", "bf16", "col", 4096, 8192, 384, "set0", "relu"),
+    ("i8", "i32", "row", 8192, 4096, 512, "set0", "relu"),
+    ("i8", "i8", "col", 4096, 8192, 768, "set0", "none"),
+    # a K that enters the loop in the middle (9 k-steps: no fetching ahead), ragged M and N, C read
+    ("f16", "f16", "row", 4112, 4400, 288, "set0", "relu"),
+    ("i8", "i32", "col", 4352, 4096, 512, "none", "relu"),
+    ("f16", "f32", "col", 4400, 4112, 256, "none", "relu"),
+])
+def test_four_wave_kernel_walking_several_tiles_with_a_column_major_a(in_type, out_type, b_layout, M, N, K, pro, epi):
+    """The multi-tile form for a column-major A (the transA rows of the reference's sweep lists,
+    /root/reference/tools/benchmarkers/accera_gemm.py:310-311), named explicitly and through the automatic choice."""
+    import accera_amd as acc
+    import torch
+    from accera_amd import _lib
+    v = [v for v, n in _variants(b_layout) if "multi-tile" in n and "A=col-major" in n]
+    assert len(v) == 1
+    pro_op, pa = {"set0": (ora.PRO_SET0, 0.0), "none": (ora.PRO_NONE, 0.0)}[pro]
+    epi_op, ea = {"relu": (ora.EPI_RELU, 0.0), "none": (ora.EPI_NONE, 0.0)}[epi]
+    rng = np.random.default_rng(M + N + K + 1)
+    A, B = np.asfortranarray(make_input(rng, (M, K), in_type)), make_input(rng, (K, N), in_type)
+    if b_layout == "col":
+        B = np.asfortranarray(B)
+    C0 = make_c0(rng, (M, N), out_type, scale=100)
+    dA, dB = to_device(A, in_type), to_device(B, in_type)
+    assert dA.stride() == (1, M)
+    want = ora.gemm_relu_exact(A, B, C0, in_type, out_type, pro_op, epi_op, prologue_arg=pa, epilogue_arg=ea)
+    for variant in (v[0], -1):
+        dC = to_device(C0, out_type)
+        call = acc.GemmCall(dA, dB, dC, prologue=pro_op, prologue_arg=pa, epilogue=epi_op, epilogue_arg=ea, variant=variant)
+        call()
+        torch.cuda.synchronize()
+        assert_matches(to_host(dC, out_type), want, out_type, K)
+    name = _lib.variant_name(acc.GemmCall(dA, dB, to_device(C0, out_type), prologue=pro_op, epilogue=epi_op, variant=-1).chosen[0])
+    assert "A=col-major" in name, name
 
 
 def test_skinny_workspaces_are_per_stream():

@@ -402,6 +402,31 @@ def test_loops_for_a_column_major_a(a_layout, b_layout):
         assert lanes == ["%[a_off]", "%[a_off1]", "%[a_off]", "%[a_off1]"]
 
 
+@pytest.mark.parametrize("a_layout,b_layout", [("mc16", "kc"), ("mc16", "mc16"), ("mc8", "kc"), ("mc8", "mc8")])
+@pytest.mark.parametrize("KT,flags,stores", [(8, 0, 0), (12, 1, 0), (128, 3, 64), (8, 2, 64), (12, 3, 47), (128, 2, 500)])
+def test_column_major_a_loops_of_a_workgroup_that_walks_several_tiles(a_layout, b_layout, KT, flags, stores):
+    """The same loops for a workgroup that walks several output tiles: closing steps that fetch the next tile's K tiles
+    0..2, first k-steps whose waits allow for the previous tile's stores -- the scalar side behaves as for a row-major A,
+    and the text around it is the one-tile loop's (same preamble of per-block read addresses, same reads per step)."""
+    g = _gen()
+    g.A_LAYOUT = a_layout
+    try:
+        fills, steps, p0 = _run_fills(g, b_layout, 8, KT, 3, persist=True, flags=flags, stores_in_flight=stores)
+        walk, one = _text(g.loop(b_layout, persist=True)), _text(g.loop(b_layout))
+    finally:
+        g.A_LAYOUT = "kc"
+    assert steps == KT and p0 == 0
+    last = KT + 3 if flags & 1 else KT
+    assert sorted(fills) == sorted([(o, t, p, t % 4) for o in "ab" for t in range(3, last) for p in range(4)])
+    assert walk[:walk.index("4:")] == one[:one.index("4:")], "same preamble: read addresses, accumulators"
+    assert sum(i.startswith("MFMA") for i in walk) == 64 * (4 + 4 + 1 + 3 + 3)
+    op = "ds_read_b64_tr_b16" if a_layout == "mc16" else "ds_read_b64_tr_b8"
+    per_step = 16 + (8 if b_layout == "kc" else 16)
+    # every k-step but the last of either set of closing steps reads the next step's fragments: 4 + 4 + 1 + 2 + 2 steps
+    assert sum(i.startswith("ds_read") for i in walk[walk.index("10:"):]) == per_step * (1 + 4 + 4 + 1 + 2 + 2)
+    assert sum(i.startswith(op) for i in walk[walk.index("13:"):]) >= 16 * 9
+
+
 def test_block_addresses_of_a_column_major_tile_differ_by_an_xor():
     """What the preamble above relies on: with the tile's k rows starting on multiples of their length, the LDS address
     of block x's transposing read is block 0's with x * 32 (16-bit) or x * 16 (8-bit) XORed in, for every lane."""
