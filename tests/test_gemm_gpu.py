@@ -155,8 +155,15 @@ def test_four_wave_kernel_column_major_a(in_type, out_type, b_layout):
     kb = 64 if in_type == "i8" else 32
     vec = 16 if in_type == "i8" else 8
     variants = [v for v, n in _variants(b_layout) if "hand-laid" in n and "A=col-major" in n]
-    assert len(variants) == 1
-    v = variants[0]
+    assert len(variants) == 2  # one tile per workgroup, and the form that walks several tiles
+    for v in variants:
+        _column_major_a_cases(v, in_type, out_type, b_layout, kb, vec)
+
+
+def _column_major_a_cases(v, in_type, out_type, b_layout, kb, vec):
+    import accera_amd as acc
+    import torch
+    from accera_amd import _lib
     for k_tiles, epi in ((4, ora.EPI_RELU), (5, ora.EPI_NONE), (6, ora.EPI_RELU), (7, ora.EPI_RELU), (8, ora.EPI_NONE), (21, ora.EPI_RELU)):
         print("variant", v, in_type, out_type, b_layout, "k tiles", k_tiles, flush=True)
         run_case(in_type, out_type, 512, 768, k_tiles * kb, a_layout="col", b_layout=b_layout, variant=v, seed=900 + k_tiles, epilogue=epi)
