@@ -319,18 +319,25 @@ int auto_mfma_variant(const Problem& pb)
         const int64_t per_cu = (tiles + kComputeUnits - 1) / kComputeUnits;
         const int wgs_per_cu = ((fp32 ? per_cu >= 2 : tiles > kComputeUnits) && v.waves_m * v.waves_n <= 4 &&
                                 2 * v.stages * (v.bm + v.bn) * v.kb <= 160 * 1024 && v.bm * v.bn <= 256 * 128) ? 2 : 1;
-        const int64_t rounds = (tiles + kComputeUnits * wgs_per_cu - 1) / (kComputeUnits * wgs_per_cu);
-        double cost = fp32 ? (double)per_cu * v.bm * v.bn : (double)rounds * wgs_per_cu * v.bm * v.bn;
+        const int64_t slots = (int64_t)kComputeUnits * wgs_per_cu;
+        double rounds = (double)((tiles + slots - 1) / slots);
+        // A last round that is not full costs less than a full one when K is long: the part is at its power limit there, and
+        // the workgroups of a half-empty chip run at a higher clock (fp16, K = 4096, tiles of 256 x 256: 256 of them 97 us,
+        // 192 78 us, 384 161 us, where whole rounds would say 97 and 194).  Half of the missing part is charged.
+        if ((int64_t)pb.g.K * elem_size(pb.g.in_type) >= 4096 && tiles > slots) rounds = 0.5 * (rounds + (double)tiles / (double)slots);
+        double cost = fp32 ? (double)per_cu * v.bm * v.bn : rounds * wgs_per_cu * v.bm * v.bn;
         if (v.edge) cost *= v.any ? 2.0 : 1.5;   // register-staged fill, bounds checks (unaligned chunks cost more requests)
         if (!v.direct) cost *= 1.2;
-        // measured on sweeps: 4-wave tiles reach about 85 % of the ping-pong kernel's rate when two
+        // measured on sweeps: 4-wave tiles reach about 80 % of the ping-pong kernel's rate when two
         // workgroups share a CU and about 70 % when a workgroup has the CU to itself
-        if (v.waves_m * v.waves_n <= 4 && !v.w4) cost /= wgs_per_cu == 2 ? 0.85 : 0.7;
+        // (fp32, bound by the MFMA rate whatever the tile: the 4-wave tiles are level or ahead -- 6144x4608x8192 3.29 ms on
+        // 128 x 128 tiles against 4.10 on the 256 x 256 ping-pong kernel, 50176x512x256 110 against 146 us)
+        if (v.waves_m * v.waves_n <= 4 && !v.w4) cost /= fp32 ? (wgs_per_cu == 2 ? 1.1 : 1.0) : (wgs_per_cu == 2 ? 0.8 : 0.7);
         // smaller tiles fetch more bytes and read more fragments per MFMA
         // (measured, 64x64 against 128x128 tiles: fp32, bound by its slow MFMAs, 1024^3 20.7 against 63.7 us and 3072x1024x1024
         // 53 against 66; 8- and 16-bit inputs win while a CU has at most two of them -- fp16 1024^3 6.6 against 9.5 us,
         // 1536x1152x2048 14.4 against 17.0 -- and lose beyond: 3072x1024x1024 13.1 against 9.8, 2048^3 30.3 against 21.2)
-        if (v.bm * v.bn <= 64 * 64) cost /= pb.g.in_type == T_F32 ? 0.9 : per_cu <= 2 ? 0.75 : 0.5;
+        if (v.bm * v.bn <= 64 * 64) cost /= pb.g.in_type == T_F32 ? 1.0 : per_cu <= 2 ? 0.75 : 0.5;
         else if (v.bm * v.bn <= 128 * 64) cost /= 0.8;
         // rank inside one tile shape: ping-pong kb64 x4 > ping-pong others > 8-wave > 4-wave (kb64 x4 first)
         int rank = v.pingpong ? (v.kb == 64 && v.stages == 4 ? 8 : 6) : (v.waves_m * v.waves_n == 8 ? 4 : 2);
@@ -339,6 +346,10 @@ int auto_mfma_variant(const Problem& pb)
         // more tiles than CUs want two workgroups per CU, which only the smaller stages leave room for; below 32 tiles of K the
         // four stages of 64 bytes are ahead (2048x2048x512 fp16: 7.5 against 8.2 us)
         if (!v.pingpong && v.direct && v.kb == 128 && v.stages == 4 && tiles <= kComputeUnits && (int64_t)pb.g.K * elem_size(pb.g.in_type) >= 4096) rank += 2;
+        // 128 x 128 tiles, two workgroups per CU: two stages of 128 bytes of K are ahead of four of 64 (3072x2304x4096 fp16:
+        // 59.8 against 69.6 us; 3072x2048x1024 19.2 against 22.0; 12544x512x1024 16.5 against 17.9)
+        if (!v.pingpong && v.direct && v.kb == 128 && v.stages == 2 && v.bm == 128 && v.bn == 128 && tiles > kComputeUnits &&
+            (int64_t)pb.g.K * elem_size(pb.g.in_type) >= 1024) rank += 2;
         // 16x16 shapes: measured 4-9 % faster than the 32x32 shapes on every large problem, in the lean build
         // (C = A*B, C = relu(A*B)); their full build reads C element by element and lost 20 % to the 32x32 form
         const bool lean = pb.g.prologue == PRO_SET && pb.g.prologue_arg == 0.f && (pb.g.epilogue == EPI_RELU || pb.g.epilogue == EPI_NONE);
@@ -417,11 +428,20 @@ int auto_mfma_splits(const MfmaVariant& v, const Problem& pb, size_t max_floats 
     if (g.batch > 1) return 1;
     const int64_t tiles = (((int64_t)g.M + v.bm - 1) / v.bm) * (((int64_t)g.N + v.bn - 1) / v.bn);
     if (tiles * 2 > kComputeUnits) return 1;
-    const int64_t steps = (int64_t)g.K * elem_size(g.in_type) / 64; // k-steps of 64 bytes
-    // (1024^3, 32 k-steps, on 64 tiles of 128 x 128: 9.8 us unsplit, 15.1 us in two slices -- the second kernel costs 3 to 5 us;
-    // with a handful of tiles a short K is still worth splitting: int8 363x64x3025, 6 tiles and 47 k-steps, 46.9 us unsplit,
-    // 10.8 in sixteen slices; a k-step of the register-staged kernels takes about four times as long as one of the direct ones)
-    if (steps * (v.direct ? 1 : 4) < 64 && tiles * 8 > kComputeUnits) return 1;
+    // K in steps of 0.1 us: what 64 bytes of K cost a 64 x 64 tile with direct fills.  The register-staged kernels take two
+    // to three times as long per step, twice that with a column-major A (which they transpose on the way), and their
+    // element-wise read of C costs as much again (the second kernel of a split reads C in rows instead); a 128 x 128 tile
+    // takes about twice, a 256 x 256 tile about five times as long per step as a 64 x 64 one.
+    const int64_t area = (int64_t)v.bm * v.bn;
+    const int64_t raw_steps = (int64_t)g.K * elem_size(g.in_type) / 64;
+    const int64_t steps = raw_steps * (v.direct ? 1 : (v.a_kc ? 2 : 4) * (g.prologue != PRO_SET ? 2 : 1)) * (area <= 64 * 64 ? 1 : area <= 128 * 128 ? 2 : 4) *
+                          (g.in_type == T_F32 ? 2 : 1); // (fp32: 512^3 on 64 tiles 8.9 us, 256^3 5.0)
+    // The second kernel costs 3 to 5 us: below 48 steps a split only loses, however few the tiles (fp16, 64 x 64 tiles,
+    // unsplit / best split in us, direct: 256^3 3.1 / 5.8; 64x1152x448 4.3 / 7.0; 289x192x1344 7.2 / 7.6; 64x320x1728
+    // 8.4 / 7.4; 576x192x3136 11.9 / 7.9; register-staged: 6272x32x512 7.3 / 9.2; 196x128x800 9.6 / 7.9; reading C:
+    // 384x288x512 9.0 / 5.9; with a column-major A: 512x128x196 8.4 / 5.8, 384x192x1225 16.6 / 7.2; int8 363x64x3025
+    // 46.9 / 10.8).
+    if (steps < 48) return 1;
     // Slices of about 32 k-steps; shorter ones, down to 4, while that keeps the workgroups at or below one per compute unit;
     // never more workgroups than the compute units hold at once (two of the 64 x 64 tiles each), never more than 32 slices.
     // Measured with 64 x 64 tiles, fp16, us by slices 4 / 8 / 16 / 32: 768x320x30522 84 / 53 / 49 / 53; 1024x80x30522
@@ -433,6 +453,9 @@ int auto_mfma_splits(const MfmaVariant& v, const Problem& pb, size_t max_floats 
     if (want > slots / tiles) want = slots / tiles;
     if (want > 32) want = 32;
     if ((size_t)want * (size_t)g.M * (size_t)g.N > ((size_t)1 << 24)) return 1; // 64 MiB of partial sums at most without being asked
+    // What the slices save against what the second kernel costs, 3.5 us and 0.65 us per MB of partial sums written and read
+    // (2048x256x1536 on 128 tiles: 8.2 us unsplit, 10.7 in two slices with their 4 MB; 2048x448x2048: 10.0 / 13.9).
+    if (v.direct && want > 1 && (double)steps * (double)(want - 1) / (double)want < 35.0 + 6.5e-6 * 4.0 * (double)want * (double)g.M * (double)g.N) return 1;
     SplitPlan sp;
     return want > 1 && plan_split(v, pb, (int)want, &sp, max_floats) ? sp.splits : 1;
 }
@@ -456,8 +479,13 @@ int choose(const Problem& pb, int variant, int k_splits, Choice* c, size_t max_s
         }
         int mv = auto_mfma_variant(pb);
         if (pb.g.in_type == T_F32 && f32_can_take(pb.g)) {
-            // fp32: the LDS-tiled kernels when their workgroups (tiles x K slices) fill at least half of the chip, else the kernel
-            // of 32 x 32 blocks (512^3: 16 tiles of 128 x 128 would keep 16 CUs busy)
+            // fp32: the kernel of 32 x 32 blocks against the LDS-tiled kernels.  Where a tiled kernel with direct fills takes
+            // the problem it is level or ahead, up to three times with a short K (1152x384x64: 4.8 against 8.2 us;
+            // 768x576x1024: 17.1 in four slices against 26.3; 2048x192x1280: 17.3 against 27.4), except when the 32 x 32 blocks
+            // are one round over most of the chip (512^3, 256 blocks: 9.4 against 10.0 to 11.4 us).  Against the register-staged
+            // tiled kernels (unaligned operands) the kernel of blocks wins while the tiles x K slices leave half of the chip
+            // idle (800x128x49 with a column-major A: 7.5 against 8.3 us; 512^3 would be 16 tiles of 128 x 128 on 16 CUs), and
+            // loses beyond (6272x256x528: 39.7 against 27.5; 256x32x784 in 32 slices: 8.7 against 17.3).
             int slices = 1;
             if (mv >= 0) {
                 int n = 0;
@@ -467,7 +495,9 @@ int choose(const Problem& pb, int variant, int k_splits, Choice* c, size_t max_s
                 const int64_t tiles = (((int64_t)pb.g.M + v.bm - 1) / v.bm) * (((int64_t)pb.g.N + v.bn - 1) / v.bn);
                 // (or more workgroups than there are 32 x 32 blocks: a small output with a long K, which only the tiled kernels split)
                 const int64_t blocks = (((int64_t)pb.g.M + 31) / 32) * (((int64_t)pb.g.N + 31) / 32);
-                if (tiles * slices * 2 < kComputeUnits && tiles * slices <= blocks) mv = -1;
+                const bool lean = pb.g.prologue == PRO_SET; // (reading C, the tiled kernels are ahead at 512^3 too: 8.9 to 9.3 against 11.1 to 12.7 us)
+                if (v.direct ? (blocks <= kComputeUnits && blocks * 2 > kComputeUnits && slices == 1 && lean && pb.g.K >= 256)
+                             : (tiles * slices * 2 < kComputeUnits && tiles * slices <= blocks)) mv = -1;
             }
             if (mv < 0) { c->variant = ACC950_VARIANT_F32_MFMA; return ACC950_OK; }
         }

@@ -20,6 +20,12 @@ tools/benchmarkers/gemm_*.csv; transX = 1 means the operand is stored column-maj
 
     python -m accera_amd.tune --input accera_amd/shapes/transformer_gemm.csv --type f16 --check --relu
 
+    python -m accera_amd.tune --audit sweep.csv
+
+reads a csv that --output wrote and compares, row by row of the shape list, the kernel and K slices the library takes
+by itself (its cost model; the table of recorded choices is left out) with the fastest (variant, slices) of the sweep:
+the geometric mean of chosen / best and the rows furthest off.  Needs no GPU: calls are bound, never launched.
+
 alpha / beta map to the fragment ops: beta 0 -> prologue SET 0, beta 1 -> none, else SCALE beta;
 alpha != 1 -> epilogue SCALE alpha (a ReLU epilogue and alpha != 1 exclude each other, as in the
 reference's table docs/Tutorials/GPU/Tensor_MatMul_ElementWiseOps_GPU.md:85-99).
@@ -172,9 +178,64 @@ def sweep(rows, in_type, relu, check, out_type=None, min_time_s=0.05, log=print,
     return results
 
 
+def own_choice(in_id, out_id, M, N, K, a_col_major, b_col_major, alpha, beta):
+    """(variant, K slices) the library's cost model takes for dense operands, without the table of recorded choices.
+    The call is bound with made-up 256-byte aligned addresses and unbound again: nothing is launched."""
+    import ctypes
+    L = _lib.lib()
+    sa = (1, M) if a_col_major else (K, 1)
+    sb = (1, K) if b_col_major else (N, 1)
+    pro, parg = (_lib.PROLOGUE_SET0, 0.0) if beta == 0 else (_lib.PROLOGUE_NONE, 0.0) if beta == 1 else (_lib.PROLOGUE_SCALE, beta)
+    epi, earg = (_lib.EPILOGUE_SCALE, alpha) if alpha != 1 else (_lib.EPILOGUE_RELU, 0.0)
+    handle, v, ks = ctypes.c_int(-1), ctypes.c_int(), ctypes.c_int()
+    P = ctypes.c_void_p
+    _lib.check(L.acc950_bind(in_id, out_id, 1, M, N, K, P(1 << 32), 0, sa[0], sa[1], P(2 << 32), 0, sb[0], sb[1], P(3 << 32), 0, N, 1,
+                             pro, float(parg), epi, float(earg), _lib.VARIANT_AUTO, 0, None, ctypes.byref(handle)))
+    try:
+        _lib.check(L.acc950_bound_choice(handle.value, ctypes.byref(v), ctypes.byref(ks)))
+    finally:
+        L.acc950_unbind(handle.value)
+    return v.value, max(ks.value, 1)
+
+
+def audit(path, worst=10, log=print):
+    """The library's own choice against the fastest entry of a sweep csv, per problem.  A choice of K slices the sweep did
+    not time (it tries 2, 4, 8, 16, 32) is read at the nearest count it did.  Returns (geometric mean of chosen / best,
+    [(ratio, problem, chosen kernel, slices, its ms, best kernel, slices, its ms), ...] worst first)."""
+    import math
+    problems = {}
+    with open(path) as f:
+        for r in csv.DictReader(f):
+            if int(r["variant"]) == -2:  # the vendor library's row
+                continue
+            key = (r["type"], r["out_type"], int(r["m"]), int(r["n"]), int(r["k"]), int(r["transA"]), int(r["transB"]), float(r["alpha"]), float(r["beta"]))
+            problems.setdefault(key, {})[(r["kernel"], max(int(r["k_splits"]), 1))] = float(r["time_ms"])
+    rows = []
+    for key, timed in problems.items():
+        t, ot, M, N, K, ta, tb, alpha, beta = key
+        v, ks = own_choice(getattr(_lib, t.upper()), getattr(_lib, ot.upper()), M, N, K, ta, tb, alpha, beta)
+        name = _lib.variant_name(v)
+        same = sorted((abs(math.log2(s) - math.log2(ks)), ms) for (n, s), ms in timed.items() if n == name)
+        if not same:
+            log(f"{M}x{N}x{K} tA={ta} tB={tb}: the sweep has no row for the chosen kernel ({name})")
+            continue
+        (best_name, best_ks), best_ms = min(timed.items(), key=lambda x: x[1])
+        rows.append((same[0][1] / best_ms, key, name, ks, same[0][1], best_name, best_ks, best_ms))
+    rows.sort(key=lambda x: -x[0])
+    if not rows:
+        return float("nan"), rows
+    geomean = math.exp(sum(math.log(r[0]) for r in rows) / len(rows))
+    for ratio, key, name, ks, ms, best_name, best_ks, best_ms in rows[:worst]:
+        log(f"{ratio:.2f}  {key[2]}x{key[3]}x{key[4]} tA={key[5]} tB={key[6]} a={key[7]} b={key[8]}: chosen {name} x{ks} {ms} ms | best {best_name} x{best_ks} {best_ms} ms")
+    log(f"{len(rows)} problems: geometric mean of chosen / best {geomean:.4f}, {sum(r[0] > 1.10 for r in rows)} more than 10 % off, "
+        f"{sum(r[0] > 1.25 for r in rows)} more than 25 % off")
+    return geomean, rows
+
+
 def main(argv=None):
     ap = argparse.ArgumentParser(description=__doc__.split("\n")[0])
-    ap.add_argument("--input", required=True, help="shape list (csv: m,n,k,transA,transB,alpha,beta,...)")
+    ap.add_argument("--input", default=None, help="shape list (csv: m,n,k,transA,transB,alpha,beta,...)")
+    ap.add_argument("--audit", default=None, metavar="CSV", help="compare the library's own choices with the best rows of a csv that --output wrote (no GPU needed)")
     ap.add_argument("--type", default="f16", choices=sorted(_OUT_FOR))
     ap.add_argument("--out-type", default=None, choices=["f32", "f16", "bf16", "i32", "i16", "i8"])
     ap.add_argument("--relu", action="store_true", help="fused ReLU epilogue (rows with alpha != 1 are rejected)")
@@ -186,6 +247,11 @@ def main(argv=None):
                     help="record the best variant per shape in the table that automatic kernel choices consult "
                          "(default: accera_amd/shapes/tuned_gfx950.json)")
     args = ap.parse_args(argv)
+    if args.audit:
+        audit(args.audit)
+        return 0
+    if not args.input:
+        ap.error("--input or --audit is required")
     with open(args.input) as f:
         rows = [r for r in csv.DictReader(f) if r.get("m")]
     _lib.check(_lib.lib().acc950_init(0))

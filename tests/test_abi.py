@@ -121,6 +121,55 @@ def test_sweep_tool_lists_the_variants_that_take_a_problem():
     assert len(rows) >= 10 and {"m", "n", "k", "transA", "transB", "alpha", "beta"} <= set(rows[0])
 
 
+def test_sweep_tool_audits_the_library_s_own_choice(tmp_path):
+    """accera_amd.tune --audit: the kernel and K slices the library takes by itself against the fastest row of a sweep csv."""
+    import csv
+    from accera_amd import tune
+    v, ks = tune.own_choice(_lib.F16, _lib.F32, 4096, 4096, 4096, False, False, 1.0, 0.0)
+    chosen = _lib.variant_name(v)
+    assert "hand-laid loop" in chosen and ks == 1
+    other = next(_lib.variant_name(i) for i in range(_lib.num_variants()) if "pingpong" in _lib.variant_name(i))
+    rows = [dict(m=4096, n=4096, k=4096, transA=0, transB=0, alpha=1.0, beta=0.0, type="f16", out_type="f32", variant=v, k_splits=0, kernel=chosen, time_ms=0.1),
+            dict(m=4096, n=4096, k=4096, transA=0, transB=0, alpha=1.0, beta=0.0, type="f16", out_type="f32", variant=0, k_splits=0, kernel=other, time_ms=0.08),
+            dict(m=4096, n=4096, k=4096, transA=0, transB=0, alpha=1.0, beta=0.0, type="f16", out_type="f16", variant=-2, k_splits=0, kernel="vendor library (torch.matmul)", time_ms=0.01)]
+    path = tmp_path / "sweep.csv"
+    with open(path, "w", newline="") as f:
+        w = csv.DictWriter(f, fieldnames=list(rows[0]))
+        w.writeheader()
+        w.writerows(rows)
+    lines = []
+    geomean, worst = tune.audit(str(path), log=lines.append)
+    assert abs(geomean - 1.25) < 1e-9 and len(worst) == 1 and worst[0][2] == chosen and worst[0][5] == other   # (the vendor row is no candidate)
+    assert "1 problems" in lines[-1] and "1.2500" in lines[-1]
+
+
+def test_choices_of_the_cost_model():
+    """What the library takes by itself where measurements decided it (numbers in capi.hip next to each rule)."""
+    from accera_amd import tune
+    name = lambda *a: (lambda v, ks: (_lib.variant_name(v), ks))(*tune.own_choice(*a))
+    # a last round that is half empty does not cost a whole round: one and a half rounds of 256 x 256 tiles stay on the four-wave kernel
+    n, ks = name(_lib.F16, _lib.F16, 2048, 12288, 4096, False, False, 1.0, 0.0)
+    assert "256x256" in n and "hand-laid loop" in n and ks == 1
+    # a short K is not split, however few the tiles; a long one is
+    assert name(_lib.F16, _lib.F16, 256, 256, 256, False, False, 1.0, 1.0)[1] == 1
+    assert name(_lib.F16, _lib.F16, 64, 1152, 448, False, False, 1.0, 0.0)[1] == 1
+    assert name(_lib.F16, _lib.F16, 2048, 256, 1536, False, False, 1.0, 0.0)[1] == 1      # (128 tiles: the partial sums cost more than the slices save)
+    assert name(_lib.F16, _lib.F16, 64, 320, 1728, False, False, 1.0, 0.0)[1] > 1
+    assert name(_lib.F16, _lib.F16, 768, 320, 30522, False, False, 1.0, 0.0)[1] >= 8
+    # register-staged kernels (unaligned K) with a column-major A that read C: their slow steps are worth splitting early
+    assert name(_lib.F16, _lib.F16, 512, 128, 196, True, False, 1.0, 1.0)[1] > 1
+    assert name(_lib.F16, _lib.F16, 6272, 32, 513, False, False, 1.0, 0.0)[1] == 1
+    # 128 x 128 tiles, two workgroups per CU: two stages of 128 bytes of K
+    n, _ = name(_lib.F16, _lib.F16, 3072, 2304, 4096, False, True, 1.0, 1.0)
+    assert ("128x128 kb128" in n and "stages=2" in n) or "256x256" in n
+    # fp32: tiled kernels with direct fills where they apply, the kernel of 32 x 32 blocks for one round of blocks (512^3) and against the register-staged kernels
+    assert "fp32 mfma 32x32" in name(_lib.F32, _lib.F32, 512, 512, 512, False, False, 1.0, 0.0)[0]
+    assert "64x64" in name(_lib.F32, _lib.F32, 1152, 384, 64, True, False, 1.0, 1.0)[0]
+    n, ks = name(_lib.F32, _lib.F32, 768, 576, 1024, False, False, 1.0, 1.0)
+    assert "fill=direct" in n and ks > 1
+    assert "fp32 mfma 32x32" in name(_lib.F32, _lib.F32, 800, 126, 49, True, False, 1.0, 1.0)[0]
+
+
 def test_bound_call_handles_without_launching():
     """acc950_bind validates and chooses once; handles are reused after acc950_unbind; unknown handles
     are reported.  (No launch here: there is no GPU on the CPU test tier.)"""
