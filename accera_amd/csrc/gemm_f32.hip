@@ -71,17 +71,42 @@ __global__ void __launch_bounds__(256) gemm_f32_kernel(GemmArgs p)
     }
     __syncthreads();
     if (wave > 0) return;
+    // The tail is laid out as passes over all 16 elements -- partial sums out of LDS, old C (only when the prologue keeps
+    // it), prologue, epilogue (one test of the op, outside the pass), stores -- so that the reads of a pass are all under
+    // way before the first is used and no store waits for another.  Written element by element (sum, test the ops, maybe
+    // load C, store) the compiler kept that order: a wait for LDS and a dozen branches per element, and every store
+    // behind the memory counter of a possible load (512^3: 9.4 us then, 7.5 now; 512 x 512 x 16: 5.9 / 3.8).
+    float v[16];
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-        float v = acc[i] + red[0][i][lane] + red[1][i][lane] + red[2][i][lane];
-        const int orow = blockIdx.y * 32 + (i >> 2) * 8 + kh * 4 + (i & 3);
-        const int ocol = blockIdx.x * 32 + r;
-        if (orow >= p.M || ocol >= p.N) continue;
-        float* C = (float*)p.C;
-        const int64_t idx = (int64_t)orow * p.c_rs + (int64_t)ocol * p.c_cs;
-        v = apply_prologue<float>(v, p.prologue, p.prologue_arg, [&]() { return C[idx]; });
-        C[idx] = apply_epilogue<float>(v, p.epilogue, p.epilogue_arg);
+    for (int i = 0; i < 16; ++i) v[i] = acc[i] + red[0][i][lane] + red[1][i][lane] + red[2][i][lane];
+    float* C = (float*)p.C;
+    const int ocol = blockIdx.x * 32 + r;
+    const int orow0 = blockIdx.y * 32 + kh * 4;
+    const int64_t idx0 = (int64_t)orow0 * p.c_rs + (int64_t)ocol * p.c_cs;
+    auto row_of = [](int i) { return (i >> 2) * 8 + (i & 3); };
+    // (rows of C this lane may touch: all 16 inside a full block, fewer at the lower edge; none for a column beyond N)
+    const int rows_in = ocol < p.N ? p.M - orow0 : 0;
+    if (p.prologue == PRO_SET) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) v[i] += p.prologue_arg;
+    } else {
+        float old[16];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) old[i] = row_of(i) < rows_in ? C[idx0 + (int64_t)row_of(i) * p.c_rs] : 0.f;
+        const float c_mul = p.prologue == PRO_SCALE ? p.prologue_arg : 1.f; // (x 1 is exact)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) v[i] += old[i] * c_mul;
     }
+    if (p.epilogue == EPI_RELU) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) v[i] = v[i] > 0.f ? v[i] : 0.f;
+    } else if (p.epilogue != EPI_NONE) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) v[i] = apply_epilogue<float>(v[i], p.epilogue, p.epilogue_arg);
+    }
+#pragma unroll
+    for (int i = 0; i < 16; ++i)
+        if (row_of(i) < rows_in) C[idx0 + (int64_t)row_of(i) * p.c_rs] = v[i];
 }
 
 bool vec_ok(const void* ptr, int64_t ld, int K, bool have_pointers = true)
