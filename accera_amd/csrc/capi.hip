@@ -479,13 +479,14 @@ int choose(const Problem& pb, int variant, int k_splits, Choice* c, size_t max_s
         }
         int mv = auto_mfma_variant(pb);
         if (pb.g.in_type == T_F32 && f32_can_take(pb.g)) {
-            // fp32: the kernel of 32 x 32 blocks against the LDS-tiled kernels.  Where a tiled kernel with direct fills takes
-            // the problem it is level or ahead, up to three times with a short K (1152x384x64: 4.8 against 8.2 us;
-            // 768x576x1024: 17.1 in four slices against 26.3; 2048x192x1280: 17.3 against 27.4), except when the 32 x 32 blocks
-            // are one round over most of the chip (512^3, 256 blocks: 9.4 against 10.0 to 11.4 us).  Against the register-staged
-            // tiled kernels (unaligned operands) the kernel of blocks wins while the tiles x K slices leave half of the chip
-            // idle (800x128x49 with a column-major A: 7.5 against 8.3 us; 512^3 would be 16 tiles of 128 x 128 on 16 CUs), and
-            // loses beyond (6272x256x528: 39.7 against 27.5; 256x32x784 in 32 slices: 8.7 against 17.3).
+            // fp32: the kernel of 32 x 32 blocks against the LDS-tiled kernels.  The kernel of blocks is ahead while its blocks
+            // are at most one round over the chip and K is short (sweep of the reference's 339 shapes: best on 81 of the 86
+            // problems with up to 256 blocks and K <= 640 -- 512^3 7.5 us against 8.9 to 10.4, 256x1024x196 with a
+            // column-major A 4.8 against 10.6 -- and on 6 of the 74 with a longer K, where the tiled kernels split K:
+            // 64x192x1728 9.9 us in 16 slices against 18.5); with more blocks the tiled kernels with direct fills win
+            // (768x576x1024: 17.1 in four slices against 26.3; 2048x192x1280: 17.3 against 27.4).  Against the
+            // register-staged tiled kernels (unaligned operands) the kernel of blocks also wins with a K up to 768, and with a
+            // longer one while the tiles x K slices leave half of the chip idle.
             int slices = 1;
             if (mv >= 0) {
                 int n = 0;
@@ -495,9 +496,10 @@ int choose(const Problem& pb, int variant, int k_splits, Choice* c, size_t max_s
                 const int64_t tiles = (((int64_t)pb.g.M + v.bm - 1) / v.bm) * (((int64_t)pb.g.N + v.bn - 1) / v.bn);
                 // (or more workgroups than there are 32 x 32 blocks: a small output with a long K, which only the tiled kernels split)
                 const int64_t blocks = (((int64_t)pb.g.M + 31) / 32) * (((int64_t)pb.g.N + 31) / 32);
-                const bool lean = pb.g.prologue == PRO_SET; // (reading C, the tiled kernels are ahead at 512^3 too: 8.9 to 9.3 against 11.1 to 12.7 us)
-                if (v.direct ? (blocks <= kComputeUnits && blocks * 2 > kComputeUnits && slices == 1 && lean && pb.g.K >= 256)
-                             : (tiles * slices * 2 < kComputeUnits && tiles * slices <= blocks)) mv = -1;
+                const bool one_round = blocks <= kComputeUnits && pb.g.K <= 640;
+                // (against the register-staged kernels a short K is enough: 2304x256x196 with a column-major A, 576 blocks,
+                // 8.4 against 14.1 us; 4608x512x49, 2304 blocks, 16.8 against 19.0; but 1728x192x1225 24.1 against 19.8)
+                if (one_round || (!v.direct && (pb.g.K <= 768 || (tiles * slices * 2 < kComputeUnits && tiles * slices <= blocks)))) mv = -1;
             }
             if (mv < 0) { c->variant = ACC950_VARIANT_F32_MFMA; return ACC950_OK; }
         }
