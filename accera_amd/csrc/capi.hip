@@ -428,20 +428,18 @@ int auto_mfma_splits(const MfmaVariant& v, const Problem& pb, size_t max_floats 
     if (g.batch > 1) return 1;
     const int64_t tiles = (((int64_t)g.M + v.bm - 1) / v.bm) * (((int64_t)g.N + v.bn - 1) / v.bn);
     if (tiles * 2 > kComputeUnits) return 1;
-    // K in steps of 0.1 us: what 64 bytes of K cost a 64 x 64 tile with direct fills.  The register-staged kernels take two
-    // to three times as long per step, twice that with a column-major A (which they transpose on the way), and their
-    // element-wise read of C costs as much again (the second kernel of a split reads C in rows instead); a 128 x 128 tile
-    // takes about twice, a 256 x 256 tile about five times as long per step as a 64 x 64 one.
+    // K in steps of 64 bytes, and in units of 0.1 us: what such a step costs a 64 x 64 tile with direct fills.  The
+    // register-staged kernels take about three times as long per step, a 128 x 128 tile about twice and a 256 x 256 tile
+    // about five times as long as a 64 x 64 one, fp32 twice as long as the 8- and 16-bit types.
     const int64_t area = (int64_t)v.bm * v.bn;
-    const int64_t raw_steps = (int64_t)g.K * elem_size(g.in_type) / 64;
-    const int64_t steps = raw_steps * (v.direct ? 1 : (v.a_kc ? 2 : 4) * (g.prologue != PRO_SET ? 2 : 1)) * (area <= 64 * 64 ? 1 : area <= 128 * 128 ? 2 : 4) *
-                          (g.in_type == T_F32 ? 2 : 1); // (fp32: 512^3 on 64 tiles 8.9 us, 256^3 5.0)
-    // The second kernel costs 3 to 5 us: below 48 steps a split only loses, however few the tiles (fp16, 64 x 64 tiles,
-    // unsplit / best split in us, direct: 256^3 3.1 / 5.8; 64x1152x448 4.3 / 7.0; 289x192x1344 7.2 / 7.6; 64x320x1728
-    // 8.4 / 7.4; 576x192x3136 11.9 / 7.9; register-staged: 6272x32x512 7.3 / 9.2; 196x128x800 9.6 / 7.9; reading C:
-    // 384x288x512 9.0 / 5.9; with a column-major A: 512x128x196 8.4 / 5.8, 384x192x1225 16.6 / 7.2; int8 363x64x3025
+    const int64_t steps = (int64_t)g.K * elem_size(g.in_type) / 64;
+    const int64_t worth = steps * (v.direct ? 1 : 3) * (area <= 64 * 64 ? 1 : area <= 128 * 128 ? 2 : 4) * (g.in_type == T_F32 ? 2 : 1);
+    // The second kernel costs 3 to 5 us: a K worth less than 48 units only loses by a split, however few the tiles (launches
+    // back to back from a C++ loop, fp16, 64 x 64 tiles, unsplit / split in us -- direct: 64x1536x256 4.1 / 6.7; 256^3
+    // 5.0 / 7.7; 64x320x1728 8.4 / 7.4; 576x192x3136 11.9 / 7.9; register-staged: 196x48x400 6.6 / 8.3; 6272x32x512
+    // 7.3 / 8.8; 512x32x196 with a column-major A 7.2 / 9.3; 196x64x800 8.5 in four slices, 7.8 in six; int8 363x64x3025
     // 46.9 / 10.8).
-    if (steps < 48) return 1;
+    if (worth < 48) return 1;
     // Slices of about 32 k-steps; shorter ones, down to 4, while that keeps the workgroups at or below one per compute unit;
     // never more workgroups than the compute units hold at once (two of the 64 x 64 tiles each), never more than 32 slices.
     // Measured with 64 x 64 tiles, fp16, us by slices 4 / 8 / 16 / 32: 768x320x30522 84 / 53 / 49 / 53; 1024x80x30522
@@ -455,7 +453,7 @@ int auto_mfma_splits(const MfmaVariant& v, const Problem& pb, size_t max_floats 
     if ((size_t)want * (size_t)g.M * (size_t)g.N > ((size_t)1 << 24)) return 1; // 64 MiB of partial sums at most without being asked
     // What the slices save against what the second kernel costs, 3.5 us and 0.65 us per MB of partial sums written and read
     // (2048x256x1536 on 128 tiles: 8.2 us unsplit, 10.7 in two slices with their 4 MB; 2048x448x2048: 10.0 / 13.9).
-    if (v.direct && want > 1 && (double)steps * (double)(want - 1) / (double)want < 35.0 + 6.5e-6 * 4.0 * (double)want * (double)g.M * (double)g.N) return 1;
+    if (want > 1 && (double)worth * (double)(want - 1) / (double)want < 35.0 + 6.5e-6 * 4.0 * (double)want * (double)g.M * (double)g.N) return 1;
     SplitPlan sp;
     return want > 1 && plan_split(v, pb, (int)want, &sp, max_floats) ? sp.splits : 1;
 }

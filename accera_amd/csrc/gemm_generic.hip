@@ -70,19 +70,36 @@ __global__ void __launch_bounds__(256) gemm_generic_kernel(GemmArgs p)
         __syncthreads();
     }
 
+    // Passes over the thread's elements: old C first (only when the prologue keeps it), then the ops, then the stores.  A
+    // load inside the loop over the elements, behind the test of the prologue op, would put every store behind the memory
+    // counter of that possible load: one store round trip after the other.
+    const bool keeps_c = p.prologue != PRO_SET;
+    AccT old[GC][GC];
 #pragma unroll
     for (int i = 0; i < GC; ++i)
 #pragma unroll
         for (int j = 0; j < GC; ++j) {
-            int m = m0 + ty + 16 * i, n = n0 + tx + 16 * j;
+            old[i][j] = AccT(0);
+            const int m = m0 + ty + 16 * i, n = n0 + tx + 16 * j;
+            if (keeps_c && m < p.M && n < p.N) {
+                const int64_t idx = m * p.c_rs + n * p.c_cs;
+                if constexpr (std::is_same<AccT, int>::value) old[i][j] = load_out_int(p.C, p.out_type, idx);
+                else old[i][j] = load_out(p.C, p.out_type, idx);
+            }
+        }
+#pragma unroll
+    for (int i = 0; i < GC; ++i)
+#pragma unroll
+        for (int j = 0; j < GC; ++j) {
+            const int m = m0 + ty + 16 * i, n = n0 + tx + 16 * j;
             if (m >= p.M || n >= p.N) continue;
-            int64_t idx = m * p.c_rs + n * p.c_cs;
-            AccT v = acc[i][j];
+            const int64_t idx = m * p.c_rs + n * p.c_cs;
+            const AccT c_old = old[i][j];
             if constexpr (std::is_same<AccT, int>::value) {
-                v = apply_prologue<int>(v, p.prologue, p.prologue_arg, [&]() { return load_out_int(p.C, p.out_type, idx); });
+                const int v = apply_prologue<int>(acc[i][j], p.prologue, p.prologue_arg, [&]() { return c_old; });
                 store_out_int(p.C, p.out_type, idx, apply_epilogue<int>(v, p.epilogue, p.epilogue_arg));
             } else {
-                v = apply_prologue<float>(v, p.prologue, p.prologue_arg, [&]() { return load_out(p.C, p.out_type, idx); });
+                const float v = apply_prologue<float>(acc[i][j], p.prologue, p.prologue_arg, [&]() { return c_old; });
                 store_out(p.C, p.out_type, idx, apply_epilogue<float>(v, p.epilogue, p.epilogue_arg));
             }
         }

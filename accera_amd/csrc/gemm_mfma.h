@@ -780,17 +780,32 @@ __global__ void __launch_bounds__(Cfg::NT, Cfg::WGS_PER_CU) gemm_mfma_kernel(Gem
             }
         };
         auto offset_of = [&](int i, int r, int j) { return lane_off + ((unsigned)(i * 32 + (r >> 2) * 8 + (r & 3)) * row_bytes + ((unsigned)(j * 32) << sh)); };
-        if constexpr (TM * TN * 16 <= 64 && !EDGE) {
+        if constexpr (TM * TN * 16 <= 64) {
             // A small wave tile (64 sums per lane) has the registers for a second copy: all of its loads are issued before the
             // first is used, so the tile of C costs one trip through memory instead of one per eight loads (left to the
-            // compiler's own order: 7 us of a 29 us launch at 2048^3 with 128 x 128 tiles).
+            // compiler's own order: 7 us of a 29 us launch at 2048^3 with 128 x 128 tiles).  The edge kernels read the same
+            // way, their tests of the edges around the load alone: with the use inside the test as well, every load waited
+            // for the one before (a wait for memory sits where the skipped and the loaded paths join), 16 to 64 trips
+            // through memory in a row -- 600x64x196 int8 with beta = 1: 10.0 us, 5.0 this way.  (Loads without any test,
+            // the descriptor's range check as the only guard, were tried too: the compiler then put a wait for memory in
+            // front of every store of the fp16 / bf16 kernels.)
             unsigned words[TM][16][TN];
 #pragma unroll
             for (int i = 0; i < TM; ++i)
 #pragma unroll
                 for (int r = 0; r < 16; ++r)
 #pragma unroll
-                    for (int j = 0; j < TN; ++j) words[i][r][j] = __builtin_amdgcn_raw_buffer_load_b32(tile.rsrc, offset_of(i, r, j) & ~3u, 0, 0);
+                    for (int j = 0; j < TN; ++j) {
+                        const bool inside = !EDGE || (m0 + row_in_tile + i * 32 + (r >> 2) * 8 + (r & 3) < p.M && n0 + col_in_tile + j * 32 < p.N);
+                        const unsigned off = offset_of(i, r, j) & ~3u;
+                        if constexpr (IN == IN_I8) {
+                            // (a lane outside reads at an offset beyond any descriptor's range: the range check answers with 0)
+                            words[i][r][j] = __builtin_amdgcn_raw_buffer_load_b32(tile.rsrc, inside ? off : 0xfffffffcu, 0, 0);
+                        } else {
+                            words[i][r][j] = 0;
+                            if (inside) words[i][r][j] = __builtin_amdgcn_raw_buffer_load_b32(tile.rsrc, off, 0, 0);
+                        }
+                    }
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int i = 0; i < TM; ++i)
