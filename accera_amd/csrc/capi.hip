@@ -106,6 +106,9 @@ int make_problem(int in_type, int out_type, int M, int N, int K,
         g.A = B; g.B = A; g.C = C; g.M = N; g.N = M; g.K = K;
         g.a_rs = b_cs; g.a_cs = b_rs; g.b_rs = a_cs; g.b_cs = a_rs; g.c_rs = c_cs; g.c_cs = c_rs;
     }
+    // (the kernels take these two strides as 32-bit arguments)
+    if (g.a_cs > 0x7fffffffll || g.b_cs > 0x7fffffffll)
+        return fail(ACC950_UNSUPPORTED, "the stride of A between consecutive k and the stride of B between consecutive columns must be below 2^31 elements");
     g.batch = batch.count;
     g.a_bs = transpose ? batch.b_bs : batch.a_bs;
     g.b_bs = transpose ? batch.a_bs : batch.b_bs;

@@ -141,11 +141,38 @@ __device__ __forceinline__ int load_out_int(const void* C, int out_type, int64_t
     return ((const int8_t*)C)[idx];
 }
 
+// The first 16 dwords of a kernel's arguments are preloaded into scalar registers when the kernel is dispatched (the
+// translation units are built with -amdgpu-kernarg-preload-count=16); what lies behind them is fetched by the kernel itself,
+// a trip through memory of about 0.4 us before its first address can be formed (an empty kernel: 2.5 us from launch to
+// launch; one that loads and stores a few bytes: 3.0 us with its arguments fetched, 2.6 with them preloaded).  Only scalar
+// and pointer arguments are preloaded, not a struct, so the kernels take the fields they need first -- operand pointers,
+// sizes, strides -- as arguments of their own in front of the struct and put them back into their copy of it.
+// (14 dwords fit beside the registers the dispatch itself needs: two pointers, three sizes, the element strides of A and B
+// along K -- 32 bits: the entry points refuse larger ones --, the stagger switch of the multi-tile kernels, which they test
+// first thing, and the two row strides.  The MFMA kernels work out their tile counts from M and N themselves.)
+#define ACC950_HEAD_PARAMS const void* head_A, const void* head_B, int head_M, int head_N, int head_K, int head_a_cs, int head_b_cs, \
+                           int head_stagger_groups, int64_t head_a_rs, int64_t head_b_rs
+#define ACC950_HEAD_OF(g) (g).A, (g).B, (g).M, (g).N, (g).K, (int)(g).a_cs, (int)(g).b_cs, (g).stagger_groups, (g).a_rs, (g).b_rs
+#define ACC950_TAKE_HEAD(p)                                                                                                      \
+    do {                                                                                                                          \
+        (p).A = head_A; (p).B = head_B; (p).M = head_M; (p).N = head_N; (p).K = head_K; (p).stagger_groups = head_stagger_groups; \
+        (p).a_rs = head_a_rs; (p).b_rs = head_b_rs; (p).a_cs = head_a_cs; (p).b_cs = head_b_cs;                                   \
+    } while (0)
+// (the MFMA kernels: tile counts as their launchers set them)
+#define ACC950_TAKE_HEAD_TILES(p, BM_, BN_)                                                   \
+    do {                                                                                      \
+        ACC950_TAKE_HEAD(p);                                                                  \
+        (p).tiles_m = ((p).M + (BM_) - 1) / (BM_); (p).tiles_n = ((p).N + (BN_) - 1) / (BN_); \
+    } while (0)
+
 // Batched launch: blockIdx.z picks the problem; the kernel then sees one plain GEMM.
 __device__ __forceinline__ int elem_bytes(int type) { return type == T_I8 ? 1 : (type == T_F16 || type == T_BF16 || type == T_I16) ? 2 : 4; }
+// (Problem 0 needs none of this -- a K split has at least two slices, so its last slice is never slice 0 -- and a plain
+// GEMM is all problem 0: its workgroups do not wait for the batch fields, which are not among the preloaded arguments.)
 __device__ __forceinline__ void select_batch(GemmArgs& p)
 {
     const int64_t z = blockIdx.z;
+    if (z == 0) return;
     p.A = (const char*)p.A + z * p.a_bs * elem_bytes(p.in_type);
     p.B = (const char*)p.B + z * p.b_bs * elem_bytes(p.in_type);
     p.C = (char*)p.C + z * p.c_bs * elem_bytes(p.out_type);

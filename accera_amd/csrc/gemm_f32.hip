@@ -34,9 +34,10 @@ __device__ __forceinline__ void load_frag(float (&f)[4], const float* X, int64_t
 }
 
 template <bool A_KC, bool B_KC>
-__global__ void __launch_bounds__(256) gemm_f32_kernel(GemmArgs p)
+__global__ void __launch_bounds__(256) gemm_f32_kernel(ACC950_HEAD_PARAMS, GemmArgs p)
 {
     __shared__ float red[3][16][64];
+    ACC950_TAKE_HEAD(p);
     select_batch(p);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int r = lane & 31, kh = lane >> 5;
@@ -132,10 +133,10 @@ hipError_t launch_f32(const GemmArgs& g, hipStream_t stream, LaunchGeom* geom, b
     // prefer the vector (K contiguous) form of an operand when its layout allows it
     const bool a_kc = g.a_cs == 1 && vec_ok(g.A, g.a_rs, g.K, true);
     const bool b_kc = g.b_rs == 1 && vec_ok(g.B, g.b_cs, g.K, true);
-    if (a_kc && b_kc) hipLaunchKernelGGL((gemm_f32_kernel<true, true>), grid, block, 0, stream, g);
-    else if (a_kc) hipLaunchKernelGGL((gemm_f32_kernel<true, false>), grid, block, 0, stream, g);
-    else if (b_kc) hipLaunchKernelGGL((gemm_f32_kernel<false, true>), grid, block, 0, stream, g);
-    else hipLaunchKernelGGL((gemm_f32_kernel<false, false>), grid, block, 0, stream, g);
+    if (a_kc && b_kc) hipLaunchKernelGGL((gemm_f32_kernel<true, true>), grid, block, 0, stream, ACC950_HEAD_OF(g), g);
+    else if (a_kc) hipLaunchKernelGGL((gemm_f32_kernel<true, false>), grid, block, 0, stream, ACC950_HEAD_OF(g), g);
+    else if (b_kc) hipLaunchKernelGGL((gemm_f32_kernel<false, true>), grid, block, 0, stream, ACC950_HEAD_OF(g), g);
+    else hipLaunchKernelGGL((gemm_f32_kernel<false, false>), grid, block, 0, stream, ACC950_HEAD_OF(g), g);
     return hipGetLastError();
 }
 

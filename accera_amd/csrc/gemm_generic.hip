@@ -28,10 +28,11 @@ __device__ __forceinline__ AccT load_in(const void* p, int type, int64_t idx)
 }
 
 template <typename AccT>
-__global__ void __launch_bounds__(256) gemm_generic_kernel(GemmArgs p)
+__global__ void __launch_bounds__(256) gemm_generic_kernel(ACC950_HEAD_PARAMS, GemmArgs p)
 {
     __shared__ AccT sA[GK][GT + 1]; // [k][m]
     __shared__ AccT sB[GK][GT + 1]; // [k][n]
+    ACC950_TAKE_HEAD(p);
     select_batch(p);
     const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
     const int m0 = blockIdx.y * GT, n0 = blockIdx.x * GT;
@@ -117,9 +118,9 @@ hipError_t launch_generic(const GemmArgs& a, hipStream_t stream, LaunchGeom* geo
     }
     if (dry_run) return hipSuccess;
     if (a.in_type == T_I8)
-        hipLaunchKernelGGL(gemm_generic_kernel<int>, grid, block, 0, stream, a);
+        hipLaunchKernelGGL(gemm_generic_kernel<int>, grid, block, 0, stream, ACC950_HEAD_OF(a), a);
     else
-        hipLaunchKernelGGL(gemm_generic_kernel<float>, grid, block, 0, stream, a);
+        hipLaunchKernelGGL(gemm_generic_kernel<float>, grid, block, 0, stream, ACC950_HEAD_OF(a), a);
     return hipGetLastError();
 }
 

@@ -48,7 +48,7 @@ struct Mfma16Config {
 };
 
 template <typename Cfg>
-__global__ void __launch_bounds__(Cfg::NT, 1) gemm_mfma16_kernel(GemmArgs p)
+__global__ void __launch_bounds__(Cfg::NT, 1) gemm_mfma16_kernel(ACC950_HEAD_PARAMS, GemmArgs p)
 {
     constexpr int IN = Cfg::IN, BM = Cfg::BM, BN = Cfg::BN, WAVES_M = Cfg::WAVES_M, WAVES_N = Cfg::WAVES_N;
     constexpr int KB = Cfg::KB, STAGES = Cfg::STAGES, NT = Cfg::NT;
@@ -66,6 +66,7 @@ __global__ void __launch_bounds__(Cfg::NT, 1) gemm_mfma16_kernel(GemmArgs p)
     constexpr int STAGE_BYTES = TA::TILE_BYTES + TB::TILE_BYTES;
 
     extern __shared__ __attribute__((aligned(1024))) char smem[];
+    ACC950_TAKE_HEAD_TILES(p, BM, BN);
     select_batch(p);
 
     const int tid = threadIdx.x;
@@ -449,7 +450,7 @@ hipError_t launch_mfma16(const GemmArgs& a, hipStream_t stream, LaunchGeom* geom
     if (dry_run) return hipSuccess;
     static LdsLimitOnce lds_limit; // per instantiation
     if (hipError_t e = lds_limit.ensure((const void*)kern, Cfg::LDS_BYTES); e != hipSuccess) return e;
-    hipLaunchKernelGGL(kern, dim3(args.tiles_m * args.tiles_n, 1, a.batch > 1 ? a.batch : 1), dim3(Cfg::NT), Cfg::LDS_BYTES, stream, args);
+    hipLaunchKernelGGL(kern, dim3(args.tiles_m * args.tiles_n, 1, a.batch > 1 ? a.batch : 1), dim3(Cfg::NT), Cfg::LDS_BYTES, stream, ACC950_HEAD_OF(args), args);
     return hipGetLastError();
 }
 

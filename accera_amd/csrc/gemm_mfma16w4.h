@@ -67,7 +67,7 @@ __device__ __forceinline__ void w4_static_for(F&& f)
 }
 
 template <typename Cfg>
-__global__ void __launch_bounds__(256, 1) gemm_mfma16w4_kernel(GemmArgs p)
+__global__ void __launch_bounds__(256, 1) gemm_mfma16w4_kernel(ACC950_HEAD_PARAMS, GemmArgs p)
 {
     constexpr int IN = Cfg::IN, BM = 256, BN = Cfg::BN, NT = 256, KB = 64, WAVES_N = 2;
     constexpr bool A_KC = Cfg::A_KC, B_KC = Cfg::B_KC;
@@ -84,6 +84,7 @@ __global__ void __launch_bounds__(256, 1) gemm_mfma16w4_kernel(GemmArgs p)
     static_assert(STAGE_BYTES == 16384 + TN * 2048 && TA::TILE_BYTES == 16384, "the loop's offsets are written for these");
 
     extern __shared__ __attribute__((aligned(1024))) char smem[];
+    ACC950_TAKE_HEAD_TILES(p, BM, BN);
     select_batch(p);
 
     const int tid = threadIdx.x;
@@ -624,7 +625,7 @@ hipError_t launch_mfma16w4(const GemmArgs& a, hipStream_t stream, LaunchGeom* ge
     if (dry_run) return hipSuccess;
     static LdsLimitOnce lds_limit; // per instantiation
     if (hipError_t e = lds_limit.ensure((const void*)kern, Cfg::LDS_BYTES); e != hipSuccess) return e;
-    hipLaunchKernelGGL(kern, dim3(grid_x, 1, a.batch > 1 ? a.batch : 1), dim3(Cfg::NT), Cfg::LDS_BYTES, stream, args);
+    hipLaunchKernelGGL(kern, dim3(grid_x, 1, a.batch > 1 ? a.batch : 1), dim3(Cfg::NT), Cfg::LDS_BYTES, stream, ACC950_HEAD_OF(args), args);
     return hipGetLastError();
 }
 

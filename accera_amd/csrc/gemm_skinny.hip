@@ -49,8 +49,9 @@ __device__ __forceinline__ float dot2(unsigned a, unsigned b, float c)
 // LPR: lanes per B row segment (8 columns each); WAVES: waves per workgroup;
 // DEPTH: ring slots (steps in flight) per wave.
 template <bool BF16, int LPR, int WAVES, int DEPTH>
-__global__ void __launch_bounds__(WAVES * 64) gemm_skinny_kernel(SkinnyArgs p)
+__global__ void __launch_bounds__(WAVES * 64) gemm_skinny_kernel(ACC950_SKINNY_HEAD_PARAMS, SkinnyArgs p)
 {
+    ACC950_SKINNY_TAKE_HEAD(p);
     constexpr int NKP = 64 / LPR;        // k pairs per wave step
     constexpr int CB = LPR * 8;          // columns per workgroup
     constexpr int VPL = 64 / NKP;        // values per lane after the butterfly
@@ -58,7 +59,7 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_skinny_kernel(SkinnyArgs p)
     constexpr int RING_BYTES = DEPTH * SLOT_BYTES;
     static_assert(3 * (DEPTH - 1) < 64, "vmcnt is a 6-bit counter");
     extern __shared__ __attribute__((aligned(16))) char smem[];
-    { // batched launch: blockIdx.z picks the problem (and its slice of the K-split workspace)
+    if (blockIdx.z != 0) { // batched launch: blockIdx.z picks the problem (and its slice of the K-split workspace); problem 0 waits for none of these fields
         const int64_t z = blockIdx.z;
         p.A = (const char*)p.A + z * p.a_bs * 2;
         p.B = (const char*)p.B + z * p.b_bs * 2;
@@ -257,7 +258,7 @@ hipError_t launch_one(const SkinnyArgs& a, hipStream_t stream, LaunchGeom* geom,
     static LdsLimitOnce lds_limit;
     if (lds > 64 * 1024)
         if (hipError_t e = lds_limit.ensure((const void*)kern, 160 * 1024); e != hipSuccess) return e;
-    hipLaunchKernelGGL(kern, grid, block, lds, stream, a);
+    hipLaunchKernelGGL(kern, grid, block, lds, stream, ACC950_SKINNY_HEAD_OF(a), a);
     return hipGetLastError();
 }
 

@@ -51,8 +51,9 @@ typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 // that wrap around like the reference's int32 accumulator: /root/reference/accera/acc-translate/src/Target/Cpp/CppPrinterUtils.h:342-360).
 // A step has the same bytes either way: a 64-column block of int8 is 32 k rows x 64 bytes where fp16 has 16 x 128.
 template <int IN, int CB, int WAVES, int DEPTH>
-__global__ void __launch_bounds__(WAVES * 64) gemm_skinny_mfma_kernel(SkinnyArgs p)
+__global__ void __launch_bounds__(WAVES * 64) gemm_skinny_mfma_kernel(ACC950_SKINNY_HEAD_PARAMS, SkinnyArgs p)
 {
+    ACC950_SKINNY_TAKE_HEAD(p);
     static_assert(CB == 64 || CB == 256, "column block of 64 or 256");
     constexpr bool I8 = IN == T_I8, BF16 = IN == T_BF16;
     constexpr int ES = I8 ? 1 : 2;                // bytes per input element
@@ -72,7 +73,7 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_skinny_mfma_kernel(SkinnyArgs
     constexpr int NT = WAVES * 64;
     static_assert(LOADS * (DEPTH - 1) < 64, "vmcnt is a 6-bit counter");
     extern __shared__ __attribute__((aligned(1024))) char smem[];
-    { // batched launch: blockIdx.z picks the problem (and its slice of the K-split workspace)
+    if (blockIdx.z != 0) { // batched launch: blockIdx.z picks the problem (and its slice of the K-split workspace); problem 0 waits for none of these fields
         const int64_t z = blockIdx.z;
         p.A = (const char*)p.A + z * p.a_bs * ES;
         p.B = (const char*)p.B + z * p.b_bs * ES;
@@ -344,7 +345,7 @@ hipError_t launch_one(const SkinnyArgs& a, hipStream_t stream, LaunchGeom* geom,
     static LdsLimitOnce lds_limit;
     if (lds > 64 * 1024)
         if (hipError_t e = lds_limit.ensure((const void*)kern, 160 * 1024); e != hipSuccess) return e;
-    hipLaunchKernelGGL(kern, grid, block, lds, stream, a);
+    hipLaunchKernelGGL(kern, grid, block, lds, stream, ACC950_SKINNY_HEAD_OF(a), a);
     return hipGetLastError();
 }
 

@@ -25,8 +25,12 @@ struct SplitReduceArgs {
 };
 
 // one thread per four consecutive columns of a row (N is padded up to a multiple of four by the test below)
-__global__ void __launch_bounds__(256) splitk_reduce_kernel(SplitReduceArgs p)
+// (ws, C, splits, M, N, c_rs, c_cs come as arguments of their own as well: the first 14 dwords of a kernel's arguments are
+// preloaded into scalar registers at dispatch, and the loads of the slices need nothing else)
+__global__ void __launch_bounds__(256) splitk_reduce_kernel(const void* head_ws, void* head_C, int head_splits, int head_M, int head_N,
+                                                            int64_t head_c_rs, int64_t head_c_cs, SplitReduceArgs p)
 {
+    p.ws = head_ws; p.C = head_C; p.splits = head_splits; p.M = head_M; p.N = head_N; p.c_rs = head_c_rs; p.c_cs = head_c_cs;
     const int groups_n = (p.N + 3) / 4;
     const int64_t id = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (id >= (int64_t)p.M * groups_n) return;
@@ -120,7 +124,7 @@ hipError_t launch_splitk_reduce(const GemmArgs& g, const void* ws, int splits, h
     const int64_t threads = (int64_t)g.M * ((g.N + 3) / 4);
     const int64_t blocks = (threads + 255) / 256;
     if (blocks <= 0 || blocks > 0x7fffffffll) return hipErrorInvalidValue;
-    hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, a);
+    hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, a.ws, a.C, a.splits, a.M, a.N, a.c_rs, a.c_cs, a);
     return hipGetLastError();
 }
 

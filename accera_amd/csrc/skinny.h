@@ -24,6 +24,17 @@ struct SkinnyArgs {
     unsigned* counters; // splits > 1: one arrival counter per column block, zero between launches
 };
 
+// What a skinny kernel needs before its first load, as arguments of their own in front of the struct: the first 14 dwords
+// of a kernel's arguments are preloaded into scalar registers at dispatch (see ACC950_HEAD_PARAMS in common.h).
+#define ACC950_SKINNY_HEAD_PARAMS const void* head_A, const void* head_B, int head_M, int head_N, int head_K, int head_splits, \
+                                  int head_extra_phase, int head_batch, int64_t head_a_rs, int64_t head_b_rs
+#define ACC950_SKINNY_HEAD_OF(a) (a).A, (a).B, (a).M, (a).N, (a).K, (a).splits, (a).extra_phase, (a).batch, (a).a_rs, (a).b_rs
+#define ACC950_SKINNY_TAKE_HEAD(p)                                                                               \
+    do {                                                                                                          \
+        (p).A = head_A; (p).B = head_B; (p).M = head_M; (p).N = head_N; (p).K = head_K; (p).splits = head_splits; \
+        (p).extra_phase = head_extra_phase; (p).batch = head_batch; (p).a_rs = head_a_rs; (p).b_rs = head_b_rs;   \
+    } while (0)
+
 typedef hipError_t (*SkinnyLaunchFn)(const SkinnyArgs&, hipStream_t, LaunchGeom*, bool);
 
 // One kernel instantiation.  Two families: "dot2" (packed dot products on the vector

@@ -10,6 +10,9 @@
  * Matrices are described the way a .hat file describes an `affine_array`
  * (/root/reference/accera/ir/src/TranslateToHeader.cpp:713-762): shape plus element
  * strides (`affine_map`); row-major M x N has strides (N, 1), column-major (1, M).
+ * Strides are 64-bit and not negative; A's stride between consecutive k and B's stride between consecutive
+ * columns (after the exchange of operands that a column-major C brings) must be below 2^31 elements, or the
+ * call is refused with ACC950_UNSUPPORTED: the kernels take those two as 32-bit arguments.
  */
 #ifndef ACCERA_MI355X_GEMM_H
 #define ACCERA_MI355X_GEMM_H
