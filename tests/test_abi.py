@@ -195,6 +195,11 @@ def test_bound_call_handles_without_launching():
     bad = list(args)
     bad[22] = 57 + 1000   # unknown variant
     assert L.acc950_bind(*bad, ctypes.byref(h)) == _lib.INVALID_ARGUMENT
+    # A's stride between consecutive k and B's between consecutive columns travel as 32-bit kernel arguments
+    for where in (9, 13):   # a_col_stride, b_col_stride
+        bad = list(args)
+        bad[where] = 1 << 31
+        assert L.acc950_bind(*bad, ctypes.byref(h)) == _lib.UNSUPPORTED and b"2^31" in L.acc950_last_error()
 
 
 def test_tuned_table_is_consulted_by_name_and_validated(tmp_path, monkeypatch):
