@@ -814,6 +814,9 @@ int acc950_release_workspaces(void)
         it = g_ws_retired.erase(it);
     }
     if (first != hipSuccess) return fail_hip(first, "hipFree");
+    // the host-pointer path's idle contexts: device copies of the largest operands they have carried, 16 MiB of pinned staging each
+    e = host_path_release_idle(dev);
+    if (e != hipSuccess) return fail_hip(e, "releasing the host-pointer path's buffers");
     return ACC950_OK;
 }
 

@@ -24,6 +24,10 @@ typedef std::function<int(void* dA, void* dB, void* dC, hipStream_t stream)> Hos
 // run side by side, each on a context of its own.
 hipError_t host_path_run(const HostOperands& h, const HostLaunchFn& launch, int* launch_status);
 
+// Frees the contexts of `device` that no call is using (their device buffers, pinned staging slots, events and streams);
+// the next call on a host pointer makes a new one.
+hipError_t host_path_release_idle(int device);
+
 // device allocations of the path's contexts are added to this counter
 void host_path_count_allocations(std::atomic<unsigned long long>* counter);
 

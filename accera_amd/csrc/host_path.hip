@@ -236,6 +236,33 @@ hipError_t download(HostContext& c, void* host, const void* dev, size_t bytes)
 
 void host_path_count_allocations(std::atomic<unsigned long long>* counter) { g_allocations = counter; }
 
+hipError_t host_path_release_idle(int device)
+{
+    std::vector<HostContext*> mine;
+    {
+        std::lock_guard<std::mutex> lock(g_pool_mutex);
+        for (size_t i = 0; i < g_idle.size();) {
+            if (g_idle[i]->device != device) { ++i; continue; }
+            mine.push_back(g_idle[i]);
+            g_idle.erase(g_idle.begin() + (long)i);
+        }
+    }
+    // (a context goes back to the pool with its stream idle: nothing of it is in use any more)
+    hipError_t first = hipSuccess;
+    auto note = [&](hipError_t e) { if (e != hipSuccess && first == hipSuccess) first = e; };
+    for (HostContext* c : mine) {
+        for (DevBuf* b : {&c->a, &c->b, &c->c})
+            if (b->p) note(hipFree(b->p));
+        for (int i = 0; i < kSlots; ++i) {
+            if (c->event[i]) note(hipEventDestroy(c->event[i]));
+            if (c->slot[i]) note(hipHostFree(c->slot[i]));
+        }
+        if (c->stream) note(hipStreamDestroy(c->stream));
+        delete c;
+    }
+    return first;
+}
+
 hipError_t host_path_run(const HostOperands& h, const HostLaunchFn& launch, int* launch_status)
 {
     HostContext* c = nullptr;

@@ -244,8 +244,10 @@ int acc950_allocation_probe(unsigned long long* count);
 
 /*
  * Frees every K-split workspace the allocating entry points have made on the current device (all streams), the blocks
- * they have outgrown included, after waiting for the device to go idle.  The next launch that needs a workspace
- * allocates a new one.  For programs that create and destroy streams or sweep over growing problems; a workspace
+ * they have outgrown included, after waiting for the device to go idle, and the buffers the host-pointer entry points
+ * keep between calls (per call that was ever in flight at once: device copies as large as the largest operands it
+ * carried, 16 MiB of pinned staging, a stream).  The next launch that needs a workspace, the next call on host
+ * pointers, allocates anew.  For programs that create and destroy streams or sweep over growing problems; a workspace
  * otherwise stays with its (device, stream) pair until the process ends (at least 4 MiB + 16 KiB per pair).  Must not
  * run while another thread launches on the device.  No counterpart in the reference, whose functions own no device state.
  */

@@ -398,6 +398,13 @@ def test_package_functions_called_from_two_host_threads_at_once(tmp_path):
     for t in threads:
         t.join()
     assert not errors, errors[0]
+    # the two contexts the calls used can be handed back; the next call on host arrays makes its own again
+    from accera_amd import _lib
+    before = _lib.allocation_probe()
+    _lib.release_workspaces()
+    worker(fa, Aa, Ba, want_a, "f32", 3072, 1)
+    assert not errors, errors[0]
+    assert _lib.allocation_probe() >= before + 3  # device copies of A, B and C
 
 
 @pytest.mark.gpu
