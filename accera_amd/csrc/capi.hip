@@ -466,9 +466,53 @@ struct Choice {
     int splits;
 };
 
+// Few rows of A, a large B (decode shapes with a long K or many columns): the 256-column blocks of the streaming kernel
+// against its 64-column default.  A 64-column block fetches B in pieces of one cache line (half a line for int8), and
+// the memory system delivers such pieces at 5.0-5.3 TB/s (int8: 3.8-4.4) however many workgroups ask for them; 256-column
+// blocks fetch 512 (256) bytes of a row per request and reach 6.2-6.6 (5.9), but there are a quarter as many of them, one
+// workgroup at a time per CU (its rings fill the LDS), so they need a K split to occupy the chip while there are fewer
+// than about 150, and the split's second trip through memory (5-11 us, more with more rows) has to be worth it.  Measured
+// on grids of N = 4096 ... 128256 x K = 2048 ... 53248 for 8, 16 and 32 rows, fp16 and int8, B out of HBM (fp16, 8 rows, us,
+// 64-column default / best 256-column form): 8x16384x8192 54.4 / 47.4 in three slices, 8x22016x8192 97.4 / 65.7 in two,
+// 8x65536x8192 216.6 / 176.3 unsplit, 8x128256x8192 394.2 / 338.9; int8 8x12288x16384 69.2 / 42.2 in four, 8x65536x16384
+// 285.2 / 185.7; while the default stays ahead for N <= 12288 with fp16 (8x11008x4096 18.0 / 22.1) and for a short K.
+// Over the grids the default alone took 1.14 (fp16, 8 rows) to 1.39 (int8) times the best form's time on average, this rule 1.01-1.03.
+// splits: what the 256-column form should run with; false: stay with the default.
+bool wide_skinny_blocks_pay(const Problem& pb, int sv_wide, size_t max_floats, size_t max_counters, int* splits)
+{
+    const GemmArgs& g = pb.g;
+    if (g.batch > 1) return false;
+    const bool i8 = g.in_type == T_I8;
+    const int nb = (g.N + 255) / 256;
+    if ((size_t)nb > max_counters) return false;
+    if (nb > 128) {
+        // no split: whole rounds of 256 blocks at the chip's rate, a last partial round no shorter than one block at a CU's rate
+        // (bytes per us, in millions); against all of B at the rate of the narrow pieces
+        const double chip_wide = i8 ? 5.9 : 6.3, cu_wide = i8 ? 0.042 : 0.050, chip_narrow = i8 ? 4.2 : 5.0;
+        const int full = nb / 256, rem = nb % 256;
+        const double t_wide = full * 256 / chip_wide + (rem ? std::max(rem / chip_wide, 1.0 / cu_wide) : 0.0);
+        if (nb < 150 || g.K < 1024 || t_wide >= 0.95 * (nb / chip_narrow)) return false;
+        *splits = 1;
+        return true;
+    }
+    // with a split: only where the default has no idle CUs to share its slow blocks with (fp16, bf16: more than 200 blocks
+    // of 64 columns) or streams half lines (int8, from 32 blocks of 256 columns), the slices stay long enough for the
+    // second trip to be worth it, and the workgroups fill most of the chip in one round
+    if (i8 ? nb < 32 : (g.N + 63) / 64 <= 200) return false;
+    const int k_min = g.M <= 8 ? 2048 : 4096;
+    const int w_min = i8 && nb <= 40 ? 128 : 160;
+    for (int s : {8, 6, 4, 3, 2}) {
+        if (nb * s > kComputeUnits || g.K / s < k_min) continue;
+        if (nb * s < w_min || skinny_scratch_floats(sv_wide, g.N, s) > max_floats) return false;
+        *splits = s;
+        return true;
+    }
+    return false;
+}
+
 // max_split_floats: 32-bit partial sums the workspace of this call holds (the built-in array of acc950_gemm_ops_static
 // is smaller than what the allocating entry points may ask for): an MFMA kernel's K split never plans more slices.
-int choose(const Problem& pb, int variant, int k_splits, Choice* c, size_t max_split_floats = kMaxSplitFloats)
+int choose(const Problem& pb, int variant, int k_splits, Choice* c, size_t max_split_floats = kMaxSplitFloats, size_t max_counters = ~(size_t)0)
 {
     c->splits = 1;
     if (variant == ACC950_VARIANT_AUTO) {
@@ -476,6 +520,12 @@ int choose(const Problem& pb, int variant, int k_splits, Choice* c, size_t max_s
         if (sv >= 0) {
             c->variant = ACC950_VARIANT_SKINNY_BASE + sv;
             c->splits = k_splits > 0 ? k_splits : auto_skinny_splits(sv, pb.g);
+            // (the table's first entry is the MFMA family's 64-column form, kSkinnyWide its 256-column one)
+            int wide_splits = 1;
+            if (k_splits == 0 && sv == 0 && skinny_can_take(pb, kSkinnyWide) && wide_skinny_blocks_pay(pb, kSkinnyWide, max_split_floats, max_counters, &wide_splits)) {
+                c->variant = ACC950_VARIANT_SKINNY_BASE + kSkinnyWide;
+                c->splits = wide_splits;
+            }
             return ACC950_OK;
         }
         int mv = auto_mfma_variant(pb);
@@ -684,7 +734,7 @@ int acc950_gemm_ops_static(int in_type, int out_type, int M, int N, int K,
                           prologue_arg, epilogue_arg);
     if (rc) return rc;
     Choice c;
-    rc = choose(pb, variant, k_splits, &c, kStaticFloats);
+    rc = choose(pb, variant, k_splits, &c, kStaticFloats, kStaticCounters);
     if (rc) return rc;
     return run(pb, c, (hipStream_t)stream, nullptr, false, true);
 }

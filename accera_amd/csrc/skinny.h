@@ -58,6 +58,9 @@ inline int skinny_k_step(const SkinnyVariant& v, int in_type) { return in_type =
 const SkinnyVariant* skinny_dot2_table(int* count);
 const SkinnyVariant* skinny_mfma_table(int* count);
 
+// place of the MFMA family's 256-column form (four waves, four ring slots) in the table: skinny_variant(kSkinnyWide)
+constexpr int kSkinnyWide = 4;
+
 int skinny_num_variants();
 const SkinnyVariant& skinny_variant(int v); // MFMA family first, then dot2
 void skinny_variant_info(int v, int* lanes_per_row, int* waves, int* depth);

@@ -169,6 +169,20 @@ def test_choices_of_the_cost_model():
     n, ks = name(_lib.F32, _lib.F32, 768, 576, 1024, False, False, 1.0, 1.0)
     assert "fill=direct" in n and ks > 1
     assert "fp32 mfma 32x32" in name(_lib.F32, _lib.F32, 800, 126, 49, True, False, 1.0, 1.0)[0]
+    # few rows of A: the streaming kernel's 64-column blocks for the decode shape of the benchmark, its 256-column blocks (with
+    # the K split that fills the chip in one round) once there are enough of them or the default would stream half lines
+    narrow, wide = "skinny mfma cols/wg=64 waves=4 depth=4", "skinny mfma cols/wg=256 waves=4 depth=4"
+    assert name(_lib.F16, _lib.F16, 8, 11008, 4096, False, False, 1.0, 0.0) == (narrow, 1)
+    assert name(_lib.F16, _lib.F16, 8, 16384, 4096, False, False, 1.0, 0.0) == (narrow, 1)     # (two slices would fill half the chip)
+    assert name(_lib.F16, _lib.F16, 8, 16384, 8192, False, False, 1.0, 0.0) == (wide, 4)
+    assert name(_lib.BF16, _lib.BF16, 8, 22016, 8192, False, False, 1.0, 0.0) == (wide, 2)
+    assert name(_lib.F16, _lib.F16, 8, 65536, 8192, False, False, 1.0, 0.0) == (wide, 1)
+    assert name(_lib.F16, _lib.F16, 8, 66048, 4096, False, False, 1.0, 0.0) == (narrow, 1)     # (258 wide blocks: a second round for two of them)
+    assert name(_lib.F16, _lib.F16, 32, 16384, 8192, False, False, 1.0, 0.0) == (narrow, 1)    # (more rows: the second trip costs more)
+    assert name(_lib.F16, _lib.F16, 32, 16384, 16384, False, False, 1.0, 0.0) == (wide, 4)
+    assert name(_lib.I8, _lib.I32, 8, 12288, 16384, False, False, 1.0, 0.0) == (wide, 4)
+    assert name(_lib.I8, _lib.I32, 8, 8192, 8192, False, False, 1.0, 0.0) == (wide, 4)
+    assert name(_lib.I8, _lib.I32, 8, 4096, 8192, False, False, 1.0, 0.0)[0] == narrow
 
 
 def test_bound_call_handles_without_launching():

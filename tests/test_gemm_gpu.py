@@ -455,6 +455,24 @@ def test_skinny_all_variants_and_splits(in_type, out_type):
     run_case(in_type, out_type, 24, 2048, 512, seed=80, dist="normal", prologue=ora.PRO_NONE, epilogue=ora.EPI_RELU_NOCOND)
 
 
+@pytest.mark.parametrize("in_type,out_type,M,N,K,cols,splits,prologue", [
+    ("f16", "f16", 8, 22016, 4096, 256, 2, ora.PRO_SET0),     # 86 wide blocks in two slices: 172 workgroups
+    ("bf16", "f32", 16, 16384, 16384, 256, 4, ora.PRO_NONE),  # accumulates into C
+    ("f16", "f32", 5, 40960 + 72, 1024, 256, 1, ora.PRO_SET0),  # enough wide blocks without a split; the last block is ragged
+    ("i8", "i32", 8, 12288, 8192, 256, 4, ora.PRO_SET0),
+    ("i8", "i16", 32, 8192, 16384, 256, 4, ora.PRO_SET0),
+    ("f16", "f16", 8, 16384, 4096, 64, 1, ora.PRO_SET0),      # two slices would fill half the chip: the default form
+])
+def test_decode_shapes_take_the_wide_blocks_of_the_streaming_kernel(in_type, out_type, M, N, K, cols, splits, prologue):
+    """Few rows of A against a large B: the library by itself takes the streaming kernel's 256-column blocks, with the K split
+    that fills the chip in one round, where they measured ahead of the 64-column default; results against the oracle."""
+    from accera_amd import _lib, tune
+    n_in, n_out = {"f16": _lib.F16, "bf16": _lib.BF16, "i8": _lib.I8}[in_type], {"f16": _lib.F16, "f32": _lib.F32, "i32": _lib.I32, "i16": _lib.I16}[out_type]
+    variant, slices = tune.own_choice(n_in, n_out, M, N, K, False, False, 1.0, 1.0 if prologue == ora.PRO_NONE else 0.0)
+    assert f"skinny mfma cols/wg={cols} " in _lib.variant_name(variant) and slices == splits, (_lib.variant_name(variant), slices)
+    run_case(in_type, out_type, M, N, K, seed=N % 97 + K % 89, dist="normal", prologue=prologue)
+
+
 @pytest.mark.parametrize("out_type", ["i32", "i16", "i8"])
 def test_skinny_int8_streaming_kernels(out_type):
     """int8 rows of A against a large row-major int8 B on the streaming kernels of the matrix-core family

@@ -70,6 +70,19 @@ def test_static_workspace_entry_point_matches_the_allocating_one():
     assert _lib.allocation_probe() == allocations_before
     rows = rng.choice(M, 16, replace=False)
     assert_matches(to_host(dC, "f16")[rows], ora.gemm_relu_exact(A[rows], B, out_zeros(16, N, "f16"), "f16", "f16", ora.PRO_SET0, ora.EPI_RELU), "f16", K)
+    # few rows against a large B: the allocating entry point takes the streaming kernel's 256-column blocks in four slices
+    # (8 MiB of partial sums), which the array does not hold; here the library stays with the 64-column default, unsplit
+    from accera_amd import tune
+    M, N, K = 8, 16384, 8192
+    v, ks = tune.own_choice(_lib.F16, _lib.F16, M, N, K, False, False, 1.0, 0.0)
+    assert "cols/wg=256" in _lib.variant_name(v) and ks == 4
+    A = make_input(rng, (M, K), "f16", "normal")
+    B = (make_input(rng, (K, N), "f16", "normal").astype(np.float32) * 0.03).astype(np.float16)
+    dA, dB, dC = to_device(A, "f16"), to_device(B, "f16"), to_device(np.full((M, N), 9, np.float16), "f16")
+    _lib.check(_call(L.acc950_gemm_ops_static, dA, dB, dC, M, N, K, 0, stream))
+    torch.cuda.synchronize()
+    assert _lib.allocation_probe() == allocations_before
+    assert_matches(to_host(dC, "f16"), ora.gemm_relu_exact(A, B, out_zeros(M, N, "f16"), "f16", "f16", ora.PRO_SET0, ora.EPI_RELU), "f16", K)
 
 
 def test_static_workspace_entry_point_under_graph_capture():
