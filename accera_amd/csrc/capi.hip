@@ -4,6 +4,8 @@
 #include "common.h"
 #include "skinny.h"
 #include "host_path.h"
+#include <algorithm>
+#include <cmath>
 #include <vector>
 #include "variants.h"
 
@@ -186,8 +188,10 @@ bool skinny_can_take(const Problem& pb, int sv)
     if (g.a_cs != 1 || g.b_cs != 1 || g.c_cs != 1) return false;
     if (g.N % vec || g.K % k_step || g.b_rs % vec) return false;
     if (g.a_rs % (v.mfma ? vec : 2)) return false; // A pieces are fetched 16 (4) bytes at a time
-    // per-lane offsets of the direct-to-LDS fills are 32-bit
-    if ((int64_t)g.K * g.b_rs * es >= (1ll << 32) || (int64_t)v.max_m * g.a_rs * es >= (1ll << 32)) return false;
+    // per-lane offsets of the direct-to-LDS fills are 32-bit: inside one step of a wave for the MFMA family (every step has
+    // its own 64-bit base, so B itself may be of any size), inside a workgroup's whole K range for the dot-product family
+    const int64_t b_reach = (v.mfma ? (int64_t)k_step : (int64_t)g.K) * g.b_rs * es + (int64_t)g.N * es;
+    if (b_reach >= (1ll << 32) || (int64_t)v.max_m * g.a_rs * es >= (1ll << 32)) return false;
     if (pb.have_pointers && (!aligned16(g.B) || (reinterpret_cast<uintptr_t>(g.A) & (v.mfma ? 15u : 3u)))) return false;
     if (g.batch > 1 && (g.b_bs % vec || g.a_bs % (v.mfma ? vec : 2))) return false;
     return true;
@@ -483,31 +487,37 @@ bool wide_skinny_blocks_pay(const Problem& pb, int sv_wide, size_t max_floats, s
     const GemmArgs& g = pb.g;
     if (g.batch > 1) return false;
     const bool i8 = g.in_type == T_I8;
-    const int nb = (g.N + 255) / 256;
+    const int nb = (g.N + 255) / 256, nb_narrow = (g.N + 63) / 64;
     if ((size_t)nb > max_counters) return false;
-    if (nb > 128) {
-        // no split: whole rounds of 256 blocks at the chip's rate, a last partial round no shorter than one block at a CU's rate
-        // (bytes per us, in millions); against all of B at the rate of the narrow pieces
-        const double chip_wide = i8 ? 5.9 : 6.3, cu_wide = i8 ? 0.042 : 0.050, chip_narrow = i8 ? 4.2 : 5.0;
-        const int full = nb / 256, rem = nb % 256;
-        const double t_wide = full * 256 / chip_wide + (rem ? std::max(rem / chip_wide, 1.0 / cu_wide) : 0.0);
-        if (nb < 150 || g.K < 1024 || t_wide >= 0.95 * (nb / chip_narrow)) return false;
-        *splits = 1;
-        return true;
-    }
     // with a split: only where the default has no idle CUs to share its slow blocks with (fp16, bf16: more than 200 blocks
     // of 64 columns) or streams half lines (int8, from 32 blocks of 256 columns), the slices stay long enough for the
     // second trip to be worth it, and the workgroups fill most of the chip in one round
-    if (i8 ? nb < 32 : (g.N + 63) / 64 <= 200) return false;
-    const int k_min = g.M <= 8 ? 2048 : 4096;
-    const int w_min = i8 && nb <= 40 ? 128 : 160;
-    for (int s : {8, 6, 4, 3, 2}) {
-        if (nb * s > kComputeUnits || g.K / s < k_min) continue;
-        if (nb * s < w_min || skinny_scratch_floats(sv_wide, g.N, s) > max_floats) return false;
-        *splits = s;
-        return true;
+    if (nb <= 128 && (i8 ? nb >= 32 : nb_narrow > 200)) {
+        const int k_min = g.M <= 8 ? 2048 : 4096;
+        const int w_min = i8 && nb <= 40 ? 128 : 160;
+        for (int s : {8, 6, 4, 3, 2}) {
+            if (nb * s > kComputeUnits || g.K / s < k_min) continue;
+            if (nb * s < w_min || skinny_scratch_floats(sv_wide, g.N, s) > max_floats) break;
+            *splits = s;
+            return true;
+        }
     }
-    return false;
+    // unsplit, from about a hundred blocks: whole rounds of 256 blocks at the chip's rate for wide pieces and a last partial
+    // round (W blocks on W CUs reach less: 64 of them 3.2 TB/s, 125 5.5, 160 5.6, 208 6.0; never shorter than one block at a
+    // CU's rate), against all of B at the rate of the narrow pieces, which also loses what its last round of 256 blocks
+    // lacks (344 narrow blocks: 3.7 TB/s, 513: 3.8, 640: 4.3; less so from three rounds on, where workgroups of different
+    // rounds share CUs).  Rates in millions of bytes per us.
+    if (nb < 100 || g.K < 1024) return false;
+    const double chip_wide = i8 ? 5.9 : 6.3, cu_wide = i8 ? 0.042 : 0.050, chip_narrow = i8 ? 4.2 : 5.3;
+    const int full = nb / kComputeUnits, rem = nb % kComputeUnits;
+    const double rem_rate = std::min(rem * cu_wide, chip_wide * (0.75 + 0.25 * rem / kComputeUnits));
+    const double t_wide = full * kComputeUnits / chip_wide + (rem ? std::max(rem / rem_rate, 1.0 / cu_wide) : 0.0);
+    const double rounds = (double)nb_narrow / kComputeUnits;
+    double lost = std::ceil(rounds) / rounds;
+    if (rounds > 3) lost = 1 + 0.5 * (lost - 1);
+    if (t_wide >= 0.92 * (nb / chip_narrow * lost)) return false;
+    *splits = 1;
+    return true;
 }
 
 // max_split_floats: 32-bit partial sums the workspace of this call holds (the built-in array of acc950_gemm_ops_static

@@ -1244,6 +1244,57 @@ def test_measurement_aids_of_the_benchmark(in_type, out_type):
         assert 0.1 * peak < rate < peak * 1.02 and 0.5 < clock < 3.0
 
 
+@pytest.mark.parametrize("in_type,out_type,M,N,K,a_col,b_col,kernel", [
+    ("f16", "f16", 1049600, 2048, 2048, False, False, "hand-laid loop"),   # A and C beyond 4 GiB on the four-wave kernel (multi-tile form)
+    ("i8", "i32", 33024, 33024, 256, False, False, "hand-laid loop"),      # C beyond 4 GiB
+    ("f16", "f32", 1100003, 72, 2049, False, False, "any-alignment"),      # A beyond 4 GiB, register-staged fills
+    ("bf16", "bf16", 2200000, 64, 1024, True, False, "A=col-major"),       # a column-major A beyond 4 GiB
+    ("f32", "f32", 600000, 128, 2048, False, False, "mfma"),               # fp32
+    ("f16", "f16", 8, 32776, 65536, False, False, "skinny mfma"),          # few rows, B beyond 4 GiB on the streaming kernel
+    ("f16", "f32", 512, 1100000, 2048, False, True, "B=col-major"),        # a column-major B beyond 4 GiB
+])
+def test_operands_beyond_four_gib(in_type, out_type, M, N, K, a_col, b_col, kernel):
+    """Maximum sizes: an A, B or C larger than 4 GiB on every kernel family (64-bit tile bases, 32-bit offsets only inside a
+    tile or a step).  B has one +-1 per column, which makes the expected C a gather of A's columns: compared exactly, on the
+    GPU, in slabs of rows.  Inputs are small integers, so every type holds the results exactly."""
+    import torch
+    from accera_amd import _lib
+    from accera_amd.gemm import GemmCall
+    tt = {"f16": torch.float16, "bf16": torch.bfloat16, "f32": torch.float32, "i8": torch.int8, "i32": torch.int32}
+    dev = "cuda"
+    g = torch.Generator(device=dev).manual_seed(M % 1000 + N + K)
+    lo, hi = (-128, 128) if in_type == "i8" else (-4, 5)
+    if a_col:
+        A = torch.randint(lo, hi, (K, M), device=dev, generator=g, dtype=torch.int8).to(tt[in_type]).t()
+    else:
+        A = torch.randint(lo, hi, (M, K), device=dev, generator=g, dtype=torch.int8).to(tt[in_type])
+    cols = torch.arange(N, device=dev)
+    src = (cols * 7 + 3) % K                      # column n of B has its one entry in row src[n]
+    sign = torch.where(cols % 3 == 0, -1, 1)
+    if b_col:
+        B = torch.zeros((N, K), device=dev, dtype=tt[in_type])
+        B[cols, src] = sign.to(tt[in_type])
+        B = B.t()
+    else:
+        B = torch.zeros((K, N), device=dev, dtype=tt[in_type])
+        B[src, cols] = sign.to(tt[in_type])
+    C = torch.full((M, N), 7, device=dev, dtype=tt[out_type])
+    assert max(t.numel() * t.element_size() for t in (A, B, C)) > 1 << 32
+    call = GemmCall(A, B, C, variant=_lib.VARIANT_AUTO)   # (the library's own choice, not a recorded one: these shapes are in no table)
+    name = _lib.variant_name(call.chosen[0])
+    print(in_type, out_type, M, N, K, name, call.chosen[1], flush=True)
+    assert kernel in name, name
+    call()
+    torch.cuda.synchronize()
+    step = max(1, (1 << 28) // N)
+    for r0 in range(0, M, step):
+        want = torch.relu(A[r0:r0 + step][:, src].to(torch.float32) * sign.to(torch.float32)).to(tt[out_type])
+        assert torch.equal(C[r0:r0 + step], want), (r0, name)
+        del want
+    del A, B, C, call
+    torch.cuda.empty_cache()
+
+
 @pytest.mark.gpu
 def test_small_tiles_are_chosen_for_problems_that_would_not_fill_the_chip():
     """64 x 64 tiles (a wave has one 32 x 32 block) while 128 x 128 tiles would leave most compute units idle; the larger
