@@ -304,7 +304,8 @@ int auto_skinny_splits(int variant, const GemmArgs& g)
 // and register budget allows it; ties go to the larger tile (more reuse per byte fetched).
 // Among equal tiles the ping-pong kernel with four 64-byte stages is preferred, then the
 // others in table order; partial tiles only fit the edge kernel.
-int auto_mfma_variant(const Problem& pb)
+// only_tile: 0, or the edge length of the (square) tiles to choose among.
+int auto_mfma_variant(const Problem& pb, int only_tile = 0)
 {
     int n = 0;
     const MfmaVariant* tab = mfma_table(pb.g.in_type, &n);
@@ -314,6 +315,7 @@ int auto_mfma_variant(const Problem& pb)
     int best_rank = 0;
     for (int i = 0; i < n; ++i) {
         const MfmaVariant& v = tab[i];
+        if (only_tile && (v.bm != only_tile || v.bn != only_tile)) continue;
         if (!mfma_can_take(v, pb)) continue;
         // (a batch is one launch: its problems' tiles fill the chip together)
         const int64_t tiles = (((int64_t)pb.g.M + v.bm - 1) / v.bm) * (((int64_t)pb.g.N + v.bn - 1) / v.bn) * (pb.g.batch > 1 ? pb.g.batch : 1);
@@ -465,6 +467,55 @@ int auto_mfma_splits(const MfmaVariant& v, const Problem& pb, size_t max_floats 
     return want > 1 && plan_split(v, pb, (int)want, &sp, max_floats) ? sp.splits : 1;
 }
 
+// A few dozen to a few hundred rows of A against a B far larger than the caches (prefill of a short prompt, a batch of decode
+// steps): the problem is a stream of B out of HBM, and what counts is that B is streamed once -- a tile as tall as A, so
+// that no second row of tiles fetches it again -- by enough workgroups to keep the memory system busy, which takes a K
+// split where the tiles are few.  The general rule above knows neither: it weighs MFMA work, takes 64 x 64 tiles for
+// 128 x 16384 x 16384 (512 of them: B is read twice; 181 us) where 128 x 128 tiles in two slices take 106, and never
+// splits more tiles than half the CUs.  Swept over M = 33 ... 256 x (N, K) = (8192, 28672) ... (65536, 4096), fp16, every
+// tile and 1 ... 32 slices (us, general rule / this rule's choice): 33x8192x28672 231 / 94, 64x16384x16384 111 / 111,
+// 96x28672x8192 167 / 110, 128x8192x28672 174 / 98, 128x16384x16384 181 / 106, 192x8192x28672 250 / 152, 256x8192x28672
+// 288 / 135.  The best forms have about 256 workgroups with direct fills and about 512 with register-staged ones.
+// Returns the tile edge to choose among (0: the general rule) and the number of workgroups to aim for.
+// (The tile only for a B of 192 MB and more, most of the 256 MB Infinity Cache, out of which a second pass over B costs little; the
+// slices from 64 MB on, whatever tile the general rule takes: 33x11008x4096, 90 MB, 44.5 us on 172 unsplit 64 x 64 tiles, 22.3 in four slices.)
+bool streamed_b(const Problem& pb, int64_t least_bytes)
+{
+    const GemmArgs& g = pb.g;
+    return g.batch <= 1 && g.in_type != T_F32 && g.M > 32 && g.M <= 256 && (int64_t)g.N * g.K * elem_size(g.in_type) >= least_bytes;
+}
+
+int streamed_b_tile(const Problem& pb)
+{
+    const GemmArgs& g = pb.g;
+    if (!streamed_b(pb, (int64_t)192 << 20)) return 0;
+    // (a tile that holds all rows of A; 64 rows exactly fit the small tiles' direct fills, fewer or up to 128 the 128 x 128
+    // tiles -- their register-staged edge form where M is not a tile multiple; between 128 and 256 rows the 128 x 128 tiles
+    // read B twice, which the 256 x 256 tiles, taking only whole rows of tiles, would do as well)
+    return g.M == 64 ? 64 : g.M == 256 ? 256 : 128;
+}
+
+// K slices for the tile the rule above has taken: about 256 workgroups for the direct-fill kernels of the larger tiles (one
+// workgroup per CU), about 512 for the 64 x 64 tiles and the register-staged kernels (two per CU, fewer bytes in flight
+// each), a power of two, none from 160 tiles on with direct fills; a slice keeps at least 1024 elements of K, and the
+// partial sums (written and read once more) stay below a sixth of B's bytes (256x32000x4096: 74 us unsplit, 87 in two
+// slices with their 65 MB; 256x28672x8192 in two slices 132 against 165).
+int streamed_b_splits(const MfmaVariant& v, const Problem& pb, size_t max_floats)
+{
+    const GemmArgs& g = pb.g;
+    const int64_t tiles = (((int64_t)g.M + v.bm - 1) / v.bm) * (((int64_t)g.N + v.bn - 1) / v.bn);
+    if (v.direct && tiles >= 160) return 1;
+    const int64_t target = v.direct && v.bm * v.bn > 64 * 64 ? kComputeUnits : 2 * kComputeUnits;
+    int64_t want = 1;
+    while (want * 2 * tiles <= target && want < 32) want *= 2;
+    const int64_t b_bytes = (int64_t)g.N * g.K * elem_size(g.in_type);
+    while (want > 1 && (g.K / want < 1024 || want * (int64_t)g.M * g.N * 4 > b_bytes / 6)) want /= 2;
+    if (want < 2) return 1;
+    if ((size_t)want * (size_t)g.M * (size_t)g.N > ((size_t)1 << 24)) return 1; // 64 MiB of partial sums at most without being asked
+    SplitPlan sp;
+    return plan_split(v, pb, (int)want, &sp, max_floats) ? sp.splits : 1;
+}
+
 struct Choice {
     int variant;
     int splits;
@@ -538,7 +589,21 @@ int choose(const Problem& pb, int variant, int k_splits, Choice* c, size_t max_s
             }
             return ACC950_OK;
         }
-        int mv = auto_mfma_variant(pb);
+        int mv = -1, streamed_splits = 0;
+        if (k_splits == 0) {
+            if (const int tile = streamed_b_tile(pb)) {
+                mv = auto_mfma_variant(pb, tile);
+                if (mv >= 0) {
+                    int n = 0;
+                    const MfmaVariant& v = mfma_table(pb.g.in_type, &n)[mv];
+                    streamed_splits = streamed_b_splits(v, pb, max_split_floats);
+                    // (too few workgroups to stream with, and no split to make more: the general rule's smaller tiles)
+                    const int64_t tiles = (((int64_t)pb.g.M + v.bm - 1) / v.bm) * (((int64_t)pb.g.N + v.bn - 1) / v.bn);
+                    if (tiles * streamed_splits < 100) { mv = -1; streamed_splits = 0; }
+                }
+            }
+        }
+        if (mv < 0) mv = auto_mfma_variant(pb);
         if (pb.g.in_type == T_F32 && f32_can_take(pb.g)) {
             // fp32: the kernel of 32 x 32 blocks against the LDS-tiled kernels.  The kernel of blocks is ahead while its blocks
             // are at most one round over the chip and K is short (sweep of the reference's 339 shapes: best on 81 of the 86
@@ -570,7 +635,10 @@ int choose(const Problem& pb, int variant, int k_splits, Choice* c, size_t max_s
             const MfmaVariant& v = mfma_table(pb.g.in_type, &n)[mv];
             SplitPlan sp;
             if (k_splits > 1) c->splits = plan_split(v, pb, k_splits, &sp, max_split_floats) ? sp.splits : 1;
-            else if (k_splits == 0) c->splits = auto_mfma_splits(v, pb, max_split_floats);
+            else if (k_splits == 0) {
+                if (!streamed_splits && streamed_b(pb, (int64_t)64 << 20)) streamed_splits = streamed_b_splits(v, pb, max_split_floats);
+                c->splits = streamed_splits > 1 ? streamed_splits : auto_mfma_splits(v, pb, max_split_floats);
+            }
         }
         return ACC950_OK;
     }

@@ -57,8 +57,8 @@ def _make(torch, rows, cols, t, col_major, gen):
 
 def candidates(in_id, out_id, M, N, K, sa, sb, sc, splits_for_skinny=(0, 2, 4, 8), splits_for_mfma=(0, 2, 4, 8, 16, 32)):
     """(variant, k_splits) pairs the library accepts for this problem.  MFMA variants are tried with K split over workgroups
-    only when the output is small (at most 128 tiles of 128 x 128): elsewhere the partial sums cost more than the idle
-    compute units."""
+    only when the output is small (at most 128 tiles of 128 x 128) or has few rows (at most 256: the partial sums are then
+    small beside B): elsewhere the partial sums cost more than the idle compute units."""
     L = _lib.lib()
     ids = list(range(_lib.num_variants())) + [_lib.VARIANT_SKINNY_BASE + i for i in range(_lib.num_skinny_variants())]
     ids += [_lib.VARIANT_F32_MFMA, _lib.VARIANT_GENERIC]
@@ -66,7 +66,7 @@ def candidates(in_id, out_id, M, N, K, sa, sb, sc, splits_for_skinny=(0, 2, 4, 8
     for v in ids:
         if _lib.VARIANT_SKINNY_BASE <= v < _lib.VARIANT_GENERIC:
             sweep = splits_for_skinny
-        elif v < _lib.num_variants() and -(-M // 128) * -(-N // 128) <= 128:
+        elif v < _lib.num_variants() and (-(-M // 128) * -(-N // 128) <= 128 or M <= 256):
             sweep = splits_for_mfma
         else:
             sweep = (0,)

@@ -183,6 +183,21 @@ def test_choices_of_the_cost_model():
     assert name(_lib.I8, _lib.I32, 8, 12288, 16384, False, False, 1.0, 0.0) == (wide, 4)
     assert name(_lib.I8, _lib.I32, 8, 8192, 8192, False, False, 1.0, 0.0) == (wide, 4)
     assert name(_lib.I8, _lib.I32, 8, 4096, 8192, False, False, 1.0, 0.0)[0] == narrow
+    # a few dozen to a few hundred rows against a B far beyond the caches: a tile as tall as A (B is streamed once) and the K
+    # slices that make about 256 workgroups (512 of the register-staged ones); the slices alone from 64 MB of B on
+    n, ks = name(_lib.F16, _lib.F16, 128, 16384, 16384, False, False, 1.0, 0.0)
+    assert "128x128" in n and "fill=direct" in n and ks == 2
+    n, ks = name(_lib.F16, _lib.F16, 33, 8192, 28672, False, False, 1.0, 0.0)
+    assert "128x128" in n and "edge" in n and ks == 8
+    n, ks = name(_lib.BF16, _lib.BF16, 256, 28672, 8192, False, False, 1.0, 0.0)
+    assert "256x256" in n and "hand-laid loop" in n and ks == 2
+    n, ks = name(_lib.F16, _lib.F16, 256, 32000, 4096, False, False, 1.0, 0.0)
+    assert "256x256" in n and ks == 1                                                    # (two slices' partial sums would be a quarter of B)
+    n, ks = name(_lib.F16, _lib.F16, 64, 8192, 28672, False, True, 1.0, 0.0)
+    assert "64x64" in n and "fill=direct" in n and ks == 4
+    assert name(_lib.F16, _lib.F16, 64, 16384, 16384, False, False, 1.0, 0.0)[1] == 1   # (256 tiles stream by themselves)
+    n, ks = name(_lib.F16, _lib.F16, 33, 11008, 4096, False, False, 1.0, 0.0)
+    assert "64x64" in n and ks == 2                                                     # (90 MB: the general rule's tile, sliced)
 
 
 def test_bound_call_handles_without_launching():

@@ -473,6 +473,25 @@ def test_decode_shapes_take_the_wide_blocks_of_the_streaming_kernel(in_type, out
     run_case(in_type, out_type, M, N, K, seed=N % 97 + K % 89, dist="normal", prologue=prologue)
 
 
+@pytest.mark.parametrize("in_type,out_type,M,N,K,b_layout,tile,splits,prologue", [
+    ("f16", "f16", 33, 8192, 12288, "row", "128x128", 8, ora.PRO_SET0),     # register-staged edge tiles: 64 of them in eight slices
+    ("bf16", "f32", 128, 12288, 8192, "row", "128x128", 2, ora.PRO_NONE),   # 96 tiles with direct fills in two slices, accumulating into C
+    ("f16", "f16", 64, 8192, 12288, "col", "64x64", 4, ora.PRO_SET0),
+    ("i8", "i32", 256, 16384, 12288, "row", "256x256", 2, ora.PRO_SET0),    # the four-wave kernel, K split
+    ("f16", "f32", 200, 12288, 8192, "row", "128x128", 1, ora.PRO_SET0),    # two rows of 128 x 128 tiles: 192 tiles stream by themselves
+    ("f16", "f16", 48, 11008, 4096, "row", "64x64", 2, ora.PRO_SET0),       # 86 MB: the general rule's tiles, sliced
+])
+def test_many_column_problems_with_few_rows_stream_b_once(in_type, out_type, M, N, K, b_layout, tile, splits, prologue):
+    """A few dozen to a few hundred rows of A against a B beyond the caches: the library takes a tile as tall as A and the
+    K slices that give the memory system enough workgroups; results against the oracle."""
+    from accera_amd import _lib, tune
+    ids = {"f16": _lib.F16, "bf16": _lib.BF16, "i8": _lib.I8, "f32": _lib.F32, "i32": _lib.I32}
+    variant, slices = tune.own_choice(ids[in_type], ids[out_type], M, N, K, False, b_layout == "col", 1.0, 1.0 if prologue == ora.PRO_NONE else 0.0)
+    name = _lib.variant_name(variant)
+    assert f"mfma {tile} " in name and slices == splits, (name, slices)
+    run_case(in_type, out_type, M, N, K, b_layout=b_layout, seed=M + N % 91, dist="normal", prologue=prologue)
+
+
 @pytest.mark.parametrize("out_type", ["i32", "i16", "i8"])
 def test_skinny_int8_streaming_kernels(out_type):
     """int8 rows of A against a large row-major int8 B on the streaming kernels of the matrix-core family
