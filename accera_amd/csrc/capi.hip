@@ -166,7 +166,10 @@ bool mfma_can_take(const MfmaVariant& v, const Problem& pb)
             // eight-wave kernels on the 16x16 shapes take whole tiles only
             const int os = elem_size(g.out_type);
             const bool movable = !v.mi16 && g.prologue == PRO_SET;
-            if (g.M % v.bm && (!movable || g.M < v.bm || (!v.a_kc && g.M % vec))) return false;
+            // (fewer rows than one 64-row tile has, A with K contiguous: the fills fetch A's last row for the missing ones,
+            // and C's descriptor drops what comes of them -- any prologue, nothing overlaps)
+            const bool short_m = g.M < v.bm && v.bm == 64 && v.a_kc && v.direct && !v.mi16;
+            if (g.M % v.bm && !short_m && (!movable || g.M < v.bm || (!v.a_kc && g.M % vec))) return false;
             if (g.N % v.bn && (!movable || g.N < v.bn || g.N % vec || (g.N * os) % 16)) return false;
         }
     }
@@ -304,6 +307,8 @@ int auto_skinny_splits(int variant, const GemmArgs& g)
 // and register budget allows it; ties go to the larger tile (more reuse per byte fetched).
 // Among equal tiles the ping-pong kernel with four 64-byte stages is preferred, then the
 // others in table order; partial tiles only fit the edge kernel.
+bool streamed_b(const Problem& pb, int64_t least_bytes);
+
 // only_tile: 0, or the edge length of the (square) tiles to choose among.
 int auto_mfma_variant(const Problem& pb, int only_tile = 0)
 {
@@ -317,6 +322,9 @@ int auto_mfma_variant(const Problem& pb, int only_tile = 0)
         const MfmaVariant& v = tab[i];
         if (only_tile && (v.bm != only_tile || v.bn != only_tile)) continue;
         if (!mfma_can_take(v, pb)) continue;
+        // (a 64-row tile with direct fills on fewer rows than it has: taken only where B is a stream out of memory, see
+        // streamed_b_tile -- elsewhere the choices stand as the sweeps of the reference's lists found them)
+        if (!v.edge && !v.w4 && pb.g.M < v.bm && !streamed_b(pb, (int64_t)64 << 20)) continue;
         // (a batch is one launch: its problems' tiles fill the chip together)
         const int64_t tiles = (((int64_t)pb.g.M + v.bm - 1) / v.bm) * (((int64_t)pb.g.N + v.bn - 1) / v.bn) * (pb.g.batch > 1 ? pb.g.batch : 1);
         // 8- and 16-bit inputs: rounds of workgroups over the compute units, two side by side where the tile leaves room and
@@ -482,17 +490,19 @@ int auto_mfma_splits(const MfmaVariant& v, const Problem& pb, size_t max_floats 
 bool streamed_b(const Problem& pb, int64_t least_bytes)
 {
     const GemmArgs& g = pb.g;
-    return g.batch <= 1 && g.in_type != T_F32 && g.M > 32 && g.M <= 256 && (int64_t)g.N * g.K * elem_size(g.in_type) >= least_bytes;
+    // (up to 32 rows the streaming kernels come first; this is for what they do not take: a column-major B or A)
+    return g.batch <= 1 && g.in_type != T_F32 && g.M <= 256 && (int64_t)g.N * g.K * elem_size(g.in_type) >= least_bytes;
 }
 
 int streamed_b_tile(const Problem& pb)
 {
     const GemmArgs& g = pb.g;
     if (!streamed_b(pb, (int64_t)192 << 20)) return 0;
-    // (a tile that holds all rows of A; 64 rows exactly fit the small tiles' direct fills, fewer or up to 128 the 128 x 128
-    // tiles -- their register-staged edge form where M is not a tile multiple; between 128 and 256 rows the 128 x 128 tiles
-    // read B twice, which the 256 x 256 tiles, taking only whole rows of tiles, would do as well)
-    return g.M == 64 ? 64 : g.M == 256 ? 256 : 128;
+    // (a tile that holds all rows of A: up to 64 rows the small tiles with direct fills, which take fewer rows than they
+    // have when A is row-major -- the caller falls back to 128 x 128 where only their register-staged form applies --, up
+    // to 128 rows the 128 x 128 tiles, in their register-staged edge form where M is not a tile multiple; between 128 and
+    // 256 rows the 128 x 128 tiles read B twice, which the 256 x 256 tiles, taking only whole rows of tiles, would do as well)
+    return g.M <= 64 ? 64 : g.M == 256 ? 256 : 128;
 }
 
 // K slices for the tile the rule above has taken: about 256 workgroups for the direct-fill kernels of the larger tiles (one
@@ -593,6 +603,10 @@ int choose(const Problem& pb, int variant, int k_splits, Choice* c, size_t max_s
         if (k_splits == 0) {
             if (const int tile = streamed_b_tile(pb)) {
                 mv = auto_mfma_variant(pb, tile);
+                if (tile == 64 && pb.g.M < 64) { // (33x16384x16384: 102 us on 128 x 128 edge tiles, 110 on the 64 x 64 ones)
+                    int n = 0;
+                    if (mv < 0 || !mfma_table(pb.g.in_type, &n)[mv].direct) mv = auto_mfma_variant(pb, 128);
+                }
                 if (mv >= 0) {
                     int n = 0;
                     const MfmaVariant& v = mfma_table(pb.g.in_type, &n)[mv];

@@ -454,7 +454,8 @@ __global__ void __launch_bounds__(Cfg::NT, Cfg::WGS_PER_CU) gemm_mfma_kernel(ACC
     // Full-tile builds: M and N need not be multiples of the tile -- the last row / column of tiles is moved to end at
     // M / N and overlaps its neighbour, and what both compute gets the same bits from both (the host allows this only when C
     // is not read, and only for sizes whose moved tile still starts on a 16-byte boundary of the operands' and C's rows).
-    const int m0 = EDGE || tile_m * BM + BM <= p.M ? tile_m * BM : p.M - BM;
+    // (fewer rows than one tile has -- the 64-row tiles with direct fills of a row-major A take that, see short_m below: the one row of tiles starts at row 0)
+    const int m0 = EDGE || tile_m * BM + BM <= p.M ? tile_m * BM : p.M >= BM ? p.M - BM : 0;
     const int n0 = EDGE || tile_n * BN + BN <= p.N ? tile_n * BN : p.N - BN;
 
     const char* Ab = (const char*)p.A;
@@ -479,6 +480,20 @@ __global__ void __launch_bounds__(Cfg::NT, Cfg::WGS_PER_CU) gemm_mfma_kernel(ACC
         b_lane_off = TB::direct_lane_offset(ldb, tid);
     }
     constexpr int FILLS_A = TA::PER_THREAD, FILLS_B = TB::PER_THREAD, FILLS = FILLS_A + FILLS_B;
+    // Fewer rows of A than the tile has (64-row tiles, A with K contiguous, direct fills): the fills of rows past the end
+    // fetch A's last row instead -- every lane its own offset from the tile's first row, per fill instruction -- and what the
+    // matrix cores make of those rows is dropped by the range check of C's descriptor, which ends with C's last row.
+    constexpr bool SHORT_M_OK = DIRECT && !EDGE && A_KC && BM <= 64 && TA::EVEN_SPLIT;
+    const bool short_m = SHORT_M_OK && p.M < BM;
+    unsigned a_short_off[SHORT_M_OK ? FILLS_A : 1];
+    if constexpr (SHORT_M_OK) {
+#pragma unroll
+        for (int f = 0; f < FILLS_A; ++f) {
+            const int row = f * TA::ROWS_PER_PASS + tid / TA::CPR, cpos = tid % TA::CPR;
+            const int row_g = short_m && row >= p.M ? p.M - 1 : row;
+            a_short_off[f] = (unsigned)TA::global_off(row_g, TA::swizzle(row, cpos), 0, 0, lda);
+        }
+    }
     // fill number f of the tile starting at K element k0 into stage buffer `stage`
     static_assert(DIRECT || (TA::EVEN_SPLIT && TB::EVEN_SPLIT), "register-staged fills need an even split");
     auto fill_one = [&](auto tile_tag, int f, unsigned lds_tile, unsigned lane_off, const char* base, int r0, int k0,
@@ -495,6 +510,12 @@ __global__ void __launch_bounds__(Cfg::NT, Cfg::WGS_PER_CU) gemm_mfma_kernel(ACC
         T::direct_issue(lds_tile + pos, lane_off, src);
     };
     auto issue_fill = [&](int f, int stage, int k0) {
+        if constexpr (SHORT_M_OK) {
+            if (short_m && f < FILLS_A) { // (every fill from the base of the first, the rows in the lanes' offsets)
+                TA::direct_issue(smem_addr + stage * STAGE_BYTES + wave_lds + f * NT * 16, a_short_off[f], TA::direct_base(Ab, 0, m0, k0, lda));
+                return;
+            }
+        }
         if (f < FILLS_A) fill_one(TA{}, f, smem_addr + stage * STAGE_BYTES, a_lane_off, Ab, m0, k0, lda);
         else fill_one(TB{}, f - FILLS_A, smem_addr + stage * STAGE_BYTES + TA::TILE_BYTES, b_lane_off, Bb, n0, k0, ldb);
     };

@@ -188,7 +188,12 @@ def test_choices_of_the_cost_model():
     n, ks = name(_lib.F16, _lib.F16, 128, 16384, 16384, False, False, 1.0, 0.0)
     assert "128x128" in n and "fill=direct" in n and ks == 2
     n, ks = name(_lib.F16, _lib.F16, 33, 8192, 28672, False, False, 1.0, 0.0)
+    assert "64x64" in n and "fill=direct" in n and ks == 4                              # (fewer rows than the tile has: direct fills all the same)
+    n, ks = name(_lib.F16, _lib.F16, 100, 8192, 28672, False, False, 1.0, 0.0)
     assert "128x128" in n and "edge" in n and ks == 8
+    n, ks = name(_lib.F16, _lib.F16, 8, 11008, 4096, False, True, 1.0, 0.0)            # a decode step against a K-contiguous B
+    assert "64x64" in n and "fill=direct" in n and ks == 1
+    assert "edge" in name(_lib.F16, _lib.F16, 8, 4096, 4096, False, True, 1.0, 0.0)[0]  # (32 MB of B: as before)
     n, ks = name(_lib.BF16, _lib.BF16, 256, 28672, 8192, False, False, 1.0, 0.0)
     assert "256x256" in n and "hand-laid loop" in n and ks == 2
     n, ks = name(_lib.F16, _lib.F16, 256, 32000, 4096, False, False, 1.0, 0.0)
@@ -196,8 +201,8 @@ def test_choices_of_the_cost_model():
     n, ks = name(_lib.F16, _lib.F16, 64, 8192, 28672, False, True, 1.0, 0.0)
     assert "64x64" in n and "fill=direct" in n and ks == 4
     assert name(_lib.F16, _lib.F16, 64, 16384, 16384, False, False, 1.0, 0.0)[1] == 1   # (256 tiles stream by themselves)
-    n, ks = name(_lib.F16, _lib.F16, 33, 11008, 4096, False, False, 1.0, 0.0)
-    assert "64x64" in n and ks == 2                                                     # (90 MB: the general rule's tile, sliced)
+    n, ks = name(_lib.F16, _lib.F16, 100, 11008, 4096, False, False, 1.0, 0.0)
+    assert "64x64" in n and "fill=direct" in n and ks == 1                              # (90 MB: the general rule's tiles, 344 of them)
 
 
 def test_bound_call_handles_without_launching():

@@ -473,13 +473,48 @@ def test_decode_shapes_take_the_wide_blocks_of_the_streaming_kernel(in_type, out
     run_case(in_type, out_type, M, N, K, seed=N % 97 + K % 89, dist="normal", prologue=prologue)
 
 
+@pytest.mark.parametrize("in_type,out_type", [("f16", "f32"), ("bf16", "bf16"), ("i8", "i32"), ("i8", "i8"), ("f32", "f32")])
+def test_small_tiles_with_direct_fills_take_fewer_rows_than_a_tile(in_type, out_type):
+    """The 64 x 64 tiles with direct fills on 1 ... 63 rows of a row-major A: the fills of the missing rows fetch A's last row, and
+    what comes of them is dropped by the range check on C.  Both layouts of B, C written and accumulated into; the rows of C
+    behind the last one (a larger allocation, poisoned) must stay as they are."""
+    import torch
+    from accera_amd import _lib
+    small = [(v, _lib.variant_name(v)) for v in range(_lib.num_variants())]
+    small = [(v, n) for v, n in small if "mfma 64x64" in n and "fill=direct" in n and "A=col-major" not in n]
+    assert len(small) >= 2
+    for v, name in small:
+        b_layout = "col" if "B=col-major" in name else "row"
+        for M in (1, 8, 33, 63):
+            for pro, epi in ((ora.PRO_SET0, ora.EPI_RELU), (ora.PRO_NONE, ora.EPI_NONE)):
+                if out_type == "i8" and pro == ora.PRO_NONE:
+                    continue
+                print(name, in_type, out_type, M, pro, flush=True)
+                run_case(in_type, out_type, M, 192, 512, b_layout=b_layout, variant=v, prologue=pro, epilogue=epi, seed=M + v, dist="normal")
+    # C as the first rows of a taller matrix: nothing behind row M may change
+    v = small[0][0]
+    rng = np.random.default_rng(9)
+    M, N, K = 5, 128, 256
+    A, B = make_input(rng, (M, K), in_type, "normal"), make_input(rng, (K, N), in_type, "normal")
+    full = to_device(np.full((64, N), 3, ora.NP_STORAGE[out_type]), out_type)
+    import accera_amd as acc
+    acc.gemm_relu(to_device(A, in_type), to_device(B, in_type), full[:M], variant=v)
+    torch.cuda.synchronize()
+    got = to_host(full, out_type)
+    assert (got[M:] == np.full((64 - M, N), 3, ora.NP_STORAGE[out_type])).all()
+    assert_matches(got[:M], ora.gemm_relu_exact(A, B, out_zeros(M, N, out_type), in_type, out_type, ora.PRO_SET0, ora.EPI_RELU), out_type, K)
+
+
 @pytest.mark.parametrize("in_type,out_type,M,N,K,b_layout,tile,splits,prologue", [
-    ("f16", "f16", 33, 8192, 12288, "row", "128x128", 8, ora.PRO_SET0),     # register-staged edge tiles: 64 of them in eight slices
+    ("f16", "f16", 33, 8192, 12288, "row", "64x64", 4, ora.PRO_SET0),       # fewer rows than the 64-row tile has: direct fills all the same
+    ("f16", "f16", 100, 8192, 12288, "row", "128x128", 8, ora.PRO_SET0),    # register-staged edge tiles: 64 of them in eight slices
+    ("f16", "f16", 8, 11008, 4096, "col", "64x64", 1, ora.PRO_SET0),        # a decode step against a K-contiguous B (the streaming kernels want a row-major one)
+    ("bf16", "bf16", 1, 8192, 12288, "col", "64x64", 4, ora.PRO_NONE),      # one row
     ("bf16", "f32", 128, 12288, 8192, "row", "128x128", 2, ora.PRO_NONE),   # 96 tiles with direct fills in two slices, accumulating into C
     ("f16", "f16", 64, 8192, 12288, "col", "64x64", 4, ora.PRO_SET0),
     ("i8", "i32", 256, 16384, 12288, "row", "256x256", 2, ora.PRO_SET0),    # the four-wave kernel, K split
     ("f16", "f32", 200, 12288, 8192, "row", "128x128", 1, ora.PRO_SET0),    # two rows of 128 x 128 tiles: 192 tiles stream by themselves
-    ("f16", "f16", 48, 11008, 4096, "row", "64x64", 2, ora.PRO_SET0),       # 86 MB: the general rule's tiles, sliced
+    ("f16", "f16", 48, 11008, 4096, "row", "64x64", 1, ora.PRO_SET0),       # 86 MB: the general rule's tiles (172 of them stream by themselves)
 ])
 def test_many_column_problems_with_few_rows_stream_b_once(in_type, out_type, M, N, K, b_layout, tile, splits, prologue):
     """A few dozen to a few hundred rows of A against a B beyond the caches: the library takes a tile as tall as A and the
@@ -1159,7 +1194,8 @@ def test_k_split_is_chosen_for_small_outputs_with_a_long_k_and_refused_where_it_
 def test_full_tile_kernels_on_sizes_that_are_not_tile_multiples(in_type, out_type):
     """The direct-fill kernels on the 32x32 instruction shapes take any M, N of at least one tile when C is only written:
     the last row / column of tiles is moved to end at M / N.  Every such variant, both layouts of B, column-major A;
-    reading C with such sizes is refused (the edge kernels take it)."""
+    reading C with such sizes is refused (the edge kernels take it), and so is less than one tile of rows, except by the
+    64-row tiles on a row-major A."""
     from accera_amd import _lib
     vec = 16 if in_type == "i8" else 8
     seen = 0
@@ -1176,8 +1212,11 @@ def test_full_tile_kernels_on_sizes_that_are_not_tile_multiples(in_type, out_typ
             run_case(in_type, out_type, bm, N, 3 * kb, a_layout=a_layout, b_layout=b_layout, variant=v, seed=1700 + v, epilogue=ora.EPI_NONE)
             with pytest.raises(_lib.Acc950Error):
                 run_case(in_type, out_type, M, N, 5 * kb, a_layout=a_layout, b_layout=b_layout, variant=v, seed=1, prologue=ora.PRO_NONE)
-            with pytest.raises(_lib.Acc950Error):   # less than one tile
+            if bm == 64 and a_layout == "row":      # less than one tile: the 64-row tiles take it when A is row-major
                 run_case(in_type, out_type, bm - vec, N, 5 * kb, a_layout=a_layout, b_layout=b_layout, variant=v, seed=1)
+            else:
+                with pytest.raises(_lib.Acc950Error):
+                    run_case(in_type, out_type, bm - vec, N, 5 * kb, a_layout=a_layout, b_layout=b_layout, variant=v, seed=1)
             seen += 1
     assert seen >= 20
 
