@@ -294,7 +294,10 @@ int auto_skinny_splits(int variant, const GemmArgs& g)
     // One workgroup per column block streams all of K unless that leaves most CUs idle;
     // splitting K costs a trip through the scratch buffer, so it is only used to reach
     // about one workgroup per CU, with at least 256 k rows per slice.
-    const int blocks = skinny_column_blocks(variant, g.N);
+    // (a batch is one launch: the column blocks of all its problems fill the chip together -- 128 problems of 8 x 128 x 4096
+    // took 96.7 us in 16 slices each, which a single problem of that shape would want, and take a quarter of that unsplit)
+    const int64_t all_blocks = (int64_t)skinny_column_blocks(variant, g.N) * (g.batch > 1 ? g.batch : 1);
+    const int blocks = all_blocks > 4096 ? 4096 : (int)all_blocks;
     int splits = blocks >= 128 ? 1 : (256 + blocks - 1) / blocks;
     const int max_splits = g.K / 256 > 0 ? g.K / 256 : 1;
     if (splits > max_splits) splits = max_splits;
@@ -309,8 +312,9 @@ int auto_skinny_splits(int variant, const GemmArgs& g)
 // others in table order; partial tiles only fit the edge kernel.
 bool streamed_b(const Problem& pb, int64_t least_bytes);
 
-// only_tile: 0, or the edge length of the (square) tiles to choose among.
-int auto_mfma_variant(const Problem& pb, int only_tile = 0)
+// only_tile: 0, or the edge length of the (square) tiles to choose among.  short_rows: also the 64-row tiles with direct fills
+// on fewer rows than they have, whatever the size of B.
+int auto_mfma_variant(const Problem& pb, int only_tile = 0, bool short_rows = false)
 {
     int n = 0;
     const MfmaVariant* tab = mfma_table(pb.g.in_type, &n);
@@ -324,7 +328,7 @@ int auto_mfma_variant(const Problem& pb, int only_tile = 0)
         if (!mfma_can_take(v, pb)) continue;
         // (a 64-row tile with direct fills on fewer rows than it has: taken only where B is a stream out of memory, see
         // streamed_b_tile -- elsewhere the choices stand as the sweeps of the reference's lists found them)
-        if (!v.edge && !v.w4 && pb.g.M < v.bm && !streamed_b(pb, (int64_t)64 << 20)) continue;
+        if (!v.edge && !v.w4 && pb.g.M < v.bm && !short_rows && !streamed_b(pb, (int64_t)64 << 20)) continue;
         // (a batch is one launch: its problems' tiles fill the chip together)
         const int64_t tiles = (((int64_t)pb.g.M + v.bm - 1) / v.bm) * (((int64_t)pb.g.N + v.bn - 1) / v.bn) * (pb.g.batch > 1 ? pb.g.batch : 1);
         // 8- and 16-bit inputs: rounds of workgroups over the compute units, two side by side where the tile leaves room and
@@ -591,6 +595,21 @@ int choose(const Problem& pb, int variant, int k_splits, Choice* c, size_t max_s
         if (sv >= 0) {
             c->variant = ACC950_VARIANT_SKINNY_BASE + sv;
             c->splits = k_splits > 0 ? k_splits : auto_skinny_splits(sv, pb.g);
+            // A batch of problems with few rows and a narrow B (rows of B of at most 512 bytes: the P x V product of a decode
+            // step's attention, 8 x 128 x 4096 per head): the streaming kernels' pieces of such short rows come in slowly
+            // (128 problems: 59.7 us, 2.3 TB/s), the 64 x 64 tiles with direct fills, which take fewer rows than a tile
+            // has, stream whole rows (22.6 us, the vendor library's batched call 22.6; 256 problems of 1 x 128 x 8192: 207 /
+            // 87.7 / 94.9) -- when the batch has enough tiles for the chip, as a batch is not split over K.
+            if (k_splits == 0 && pb.g.batch > 1 && pb.g.N <= 256 && pb.g.N * elem_size(pb.g.in_type) <= 512) {
+                const int mv = auto_mfma_variant(pb, 64, true);
+                int n = 0;
+                const MfmaVariant* tab = mfma_table(pb.g.in_type, &n);
+                if (mv >= 0 && tab[mv].direct && (int64_t)((pb.g.N + 63) / 64) * pb.g.batch >= kComputeUnits / 2) {
+                    c->variant = mv;
+                    c->splits = 1;
+                    return ACC950_OK;
+                }
+            }
             // (the table's first entry is the MFMA family's 64-column form, kSkinnyWide its 256-column one)
             int wide_splits = 1;
             if (k_splits == 0 && sv == 0 && skinny_can_take(pb, kSkinnyWide) && wide_skinny_blocks_pay(pb, kSkinnyWide, max_split_floats, max_counters, &wide_splits)) {

@@ -782,7 +782,10 @@ def test_benchmark_configurations_at_full_size(cfg):
                                   ("i8", "i16", 3, 256, 256, 512, -1), ("i8", "i8", 5, 128, 384, 256, -1),
                                   ("f32", "f32", 32, 128, 128, 128, -1), ("f16", "f16", 5, 100, 72, 40, -1), ("f16", "f16", 6, 8, 1088, 512, -1),
                                   ("f16", "f16", 3, 8, 1088, 512, 100), ("bf16", "f32", 2, 5, 1000, 998, -1), ("f16", "f32", 1, 64, 64, 64, -1),
-                                  ("f16", "f32", 3, 512, 768, 512, "hand-laid"), ("i8", "i32", 2, 256, 512, 1024, "hand-laid")])
+                                  ("f16", "f32", 3, 512, 768, 512, "hand-laid"), ("i8", "i32", 2, 256, 512, 1024, "hand-laid"),
+                                  # a decode step's attention, P x V per head: few rows, a narrow B, many problems -- the 64 x 64 tiles with direct
+                                  # fills on fewer rows than they have (the streaming kernels read such short rows slowly)
+                                  ("f16", "f16", 80, 8, 128, 512, -1), ("i8", "i32", 70, 1, 256, 256, -1), ("bf16", "f32", 140, 20, 64, 192, -1)])
 def test_batched_gemm(case):
     """C[b] = relu(A[b] @ B[b]) in one launch: the reference's batch matmul nest
     (mfma_tests.py:435-549; shapes 3 x 1280x768x1024, 8 x ..., 32 x 128^3, 1 x 64^3 from :2519-2549) on
@@ -798,6 +801,11 @@ def test_batched_gemm(case):
     C0 = np.stack([make_c0(rng, (M, N), out_type, scale=1) for _ in range(batch)])
     up = lambda x, t: torch.stack([to_device(m, t) for m in x])
     dA, dB, dC = up(A, in_type), up(B, in_type), up(C0, out_type)
+    if batch >= 64:
+        from accera_amd.gemm import GemmCall
+        from accera_amd import _lib
+        name = _lib.variant_name(GemmCall(dA, dB, dC).chosen[0])
+        assert "mfma 64x64" in name and "fill=direct" in name, name
     acc.gemm_relu(dA, dB, dC, variant=variant, k_splits=3 if variant >= 100 else 0)
     torch.cuda.synchronize()
     got = [to_host(dC[b], out_type) for b in range(batch)]
