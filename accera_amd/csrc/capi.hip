@@ -166,9 +166,9 @@ bool mfma_can_take(const MfmaVariant& v, const Problem& pb)
             // eight-wave kernels on the 16x16 shapes take whole tiles only
             const int os = elem_size(g.out_type);
             const bool movable = !v.mi16 && g.prologue == PRO_SET;
-            // (fewer rows than one 64-row tile has, A with K contiguous: the fills fetch A's last row for the missing ones,
+            // (fewer rows than one 64- or 128-row tile has, A with K contiguous: the fills fetch A's last row for the missing ones,
             // and C's descriptor drops what comes of them -- any prologue, nothing overlaps)
-            const bool short_m = g.M < v.bm && v.bm == 64 && v.a_kc && v.direct && !v.mi16;
+            const bool short_m = g.M < v.bm && v.bm <= 128 && v.a_kc && v.direct && !v.mi16 && !v.pingpong;
             if (g.M % v.bm && !short_m && (!movable || g.M < v.bm || (!v.a_kc && g.M % vec))) return false;
             if (g.N % v.bn && (!movable || g.N < v.bn || g.N % vec || (g.N * os) % 16)) return false;
         }
@@ -502,10 +502,10 @@ int streamed_b_tile(const Problem& pb)
 {
     const GemmArgs& g = pb.g;
     if (!streamed_b(pb, (int64_t)192 << 20)) return 0;
-    // (a tile that holds all rows of A: up to 64 rows the small tiles with direct fills, which take fewer rows than they
-    // have when A is row-major -- the caller falls back to 128 x 128 where only their register-staged form applies --, up
-    // to 128 rows the 128 x 128 tiles, in their register-staged edge form where M is not a tile multiple; between 128 and
-    // 256 rows the 128 x 128 tiles read B twice, which the 256 x 256 tiles, taking only whole rows of tiles, would do as well)
+    // (a tile that holds all rows of A: up to 64 rows the small tiles, up to 128 rows the 128 x 128 tiles; with direct fills
+    // both take fewer rows than they have when A is row-major, else their register-staged edge forms apply -- of which the
+    // caller prefers the 128 x 128 one; between 128 and 256 rows the 128 x 128 tiles read B twice, which the 256 x 256
+    // tiles, taking only whole rows of tiles, would do as well)
     return g.M <= 64 ? 64 : g.M == 256 ? 256 : 128;
 }
 

@@ -454,7 +454,7 @@ __global__ void __launch_bounds__(Cfg::NT, Cfg::WGS_PER_CU) gemm_mfma_kernel(ACC
     // Full-tile builds: M and N need not be multiples of the tile -- the last row / column of tiles is moved to end at
     // M / N and overlaps its neighbour, and what both compute gets the same bits from both (the host allows this only when C
     // is not read, and only for sizes whose moved tile still starts on a 16-byte boundary of the operands' and C's rows).
-    // (fewer rows than one tile has -- the 64-row tiles with direct fills of a row-major A take that, see short_m below: the one row of tiles starts at row 0)
+    // (fewer rows than one tile has -- the 64- and 128-row tiles with direct fills of a row-major A take that, see short_m below: the one row of tiles starts at row 0)
     const int m0 = EDGE || tile_m * BM + BM <= p.M ? tile_m * BM : p.M >= BM ? p.M - BM : 0;
     const int n0 = EDGE || tile_n * BN + BN <= p.N ? tile_n * BN : p.N - BN;
 
@@ -480,10 +480,10 @@ __global__ void __launch_bounds__(Cfg::NT, Cfg::WGS_PER_CU) gemm_mfma_kernel(ACC
         b_lane_off = TB::direct_lane_offset(ldb, tid);
     }
     constexpr int FILLS_A = TA::PER_THREAD, FILLS_B = TB::PER_THREAD, FILLS = FILLS_A + FILLS_B;
-    // Fewer rows of A than the tile has (64-row tiles, A with K contiguous, direct fills): the fills of rows past the end
+    // Fewer rows of A than the tile has (64- and 128-row tiles, A with K contiguous, direct fills): the fills of rows past the end
     // fetch A's last row instead -- every lane its own offset from the tile's first row, per fill instruction -- and what the
     // matrix cores make of those rows is dropped by the range check of C's descriptor, which ends with C's last row.
-    constexpr bool SHORT_M_OK = DIRECT && !EDGE && A_KC && BM <= 64 && TA::EVEN_SPLIT;
+    constexpr bool SHORT_M_OK = DIRECT && !EDGE && A_KC && BM <= 128 && TA::EVEN_SPLIT;
     const bool short_m = SHORT_M_OK && p.M < BM;
     unsigned a_short_off[SHORT_M_OK ? FILLS_A : 1];
     if constexpr (SHORT_M_OK) {

@@ -190,6 +190,8 @@ def test_choices_of_the_cost_model():
     n, ks = name(_lib.F16, _lib.F16, 33, 8192, 28672, False, False, 1.0, 0.0)
     assert "64x64" in n and "fill=direct" in n and ks == 4                              # (fewer rows than the tile has: direct fills all the same)
     n, ks = name(_lib.F16, _lib.F16, 100, 8192, 28672, False, False, 1.0, 0.0)
+    assert "128x128" in n and "fill=direct" in n and ks == 4
+    n, ks = name(_lib.F16, _lib.F16, 100, 8192, 28672, True, False, 1.0, 0.0)           # (a column-major A: the register-staged edge form)
     assert "128x128" in n and "edge" in n and ks == 8
     n, ks = name(_lib.F16, _lib.F16, 8, 11008, 4096, False, True, 1.0, 0.0)            # a decode step against a K-contiguous B
     assert "64x64" in n and "fill=direct" in n and ks == 1

@@ -475,24 +475,25 @@ def test_decode_shapes_take_the_wide_blocks_of_the_streaming_kernel(in_type, out
 
 @pytest.mark.parametrize("in_type,out_type", [("f16", "f32"), ("bf16", "bf16"), ("i8", "i32"), ("i8", "i8"), ("f32", "f32")])
 def test_small_tiles_with_direct_fills_take_fewer_rows_than_a_tile(in_type, out_type):
-    """The 64 x 64 tiles with direct fills on 1 ... 63 rows of a row-major A: the fills of the missing rows fetch A's last row, and
+    """The 64- and 128-row tiles with direct fills on fewer rows of a row-major A than they have: the fills of the missing rows fetch A's last row, and
     what comes of them is dropped by the range check on C.  Both layouts of B, C written and accumulated into; the rows of C
     behind the last one (a larger allocation, poisoned) must stay as they are."""
     import torch
     from accera_amd import _lib
     small = [(v, _lib.variant_name(v)) for v in range(_lib.num_variants())]
-    small = [(v, n) for v, n in small if "mfma 64x64" in n and "fill=direct" in n and "A=col-major" not in n]
-    assert len(small) >= 2
+    small = [(v, n) for v, n in small if re.search(r"mfma (64|128)x", n) and "fill=direct" in n and "A=col-major" not in n and "pingpong" not in n and "mi16" not in n]
+    assert len(small) >= 6
     for v, name in small:
         b_layout = "col" if "B=col-major" in name else "row"
-        for M in (1, 8, 33, 63):
+        bm, bn = map(int, re.search(r"mfma (\d+)x(\d+)", name).groups())
+        for M in ((1, 8, 33, 63) if bm == 64 else (5, 65, 127)):
             for pro, epi in ((ora.PRO_SET0, ora.EPI_RELU), (ora.PRO_NONE, ora.EPI_NONE)):
                 if out_type == "i8" and pro == ora.PRO_NONE:
                     continue
                 print(name, in_type, out_type, M, pro, flush=True)
-                run_case(in_type, out_type, M, 192, 512, b_layout=b_layout, variant=v, prologue=pro, epilogue=epi, seed=M + v, dist="normal")
+                run_case(in_type, out_type, M, 3 * bn, 512, b_layout=b_layout, variant=v, prologue=pro, epilogue=epi, seed=M + v, dist="normal")
     # C as the first rows of a taller matrix: nothing behind row M may change
-    v = small[0][0]
+    v = next(v for v, n in small if "mfma 64x64" in n)
     rng = np.random.default_rng(9)
     M, N, K = 5, 128, 256
     A, B = make_input(rng, (M, K), in_type, "normal"), make_input(rng, (K, N), in_type, "normal")
@@ -507,7 +508,7 @@ def test_small_tiles_with_direct_fills_take_fewer_rows_than_a_tile(in_type, out_
 
 @pytest.mark.parametrize("in_type,out_type,M,N,K,b_layout,tile,splits,prologue", [
     ("f16", "f16", 33, 8192, 12288, "row", "64x64", 4, ora.PRO_SET0),       # fewer rows than the 64-row tile has: direct fills all the same
-    ("f16", "f16", 100, 8192, 12288, "row", "128x128", 8, ora.PRO_SET0),    # register-staged edge tiles: 64 of them in eight slices
+    ("f16", "f16", 100, 8192, 12288, "row", "128x128", 4, ora.PRO_SET0),    # 128-row tiles on 100 rows, direct fills: 64 of them in four slices
     ("f16", "f16", 8, 11008, 4096, "col", "64x64", 1, ora.PRO_SET0),        # a decode step against a K-contiguous B (the streaming kernels want a row-major one)
     ("bf16", "bf16", 1, 8192, 12288, "col", "64x64", 4, ora.PRO_NONE),      # one row
     ("bf16", "f32", 128, 12288, 8192, "row", "128x128", 2, ora.PRO_NONE),   # 96 tiles with direct fills in two slices, accumulating into C
@@ -1203,7 +1204,7 @@ def test_full_tile_kernels_on_sizes_that_are_not_tile_multiples(in_type, out_typ
     """The direct-fill kernels on the 32x32 instruction shapes take any M, N of at least one tile when C is only written:
     the last row / column of tiles is moved to end at M / N.  Every such variant, both layouts of B, column-major A;
     reading C with such sizes is refused (the edge kernels take it), and so is less than one tile of rows, except by the
-    64-row tiles on a row-major A."""
+    64- and 128-row tiles on a row-major A."""
     from accera_amd import _lib
     vec = 16 if in_type == "i8" else 8
     seen = 0
@@ -1220,7 +1221,7 @@ def test_full_tile_kernels_on_sizes_that_are_not_tile_multiples(in_type, out_typ
             run_case(in_type, out_type, bm, N, 3 * kb, a_layout=a_layout, b_layout=b_layout, variant=v, seed=1700 + v, epilogue=ora.EPI_NONE)
             with pytest.raises(_lib.Acc950Error):
                 run_case(in_type, out_type, M, N, 5 * kb, a_layout=a_layout, b_layout=b_layout, variant=v, seed=1, prologue=ora.PRO_NONE)
-            if bm == 64 and a_layout == "row":      # less than one tile: the 64-row tiles take it when A is row-major
+            if bm <= 128 and a_layout == "row" and "pingpong" not in name:   # less than one tile: the 64- and 128-row tiles take it when A is row-major
                 run_case(in_type, out_type, bm - vec, N, 5 * kb, a_layout=a_layout, b_layout=b_layout, variant=v, seed=1)
             else:
                 with pytest.raises(_lib.Acc950Error):
