@@ -170,7 +170,11 @@ bool mfma_can_take(const MfmaVariant& v, const Problem& pb)
             // and C's descriptor drops what comes of them -- any prologue, nothing overlaps)
             const bool short_m = g.M < v.bm && v.bm <= 128 && v.a_kc && v.direct && !v.mi16 && !v.pingpong;
             if (g.M % v.bm && !short_m && (!movable || g.M < v.bm || (!v.a_kc && g.M % vec))) return false;
-            if (g.N % v.bn && (!movable || g.N < v.bn || g.N % vec || (g.N * os) % 16)) return false;
+            // (a K-contiguous B has no row that the moved tile's first column could split, and a C of 16- or 32-bit elements
+            // is then stored element by element where the tile does not start on a 16-byte boundary: any N -- the odd
+            // vocabulary sizes of language-model heads, 4096x50257x4096 with B as the framework keeps it)
+            const bool any_n = v.b_kc && os >= 2;
+            if (g.N % v.bn && (!movable || g.N < v.bn || (!any_n && (g.N % vec || (g.N * os) % 16)))) return false;
         }
     }
     // offsets inside one output tile are 32-bit in the write-back

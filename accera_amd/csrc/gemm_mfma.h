@@ -955,7 +955,8 @@ __global__ void __launch_bounds__(Cfg::NT, Cfg::WGS_PER_CU) gemm_mfma_kernel(ACC
     auto store_all = [&](auto relu_tag) {
         auto fin = [&](scalar_t v) { return decltype(relu_tag)::value ? (v > scalar_t(0) ? v : scalar_t(0)) : v; };
         const unsigned os = p.out_type == T_I8 ? 1 : (p.out_type == T_F32 || p.out_type == T_I32) ? 4 : 2;
-        const bool staged = CAN_STAGE && (p.c_rs * os) % 16 == 0 && ((size_t)p.C & 15) == 0;
+        // (whole 16-byte pieces of rows: rows 16 bytes apart, and a tile -- a moved last one may start at any column when B is K-contiguous -- on a 16-byte boundary)
+        const bool staged = CAN_STAGE && (p.c_rs * os) % 16 == 0 && ((size_t)p.C & 15) == 0 && ((unsigned)n0 * os) % 16 == 0;
         if constexpr (IN == IN_I8) {
             if (p.out_type == T_I32) for_each_element(int{}, [&](CTile t, unsigned vo, unsigned so, int v) { c_store<int, EDGE ? 0 : C_STORE_AUX>(t, vo, so, fin(v)); return v; });
             else if (CAN_STAGE && staged) {

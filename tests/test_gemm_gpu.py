@@ -1230,6 +1230,34 @@ def test_full_tile_kernels_on_sizes_that_are_not_tile_multiples(in_type, out_typ
     assert seen >= 20
 
 
+@pytest.mark.parametrize("in_type,out_type", [("f16", "f16"), ("f16", "f32"), ("bf16", "bf16"), ("i8", "i32"), ("i8", "i16"), ("f32", "f32")])
+def test_direct_fill_kernels_take_any_n_with_a_k_contiguous_b(in_type, out_type):
+    """A column-major (K-contiguous) B has no row that a moved last tile's first column could split: the direct-fill kernels
+    on the 32x32 instruction shapes take any N of at least one tile with it when C is only written -- odd vocabulary sizes
+    of language-model heads.  C's rows are then not 16 bytes apart and are stored element by element; every such variant."""
+    from accera_amd import _lib
+    seen = 0
+    for v, name in _variants("col"):
+        if "fill=direct" not in name or "mi16" in name or "edge" in name:
+            continue
+        bm, bn = map(int, re.search(r"mfma (\d+)x(\d+)", name).groups())
+        kb = int(re.search(r"kb(\d+)", name).group(1)) // {"f16": 2, "bf16": 2, "i8": 1, "f32": 4}[in_type]
+        a_layout = "col" if "A=col-major" in name else "row"
+        for N in (2 * bn + 37, bn + 1):
+            print("variant", v, name, in_type, out_type, N, flush=True)
+            run_case(in_type, out_type, 2 * bm, N, 3 * kb, a_layout=a_layout, b_layout="col", variant=v, seed=N + v, dist="normal")
+        seen += 1
+    assert seen >= 8
+    if out_type == "f16":   # the library by itself: a prefill step's language-model head with GPT-2's vocabulary, scaled down in M and K
+        from accera_amd import tune
+        name = _lib.variant_name(tune.own_choice(_lib.F16, _lib.F16, 4096, 50257, 4096, False, True, 1.0, 0.0)[0])
+        assert "fill=direct" in name and "edge" not in name, name
+        run_case("f16", "f16", 300, 50257, 256, b_layout="col", seed=3, dist="normal")
+    if out_type == "i16":   # an int8 C keeps its rule: rows 16 bytes apart, or the thread-bound kernel
+        with pytest.raises(_lib.Acc950Error):
+            run_case("i8", "i8", 256, 293, 256, b_layout="col", variant=next(v for v, n in _variants("col") if "mfma 128x128" in n and "fill=direct" in n and "mi16" not in n), seed=1)
+
+
 @pytest.mark.parametrize("b_layout", ["row", "col"])
 def test_fp32_on_the_tiled_mfma_kernels(b_layout):
     """fp32 inputs on the LDS-tiled kernels (v_mfma_f32_32x32x2_f32; four instructions per 32-byte k-step): every variant
