@@ -166,9 +166,9 @@ bool mfma_can_take(const MfmaVariant& v, const Problem& pb)
             // eight-wave kernels on the 16x16 shapes take whole tiles only
             const int os = elem_size(g.out_type);
             const bool movable = !v.mi16 && g.prologue == PRO_SET;
-            // (fewer rows than one 64- or 128-row tile has, A with K contiguous: the fills fetch A's last row for the missing ones,
+            // (fewer rows than one tile has, A with K contiguous: the fills fetch A's last row for the missing ones,
             // and C's descriptor drops what comes of them -- any prologue, nothing overlaps)
-            const bool short_m = g.M < v.bm && v.bm <= 128 && v.a_kc && v.direct && !v.mi16 && !v.pingpong;
+            const bool short_m = g.M < v.bm && v.a_kc && v.direct && !v.mi16;
             if (g.M % v.bm && !short_m && (!movable || g.M < v.bm || (!v.a_kc && g.M % vec))) return false;
             // (a K-contiguous B has no row that the moved tile's first column could split, and a C of 16- or 32-bit elements
             // is then stored element by element where the tile does not start on a 16-byte boundary: any N -- the odd
@@ -506,11 +506,11 @@ int streamed_b_tile(const Problem& pb)
 {
     const GemmArgs& g = pb.g;
     if (!streamed_b(pb, (int64_t)192 << 20)) return 0;
-    // (a tile that holds all rows of A: up to 64 rows the small tiles, up to 128 rows the 128 x 128 tiles; with direct fills
-    // both take fewer rows than they have when A is row-major, else their register-staged edge forms apply -- of which the
-    // caller prefers the 128 x 128 one; between 128 and 256 rows the 128 x 128 tiles read B twice, which the 256 x 256
-    // tiles, taking only whole rows of tiles, would do as well)
-    return g.M <= 64 ? 64 : g.M == 256 ? 256 : 128;
+    // (a tile that holds all rows of A: up to 64 rows the small tiles, up to 128 rows the 128 x 128 tiles, up to 256 the
+    // 256 x 256 ones; with direct fills all take fewer rows than they have when A is row-major (the four-wave kernel, which
+    // moves its last row of tiles instead, only from 256 rows on), else the register-staged edge forms apply -- of which
+    // the caller prefers the 128 x 128 one -- or, beyond 128 rows, the general rule)
+    return g.M <= 64 ? 64 : g.M <= 128 ? 128 : 256;
 }
 
 // K slices for the tile the rule above has taken: about 256 workgroups for the direct-fill kernels of the larger tiles (one

@@ -409,6 +409,14 @@ __device__ __forceinline__ void c_store(CTile t, unsigned voff, unsigned soff, T
     else __builtin_amdgcn_raw_buffer_store_b8(__builtin_bit_cast(unsigned char, v), t.rsrc, voff, soff, AUX);
 }
 
+// Whether a kernel takes fewer rows of A than its tile has (see short_m in the kernel): direct fills of a row-major A whose
+// fill instructions split evenly over the workgroup.  The launcher refuses such a problem for every other instantiation.
+template <typename Cfg>
+constexpr bool mfma_takes_short_m()
+{
+    return Cfg::DIRECT && !Cfg::EDGE && Cfg::A_KC && OperandTile<Cfg::IN, Cfg::BM, Cfg::A_KC, Cfg::NT, Cfg::KB>::EVEN_SPLIT;
+}
+
 template <typename Cfg>
 __global__ void __launch_bounds__(Cfg::NT, Cfg::WGS_PER_CU) gemm_mfma_kernel(ACC950_HEAD_PARAMS, GemmArgs p)
 {
@@ -454,7 +462,7 @@ __global__ void __launch_bounds__(Cfg::NT, Cfg::WGS_PER_CU) gemm_mfma_kernel(ACC
     // Full-tile builds: M and N need not be multiples of the tile -- the last row / column of tiles is moved to end at
     // M / N and overlaps its neighbour, and what both compute gets the same bits from both (the host allows this only when C
     // is not read, and only for sizes whose moved tile still starts on a 16-byte boundary of the operands' and C's rows).
-    // (fewer rows than one tile has -- the 64- and 128-row tiles with direct fills of a row-major A take that, see short_m below: the one row of tiles starts at row 0)
+    // (fewer rows than one tile has -- the tiles with direct fills of a row-major A take that, see short_m below: the one row of tiles starts at row 0)
     const int m0 = EDGE || tile_m * BM + BM <= p.M ? tile_m * BM : p.M >= BM ? p.M - BM : 0;
     const int n0 = EDGE || tile_n * BN + BN <= p.N ? tile_n * BN : p.N - BN;
 
@@ -480,10 +488,10 @@ __global__ void __launch_bounds__(Cfg::NT, Cfg::WGS_PER_CU) gemm_mfma_kernel(ACC
         b_lane_off = TB::direct_lane_offset(ldb, tid);
     }
     constexpr int FILLS_A = TA::PER_THREAD, FILLS_B = TB::PER_THREAD, FILLS = FILLS_A + FILLS_B;
-    // Fewer rows of A than the tile has (64- and 128-row tiles, A with K contiguous, direct fills): the fills of rows past the end
+    // Fewer rows of A than the tile has (A with K contiguous, direct fills): the fills of rows past the end
     // fetch A's last row instead -- every lane its own offset from the tile's first row, per fill instruction -- and what the
     // matrix cores make of those rows is dropped by the range check of C's descriptor, which ends with C's last row.
-    constexpr bool SHORT_M_OK = DIRECT && !EDGE && A_KC && BM <= 128 && TA::EVEN_SPLIT;
+    constexpr bool SHORT_M_OK = mfma_takes_short_m<Cfg>();
     const bool short_m = SHORT_M_OK && p.M < BM;
     unsigned a_short_off[SHORT_M_OK ? FILLS_A : 1];
     if constexpr (SHORT_M_OK) {
@@ -1002,6 +1010,8 @@ hipError_t launch_mfma(const GemmArgs& a, hipStream_t stream, LaunchGeom* geom, 
     auto kern = gemm_mfma_kernel<Cfg>;
     // an int8 C is written in 16-byte pieces of 16-byte aligned rows; no kernel here has a path for anything else
     if (a.out_type == T_I8 && (a.c_rs % 16 || ((size_t)a.C & 15) || (a.batch > 1 && a.c_bs % 16))) return hipErrorInvalidValue;
+    // fewer rows than one tile: only where the fills fetch A's last row for the missing ones (or the edge build tests every row)
+    if (!Cfg::EDGE && a.M < Cfg::BM && !mfma_takes_short_m<Cfg>()) return hipErrorInvalidValue;
     GemmArgs args = a;
     args.tiles_m = (a.M + Cfg::BM - 1) / Cfg::BM;
     args.tiles_n = (a.N + Cfg::BN - 1) / Cfg::BN;

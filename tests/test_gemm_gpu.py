@@ -475,18 +475,18 @@ def test_decode_shapes_take_the_wide_blocks_of_the_streaming_kernel(in_type, out
 
 @pytest.mark.parametrize("in_type,out_type", [("f16", "f32"), ("bf16", "bf16"), ("i8", "i32"), ("i8", "i8"), ("f32", "f32")])
 def test_small_tiles_with_direct_fills_take_fewer_rows_than_a_tile(in_type, out_type):
-    """The 64- and 128-row tiles with direct fills on fewer rows of a row-major A than they have: the fills of the missing rows fetch A's last row, and
+    """The tiles with direct fills (32x32 instruction shapes) on fewer rows of a row-major A than they have: the fills of the missing rows fetch A's last row, and
     what comes of them is dropped by the range check on C.  Both layouts of B, C written and accumulated into; the rows of C
     behind the last one (a larger allocation, poisoned) must stay as they are."""
     import torch
     from accera_amd import _lib
     small = [(v, _lib.variant_name(v)) for v in range(_lib.num_variants())]
-    small = [(v, n) for v, n in small if re.search(r"mfma (64|128)x", n) and "fill=direct" in n and "A=col-major" not in n and "pingpong" not in n and "mi16" not in n]
-    assert len(small) >= 6
+    small = [(v, n) for v, n in small if "fill=direct" in n and "A=col-major" not in n and "mi16" not in n and "edge" not in n]
+    assert len(small) >= 10
     for v, name in small:
         b_layout = "col" if "B=col-major" in name else "row"
         bm, bn = map(int, re.search(r"mfma (\d+)x(\d+)", name).groups())
-        for M in ((1, 8, 33, 63) if bm == 64 else (5, 65, 127)):
+        for M in ((1, 8, 33, 63) if bm == 64 else (5, 65, 127) if bm == 128 else (3, 129, 255)):
             for pro, epi in ((ora.PRO_SET0, ora.EPI_RELU), (ora.PRO_NONE, ora.EPI_NONE)):
                 if out_type == "i8" and pro == ora.PRO_NONE:
                     continue
@@ -1203,8 +1203,7 @@ def test_k_split_is_chosen_for_small_outputs_with_a_long_k_and_refused_where_it_
 def test_full_tile_kernels_on_sizes_that_are_not_tile_multiples(in_type, out_type):
     """The direct-fill kernels on the 32x32 instruction shapes take any M, N of at least one tile when C is only written:
     the last row / column of tiles is moved to end at M / N.  Every such variant, both layouts of B, column-major A;
-    reading C with such sizes is refused (the edge kernels take it), and so is less than one tile of rows, except by the
-    64- and 128-row tiles on a row-major A."""
+    reading C with such sizes is refused (the edge kernels take it), and so is less than one tile of rows of a column-major A."""
     from accera_amd import _lib
     vec = 16 if in_type == "i8" else 8
     seen = 0
@@ -1221,7 +1220,7 @@ def test_full_tile_kernels_on_sizes_that_are_not_tile_multiples(in_type, out_typ
             run_case(in_type, out_type, bm, N, 3 * kb, a_layout=a_layout, b_layout=b_layout, variant=v, seed=1700 + v, epilogue=ora.EPI_NONE)
             with pytest.raises(_lib.Acc950Error):
                 run_case(in_type, out_type, M, N, 5 * kb, a_layout=a_layout, b_layout=b_layout, variant=v, seed=1, prologue=ora.PRO_NONE)
-            if bm <= 128 and a_layout == "row" and "pingpong" not in name:   # less than one tile: the 64- and 128-row tiles take it when A is row-major
+            if a_layout == "row":   # less than one tile: taken when A is row-major
                 run_case(in_type, out_type, bm - vec, N, 5 * kb, a_layout=a_layout, b_layout=b_layout, variant=v, seed=1)
             else:
                 with pytest.raises(_lib.Acc950Error):
