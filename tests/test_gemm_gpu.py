@@ -504,6 +504,21 @@ def test_small_tiles_with_direct_fills_take_fewer_rows_than_a_tile(in_type, out_
     got = to_host(full, out_type)
     assert (got[M:] == np.full((64 - M, N), 3, ora.NP_STORAGE[out_type])).all()
     assert_matches(got[:M], ora.gemm_relu_exact(A, B, out_zeros(M, N, out_type), in_type, out_type, ora.PRO_SET0, ora.EPI_RELU), out_type, K)
+    # A and C as the left columns of wider matrices (rows further apart than they are long), and a batch of such problems
+    batch, pad = 3, 64
+    As = np.stack([make_input(rng, (M, K + pad), in_type, "normal") for _ in range(batch)])
+    Bs = np.stack([make_input(rng, (K, N), in_type, "normal") for _ in range(batch)])
+    dA = torch.stack([to_device(a, in_type) for a in As])[:, :, :K]
+    dB = torch.stack([to_device(b, in_type) for b in Bs])
+    dC = torch.stack([to_device(np.full((M, N + 16), 3, ora.NP_STORAGE[out_type]), out_type) for _ in range(batch)])
+    assert dA.stride(1) == K + pad and dC.stride(1) == N + 16
+    acc.gemm_relu(dA, dB, dC[:, :, :N], variant=v)
+    torch.cuda.synchronize()
+    for b in range(batch):
+        got = to_host(dC[b], out_type)
+        assert (got[:, N:] == 3).all()
+        want = ora.gemm_relu_exact(np.ascontiguousarray(As[b][:, :K]), Bs[b], out_zeros(M, N, out_type), in_type, out_type, ora.PRO_SET0, ora.EPI_RELU)
+        assert_matches(got[:, :N], want, out_type, K)
 
 
 @pytest.mark.parametrize("in_type,out_type,M,N,K,b_layout,tile,splits,prologue", [
