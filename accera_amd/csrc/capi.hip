@@ -333,6 +333,13 @@ int auto_mfma_variant(const Problem& pb, int only_tile = 0, bool short_rows = fa
         // (a 64-row tile with direct fills on fewer rows than it has: taken only where B is a stream out of memory, see
         // streamed_b_tile -- elsewhere the choices stand as the sweeps of the reference's lists found them)
         if (!v.edge && !v.w4 && pb.g.M < v.bm && !short_rows && !streamed_b(pb, (int64_t)64 << 20)) continue;
+        // (the any-alignment form on 256 x 256 tiles pays where the K-contiguous operands' rows are 16 bytes aligned and the
+        // odd size is N or M -- 4096x50257x4096 with a row-major B: 2397 us on 128 x 128 tiles, 1832 on these -- and loses
+        // where every row of a K-contiguous operand starts unaligned: 4100^3 326 / 361, 1234x5678x4321 205 / 256)
+        if (v.any && v.bm == 256) {
+            const int vec_k = 16 / elem_size(pb.g.in_type);
+            if ((v.a_kc && pb.g.a_rs % vec_k) || (v.b_kc && pb.g.b_cs % vec_k)) continue;
+        }
         // (a batch is one launch: its problems' tiles fill the chip together)
         const int64_t tiles = (((int64_t)pb.g.M + v.bm - 1) / v.bm) * (((int64_t)pb.g.N + v.bn - 1) / v.bn) * (pb.g.batch > 1 ? pb.g.batch : 1);
         // 8- and 16-bit inputs: rounds of workgroups over the compute units, two side by side where the tile leaves room and

@@ -55,6 +55,10 @@ namespace acc950 {
 #define VANY64(AKC, BKC)                                                                                \
     { 64, 64, 2, 2, AKC, BKC, false, true, 128, 2, false, false, false, false, true,                   \
       &launch_mfma<MfmaConfig<ACC950_IN, 64, 64, 2, 2, AKC, BKC, false, true, 128, 2, false, false, true>>, nullptr }
+// the same on 256x256 tiles, eight waves: large problems of odd sizes (half the fill work per MFMA of the 128x128 form)
+#define VANY256(AKC, BKC)                                                                               \
+    { 256, 256, 2, 4, AKC, BKC, false, true, 128, 2, false, false, false, false, true,                 \
+      &launch_mfma<MfmaConfig<ACC950_IN, 256, 256, 2, 4, AKC, BKC, false, true, 128, 2, false, false, true>>, nullptr }
 #define V(BM, BN, WM, WN, BKC, DIRECT, EDGE, KB, STAGES) VA(true, BM, BN, WM, WN, BKC, DIRECT, EDGE, KB, STAGES)
 #define VP(BM, BN, WM, WN, BKC, KB, STAGES) VPA(true, BM, BN, WM, WN, BKC, KB, STAGES)
 // column-major A (M contiguous; the "transA" shapes of the reference's sweep lists,
@@ -131,6 +135,9 @@ static const MfmaVariant kVariants[] = {
     // four-wave kernel for a column-major A, one workgroup per CU walking several output tiles
     V16W4PA(false),
     V16W4PA(true),
+    // any sizes, leading dimensions and alignments on 256x256 tiles
+    VANY256(true, false),
+    VANY256(true, true),
 };
 #undef LAYOUT_AT
 #undef VA
@@ -143,6 +150,7 @@ static const MfmaVariant kVariants[] = {
 #undef V16W4PA
 #undef VANY
 #undef VANY64
+#undef VANY256
 #undef LAYOUT
 #undef V
 #undef VP
