@@ -519,7 +519,9 @@ __global__ void __launch_bounds__(Cfg::NT, Cfg::WGS_PER_CU) gemm_mfma_kernel(ACC
     };
     auto issue_fill = [&](int f, int stage, int k0) {
         if constexpr (SHORT_M_OK) {
-            if (short_m && f < FILLS_A) { // (every fill from the base of the first, the rows in the lanes' offsets)
+            // (always this way, short rows or not: every fill of A from the base of the first, the rows in the lanes' offsets
+            // -- a test of short_m here would split the K loop into blocks and put waits for memory where they join)
+            if (f < FILLS_A) {
                 TA::direct_issue(smem_addr + stage * STAGE_BYTES + wave_lds + f * NT * 16, a_short_off[f], TA::direct_base(Ab, 0, m0, k0, lda));
                 return;
             }
