@@ -848,7 +848,7 @@ def test_sweep_tool_checks_and_times_every_variant():
     assert res and all(r["correct"] is True for r in res)
     res = tune.sweep(rows[:1], "i8", relu=True, check=True, out_type="i16", min_time_s=0.002, log=lambda *_: None)
     assert res and all(r["correct"] is True for r in res)
-    # the vendor-library yardstick adds one row per shape and does not touch the verdicts
+    # the vendor-library yardstick adds one row per shape and does not touch the checks
     lines = []
     res = tune.sweep(rows[:2], "f16", relu=False, check=True, min_time_s=0.002, log=lines.append, baseline=True)
     assert sum(r["variant"] == -2 for r in res) == 2 and all("vendor library" in l for l in lines)
