@@ -330,9 +330,9 @@ int auto_mfma_variant(const Problem& pb, int only_tile = 0, bool short_rows = fa
         const MfmaVariant& v = tab[i];
         if (only_tile && (v.bm != only_tile || v.bn != only_tile)) continue;
         if (!mfma_can_take(v, pb)) continue;
-        // (a 64-row tile with direct fills on fewer rows than it has: taken only where B is a stream out of memory, see
-        // streamed_b_tile -- elsewhere the choices stand as the sweeps of the reference's lists found them)
-        if (!v.edge && !v.w4 && pb.g.M < v.bm && !short_rows && !streamed_b(pb, (int64_t)64 << 20)) continue;
+        // (a tile with direct fills on fewer rows than it has: taken only where B has at least 16 MB, see streamed_b_tile --
+        // elsewhere the choices stand as the sweeps of the reference's lists found them, none of whose rows is of this kind)
+        if (!v.edge && !v.w4 && pb.g.M < v.bm && !short_rows && !streamed_b(pb, (int64_t)16 << 20)) continue;
         // (the any-alignment form on 256 x 256 tiles pays where the K-contiguous operands' rows are 16 bytes aligned and the
         // odd size is N or M -- 4096x50257x4096 with a row-major B: 2397 us on 128 x 128 tiles, 1832 on these -- and loses
         // where every row of a K-contiguous operand starts unaligned: 4100^3 326 / 361, 1234x5678x4321 205 / 256)
@@ -501,7 +501,8 @@ int auto_mfma_splits(const MfmaVariant& v, const Problem& pb, size_t max_floats 
 // 288 / 135.  The best forms have about 256 workgroups with direct fills and about 512 with register-staged ones.
 // Returns the tile edge to choose among (0: the general rule) and the number of workgroups to aim for.
 // (The tile only for a B of 192 MB and more, most of the 256 MB Infinity Cache, out of which a second pass over B costs little; the
-// slices from 64 MB on, whatever tile the general rule takes: 33x11008x4096, 90 MB, 44.5 us on 172 unsplit 64 x 64 tiles, 22.3 in four slices.)
+// slices from 64 MB on -- 16 MB with fewer than 64 rows --, whatever tile the general rule takes: 33x11008x4096, 90 MB, 44.5 us on
+// 172 unsplit 64 x 64 tiles, 22.3 in four slices.)
 bool streamed_b(const Problem& pb, int64_t least_bytes)
 {
     const GemmArgs& g = pb.g;
@@ -680,7 +681,11 @@ int choose(const Problem& pb, int variant, int k_splits, Choice* c, size_t max_s
             SplitPlan sp;
             if (k_splits > 1) c->splits = plan_split(v, pb, k_splits, &sp, max_split_floats) ? sp.splits : 1;
             else if (k_splits == 0) {
-                if (!streamed_splits && streamed_b(pb, (int64_t)64 << 20)) streamed_splits = streamed_b_splits(v, pb, max_split_floats);
+                // (from 64 MB of B on; with fewer than 64 rows, where the tiles with direct fills on short rows come into play and
+                // the general rule never splits more tiles than half the CUs, from 16 MB: 33x4096x4096 17.1 -> 10.8 us in four
+                // slices, 8x11008x2048 with a K-contiguous B 22.8 -> 10.6 on direct fills; with 64 rows and more the smaller
+                // problems keep the general rule's slices -- 64x8192x2048 10.9 us unsplit, 12.7 in two)
+                if (!streamed_splits && streamed_b(pb, (int64_t)(pb.g.M < 64 ? 16 : 64) << 20)) streamed_splits = streamed_b_splits(v, pb, max_split_floats);
                 c->splits = streamed_splits > 1 ? streamed_splits : auto_mfma_splits(v, pb, max_split_floats);
             }
         }

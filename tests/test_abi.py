@@ -195,7 +195,10 @@ def test_choices_of_the_cost_model():
     assert "128x128" in n and "edge" in n and ks == 8
     n, ks = name(_lib.F16, _lib.F16, 8, 11008, 4096, False, True, 1.0, 0.0)            # a decode step against a K-contiguous B
     assert "64x64" in n and "fill=direct" in n and ks == 1
-    assert "edge" in name(_lib.F16, _lib.F16, 8, 4096, 4096, False, True, 1.0, 0.0)[0]  # (32 MB of B: as before)
+    n, ks = name(_lib.F16, _lib.F16, 8, 4096, 4096, False, True, 1.0, 0.0)             # (fewer than 64 rows: from 16 MB of B on)
+    assert "64x64" in n and "fill=direct" in n and ks == 4
+    assert "edge" in name(_lib.F16, _lib.F16, 8, 2048, 2048, False, True, 1.0, 0.0)[0]  # (8 MB of B: as before)
+    assert name(_lib.F16, _lib.F16, 64, 8192, 2048, False, False, 1.0, 0.0)[1] == 1     # (64 rows and 32 MB: the general rule's slices)
     n, ks = name(_lib.BF16, _lib.BF16, 256, 28672, 8192, False, False, 1.0, 0.0)
     assert "256x256" in n and "hand-laid loop" in n and ks == 2
     n, ks = name(_lib.F16, _lib.F16, 256, 32000, 4096, False, False, 1.0, 0.0)
